@@ -1,0 +1,143 @@
+/*
+ * C ABI of libs2cnn_hip.so - the MI355X (gfx950) kernels behind the spectral path
+ * of spherical CNNs.  Plain pointers and sizes only; every pointer is DEVICE memory
+ * unless stated, every tensor is dense fp32, complex numbers are (re, im) pairs.
+ *
+ * The reference has no C interface: its boundary is Python, and each entry point
+ * below replaces one of the run-time compiled CUDA strings (or cuFFT/cuBLAS calls)
+ * behind a reference function, cited per entry as file:line under s2cnn/.
+ *
+ * Conventions
+ *   - return value: 0 on success, a negative S2CNN_E* code for rejected arguments,
+ *     or a positive hipError_t reported by the launch;
+ *   - launches are asynchronous on `stream` (a hipStream_t passed as void*;
+ *     NULL = the default stream); nothing synchronises, nothing allocates;
+ *   - inputs are never written; outputs are fully overwritten;
+ *   - spectral index order is degree-major, then m, then n, with m, n in -l..l:
+ *       SO(3): lmn = l(4l^2-1)/3 + (l+m)(2l+1) + (l+n),  nspec(b) = b(4b^2-1)/3
+ *       S^2  : lm  = l^2 + l + m,                         nspec(b) = b^2
+ *   - grids are [batch, beta, alpha, gamma] (SO(3)) or [batch, beta, alpha] (S^2),
+ *     2b samples per axis.
+ */
+#ifndef S2CNN_HIP_H
+#define S2CNN_HIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define S2CNN_OK 0
+#define S2CNN_EINVAL (-1)      /* a size is out of range or inconsistent              */
+#define S2CNN_EWORKSPACE (-2)  /* workspace pointer NULL or smaller than required     */
+#define S2CNN_EALIGN (-3)      /* a pointer is not aligned to 8 bytes                  */
+
+/* ABI version of this header; bumped when a signature changes. */
+int s2cnn_abi_version(void);
+
+/* Human-readable text for a return code of this library (static storage). */
+const char *s2cnn_strerror(int code);
+
+/* ---- block-diagonal spectral products on SO(3) ------------------------------------
+ * x  [nspec(nl), nbatch, f_in , 2]
+ * y  [nspec(nl), f_in  , f_out, 2]
+ * z  [nspec(nl), nbatch, f_out, 2]
+ *
+ * fwd   : z [l,m,n,i,j] = sum_{p,k} x[l,m,p,i,k] * conj(y[l,n,p,k,j])
+ *         replaces the forward launch of so3_mm.py:66-93 (kernel so3_mm.py:125-261
+ *         with conj_y, trans_y_spec); CPU statement so3_mm.py:31-61.
+ * gradx : gx[l,m,p,i,k] = sum_{n,j} gz[l,m,n,i,j] * y[l,n,p,k,j]
+ *         replaces so3_mm.py:108-113 (trans_y_feature).
+ * grady : gy[l,n,p,k,j] = sum_{m,i} conj(gz[l,m,n,i,j]) * x[l,m,p,i,k]
+ *         replaces so3_mm.py:115-120 (trans_out_feature, conj_x, trans_x_spec,
+ *         trans_x_feature).
+ */
+int s2cnn_so3_mm_fwd(const float *x, const float *y, float *z,
+                     int nl, int nbatch, int f_in, int f_out, void *stream);
+int s2cnn_so3_mm_gradx(const float *gz, const float *y, float *gx,
+                       int nl, int nbatch, int f_in, int f_out, void *stream);
+int s2cnn_so3_mm_grady(const float *gz, const float *x, float *gy,
+                       int nl, int nbatch, int f_in, int f_out, void *stream);
+
+/* ---- S^2 x S^2 -> SO(3) spectral outer products -------------------------------------
+ * x  [nl^2, nbatch, f_in , 2]
+ * y  [nl^2, f_in  , f_out, 2]
+ * z  [nspec_so3(nl), nbatch, f_out, 2]
+ *
+ * fwd   : z [l,m,n,i,j] = sum_k x[l,m,i,k] * conj(y[l,n,k,j])        s2_mm.py:104-198
+ * gradx : gx[l,m,i,k]   = sum_{n,j} gz[l,m,n,i,j] * y[l,n,k,j]       s2_mm.py:201-255
+ * grady : gy[l,n,k,j]   = sum_{m,i} conj(gz[l,m,n,i,j]) * x[l,m,i,k] s2_mm.py:258-312
+ */
+int s2cnn_s2_mm_fwd(const float *x, const float *y, float *z,
+                    int nl, int nbatch, int f_in, int f_out, void *stream);
+int s2cnn_s2_mm_gradx(const float *gz, const float *y, float *gx,
+                      int nl, int nbatch, int f_in, int f_out, void *stream);
+int s2cnn_s2_mm_grady(const float *gz, const float *x, float *gy,
+                      int nl, int nbatch, int f_in, int f_out, void *stream);
+
+/* ---- SO(3) Fourier analysis: grid -> spectrum --------------------------------------
+ * x     [nbatch, 2b_in, 2b_in, 2b_in]      (complex_in = 0)
+ *       [nbatch, 2b_in, 2b_in, 2b_in, 2]   (complex_in = 1)
+ * table [2b_in, nspec(b_out)]  row beta_j, entries scale * d^l_{mn}(beta_j); must satisfy
+ *       table[j, l,-m,-n] = (-1)^(m-n) table[j, l,m,n] (true of Wigner small-d)
+ * out   [nspec(b_out), nbatch, 2]
+ *       out[l,m,n,z] = sum_beta table[beta,lmn] sum_{alpha,gamma} x[z,beta,alpha,gamma]
+ *                      exp(-i(m alpha + n gamma)),   0 where |m| or |n| >= b_in
+ * Replaces cuFFT + the kernel at soft/so3_fft.py:247-350 behind so3_rfft (so3_fft.py:64-112)
+ * and so3_fft (so3_fft.py:12-61).
+ * workspace: s2cnn_so3_analysis_workspace(...) bytes of device scratch, 256-byte aligned.
+ */
+size_t s2cnn_so3_analysis_workspace(int b_in, int b_out, long nbatch, int complex_in);
+int s2cnn_so3_analysis(const float *x, const float *table, float *out,
+                       void *workspace, size_t workspace_bytes,
+                       int b_in, int b_out, long nbatch, int complex_in, void *stream);
+
+/* ---- SO(3) Fourier synthesis: spectrum -> grid -------------------------------------
+ * xhat  [nspec(b_in), nbatch, 2]
+ * table [2b_out, nspec(b_in)]   (same symmetry requirement as above)
+ * out   [nbatch, 2b_out, 2b_out, 2b_out]     (complex_out = 0): the REAL PART of
+ *       [nbatch, 2b_out, 2b_out, 2b_out, 2]  (complex_out = 1):
+ *       y[z,beta,alpha,gamma] = sum_{l < min(b_in,b_out)} sum_{m,n} xhat[l,m,n,z]
+ *                               table[beta,lmn] exp(+i(m alpha + n gamma))
+ * (no symmetry of xhat is assumed in either mode).
+ * Replaces the kernel at soft/so3_fft.py:353-443 + cuFFT behind so3_rifft
+ * (so3_fft.py:158-202, CPU-branch semantics) and so3_ifft (so3_fft.py:115-155).
+ */
+size_t s2cnn_so3_synthesis_workspace(int b_in, int b_out, long nbatch, int complex_out);
+int s2cnn_so3_synthesis(const float *xhat, const float *table, float *out,
+                        void *workspace, size_t workspace_bytes,
+                        int b_in, int b_out, long nbatch, int complex_out, void *stream);
+
+/* ---- S^2 Fourier analysis / synthesis ----------------------------------------------
+ * analysis : x [nbatch, 2b_in, 2b_in] (complex_in = 0) or [..., 2] (complex_in = 1),
+ *            table [2b_in, b_out^2] (entries scale * d^l_{m0}), b_out <= b_in,
+ *            out [b_out^2, nbatch, 2]:
+ *            out[l,m,z] = sum_beta table[beta,lm] sum_alpha x[z,beta,alpha] exp(-i m alpha)
+ *            replaces cuFFT + soft/s2_fft.py:150-185 behind s2_fft (s2_fft.py:13-58).
+ * synthesis: xhat [b_in^2, nbatch, 2], table [2b_out, b_in^2], b_out >= b_in,
+ *            out [nbatch, 2b_out, 2b_out] (real part, complex_out = 0) or [..., 2]:
+ *            y[z,beta,alpha] = sum_{l,m} xhat[l,m,z] table[beta,lm] exp(+i m alpha)
+ *            replaces soft/s2_fft.py:188-223 + cuFFT behind s2_ifft (s2_fft.py:61-106).
+ */
+size_t s2cnn_s2_analysis_workspace(int b_in, int b_out, long nbatch, int complex_in);
+int s2cnn_s2_analysis(const float *x, const float *table, float *out,
+                      void *workspace, size_t workspace_bytes,
+                      int b_in, int b_out, long nbatch, int complex_in, void *stream);
+size_t s2cnn_s2_synthesis_workspace(int b_in, int b_out, long nbatch, int complex_out);
+int s2cnn_s2_synthesis(const float *xhat, const float *table, float *out,
+                       void *workspace, size_t workspace_bytes,
+                       int b_in, int b_out, long nbatch, int complex_out, void *stream);
+
+/* ---- Haar integral over SO(3) -------------------------------------------------------
+ * x [n, 2b, 2b, 2b], w [2b] -> out [n]:  out[z] = sum_beta w[beta] sum_{alpha,gamma} x[z,...]
+ * replaces the two torch.sum + torch.mm of soft/so3_integrate.py:21-27.
+ * grad : gx[z,beta,alpha,gamma] = g[z] * w[beta]   (its adjoint)
+ */
+int s2cnn_so3_integrate(const float *x, const float *w, float *out, int b, long n, void *stream);
+int s2cnn_so3_integrate_grad(const float *g, const float *w, float *gx, int b, long n, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* S2CNN_HIP_H */

@@ -1,0 +1,82 @@
+"""ctypes binding of libs2cnn_hip.so (the C ABI declared in include/s2cnn_hip.h).
+
+There is no CPU fallback: if the library is not built, or a tensor is not a
+float32 tensor on a GPU, the call raises.  Takes the place of the run-time
+kernel compiler of the reference (s2cnn/utils/cuda.py:19-27).
+"""
+import ctypes
+import os
+from functools import lru_cache
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "csrc", "libs2cnn_hip.so")
+
+_c_float_p = ctypes.c_void_p
+_int, _long, _size_t, _vp = ctypes.c_int, ctypes.c_long, ctypes.c_size_t, ctypes.c_void_p
+
+_MM_SIG = [_c_float_p, _c_float_p, _c_float_p, _int, _int, _int, _int, _vp]
+_FT_SIG = [_c_float_p, _c_float_p, _c_float_p, _vp, _size_t, _int, _int, _long, _int, _vp]
+_WS_SIG = [_int, _int, _long, _int]
+
+SIGNATURES = {
+    "s2cnn_abi_version": (_int, []),
+    "s2cnn_strerror": (ctypes.c_char_p, [_int]),
+    "s2cnn_so3_mm_fwd": (_int, _MM_SIG),
+    "s2cnn_so3_mm_gradx": (_int, _MM_SIG),
+    "s2cnn_so3_mm_grady": (_int, _MM_SIG),
+    "s2cnn_s2_mm_fwd": (_int, _MM_SIG),
+    "s2cnn_s2_mm_gradx": (_int, _MM_SIG),
+    "s2cnn_s2_mm_grady": (_int, _MM_SIG),
+    "s2cnn_so3_analysis_workspace": (_size_t, _WS_SIG),
+    "s2cnn_so3_analysis": (_int, _FT_SIG),
+    "s2cnn_so3_synthesis_workspace": (_size_t, _WS_SIG),
+    "s2cnn_so3_synthesis": (_int, _FT_SIG),
+    "s2cnn_s2_analysis_workspace": (_size_t, _WS_SIG),
+    "s2cnn_s2_analysis": (_int, _FT_SIG),
+    "s2cnn_s2_synthesis_workspace": (_size_t, _WS_SIG),
+    "s2cnn_s2_synthesis": (_int, _FT_SIG),
+    "s2cnn_so3_integrate": (_int, [_c_float_p, _c_float_p, _c_float_p, _int, _long, _vp]),
+    "s2cnn_so3_integrate_grad": (_int, [_c_float_p, _c_float_p, _c_float_p, _int, _long, _vp]),
+}
+
+
+@lru_cache(maxsize=1)
+def lib():
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            "libs2cnn_hip.so is not built (%s); run `python -m s2cnn_amd.csrc.build`. "
+            "There is no CPU fallback." % LIB_PATH)
+    handle = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(handle, name)
+        fn.restype = res
+        fn.argtypes = args
+    return handle
+
+
+def check(code):
+    if code != 0:
+        raise RuntimeError("libs2cnn_hip: %s (code %d)" % (lib().s2cnn_strerror(code).decode(), code))
+
+
+def require_gpu_f32(*tensors):
+    for t in tensors:
+        if not (t.is_cuda and t.dtype == torch.float32):
+            raise RuntimeError(
+                "s2cnn_amd runs float32 tensors on the GPU only (got %s on %s); there is no CPU path"
+                % (t.dtype, t.device))
+
+
+def stream_ptr():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def ptr(t):
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def workspace(nbytes, device):
+    """Scratch from torch's caching allocator (stream-ordered, so reuse after the call is safe)."""
+    return torch.empty(max(int(nbytes), 8), dtype=torch.uint8, device=device)

@@ -1,0 +1,361 @@
+// SO(3) Fourier analysis and synthesis on the SOFT grid.
+//
+// Analysis   out[l,m,n,z]  = sum_beta T[beta,lmn] * X[z,beta,m,n],
+//            X[z,beta,m,n] = sum_{alpha,gamma} x[z,beta,alpha,gamma] e^{-i(m alpha + n gamma)}
+// Synthesis  y[z,beta,alpha,gamma] = sum_{m,n} e^{+i(m alpha + n gamma)} S[z,beta,m,n],
+//            S[z,beta,m,n] = sum_l T[beta,lmn] * xhat[l,m,n,z]
+//
+// Only frequencies |m|,|n| < nb = min(b_in, b_out) are ever consumed, so the (alpha,gamma)
+// transform is a DFT pruned to those bins, done per (z,beta) plane inside LDS, and the
+// intermediate X / S lives in a workspace laid out [z][beta][m][n] (n fastest).
+//
+// Real signals use the half plane n >= 0:
+//   analysis : the other half follows from X[-m,-n] = conj X[m,n] and
+//              T[l,-m,-n] = (-1)^(m-n) T[l,m,n]  =>  out[l,-m,-n] = (-1)^(m-n) conj out[l,m,n];
+//   synthesis: Re sum_{m,n} e^{i.}S[m,n] = sum_{m,n} e^{i.}G[m,n] with the Hermitian
+//              G[m,n] = (S[m,n] + conj S[-m,-n])/2, and by the same table symmetry
+//              G = sum_l T[l,m,n] (xhat[l,m,n] + (-1)^(m-n) conj xhat[l,-m,-n])/2,
+//              so the spectrum is symmetrised on load and no symmetry of xhat is assumed.
+#include "common.h"
+
+namespace {
+
+constexpr float kTwoPi = 6.283185307179586476925286766559f;
+
+__device__ inline float2 cmul(float2 a, float2 b) { return make_float2(a.x * b.x - a.y * b.y, a.x * b.y + a.y * b.x); }
+__device__ inline float2 cmul_conj(float2 a, float2 b) { return make_float2(a.x * b.x + a.y * b.y, a.y * b.x - a.x * b.y); }  // a*conj(b)
+
+__device__ inline int lmn_index(int l, int m, int n) { return l * (4 * l * l - 1) / 3 + (l + m) * (2 * l + 1) + (l + n); }
+
+// w[k] = e^{-2 pi i k / n2}
+__device__ inline void fill_twiddles(float2* w, int n2) {
+  for (int k = threadIdx.x; k < n2; k += blockDim.x) {
+    float s, c;
+    sincospif(2.0f * (float)k / (float)n2, &s, &c);
+    w[k] = make_float2(c, -s);
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// analysis stage 1: one workgroup per (z,beta) plane
+//   x plane [n2][n2] (real or complex) -> X[mi][ni], mi = m + nb-1, ni = n (real) or n + nb-1
+// LDS: twiddles n2 | plane n2*n2 (float or float2) | Y n2*NW
+// ---------------------------------------------------------------------------------------
+template <bool CPLX>
+__global__ __launch_bounds__(256) void so3_plane_dft_fwd(const float* __restrict__ x, float2* __restrict__ X,
+                                                         int n2, int nb) {
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  const int MW = 2 * nb - 1;
+  const int NW = CPLX ? MW : nb;
+  float2* w = reinterpret_cast<float2*>(smem);
+  float* plane = smem + 2 * n2;
+  float2* Y = reinterpret_cast<float2*>(plane + (CPLX ? 2 : 1) * n2 * n2);
+  const size_t pl = blockIdx.x;
+
+  fill_twiddles(w, n2);
+  const int nin = (CPLX ? 2 : 1) * n2 * n2;
+  const float* src = x + pl * nin;
+  for (int i = threadIdx.x; i < nin; i += blockDim.x) plane[i] = src[i];
+  __syncthreads();
+
+  // Y[alpha][ni] = sum_gamma x[alpha][gamma] w^(n gamma)
+  for (int o = threadIdx.x; o < n2 * NW; o += blockDim.x) {
+    const int a = o / NW, ni = o - a * NW;
+    const int n = CPLX ? ni - (nb - 1) : ni;
+    const int step = ((n % n2) + n2) % n2;
+    int tw = 0;
+    float2 acc = make_float2(0.f, 0.f);
+    for (int g = 0; g < n2; ++g) {
+      const float2 t = w[tw];
+      if (CPLX) {
+        const float2 v = reinterpret_cast<const float2*>(plane)[a * n2 + g];
+        const float2 pr = cmul(v, t);
+        acc.x += pr.x; acc.y += pr.y;
+      } else {
+        const float v = plane[a * n2 + g];
+        acc.x += v * t.x; acc.y += v * t.y;
+      }
+      tw += step; if (tw >= n2) tw -= n2;
+    }
+    Y[o] = acc;
+  }
+  __syncthreads();
+
+  // X[mi][ni] = sum_alpha Y[alpha][ni] w^(m alpha)
+  float2* dst = X + pl * (size_t)(MW * NW);
+  for (int o = threadIdx.x; o < MW * NW; o += blockDim.x) {
+    const int mi = o / NW, ni = o - mi * NW;
+    const int m = mi - (nb - 1);
+    const int step = ((m % n2) + n2) % n2;
+    int tw = 0;
+    float2 acc = make_float2(0.f, 0.f);
+    for (int a = 0; a < n2; ++a) {
+      const float2 pr = cmul(Y[a * NW + ni], w[tw]);
+      acc.x += pr.x; acc.y += pr.y;
+      tw += step; if (tw >= n2) tw -= n2;
+    }
+    dst[o] = acc;
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// analysis stage 2: contraction over beta with the Wigner table.
+// block (16 ni, 16 z); grid (ceil(NW/16), MW, ceil(nbatch/16))
+// ---------------------------------------------------------------------------------------
+constexpr int LG = 8;  // degrees accumulated per pass over beta
+
+template <bool CPLX>
+__global__ __launch_bounds__(256) void so3_wigner_fwd(const float2* __restrict__ X, const float* __restrict__ T,
+                                                      float2* __restrict__ out, int n2, int nb, int b_out,
+                                                      long nbatch) {
+  const int MW = 2 * nb - 1;
+  const int NW = CPLX ? MW : nb;
+  const int ni = blockIdx.x * 16 + threadIdx.x;
+  const int mi = blockIdx.y;
+  const long z = (long)blockIdx.z * 16 + threadIdx.y;
+  if (ni >= NW || z >= nbatch) return;
+  const int m = mi - (nb - 1);
+  const int n = CPLX ? ni - (nb - 1) : ni;
+  if (!CPLX && n == 0 && m < 0) return;  // written as the mirror of (-m, 0)
+  const int lmin = max(abs(m), abs(n));
+  const long nspec = (long)b_out * (4L * b_out * b_out - 1) / 3;
+  const float2* xp = X + ((size_t)z * n2 * MW + mi) * NW + ni;  // + beta * MW*NW
+  const size_t xstride = (size_t)MW * NW;
+  const float sgn = ((m - n) & 1) ? -1.f : 1.f;
+
+  for (int l0 = lmin; l0 < b_out; l0 += LG) {
+    float2 acc[LG];
+    int idx[LG];
+#pragma unroll
+    for (int u = 0; u < LG; ++u) {
+      acc[u] = make_float2(0.f, 0.f);
+      const int l = min(l0 + u, b_out - 1);
+      idx[u] = lmn_index(l, m, n);
+    }
+    for (int bt = 0; bt < n2; ++bt) {
+      const float2 v = xp[bt * xstride];
+      const float* Tr = T + (size_t)bt * nspec;
+#pragma unroll
+      for (int u = 0; u < LG; ++u) {
+        const float t = Tr[idx[u]];
+        acc[u].x += t * v.x; acc[u].y += t * v.y;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < LG; ++u) {
+      const int l = l0 + u;
+      if (l < b_out) {
+        out[(size_t)idx[u] * nbatch + z] = acc[u];
+        if (!CPLX && (n > 0 || m > 0))
+          out[(size_t)lmn_index(l, -m, -n) * nbatch + z] = make_float2(sgn * acc[u].x, -sgn * acc[u].y);
+      }
+    }
+  }
+}
+
+__global__ void fill_zero(float* p, size_t n) {
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = 0.f;
+}
+
+// ---------------------------------------------------------------------------------------
+// synthesis stage 1: S[z][beta][mi][ni] = sum_l T[beta,lmn] xs[lmn][z]
+// block (16 ni, 16 z); grid (ceil(NW/16), MW, ceil(nbatch/16))
+// ---------------------------------------------------------------------------------------
+constexpr int BG = 8;  // betas accumulated per pass over l
+
+template <bool CPLX>
+__global__ __launch_bounds__(256) void so3_wigner_inv(const float2* __restrict__ xh, const float* __restrict__ T,
+                                                      float2* __restrict__ S, int n2, int nb, int b_spec,
+                                                      long nbatch) {
+  const int MW = 2 * nb - 1;
+  const int NW = CPLX ? MW : nb;
+  const int ni = blockIdx.x * 16 + threadIdx.x;
+  const int mi = blockIdx.y;
+  const long z = (long)blockIdx.z * 16 + threadIdx.y;
+  if (ni >= NW || z >= nbatch) return;
+  const int m = mi - (nb - 1);
+  const int n = CPLX ? ni - (nb - 1) : ni;
+  const int lmin = max(abs(m), abs(n));
+  const long nspec = (long)b_spec * (4L * b_spec * b_spec - 1) / 3;
+  float2* sp = S + ((size_t)z * n2 * MW + mi) * NW + ni;
+  const size_t sstride = (size_t)MW * NW;
+  const float sgn = ((m - n) & 1) ? -0.5f : 0.5f;
+
+  for (int b0 = 0; b0 < n2; b0 += BG) {
+    float2 acc[BG];
+#pragma unroll
+    for (int u = 0; u < BG; ++u) acc[u] = make_float2(0.f, 0.f);
+    for (int l = lmin; l < nb; ++l) {
+      const int i1 = lmn_index(l, m, n);
+      float2 v = xh[(size_t)i1 * nbatch + z];
+      if (!CPLX) {
+        const float2 u2 = xh[(size_t)lmn_index(l, -m, -n) * nbatch + z];
+        v = make_float2(0.5f * v.x + sgn * u2.x, 0.5f * v.y - sgn * u2.y);
+      }
+#pragma unroll
+      for (int u = 0; u < BG; ++u) {
+        const int bt = min(b0 + u, n2 - 1);
+        const float t = T[(size_t)bt * nspec + i1];
+        acc[u].x += t * v.x; acc[u].y += t * v.y;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < BG; ++u)
+      if (b0 + u < n2) sp[(size_t)(b0 + u) * sstride] = acc[u];
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// synthesis stage 2: one workgroup per (z,beta) plane, S[mi][ni] -> y[alpha][gamma]
+// LDS: twiddles n2 | S MW*NW | U n2*NW
+// ---------------------------------------------------------------------------------------
+template <bool CPLX>
+__global__ __launch_bounds__(256) void so3_plane_dft_inv(const float2* __restrict__ S, float* __restrict__ y,
+                                                         int n2, int nb) {
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  const int MW = 2 * nb - 1;
+  const int NW = CPLX ? MW : nb;
+  float2* w = reinterpret_cast<float2*>(smem);
+  float2* Sp = w + n2;
+  float2* U = Sp + MW * NW;
+  const size_t pl = blockIdx.x;
+
+  fill_twiddles(w, n2);
+  const float2* src = S + pl * (size_t)(MW * NW);
+  for (int i = threadIdx.x; i < MW * NW; i += blockDim.x) Sp[i] = src[i];
+  __syncthreads();
+
+  // U[alpha][ni] = sum_mi S[mi][ni] conj(w)^(m alpha)
+  for (int o = threadIdx.x; o < n2 * NW; o += blockDim.x) {
+    const int a = o / NW, ni = o - a * NW;
+    const int step = a;                                  // m -> m+1 advances the phase by alpha
+    int tw = (int)(((long)(-(nb - 1)) * a) % n2); if (tw < 0) tw += n2;
+    float2 acc = make_float2(0.f, 0.f);
+    for (int mi = 0; mi < MW; ++mi) {
+      const float2 pr = cmul_conj(Sp[mi * NW + ni], w[tw]);
+      acc.x += pr.x; acc.y += pr.y;
+      tw += step; if (tw >= n2) tw -= n2;
+    }
+    U[o] = acc;
+  }
+  __syncthreads();
+
+  if (CPLX) {
+    float2* dst = reinterpret_cast<float2*>(y) + pl * (size_t)(n2 * n2);
+    for (int o = threadIdx.x; o < n2 * n2; o += blockDim.x) {
+      const int a = o / n2, g = o - a * n2;
+      int tw = (int)(((long)(-(nb - 1)) * g) % n2); if (tw < 0) tw += n2;
+      float2 acc = make_float2(0.f, 0.f);
+      for (int ni = 0; ni < NW; ++ni) {
+        const float2 pr = cmul_conj(U[a * NW + ni], w[tw]);
+        acc.x += pr.x; acc.y += pr.y;
+        tw += g; if (tw >= n2) tw -= n2;
+      }
+      dst[o] = acc;
+    }
+  } else {
+    float* dst = y + pl * (size_t)(n2 * n2);
+    for (int o = threadIdx.x; o < n2 * n2; o += blockDim.x) {
+      const int a = o / n2, g = o - a * n2;
+      float acc = U[a * NW].x;
+      int tw = g;
+      float part = 0.f;
+      for (int ni = 1; ni < NW; ++ni) {
+        const float2 u = U[a * NW + ni];
+        const float2 t = w[tw];                          // conj(t) = e^{+i n gamma}
+        part += u.x * t.x + u.y * t.y;                  // Re(u * conj(t))
+        tw += g; if (tw >= n2) tw -= n2;
+      }
+      dst[o] = acc + 2.f * part;
+    }
+  }
+}
+
+size_t ws_bytes(int b_grid, int b_spec, long nbatch, int cplx) {
+  if (b_grid < 1 || b_spec < 1 || nbatch < 1) return 0;
+  const long nb = b_grid < b_spec ? b_grid : b_spec;
+  const long MW = 2 * nb - 1, NW = cplx ? MW : nb;
+  return (size_t)nbatch * (2 * b_grid) * MW * NW * sizeof(float2);
+}
+
+bool sizes_ok(int b_grid, int b_spec, long nbatch) {
+  return b_grid >= 1 && b_spec >= 1 && nbatch >= 1 && b_grid <= 512 && b_spec <= 512 &&
+         nbatch * 2L * b_grid < (1L << 31) && (nbatch + 15) / 16 <= 65535;
+}
+
+}  // namespace
+
+extern "C" size_t s2cnn_so3_analysis_workspace(int b_in, int b_out, long nbatch, int complex_in) {
+  return ws_bytes(b_in, b_out, nbatch, complex_in);
+}
+
+extern "C" size_t s2cnn_so3_synthesis_workspace(int b_in, int b_out, long nbatch, int complex_out) {
+  return ws_bytes(b_out, b_in, nbatch, complex_out);
+}
+
+extern "C" int s2cnn_so3_analysis(const float* x, const float* table, float* out, void* workspace,
+                                  size_t workspace_bytes, int b_in, int b_out, long nbatch, int complex_in,
+                                  void* stream) {
+  if (!x || !table || !out || !sizes_ok(b_in, b_out, nbatch)) return S2CNN_EINVAL;
+  if (!s2cnn::aligned8(out) || (complex_in && !s2cnn::aligned8(x))) return S2CNN_EALIGN;
+  const size_t need = ws_bytes(b_in, b_out, nbatch, complex_in);
+  if (!workspace || workspace_bytes < need || !s2cnn::aligned8(workspace)) return S2CNN_EWORKSPACE;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int n2 = 2 * b_in, nb = b_in < b_out ? b_in : b_out;
+  const int MW = 2 * nb - 1, NW = complex_in ? MW : nb;
+  float2* X = static_cast<float2*>(workspace);
+  const size_t lds = sizeof(float) * (2 * n2 + (complex_in ? 2 : 1) * n2 * n2 + 2 * n2 * NW);
+  if (lds > 160 * 1024) return S2CNN_EINVAL;
+  const unsigned planes = (unsigned)(nbatch * n2);
+  if (complex_in) {
+    if (lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)so3_plane_dft_fwd<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipLaunchKernelGGL(so3_plane_dft_fwd<true>, dim3(planes), dim3(256), lds, st, x, X, n2, nb);
+  } else {
+    if (lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)so3_plane_dft_fwd<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipLaunchKernelGGL(so3_plane_dft_fwd<false>, dim3(planes), dim3(256), lds, st, x, X, n2, nb);
+  }
+  int rc = s2cnn::launch_status();
+  if (rc) return rc;
+  if (b_out > b_in) {  // entries with |m| or |n| >= b_in are never touched by stage 2
+    const size_t nfl = (size_t)s2cnn::so3_nspec(b_out) * nbatch * 2;
+    hipLaunchKernelGGL(fill_zero, dim3(1024), dim3(256), 0, st, out, nfl);
+  }
+  dim3 grid(s2cnn::ceil_div(NW, 16), MW, (unsigned)((nbatch + 15) / 16));
+  if (complex_in)
+    hipLaunchKernelGGL(so3_wigner_fwd<true>, grid, dim3(16, 16), 0, st, X, table, reinterpret_cast<float2*>(out), n2, nb, b_out, nbatch);
+  else
+    hipLaunchKernelGGL(so3_wigner_fwd<false>, grid, dim3(16, 16), 0, st, X, table, reinterpret_cast<float2*>(out), n2, nb, b_out, nbatch);
+  return s2cnn::launch_status();
+}
+
+extern "C" int s2cnn_so3_synthesis(const float* xhat, const float* table, float* out, void* workspace,
+                                   size_t workspace_bytes, int b_in, int b_out, long nbatch, int complex_out,
+                                   void* stream) {
+  if (!xhat || !table || !out || !sizes_ok(b_out, b_in, nbatch)) return S2CNN_EINVAL;
+  if (!s2cnn::aligned8(xhat) || (complex_out && !s2cnn::aligned8(out))) return S2CNN_EALIGN;
+  const size_t need = ws_bytes(b_out, b_in, nbatch, complex_out);
+  if (!workspace || workspace_bytes < need || !s2cnn::aligned8(workspace)) return S2CNN_EWORKSPACE;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int n2 = 2 * b_out, nb = b_in < b_out ? b_in : b_out;
+  const int MW = 2 * nb - 1, NW = complex_out ? MW : nb;
+  float2* S = static_cast<float2*>(workspace);
+  const size_t lds = sizeof(float2) * (n2 + MW * NW + n2 * NW);
+  if (lds > 160 * 1024) return S2CNN_EINVAL;
+  dim3 grid(s2cnn::ceil_div(NW, 16), MW, (unsigned)((nbatch + 15) / 16));
+  const float2* xh = reinterpret_cast<const float2*>(xhat);
+  if (complex_out)
+    hipLaunchKernelGGL(so3_wigner_inv<true>, grid, dim3(16, 16), 0, st, xh, table, S, n2, nb, b_in, nbatch);
+  else
+    hipLaunchKernelGGL(so3_wigner_inv<false>, grid, dim3(16, 16), 0, st, xh, table, S, n2, nb, b_in, nbatch);
+  int rc = s2cnn::launch_status();
+  if (rc) return rc;
+  const unsigned planes = (unsigned)(nbatch * n2);
+  if (complex_out) {
+    if (lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)so3_plane_dft_inv<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipLaunchKernelGGL(so3_plane_dft_inv<true>, dim3(planes), dim3(256), lds, st, S, out, n2, nb);
+  } else {
+    if (lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)so3_plane_dft_inv<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipLaunchKernelGGL(so3_plane_dft_inv<false>, dim3(planes), dim3(256), lds, st, S, out, n2, nb);
+  }
+  return s2cnn::launch_status();
+}

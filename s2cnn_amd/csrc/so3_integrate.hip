@@ -1,0 +1,64 @@
+// Haar integral over SO(3) on the SOFT grid and its adjoint:
+//   out[z] = sum_beta w[beta] sum_{alpha,gamma} x[z,beta,alpha,gamma]
+//   gx[z,beta,alpha,gamma] = g[z] w[beta]
+// A pure read-reduce (write-broadcast) pass: one workgroup per volume.
+#include "common.h"
+
+namespace {
+
+__global__ __launch_bounds__(256) void so3_integrate_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                            float* __restrict__ out, int n2) {
+  __shared__ float part[256];
+  const size_t plane = (size_t)n2 * n2;
+  const float* xs = x + blockIdx.x * plane * n2;
+  float acc = 0.f;
+  for (int bt = 0; bt < n2; ++bt) {
+    float s = 0.f;
+    for (size_t i = threadIdx.x; i < plane; i += blockDim.x) s += xs[bt * plane + i];
+    acc += w[bt] * s;
+  }
+  part[threadIdx.x] = acc;
+  __syncthreads();
+  for (int s = 128; s > 0; s >>= 1) {
+    if ((int)threadIdx.x < s) part[threadIdx.x] += part[threadIdx.x + s];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) out[blockIdx.x] = part[0];
+}
+
+__global__ __launch_bounds__(256) void so3_integrate_grad_kernel(const float* __restrict__ g, const float* __restrict__ w,
+                                                                 float* __restrict__ gx, int n2) {
+  const size_t plane = (size_t)n2 * n2;
+  float* dst = gx + blockIdx.x * plane * n2;
+  const float gv = g[blockIdx.x];
+  for (int bt = 0; bt < n2; ++bt) {
+    const float v = gv * w[bt];
+    for (size_t i = threadIdx.x; i < plane; i += blockDim.x) dst[bt * plane + i] = v;
+  }
+}
+
+}  // namespace
+
+extern "C" int s2cnn_so3_integrate(const float* x, const float* w, float* out, int b, long n, void* stream) {
+  if (!x || !w || !out || b < 1 || b > 1024 || n < 1 || n >= (1L << 31)) return S2CNN_EINVAL;
+  hipLaunchKernelGGL(so3_integrate_kernel, dim3((unsigned)n), dim3(256), 0, static_cast<hipStream_t>(stream), x, w, out, 2 * b);
+  return s2cnn::launch_status();
+}
+
+extern "C" int s2cnn_so3_integrate_grad(const float* g, const float* w, float* gx, int b, long n, void* stream) {
+  if (!g || !w || !gx || b < 1 || b > 1024 || n < 1 || n >= (1L << 31)) return S2CNN_EINVAL;
+  hipLaunchKernelGGL(so3_integrate_grad_kernel, dim3((unsigned)n), dim3(256), 0, static_cast<hipStream_t>(stream), g, w, gx, 2 * b);
+  return s2cnn::launch_status();
+}
+
+extern "C" int s2cnn_abi_version(void) { return 1; }
+
+extern "C" const char* s2cnn_strerror(int code) {
+  switch (code) {
+    case S2CNN_OK: return "ok";
+    case S2CNN_EINVAL: return "a size is out of range or inconsistent, or a pointer is NULL";
+    case S2CNN_EWORKSPACE: return "workspace is NULL, misaligned or smaller than the *_workspace() size";
+    case S2CNN_EALIGN: return "a complex tensor is not aligned to 8 bytes";
+    default: return code > 0 ? hipGetErrorString(static_cast<hipError_t>(code)) : "unknown s2cnn error";
+  }
+}

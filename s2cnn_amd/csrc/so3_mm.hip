@@ -1,0 +1,312 @@
+// Block-diagonal complex products over the (2l+1)x(2l+1) blocks of an SO(3) spectrum,
+// on the fp32 matrix cores of gfx950 (v_mfma_f32_32x32x2_f32).
+//
+// For one degree l (L = 2l+1) each of the three products is a complex GEMM whose three
+// index spaces are pairs (spectral index, feature index):
+//
+//   fwd   : Z[(m,i),(n,j)] = sum_{(p,k)} X [(m,i),(p,k)] * conj(Y[(p,k),(n,j)])
+//   gradx : GX[(m,i),(p,k)] = sum_{(n,j)} GZ[(m,i),(n,j)] *      Y[(n,j),(p,k)]
+//   grady : GY[(p,k),(n,j)] = sum_{(m,i)} X [(p,k),(m,i)] * conj(GZ[(m,i),(n,j)])
+//
+// with tensors stored as [l, spectral row, spectral col, feature row, feature col, 2].
+// An operand is therefore an L x L grid of dense feature blocks; within a block either the
+// contraction index ("K-contiguous") or the free index ("MN-contiguous") is the fast one.
+// The kernel keeps each operand tile in LDS in the orientation it has in memory, so loads
+// from HBM are coalesced and nothing is transposed on the way.
+//
+// Complex arithmetic on a real matrix core: one MFMA 32x32x2 takes two contraction steps,
+// one per half-wave.  The lower half is fed the real parts and the upper half the
+// imaginary parts of the same complex column, so that with b' = (br, bi) the instruction
+// accumulates ar*br + ai*bi (the real part of a*conj(b)), and with b'' = (-bi, br) the
+// imaginary part; without conjugation b' = (br, -bi), b'' = (bi, br).  Four real MACs per
+// complex MAC - the algorithmic minimum - and the A operand register is shared by both.
+#include <type_traits>
+#include "common.h"
+
+namespace {
+
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int TM = 128;           // tile rows   (flattened (spectral, feature) index)
+constexpr int TN = 128;           // tile cols
+constexpr int TK = 16;            // complex contraction steps per LDS stage
+constexpr int NT = 256;           // threads: 4 waves, each a 64x64 complex sub-tile
+constexpr int KC_LD = TK + 2;     // leading dim (complex) of a K-contiguous LDS tile: 144 B rows
+constexpr int MN_LD = 128;        // leading dim of an MN-contiguous LDS tile
+constexpr int TILE_ELEMS = (TM * KC_LD > TK * MN_LD) ? TM * KC_LD : TK * MN_LD;
+
+enum Mode { FWD = 0, GRADX = 1, GRADY = 2 };
+
+struct MmParams {
+  const float2* A;
+  const float2* B;
+  float2* C;
+  int nl;
+  int RI;  // feature rows per block of C (and of A)
+  int CI;  // feature cols per block of C (and of B)
+  int KI;  // contraction features per block
+};
+
+template <int MODE> struct Cfg;
+// A block (rb,kb) at rb*L+kb (MNMAJOR) or kb*L+rb; same for B with (cb,kb); C (rb,cb) at rb*L+cb or cb*L+rb.
+template <> struct Cfg<FWD>   { static constexpr bool A_KC = true,  B_KC = false, A_MNMAJ = true,  B_MNMAJ = true,  C_RMAJ = true,  CONJ = true;  };
+template <> struct Cfg<GRADX> { static constexpr bool A_KC = true,  B_KC = true,  A_MNMAJ = true,  B_MNMAJ = false, C_RMAJ = true,  CONJ = false; };
+template <> struct Cfg<GRADY> { static constexpr bool A_KC = false, B_KC = false, A_MNMAJ = false, B_MNMAJ = false, C_RMAJ = false, CONJ = true;  };
+
+// One operand's tile loader: global -> registers -> LDS.  VEC = complex numbers per access.
+template <bool KC, bool MNMAJ, int VEC>
+struct TileLoader {
+  static constexpr int NSLOT = TM * TK / (NT * VEC);
+  typedef typename std::conditional<VEC == 2, float4, float2>::type vec_t;
+
+  const float2* base;   // start of degree l
+  int off[KC ? NSLOT : 1];
+  unsigned valid_mn;    // bit q: slot q's row is inside the matrix (KC) / bit 0 (MN-contiguous)
+  int kk;               // KC: this thread's k inside the stage; else k of slot 0
+  int lds_off;          // LDS offset (complex) of slot 0
+  int blk_k_stride;     // elements between consecutive contraction blocks
+  int MNI, KI;
+  vec_t reg[NSLOT];
+
+  __device__ void init(const float2* base_l, int L, int MNI_, int KI_, int tile0) {
+    base = base_l; MNI = MNI_; KI = KI_;
+    const int t = threadIdx.x;
+    const int blk_elems = MNI * KI;
+    const int blk_mn_stride = (MNMAJ ? L : 1) * blk_elems;
+    blk_k_stride = (MNMAJ ? 1 : L) * blk_elems;
+    valid_mn = 0;
+    if (KC) {
+      constexpr int TPR = TK / VEC;          // threads per tile row
+      kk = (t % TPR) * VEC;
+      const int r0 = t / TPR;
+      lds_off = r0 * KC_LD + kk;
+#pragma unroll
+      for (int q = 0; q < NSLOT; ++q) {
+        const int row = tile0 + r0 + q * (NT / TPR);
+        const int mb = row / MNI, mi = row - mb * MNI;
+        off[q] = mb * blk_mn_stride + mi * KI + kk;
+        if (row < L * MNI) valid_mn |= 1u << q;
+      }
+    } else {
+      constexpr int TPR = TM / VEC;          // threads per k-row of the tile
+      const int mn = tile0 + (t % TPR) * VEC;
+      kk = t / TPR;
+      lds_off = kk * MN_LD + (t % TPR) * VEC;
+      const int mb = mn / MNI, mi = mn - mb * MNI;
+      off[0] = mb * blk_mn_stride + mi;
+      if (mn < L * MNI) valid_mn = 1u;
+    }
+  }
+
+  __device__ void load(int kb, int k0) {
+    const float2* p = base + (size_t)kb * blk_k_stride;
+    if (KC) {
+      const bool kvalid = (k0 + kk) < KI;
+#pragma unroll
+      for (int q = 0; q < NSLOT; ++q) {
+        vec_t v = {};
+        if (kvalid && ((valid_mn >> q) & 1u)) v = *reinterpret_cast<const vec_t*>(p + off[q] + k0);
+        reg[q] = v;
+      }
+    } else {
+      constexpr int KSTEP = NT * VEC / TM;
+#pragma unroll
+      for (int q = 0; q < NSLOT; ++q) {
+        const int k = k0 + kk + q * KSTEP;
+        vec_t v = {};
+        if (valid_mn && k < KI) v = *reinterpret_cast<const vec_t*>(p + off[0] + (size_t)k * MNI);
+        reg[q] = v;
+      }
+    }
+  }
+
+  __device__ void store(float2* tile) const {
+    if (KC) {
+      constexpr int RSTEP = NT * VEC / TK;
+#pragma unroll
+      for (int q = 0; q < NSLOT; ++q)
+        *reinterpret_cast<vec_t*>(tile + lds_off + q * RSTEP * KC_LD) = reg[q];
+    } else {
+      constexpr int KSTEP = NT * VEC / TM;
+#pragma unroll
+      for (int q = 0; q < NSLOT; ++q)
+        *reinterpret_cast<vec_t*>(tile + lds_off + q * KSTEP * MN_LD) = reg[q];
+    }
+  }
+};
+
+// The four reals (re k0, im k0, re k0+1, im k0+1) one lane feeds to four consecutive MFMAs,
+// for tile row/col `idx` and the lane's pair of contraction steps k0 = 4s + 2h.
+template <bool KC>
+__device__ inline float4 fetch_operand(const float2* tile, int idx, int k0) {
+  if (KC) {
+    return *reinterpret_cast<const float4*>(tile + idx * KC_LD + k0);
+  } else {
+    const float2 a = tile[k0 * MN_LD + idx];
+    const float2 b = tile[(k0 + 1) * MN_LD + idx];
+    return make_float4(a.x, a.y, b.x, b.y);
+  }
+}
+
+template <int MODE, int VEC>
+__global__ __launch_bounds__(NT) void so3_block_mm_kernel(MmParams p) {
+  typedef Cfg<MODE> C_;
+  __shared__ __attribute__((aligned(16))) float2 As[TILE_ELEMS];
+  __shared__ __attribute__((aligned(16))) float2 Bs[TILE_ELEMS];
+
+  // ---- which tile: degrees in descending order so the heaviest tiles are dispatched first
+  int t = blockIdx.x;
+  int l = p.nl - 1, tm = 0, tn = 0;
+  for (;; --l) {
+    const int L_ = 2 * l + 1;
+    tm = s2cnn::ceil_div(L_ * p.RI, TM);
+    tn = s2cnn::ceil_div(L_ * p.CI, TN);
+    if (t < tm * tn || l == 0) break;
+    t -= tm * tn;
+  }
+  const int L = 2 * l + 1;
+  const int tile_m = (t % tm) * TM;
+  const int tile_n = (t / tm) * TN;
+  const size_t L0 = (size_t)l * (4 * l * l - 1) / 3;
+  const int M = L * p.RI, N = L * p.CI;
+
+  TileLoader<C_::A_KC, C_::A_MNMAJ, VEC> la;
+  TileLoader<C_::B_KC, C_::B_MNMAJ, VEC> lb;
+  la.init(p.A + L0 * p.RI * p.KI, L, p.RI, p.KI, tile_m);
+  lb.init(p.B + L0 * p.CI * p.KI, L, p.CI, p.KI, tile_n);
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int r32 = lane & 31, h = lane >> 5;
+  const int wrow = (wave >> 1) * 64, wcol = (wave & 1) * 64;
+
+  v16f acc_re[2][2], acc_im[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) { acc_re[i][j][v] = 0.f; acc_im[i][j][v] = 0.f; }
+
+  const int nkc = s2cnn::ceil_div(p.KI, TK);
+  const int nstage = L * nkc;
+  la.load(0, 0);
+  lb.load(0, 0);
+  int kb = 0, kc = 0;
+  for (int stage = 0; stage < nstage; ++stage) {
+    __syncthreads();
+    la.store(As);
+    lb.store(Bs);
+    __syncthreads();
+    if (++kc == nkc) { kc = 0; ++kb; }
+    if (stage + 1 < nstage) {
+      la.load(kb, kc * TK);
+      lb.load(kb, kc * TK);
+    }
+#pragma unroll
+    for (int s = 0; s < TK / 4; ++s) {
+      const int k0 = 4 * s + 2 * h;
+      float4 a[2], bre[2], bim[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) a[i] = fetch_operand<C_::A_KC>(As, wrow + 32 * i + r32, k0);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const float4 b = fetch_operand<C_::B_KC>(Bs, wcol + 32 * j + r32, k0);
+        if (C_::CONJ) {
+          bre[j] = b;
+          bim[j] = make_float4(-b.y, b.x, -b.w, b.z);
+        } else {
+          bre[j] = make_float4(b.x, -b.y, b.z, -b.w);
+          bim[j] = make_float4(b.y, b.x, b.w, b.z);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          acc_re[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i].x, bre[j].x, acc_re[i][j], 0, 0, 0);
+          acc_im[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i].x, bim[j].x, acc_im[i][j], 0, 0, 0);
+          acc_re[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i].y, bre[j].y, acc_re[i][j], 0, 0, 0);
+          acc_im[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i].y, bim[j].y, acc_im[i][j], 0, 0, 0);
+          acc_re[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i].z, bre[j].z, acc_re[i][j], 0, 0, 0);
+          acc_im[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i].z, bim[j].z, acc_im[i][j], 0, 0, 0);
+          acc_re[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i].w, bre[j].w, acc_re[i][j], 0, 0, 0);
+          acc_im[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i].w, bim[j].w, acc_im[i][j], 0, 0, 0);
+        }
+    }
+  }
+
+  // ---- write the 64x64 complex sub-tile.  Accumulator register v of lane (r32, h) holds
+  // row 8*(v/4) + 4*h + v%4 and column r32 of its 32x32 tile.
+  float2* Cl = p.C + L0 * p.RI * p.CI;
+  const int blk_elems = p.RI * p.CI;
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int col = tile_n + wcol + 32 * j + r32;
+    if (col >= N) continue;
+    const int cb = col / p.CI, ci = col - cb * p.CI;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int row = tile_m + wrow + 32 * i + 8 * (v / 4) + 4 * h + (v % 4);
+        if (row < M) {
+          const int rb = row / p.RI, ri = row - rb * p.RI;
+          const int blk = C_::C_RMAJ ? rb * L + cb : cb * L + rb;
+          Cl[(size_t)blk * blk_elems + ri * p.CI + ci] = make_float2(acc_re[i][j][v], acc_im[i][j][v]);
+        }
+      }
+    }
+  }
+}
+
+int total_tiles(int nl, int RI, int CI) {
+  long n = 0;
+  for (int l = 0; l < nl; ++l) {
+    const int L = 2 * l + 1;
+    n += (long)s2cnn::ceil_div(L * RI, TM) * s2cnn::ceil_div(L * CI, TN);
+  }
+  return n > 0x7fffffffL ? -1 : (int)n;
+}
+
+template <int MODE>
+int run(const float* a, const float* b, float* c, int nl, int RI, int CI, int KI, void* stream) {
+  if (!a || !b || !c || nl < 1 || RI < 1 || CI < 1 || KI < 1) return S2CNN_EINVAL;
+  if (nl > 512 || (long)RI * KI > (1L << 24) || (long)CI * KI > (1L << 24) || (long)RI * CI > (1L << 24)) return S2CNN_EINVAL;
+  // per-degree operand slabs are indexed with 32-bit offsets
+  const long Lmax = 2L * nl - 1;
+  if (Lmax * Lmax * RI * KI >= (1L << 31) || Lmax * Lmax * CI * KI >= (1L << 31)) return S2CNN_EINVAL;
+  if (!s2cnn::aligned8(a) || !s2cnn::aligned8(b) || !s2cnn::aligned8(c)) return S2CNN_EALIGN;
+  const int tiles = total_tiles(nl, RI, CI);
+  if (tiles < 1) return S2CNN_EINVAL;
+  MmParams p{reinterpret_cast<const float2*>(a), reinterpret_cast<const float2*>(b),
+             reinterpret_cast<float2*>(c), nl, RI, CI, KI};
+  typedef Cfg<MODE> C_;
+  // two complex numbers per access need the fast index of each operand to be even and 16-byte bases
+  const bool a_even = C_::A_KC ? (KI % 2 == 0) : (RI % 2 == 0);
+  const bool b_even = C_::B_KC ? (KI % 2 == 0) : (CI % 2 == 0);
+  const bool vec2 = a_even && b_even && s2cnn::aligned16(a) && s2cnn::aligned16(b);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (vec2)
+    hipLaunchKernelGGL((so3_block_mm_kernel<MODE, 2>), dim3(tiles), dim3(NT), 0, st, p);
+  else
+    hipLaunchKernelGGL((so3_block_mm_kernel<MODE, 1>), dim3(tiles), dim3(NT), 0, st, p);
+  return s2cnn::launch_status();
+}
+
+}  // namespace
+
+extern "C" int s2cnn_so3_mm_fwd(const float* x, const float* y, float* z, int nl, int nbatch, int f_in,
+                                int f_out, void* stream) {
+  return run<FWD>(x, y, z, nl, nbatch, f_out, f_in, stream);
+}
+
+extern "C" int s2cnn_so3_mm_gradx(const float* gz, const float* y, float* gx, int nl, int nbatch, int f_in,
+                                  int f_out, void* stream) {
+  return run<GRADX>(gz, y, gx, nl, nbatch, f_in, f_out, stream);
+}
+
+extern "C" int s2cnn_so3_mm_grady(const float* gz, const float* x, float* gy, int nl, int nbatch, int f_in,
+                                  int f_out, void* stream) {
+  return run<GRADY>(x, gz, gy, nl, f_in, f_out, nbatch, stream);
+}

@@ -1,0 +1,136 @@
+"""SO(3) Fourier transforms on the SOFT grid: mirrors s2cnn/soft/so3_fft.py of the reference
+(same functions, arguments, layouts and autograd rules), running on the HIP kernels behind
+s2cnn_so3_analysis / s2cnn_so3_synthesis."""
+from functools import lru_cache
+
+import torch
+
+from .. import _hip, wigner
+
+
+def _nspec(b):
+    return b * (4 * b ** 2 - 1) // 3
+
+
+@lru_cache(maxsize=32)
+def _setup_wigner(b, nl, weighted, device):
+    """[2b, nspec(nl)] float32 on `device`, computed in float64 (s2cnn/soft/so3_fft.py:205-243)."""
+    dss = wigner.so3_wigner_table(b, nl, bool(weighted))
+    return torch.tensor(dss, dtype=torch.float32, device=device).contiguous()
+
+
+def _analysis(x, b_in, b_out, nbatch, for_grad, complex_in):
+    _hip.require_gpu_f32(x)
+    L = _hip.lib()
+    table = _setup_wigner(b_in, nl=b_out, weighted=not for_grad, device=x.device)
+    out = x.new_empty((_nspec(b_out), nbatch, 2))
+    ws = _hip.workspace(L.s2cnn_so3_analysis_workspace(b_in, b_out, nbatch, complex_in), x.device)
+    _hip.check(L.s2cnn_so3_analysis(_hip.ptr(x), _hip.ptr(table), _hip.ptr(out), _hip.ptr(ws), ws.numel(),
+                                    b_in, b_out, nbatch, complex_in, _hip.stream_ptr()))
+    return out
+
+
+def _synthesis(x, b_in, b_out, nbatch, for_grad, complex_out):
+    _hip.require_gpu_f32(x)
+    L = _hip.lib()
+    table = _setup_wigner(b_out, nl=b_in, weighted=for_grad, device=x.device)
+    shape = (nbatch, 2 * b_out, 2 * b_out, 2 * b_out) + ((2,) if complex_out else ())
+    out = x.new_empty(shape)
+    ws = _hip.workspace(L.s2cnn_so3_synthesis_workspace(b_in, b_out, nbatch, complex_out), x.device)
+    _hip.check(L.s2cnn_so3_synthesis(_hip.ptr(x), _hip.ptr(table), _hip.ptr(out), _hip.ptr(ws), ws.numel(),
+                                     b_in, b_out, nbatch, complex_out, _hip.stream_ptr()))
+    return out
+
+
+def so3_fft(x, for_grad=False, b_out=None):
+    '''
+    :param x: [..., beta, alpha, gamma, complex]
+    :return: [l * m * n, ..., complex]
+    '''
+    assert x.size(-1) == 2, x.size()
+    b_in = x.size(-2) // 2
+    assert x.size(-2) == 2 * b_in
+    assert x.size(-3) == 2 * b_in
+    assert x.size(-4) == 2 * b_in
+    if b_out is None:
+        b_out = b_in
+    batch_size = x.size()[:-4]
+    x = x.contiguous().view(-1, 2 * b_in, 2 * b_in, 2 * b_in, 2)
+    out = _analysis(x, b_in, b_out, x.size(0), for_grad, 1)
+    return out.view(-1, *batch_size, 2)
+
+
+def so3_rfft(x, for_grad=False, b_out=None):
+    '''
+    :param x: [..., beta, alpha, gamma]
+    :return: [l * m * n, ..., complex]
+    '''
+    b_in = x.size(-1) // 2
+    assert x.size(-1) == 2 * b_in
+    assert x.size(-2) == 2 * b_in
+    assert x.size(-3) == 2 * b_in
+    if b_out is None:
+        b_out = b_in
+    batch_size = x.size()[:-3]
+    x = x.contiguous().view(-1, 2 * b_in, 2 * b_in, 2 * b_in)
+    out = _analysis(x, b_in, b_out, x.size(0), for_grad, 0)
+    return out.view(-1, *batch_size, 2)
+
+
+def _spectrum_args(x, b_out):
+    assert x.size(-1) == 2
+    nspec = x.size(0)
+    b_in = round((3 / 4 * nspec) ** (1 / 3))
+    assert nspec == b_in * (4 * b_in ** 2 - 1) // 3
+    if b_out is None:
+        b_out = b_in
+    batch_size = x.size()[1:-1]
+    x = x.contiguous().view(nspec, -1, 2)
+    return x, b_in, b_out, batch_size
+
+
+def so3_ifft(x, for_grad=False, b_out=None):
+    '''
+    :param x: [l * m * n, ..., complex]
+    :return: [..., beta, alpha, gamma, complex]
+    '''
+    x, b_in, b_out, batch_size = _spectrum_args(x, b_out)
+    out = _synthesis(x, b_in, b_out, x.size(1), for_grad, 1)
+    return out.view(*batch_size, 2 * b_out, 2 * b_out, 2 * b_out, 2)
+
+
+def so3_rifft(x, for_grad=False, b_out=None):
+    '''
+    :param x: [l * m * n, ..., complex]
+    :return: [..., beta, alpha, gamma]  (the real part of so3_ifft, whatever the symmetry of x)
+    '''
+    x, b_in, b_out, batch_size = _spectrum_args(x, b_out)
+    out = _synthesis(x, b_in, b_out, x.size(1), for_grad, 0)
+    return out.view(*batch_size, 2 * b_out, 2 * b_out, 2 * b_out)
+
+
+class SO3_fft_real(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, b_out=None):  # pylint: disable=W
+        ctx.b_out = b_out
+        ctx.b_in = x.size(-1) // 2
+        return so3_rfft(x, b_out=ctx.b_out)
+
+    @staticmethod
+    def backward(ctx, grad_output):  # pylint: disable=W
+        # real part of the complex inverse of a spectrum that need not be Hermitian
+        # (s2cnn/soft/so3_fft.py:453-456); the real-output kernel computes exactly that
+        return so3_rifft(grad_output, for_grad=True, b_out=ctx.b_in), None
+
+
+class SO3_ifft_real(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, b_out=None):  # pylint: disable=W
+        nspec = x.size(0)
+        ctx.b_out = b_out
+        ctx.b_in = round((3 / 4 * nspec) ** (1 / 3))
+        return so3_rifft(x, b_out=ctx.b_out)
+
+    @staticmethod
+    def backward(ctx, grad_output):  # pylint: disable=W
+        return so3_rfft(grad_output, for_grad=True, b_out=ctx.b_in), None

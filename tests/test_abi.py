@@ -1,0 +1,68 @@
+"""The C-ABI library loads and exports every symbol include/s2cnn_hip.h declares; argument
+checks that need no GPU (they return before any launch)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "s2cnn_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(s2cnn_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from s2cnn_amd import _hip
+    lib = _hip.lib()
+    names = _declared()
+    assert len(names) >= 18
+    for n in names:
+        assert hasattr(lib, n), n
+    assert sorted(_hip.SIGNATURES) == names
+    assert lib.s2cnn_abi_version() == 1
+
+
+def test_argument_rejection_without_gpu():
+    from s2cnn_amd import _hip
+    lib = _hip.lib()
+    null = ctypes.c_void_p(0)
+    assert lib.s2cnn_so3_mm_fwd(null, null, null, 4, 2, 3, 5, null) == -1
+    assert lib.s2cnn_s2_mm_fwd(null, null, null, 4, 2, 3, 5, null) == -1
+    assert lib.s2cnn_so3_analysis(null, null, null, null, 0, 4, 4, 1, 0, null) == -1
+    assert lib.s2cnn_so3_integrate(null, null, null, 4, 1, null) == -1
+    fake = ctypes.c_void_p(0x1000)
+    assert lib.s2cnn_so3_mm_fwd(fake, fake, fake, 0, 2, 3, 5, null) == -1          # nl < 1
+    assert lib.s2cnn_so3_mm_fwd(ctypes.c_void_p(0x1004), fake, fake, 2, 2, 3, 5, null) == -3
+    assert lib.s2cnn_so3_analysis(fake, fake, fake, null, 0, 4, 4, 1, 0, null) == -2  # no workspace
+    assert lib.s2cnn_s2_analysis(fake, fake, fake, fake, 1 << 30, 4, 5, 1, 0, null) == -1  # b_out > b_in
+    assert lib.s2cnn_so3_analysis_workspace(32, 32, 256, 0) == 256 * 64 * 63 * 32 * 8
+    assert lib.s2cnn_so3_synthesis_workspace(4, 6, 3, 1) == 3 * 12 * 7 * 7 * 8
+    assert b"workspace" in lib.s2cnn_strerror(-2)
+
+
+def test_product_has_no_cpu_path():
+    import torch
+    import s2cnn_amd
+    from s2cnn_amd.soft.so3_fft import so3_rfft
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        so3_rfft(torch.zeros(4, 4, 4))
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        s2cnn_amd.so3_mm(torch.zeros(1, 1, 1, 2), torch.zeros(1, 1, 1, 2))
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        s2cnn_amd.so3_integrate(torch.zeros(2, 4, 4, 4))
+
+
+def test_product_does_not_import_oracle():
+    import subprocess
+    import sys
+    code = ("import sys; sys.path.insert(0, %r); import s2cnn_amd, s2cnn_amd.soft.so3_fft, s2cnn_amd.soft.s2_fft; "
+            "assert not any(m == 'oracle' or m.startswith('oracle.') for m in sys.modules)" % ROOT)
+    subprocess.run([sys.executable, "-c", code], check=True)
+    for dirpath, _, files in os.walk(os.path.join(ROOT, "s2cnn_amd")):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h")):
+                assert "oracle" not in open(os.path.join(dirpath, f)).read(), f

@@ -1,0 +1,270 @@
+"""Parity of the HIP path (through the C ABI) against the CPU oracle on identical seeded
+inputs.  Bar: max|d| / std(ref) < 1e-4 (the reference's own CPU-vs-GPU metric,
+tests/so3_fft.py:95-100, so3_mm.py:264-271 of the reference) and relative L2 < 1e-4."""
+import pytest
+import torch
+
+import s2cnn_amd
+from oracle import cpu_path as O
+from s2cnn_amd.soft import s2_fft as PS2
+from s2cnn_amd.soft import so3_fft as PSO3
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+
+
+def close(got, want, what=""):
+    got = got.detach().double().cpu()
+    want = want.detach().double()
+    assert got.shape == want.shape, (what, got.shape, want.shape)
+    scale = want.std().item() if want.numel() > 1 else abs(want.item())
+    q = (got - want).abs().max().item() / max(scale, 1e-30)
+    r = (got - want).norm().item() / max(want.norm().item(), 1e-30)
+    print(f"{what}: max|d|/std={q:.2e} relL2={r:.2e}", flush=True)
+    assert q < TOL and r < TOL, (what, q, r)
+
+
+def rnd(shape, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(*shape, generator=g) * scale
+
+
+# ------------------------------------------------------------------ so3_mm
+MM_SHAPES = [(4, 2, 3, 5),        # the reference's in-module test (so3_mm.py:264-271): odd sizes
+             (3, 32, 20, 40),     # config 1 layer 2 features
+             (6, 3, 7, 55),       # odd everything
+             (8, 16, 64, 64),     # config 3/4 features at a small bandwidth
+             (5, 1, 1, 1),
+             (12, 16, 32, 48)]
+
+
+@pytest.mark.parametrize("nl,B,Fi,Fo", MM_SHAPES)
+def test_so3_mm_forward_backward(hip, nl, B, Fi, Fo):
+    print(f"so3_mm nl={nl} B={B} Fi={Fi} Fo={Fo}", flush=True)
+    ns = O.nspec_so3(nl)
+    x = rnd((ns, B, Fi, 2), 3)
+    y = rnd((ns, Fi, Fo, 2), 4, Fi ** -0.5)
+    gz = rnd((ns, B, Fo, 2), 5)
+    xo, yo = x.double().requires_grad_(), y.double().requires_grad_()
+    zo = O.so3_mm(xo, yo)
+    gxo, gyo = torch.autograd.grad(zo, (xo, yo), gz.double())
+    xg, yg = x.cuda().requires_grad_(), y.cuda().requires_grad_()
+    zg = s2cnn_amd.so3_mm(xg, yg)
+    gxg, gyg = torch.autograd.grad(zg, (xg, yg), gz.cuda())
+    close(zg, zo, "z")
+    close(gxg, gxo, "gx")
+    close(gyg, gyo, "gy")
+
+
+@pytest.mark.parametrize("nl,B,Fi,Fo", [(4, 2, 3, 5), (10, 32, 1, 20), (7, 5, 6, 9), (6, 16, 12, 15)])
+def test_s2_mm_forward_backward(hip, nl, B, Fi, Fo):
+    print(f"s2_mm nl={nl} B={B} Fi={Fi} Fo={Fo}", flush=True)
+    x = rnd((nl * nl, B, Fi, 2), 6)
+    y = rnd((nl * nl, Fi, Fo, 2), 7)
+    gz = rnd((O.nspec_so3(nl), B, Fo, 2), 8)
+    xo, yo = x.double().requires_grad_(), y.double().requires_grad_()
+    gxo, gyo = torch.autograd.grad(O.s2_mm(xo, yo), (xo, yo), gz.double())
+    xg, yg = x.cuda().requires_grad_(), y.cuda().requires_grad_()
+    zg = s2cnn_amd.s2_mm(xg, yg)
+    gxg, gyg = torch.autograd.grad(zg, (xg, yg), gz.cuda())
+    close(zg, O.s2_mm(x.double(), y.double()), "z")
+    close(gxg, gxo, "gx")
+    close(gyg, gyo, "gy")
+
+
+# ------------------------------------------------------------------ SO(3) transforms
+SO3_PAIRS = [(2, 9), (6, 6), (9, 2), (10, 11), (11, 10), (7, 5), (4, 6), (16, 16)]   # first five: tests/so3_fft.py:102
+
+
+@pytest.mark.parametrize("b_in,b_out", SO3_PAIRS)
+@pytest.mark.parametrize("for_grad", [False, True])
+def test_so3_transforms(hip, b_in, b_out, for_grad):
+    print(f"so3 transforms b_in={b_in} b_out={b_out} for_grad={for_grad}", flush=True)
+    nz = 3
+    x = rnd((nz, 2 * b_in, 2 * b_in, 2 * b_in, 2), 10)
+    close(PSO3.so3_fft(x.cuda(), for_grad, b_out), O.so3_fft(x.double(), for_grad, b_out), "so3_fft")
+    xr = x[..., 0].contiguous()
+    close(PSO3.so3_rfft(xr.cuda(), for_grad, b_out), O.so3_rfft(xr.double(), for_grad, b_out), "so3_rfft")
+    s = rnd((O.nspec_so3(b_in), nz, 2), 11)
+    close(PSO3.so3_ifft(s.cuda(), for_grad, b_out), O.so3_ifft(s.double(), for_grad, b_out), "so3_ifft")
+    close(PSO3.so3_rifft(s.cuda(), for_grad, b_out), O.so3_rifft(s.double(), for_grad, b_out), "so3_rifft (generic spectrum)")
+    sh = O.so3_rfft(rnd((nz, 2 * b_in, 2 * b_in, 2 * b_in), 12).double()).float()      # Hermitian spectrum, tests/so3_fft.py:112-114
+    close(PSO3.so3_rifft(sh.cuda(), for_grad, b_out), O.so3_rifft(sh.double(), for_grad, b_out), "so3_rifft (real signal)")
+
+
+def test_so3_transform_batch_dims_and_ragged(hip):
+    x = rnd((2, 3, 8, 8, 8), 13)
+    close(PSO3.so3_rfft(x.cuda(), b_out=3), O.so3_rfft(x.double(), b_out=3), "lead dims")
+    x1 = rnd((17, 6, 6, 6), 14)              # nbatch not a multiple of the z tile
+    close(PSO3.so3_rfft(x1.cuda()), O.so3_rfft(x1.double()), "ragged batch")
+    s1 = rnd((O.nspec_so3(3), 17, 2), 15)
+    close(PSO3.so3_rifft(s1.cuda()), O.so3_rifft(s1.double()), "ragged batch inv")
+    x0 = rnd((1, 2, 2, 2), 16)               # b = 1: a single coefficient
+    close(PSO3.so3_rfft(x0.cuda()), O.so3_rfft(x0.double()), "b=1")
+
+
+def test_so3_reference_identities_on_gpu(hip):
+    """tests/so3_fft.py:8-24 and :34-91 of the reference, run on the HIP path."""
+    b_in, b_out = 7, 5
+    x = rnd((2 * b_in, 2 * b_in, 2 * b_in), 20).cuda()
+    y1 = PSO3.so3_rfft(x, b_out=b_out)
+    w = torch.tensor(s2cnn_amd.wigner.quadrature_weights(b_in), dtype=torch.float32).cuda()
+    y2 = s2cnn_amd.so3_rft((x * w.view(-1, 1, 1)).view(-1), b_out, s2cnn_amd.so3_soft_grid(b_in))
+    assert (y1 - y2).abs().max().item() < 1e-4 * y1.abs().mean().item()
+    for f, g, cplx, pairs in ((PSO3.so3_fft, PSO3.so3_ifft, True, [(7, 7), (5, 4), (7, 4), (7, 5), (4, 6)]),
+                              (PSO3.so3_rfft, PSO3.so3_rifft, False, [(7, 7), (5, 4), (4, 6)])):
+        for bi, bo in pairs:
+            x = rnd((2 * bi,) * 3 + ((2,) if cplx else ()), 21).cuda()
+            x = g(f(x, b_out=bo), b_out=bi)
+            y = g(f(x, b_out=bo), b_out=bi)
+            assert (x - y).abs().max().item() < 1e-4 * y.abs().mean().item(), (bi, bo, cplx)
+    for f, g in ((PSO3.so3_ifft, PSO3.so3_fft), (PSO3.so3_rifft, PSO3.so3_rfft)):
+        for bi, bo in [(7, 7), (5, 4), (4, 7)]:
+            x = rnd((O.nspec_so3(bi), 2), 22).cuda()
+            x = g(f(x, b_out=bo), b_out=bi)
+            y = g(f(x, b_out=bo), b_out=bi)
+            assert (x - y).abs().max().item() < 1e-4 * y.abs().mean().item(), (bi, bo)
+
+
+# ------------------------------------------------------------------ S^2 transforms
+@pytest.mark.parametrize("b_in,b_out", [(6, 5), (12, 12), (13, 12), (30, 10), (4, 1), (64, 16)])   # (6,5): s2_fft.py:253-259
+@pytest.mark.parametrize("for_grad", [False, True])
+def test_s2_transforms(hip, b_in, b_out, for_grad):
+    print(f"s2 transforms b_in={b_in} b_out={b_out} for_grad={for_grad}", flush=True)
+    x = rnd((1, 2, 2 * b_in, 2 * b_in, 2), 30)
+    close(PS2.s2_fft(x.cuda(), for_grad, b_out), O.s2_fft(x.double(), for_grad, b_out), "s2_fft")
+    xr = x[..., 0].contiguous()
+    close(PS2.s2_rfft(xr.cuda(), for_grad, b_out), O.s2_fft(O.as_complex(xr.double()), for_grad, b_out), "s2_rfft")
+    s = rnd((b_out ** 2, 10, 2), 31)                                                    # s2_fft.py:262-268 uses (12 -> 13)
+    close(PS2.s2_ifft(s.cuda(), for_grad, b_in), O.s2_ifft(s.double(), for_grad, b_in), "s2_ifft")
+    close(PS2.s2_rifft(s.cuda(), for_grad, b_in), O.s2_ifft(s.double(), for_grad, b_in)[..., 0], "s2_rifft")
+
+
+def test_so3_integrate(hip):
+    for b in (1, 3, 6, 16):
+        x = rnd((2, 5, 2 * b, 2 * b, 2 * b), 40 + b)
+        xg = x.cuda().requires_grad_()
+        out = s2cnn_amd.so3_integrate(xg)
+        close(out, O.so3_integrate(x.double()), f"integrate b={b}")
+        g = rnd((2, 5), 41)
+        (gx,) = torch.autograd.grad(out, xg, g.cuda())
+        xo = x.double().requires_grad_()
+        (gxo,) = torch.autograd.grad(O.so3_integrate(xo), xo, g.double())
+        close(gx, gxo, f"integrate grad b={b}")
+    ones = torch.ones(3, 8, 8, 8, device="cuda")
+    assert (s2cnn_amd.so3_integrate(ones) - 1).abs().max().item() < 1e-5
+
+
+# ------------------------------------------------------------------ layers, forward and gradients
+def _conv_case(kind, B, Fi, Fo, b_in, b_out, grid, seed):
+    if kind == "so3":
+        x = rnd((B, Fi, 2 * b_in, 2 * b_in, 2 * b_in), seed)
+        layer = s2cnn_amd.SO3Convolution(Fi, Fo, b_in, b_out, grid)
+        ofun = O.so3_conv
+    else:
+        x = rnd((B, Fi, 2 * b_in, 2 * b_in), seed)
+        layer = s2cnn_amd.S2Convolution(Fi, Fo, b_in, b_out, grid)
+        ofun = O.s2_conv
+    k = torch.rand(Fi, Fo, len(grid), generator=torch.Generator().manual_seed(seed + 1)) * 2 - 1
+    bias = rnd((1, Fo, 1, 1, 1), seed + 2, 0.1)
+    with torch.no_grad():
+        layer.kernel.copy_(k)
+        layer.bias.copy_(bias)
+    layer = layer.cuda()
+    xg = x.cuda().requires_grad_()
+    out = layer(xg)
+    (out ** 2).sum().backward()
+    xo, ko, bo = x.double().requires_grad_(), k.double().requires_grad_(), bias.double().requires_grad_()
+    outo = ofun(xo, ko, bo, b_in, b_out, grid)
+    (outo ** 2).sum().backward()
+    close(out, outo, kind + " conv out")
+    close(xg.grad, xo.grad, kind + " conv grad x")
+    close(layer.kernel.grad, ko.grad, kind + " conv grad kernel")
+    close(layer.bias.grad, bo.grad, kind + " conv grad bias")
+
+
+def test_so3_convolution_parity(hip):
+    _conv_case("so3", 2, 3, 4, 5, 4, s2cnn_amd.so3_near_identity_grid(n_alpha=4, n_beta=2, n_gamma=3), 50)
+    _conv_case("so3", 3, 8, 8, 6, 6, s2cnn_amd.so3_near_identity_grid(), 53)
+    _conv_case("so3", 2, 4, 6, 4, 4, s2cnn_amd.so3_equatorial_grid(n_alpha=8), 56)
+
+
+def test_s2_convolution_parity(hip):
+    _conv_case("s2", 2, 1, 4, 8, 4, s2cnn_amd.s2_near_identity_grid(), 60)
+    _conv_case("s2", 3, 6, 5, 10, 5, s2cnn_amd.s2_equatorial_grid(n_alpha=16), 63)
+
+
+def test_config1_shaped_network(hip):
+    """BASELINE config 1 shapes at reduced batch: S2Conv 1->20 (b 30->10), ReLU, SO3Conv 20->40
+    (b 10->6), ReLU, so3_integrate; forward only."""
+    g = torch.Generator().manual_seed(1)
+    x = torch.rand(4, 1, 60, 60, generator=g) * (torch.rand(4, 1, 60, 60, generator=g) < 0.3)
+    g1 = s2cnn_amd.s2_near_identity_grid(max_beta=3.141592653589793 / 8, n_alpha=8, n_beta=3)
+    g2 = s2cnn_amd.so3_near_identity_grid(max_beta=3.141592653589793 / 8, max_gamma=2 * 3.141592653589793, n_alpha=8, n_beta=3, n_gamma=8)
+    torch.manual_seed(0)
+    c1 = s2cnn_amd.S2Convolution(1, 20, 30, 10, g1)
+    c2 = s2cnn_amd.SO3Convolution(20, 40, 10, 6, g2)
+    want = O.so3_integrate(torch.relu(O.so3_conv(torch.relu(O.s2_conv(x.double(), c1.kernel.detach().double(), c1.bias.detach().double(), 30, 10, g1)),
+                                                 c2.kernel.detach().double(), c2.bias.detach().double(), 10, 6, g2)))
+    c1, c2 = c1.cuda(), c2.cuda()
+    with torch.no_grad():
+        got = s2cnn_amd.so3_integrate(torch.relu(c2(torch.relu(c1(x.cuda())))))
+    close(got, want, "config-1 features")
+
+
+def test_z_rotation_equivariance_on_gpu(hip):
+    """examples/equivariance_error/main.py:18-46 of the reference at reduced sizes."""
+    torch.manual_seed(2)
+    c1 = s2cnn_amd.S2Convolution(3, 5, 16, 8, s2cnn_amd.s2_equatorial_grid(max_beta=0, n_alpha=32, n_beta=1)).cuda()
+    c2 = s2cnn_amd.SO3Convolution(5, 4, 8, 4, s2cnn_amd.so3_equatorial_grid(max_beta=0, max_gamma=0, n_alpha=32, n_beta=1, n_gamma=1)).cuda()
+
+    def phi(t):
+        return c2(torch.relu(c1(t)))
+
+    def rot(t, n):
+        return torch.cat([t[:, :, :, n:], t[:, :, :, :n]], dim=3)
+
+    with torch.no_grad():
+        x = torch.randn(1, 3, 32, 32, device="cuda")
+        y = phi(x)
+        rel = (rot(phi(x), 2) - phi(rot(x, 8))).std() / y.std()     # a quarter turn: 8 of 32 input samples, 2 of 8 output samples
+    assert rel.item() < 1e-4
+
+
+def test_size_independent_properties_at_config_sizes(hip):
+    """Config 2 (b = 32) at a reduced batch: fft -> ifft -> fft reproduces the spectrum (projector),
+    linearity, and the Hermitian symmetry of the spectrum of a real signal."""
+    b = 32
+    x = rnd((8, 2 * b, 2 * b, 2 * b), 70).cuda()
+    s = PSO3.so3_rfft(x)
+    assert s.shape == (43680, 8, 2)
+    s2 = PSO3.so3_rfft(PSO3.so3_rifft(s))
+    assert (s2 - s).abs().max().item() < 1e-4 * s.abs().mean().item() * 10
+    x2 = rnd((8, 2 * b, 2 * b, 2 * b), 71).cuda()
+    lin = PSO3.so3_rfft(2 * x - 3 * x2) - (2 * s - 3 * PSO3.so3_rfft(x2))
+    assert lin.abs().max().item() < 1e-4 * s.abs().mean().item() * 10
+    l, m, n = 17, 5, -9
+    i1 = O.nspec_so3(l) + (l + m) * (2 * l + 1) + (l + n)
+    i2 = O.nspec_so3(l) + (l - m) * (2 * l + 1) + (l - n)
+    sign = (-1) ** (m - n)
+    assert torch.allclose(s[i2, :, 0], sign * s[i1, :, 0]) and torch.allclose(s[i2, :, 1], -sign * s[i1, :, 1])
+
+
+def test_so3_mm_at_config3_features_linearity(hip):
+    """Config 3 feature sizes (batch 16, 64 -> 64) at nl = 16: bilinearity and agreement with a
+    per-degree complex einsum on the GPU in float64."""
+    nl, B, F = 16, 16, 64
+    ns = O.nspec_so3(nl)
+    x = rnd((ns, B, F, 2), 80).cuda()
+    y = (rnd((ns, F, F, 2), 81) * 0.125).cuda()
+    z = s2cnn_amd.so3_mm(x, y)
+    xc = torch.view_as_complex(x.double())
+    yc = torch.view_as_complex(y.double())
+    for l in (0, 1, 7, 15):
+        L = 2 * l + 1
+        lo = O.nspec_so3(l)
+        want = torch.einsum("mpik,npkj->mnij", xc[lo:lo + L * L].view(L, L, B, F), yc[lo:lo + L * L].view(L, L, F, F).conj())
+        got = torch.view_as_complex(z[lo:lo + L * L].double()).view(L, L, B, F)
+        assert (got - want).abs().max().item() < 1e-4 * want.abs().std().item(), l
+    z2 = s2cnn_amd.so3_mm(2 * x, y) - 2 * z
+    assert z2.abs().max().item() < 1e-4 * z.std().item()
