@@ -1,0 +1,176 @@
+"""Headline benchmark: one SO3Convolution layer, forward + backward, fp32, b_in = b_out = 32,
+64 -> 64 features, batch 16, default near-identity grid (192 points), Kaiming-normal kernel,
+loss = sum(out^2) - BASELINE config "Single SO3Convolution layer".  One step = one forward +
+backward over one synthetic batch that is already resident in HBM.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-fft]
+
+Prints ONE JSON line.  `roofline` is for the dominant kernel (the block-diagonal spectral
+product so3_mm, bound by the fp32 matrix cores), timed with events on the launch stream inside
+the timed steps; `so3_fft` reports the standalone SO(3) FFT round trip of BASELINE config 2
+against HBM bandwidth; `cpu_baseline` is the CPU oracle timed on this host on a bounded sample.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X dense fp32 matrix
+PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
+
+
+def nspec(b):
+    return b * (4 * b * b - 1) // 3
+
+
+def mm_flops(nl, B, Fi, Fo):
+    """Algorithmic flops of one so3_mm pass: 8 B Fi Fo sum_l (2l+1)^3 = 8 B Fi Fo nl^2 (2 nl^2 - 1)."""
+    return 8.0 * B * Fi * Fo * nl * nl * (2 * nl * nl - 1)
+
+
+def so3_fft_bytes(b_in, b_out, n):
+    """Algorithmic bytes of one SO(3) transform: real grid + complex spectrum."""
+    return 4.0 * n * (2 * b_in) ** 3 + 8.0 * n * nspec(b_out)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-fft", action="store_true", help="skip the standalone FFT round trip")
+    ap.add_argument("--batch", type=int, default=16)
+    ap.add_argument("--b", type=int, default=32)
+    ap.add_argument("--features", type=int, default=64)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU only (no collectives exist on this path); "
+              "--gpus %d is not supported" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    import s2cnn_amd
+    from s2cnn_amd import _hip
+    from s2cnn_amd.soft import so3_fft as PSO3
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    _hip.lib()
+    dev = torch.device("cuda:0")
+    B, F, b = args.batch, args.features, args.b
+    grid = s2cnn_amd.so3_near_identity_grid()            # 3 * 8 * 8 = 192 points
+    gen = torch.Generator().manual_seed(6)
+    x_cpu = torch.randn(B, F, 2 * b, 2 * b, 2 * b, generator=gen)
+    k_cpu = torch.randn(F, F, len(grid), generator=torch.Generator().manual_seed(7)) * math.sqrt(2.0 / (F * len(grid)))
+    layer = s2cnn_amd.SO3Convolution(F, F, b, b, grid)
+    with torch.no_grad():
+        layer.kernel.copy_(k_cpu)
+    layer = layer.to(dev)
+    x = x_cpu.to(dev).requires_grad_()
+
+    def step():
+        layer.zero_grad(set_to_none=True)
+        x.grad = None
+        out = layer(x)
+        (out ** 2).sum().backward()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    timer = _hip.KernelTimer()
+    t0 = time.perf_counter()
+    with timer:
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    value = B / (ms_per_step * 1e-3)
+
+    per_call = {k: sum(v) / len(v) for k, v in timer.summary().items()}
+    flops = mm_flops(b, B, F, F)
+    mm_names = ["s2cnn_so3_mm_fwd", "s2cnn_so3_mm_gradx", "s2cnn_so3_mm_grady"]
+    dominant = max(mm_names, key=lambda n: per_call[n])
+    ach = flops / (per_call[dominant] * 1e-3) / 1e12
+    roofline = {"bound": "mfma", "kernel": dominant, "achieved": round(ach, 2), "peak": PEAK_FP32_MFMA_TFLOPS,
+                "unit": "TFLOP/s", "frac": round(ach / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None,
+                "flop_per_launch": flops, "ms_per_launch": round(per_call[dominant], 3)}
+    kernels = {n: {"ms": round(ms, 3)} for n, ms in per_call.items()}
+    for n in mm_names:
+        kernels[n]["tflops"] = round(flops / (per_call[n] * 1e-3) / 1e12, 2)
+    for n in ("s2cnn_so3_analysis", "s2cnn_so3_synthesis"):
+        kernels[n]["gbs"] = round(so3_fft_bytes(b, b, B * F) / (per_call[n] * 1e-3) / 1e9, 1)
+
+    result = {
+        "metric": "SO3Conv fwd+bwd samples/s (b=32, 64->64 ch); SO(3) FFT achieved HBM GB/s",
+        "value": round(value, 2), "unit": "samples/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "SO3Convolution fwd+bwd, batch %d, %d->%d features, b_in=b_out=%d, 192-point "
+                               "near-identity grid, loss=sum(out^2) (BASELINE config 4)" % (B, F, F, b)},
+        "roofline": roofline, "kernels": kernels,
+    }
+
+    # ---- standalone SO(3) FFT round trip (BASELINE config 2: [256, 64, 64, 64] -> [43680, 256, 2] -> back)
+    if not args.no_fft:
+        del x, layer
+        torch.cuda.empty_cache()
+        n_fft = 256
+        xf = torch.randn(n_fft, 2 * b, 2 * b, 2 * b, generator=torch.Generator().manual_seed(2)).to(dev)
+        for _ in range(2):
+            PSO3.so3_rifft(PSO3.so3_rfft(xf))
+        torch.cuda.synchronize()
+        ft = _hip.KernelTimer()
+        with ft:
+            for _ in range(10):
+                PSO3.so3_rifft(PSO3.so3_rfft(xf))
+            torch.cuda.synchronize()
+        pc = {k: sum(v) / len(v) for k, v in ft.summary().items()}
+        bytes_dir = so3_fft_bytes(b, b, n_fft)
+        rt_ms = pc["s2cnn_so3_analysis"] + pc["s2cnn_so3_synthesis"]
+        gbs = 2 * bytes_dir / (rt_ms * 1e-3) / 1e9
+        result["so3_fft"] = {"workload": "SO3_fft_real -> SO3_ifft_real, [256,64,64,64] fp32 (BASELINE config 2)",
+                             "bound": "hbm", "bytes_round_trip": 2 * bytes_dir, "ms_round_trip": round(rt_ms, 4),
+                             "analysis_ms": round(pc["s2cnn_so3_analysis"], 4), "synthesis_ms": round(pc["s2cnn_so3_synthesis"], 4),
+                             "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4)}
+        del xf
+        torch.cuda.empty_cache()
+
+    # ---- CPU baseline: the oracle (a restatement of the reference's CPU branches) on a bounded sample
+    if not args.no_cpu:
+        from oracle import cpu_path as O
+        cores = os.cpu_count() or 1
+        env = os.environ.get("OMP_NUM_THREADS")
+        if env:
+            cores = min(cores, int(env))
+        torch.set_num_threads(cores)
+        Bc = 1                                           # one sample of the batch of 16
+        xc = x_cpu[:Bc].clone().requires_grad_()
+        kc = k_cpu.clone().requires_grad_()
+        bc = torch.zeros(1, F, 1, 1, 1, requires_grad=True)
+        O.so3_table(b, b, True), O.so3_table(b, b, False), O._so3_ft_matrix64(b, grid)   # tables are setup, not timed
+
+        def cpu_step():
+            xc.grad = kc.grad = bc.grad = None
+            out = O.so3_conv(xc, kc, bc, b, b, grid)
+            (out ** 2).sum().backward()
+
+        c0 = time.perf_counter()
+        cpu_step()
+        c1 = time.perf_counter()
+        result["cpu_baseline"] = {"value": round(Bc / (c1 - c0), 4), "unit": "samples/s", "cores": cores, "kind": "port",
+                                  "sample": "same layer and sizes at batch %d of %d, one fwd+bwd (%.1f s), fp32, "
+                                            "torch threads = %d" % (Bc, B, c1 - c0, cores)}
+
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

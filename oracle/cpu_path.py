@@ -95,9 +95,14 @@ def quadrature_weights(b, dtype=torch.float32):
     return torch.tensor(wigner_ref.quadrature_weights_ref(b), dtype=dtype)
 
 
+@lru_cache(maxsize=4096)
+def _d_jacobi_cached(l, beta):
+    return wigner_ref.wigner_d_jacobi(l, beta)
+
+
 def _wigner_D64(l, alpha, beta, gamma):
     """D^l_mn = exp(i m alpha) d^l_mn(beta) exp(i n gamma) (s2cnn/soft/so3_rotation.py:58)."""
-    d = wigner_ref.wigner_d_jacobi(l, float(beta))
+    d = _d_jacobi_cached(l, float(beta))
     m = np.arange(-l, l + 1)
     return np.exp(1j * m * alpha)[:, None] * d * np.exp(1j * m * gamma)[None, :]
 

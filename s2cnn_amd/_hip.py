@@ -56,6 +56,44 @@ def lib():
     return handle
 
 
+class KernelTimer:
+    """Optional per-call device timing: while active, every C-ABI call made through `call` is
+    bracketed by two events recorded on the stream the kernels are launched on (torch's current
+    stream).  Read the durations with `summary()` after a synchronize."""
+    active = None
+
+    def __init__(self):
+        self.records = []
+
+    def __enter__(self):
+        KernelTimer.active = self
+        return self
+
+    def __exit__(self, *exc):
+        KernelTimer.active = None
+
+    def summary(self):
+        out = {}
+        for name, e0, e1 in self.records:
+            out.setdefault(name, []).append(e0.elapsed_time(e1))
+        return out
+
+
+def call(name, *args):
+    """Invoke one entry point of the library and raise on a non-zero return code."""
+    fn = getattr(lib(), name)
+    timer = KernelTimer.active
+    if timer is None:
+        check(fn(*args))
+        return
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    check(fn(*args))
+    e1.record()
+    timer.records.append((name, e0, e1))
+
+
 def check(code):
     if code != 0:
         raise RuntimeError("libs2cnn_hip: %s (code %d)" % (lib().s2cnn_strerror(code).decode(), code))

@@ -25,8 +25,8 @@ def _analysis(x, b_in, b_out, nbatch, for_grad, complex_in):
     table = _setup_wigner(b_in, nl=b_out, weighted=not for_grad, device=x.device)
     out = x.new_empty((_nspec(b_out), nbatch, 2))
     ws = _hip.workspace(L.s2cnn_so3_analysis_workspace(b_in, b_out, nbatch, complex_in), x.device)
-    _hip.check(L.s2cnn_so3_analysis(_hip.ptr(x), _hip.ptr(table), _hip.ptr(out), _hip.ptr(ws), ws.numel(),
-                                    b_in, b_out, nbatch, complex_in, _hip.stream_ptr()))
+    _hip.call("s2cnn_so3_analysis", _hip.ptr(x), _hip.ptr(table), _hip.ptr(out), _hip.ptr(ws), ws.numel(),
+                  b_in, b_out, nbatch, complex_in, _hip.stream_ptr())
     return out
 
 
@@ -37,8 +37,8 @@ def _synthesis(x, b_in, b_out, nbatch, for_grad, complex_out):
     shape = (nbatch, 2 * b_out, 2 * b_out, 2 * b_out) + ((2,) if complex_out else ())
     out = x.new_empty(shape)
     ws = _hip.workspace(L.s2cnn_so3_synthesis_workspace(b_in, b_out, nbatch, complex_out), x.device)
-    _hip.check(L.s2cnn_so3_synthesis(_hip.ptr(x), _hip.ptr(table), _hip.ptr(out), _hip.ptr(ws), ws.numel(),
-                                     b_in, b_out, nbatch, complex_out, _hip.stream_ptr()))
+    _hip.call("s2cnn_so3_synthesis", _hip.ptr(x), _hip.ptr(table), _hip.ptr(out), _hip.ptr(ws), ws.numel(),
+                  b_in, b_out, nbatch, complex_out, _hip.stream_ptr())
     return out
 
 

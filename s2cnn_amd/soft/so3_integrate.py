@@ -22,8 +22,8 @@ class _SO3_integrate(torch.autograd.Function):
         x = x.contiguous().view(-1, 2 * b, 2 * b, 2 * b)
         w = _setup_so3_integrate(b, x.device)
         out = x.new_empty((x.size(0),))
-        _hip.check(_hip.lib().s2cnn_so3_integrate(_hip.ptr(x), _hip.ptr(w), _hip.ptr(out), b, x.size(0),
-                                                  _hip.stream_ptr()))
+        _hip.call("s2cnn_so3_integrate", _hip.ptr(x), _hip.ptr(w), _hip.ptr(out), b, x.size(0),
+                  _hip.stream_ptr())
         return out.view(*lead)
 
     @staticmethod
@@ -32,8 +32,8 @@ class _SO3_integrate(torch.autograd.Function):
         g = g.contiguous().view(-1)
         w = _setup_so3_integrate(b, g.device)
         gx = g.new_empty((g.numel(), 2 * b, 2 * b, 2 * b))
-        _hip.check(_hip.lib().s2cnn_so3_integrate_grad(_hip.ptr(g), _hip.ptr(w), _hip.ptr(gx), b, g.numel(),
-                                                       _hip.stream_ptr()))
+        _hip.call("s2cnn_so3_integrate_grad", _hip.ptr(g), _hip.ptr(w), _hip.ptr(gx), b, g.numel(),
+                  _hip.stream_ptr())
         return gx.view(ctx.shape)
 
 
