@@ -17,10 +17,10 @@
 //              G = sum_l T[l,m,n] (xhat[l,m,n] + (-1)^(m-n) conj xhat[l,-m,-n])/2,
 //              so the spectrum is symmetrised on load and no symmetry of xhat is assumed.
 #include "common.h"
+#include "so3_plane_fft64.h"
+#include "so3_wigner_tiled.h"
 
 namespace {
-
-constexpr float kTwoPi = 6.283185307179586476925286766559f;
 
 __device__ inline float2 cmul(float2 a, float2 b) { return make_float2(a.x * b.x - a.y * b.y, a.x * b.y + a.y * b.x); }
 __device__ inline float2 cmul_conj(float2 a, float2 b) { return make_float2(a.x * b.x + a.y * b.y, a.y * b.x - a.x * b.y); }  // a*conj(b)
@@ -307,9 +307,13 @@ extern "C" int s2cnn_so3_analysis(const float* x, const float* table, float* out
   const size_t lds = sizeof(float) * (2 * n2 + (complex_in ? 2 : 1) * n2 * n2 + 2 * n2 * NW);
   if (lds > 160 * 1024) return S2CNN_EINVAL;
   const unsigned planes = (unsigned)(nbatch * n2);
+  const bool tiled = !complex_in && nb <= 32 && b_out <= 32;
   if (complex_in) {
     if (lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)so3_plane_dft_fwd<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     hipLaunchKernelGGL(so3_plane_dft_fwd<true>, dim3(planes), dim3(256), lds, st, x, X, n2, nb);
+  } else if (n2 == 64) {
+    const long npairs = nbatch * 32;
+    hipLaunchKernelGGL(fft64::plane_fft64_fwd, dim3((unsigned)(npairs < 2048 ? npairs : 2048)), dim3(fft64::THREADS), 0, st, x, X, npairs, nb);
   } else {
     if (lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)so3_plane_dft_fwd<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     hipLaunchKernelGGL(so3_plane_dft_fwd<false>, dim3(planes), dim3(256), lds, st, x, X, n2, nb);
@@ -321,7 +325,10 @@ extern "C" int s2cnn_so3_analysis(const float* x, const float* table, float* out
     hipLaunchKernelGGL(fill_zero, dim3(1024), dim3(256), 0, st, out, nfl);
   }
   dim3 grid(s2cnn::ceil_div(NW, 16), MW, (unsigned)((nbatch + 15) / 16));
-  if (complex_in)
+  if (tiled)
+    hipLaunchKernelGGL(wigner_tiled::wigner_fwd_tiled, dim3(wigner_tiled::grid_size(MW, nbatch)), dim3(256), 0, st, X, table,
+                       reinterpret_cast<float2*>(out), n2, nb, b_out, nbatch);
+  else if (complex_in)
     hipLaunchKernelGGL(so3_wigner_fwd<true>, grid, dim3(16, 16), 0, st, X, table, reinterpret_cast<float2*>(out), n2, nb, b_out, nbatch);
   else
     hipLaunchKernelGGL(so3_wigner_fwd<false>, grid, dim3(16, 16), 0, st, X, table, reinterpret_cast<float2*>(out), n2, nb, b_out, nbatch);
@@ -345,6 +352,9 @@ extern "C" int s2cnn_so3_synthesis(const float* xhat, const float* table, float*
   const float2* xh = reinterpret_cast<const float2*>(xhat);
   if (complex_out)
     hipLaunchKernelGGL(so3_wigner_inv<true>, grid, dim3(16, 16), 0, st, xh, table, S, n2, nb, b_in, nbatch);
+  else if (nb <= 32 && n2 <= 64)
+    hipLaunchKernelGGL(wigner_tiled::wigner_inv_tiled, dim3(wigner_tiled::grid_size(MW, nbatch)), dim3(512), 0, st, xh, table, S,
+                       n2, nb, b_in, nbatch);
   else
     hipLaunchKernelGGL(so3_wigner_inv<false>, grid, dim3(16, 16), 0, st, xh, table, S, n2, nb, b_in, nbatch);
   int rc = s2cnn::launch_status();
@@ -353,6 +363,9 @@ extern "C" int s2cnn_so3_synthesis(const float* xhat, const float* table, float*
   if (complex_out) {
     if (lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)so3_plane_dft_inv<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     hipLaunchKernelGGL(so3_plane_dft_inv<true>, dim3(planes), dim3(256), lds, st, S, out, n2, nb);
+  } else if (n2 == 64) {
+    const long npairs = nbatch * 32;
+    hipLaunchKernelGGL(fft64::plane_fft64_inv, dim3((unsigned)(npairs < 2048 ? npairs : 2048)), dim3(fft64::THREADS), 0, st, S, out, npairs, nb);
   } else {
     if (lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)so3_plane_dft_inv<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     hipLaunchKernelGGL(so3_plane_dft_inv<false>, dim3(planes), dim3(256), lds, st, S, out, n2, nb);

@@ -1,0 +1,230 @@
+// Contraction with the Wigner table for real signals, tiled through LDS (FMA bound work that must
+// not re-read HBM): a workgroup owns one frequency m, all n >= 0, a tile of 16 batch items and
+// streams the reduction index (beta for analysis, l for synthesis) in chunks.
+//
+//   analysis : out[l,m,n,z] = sum_beta T[beta, lmn] X[z,beta,m,n]          (accumulators over l)
+//   synthesis: S[z,beta,m,n] = sum_l   T[beta, lmn] xs[l,m,n,z]            (accumulators over beta)
+//              xs = (xhat[l,m,n] + (-1)^(m-n) conj xhat[l,-m,-n]) / 2
+//
+// The table is read in its public layout [2b][nspec]; for fixed (beta, l, m) the entries n = 0..l
+// are contiguous.  Requirements: nb = min(b_grid, b_spec) <= 32, degrees <= 32 (analysis),
+// 2 b_grid <= 64 (synthesis).
+#pragma once
+#include <hip/hip_runtime.h>
+
+namespace wigner_tiled {
+
+constexpr int ZT = 16;        // batch items per workgroup
+constexpr int XLD = 36;       // analysis: z stride (complex) of the X chunk -> 2-way minimum on 8-byte reads
+constexpr int TLD = 36;       // analysis: n stride (floats) of the T chunk, 16-byte aligned rows of 32 degrees
+constexpr int KB = 8;         // analysis: betas per chunk
+constexpr int SLD = 33;       // synthesis: z stride (complex) of the spectrum chunk
+constexpr int QLD = 68;       // synthesis: n stride (floats) of the T chunk, 64 betas + pad
+constexpr int LC = 4;         // synthesis: degrees per chunk (LDS stays under 64 KB)
+
+__device__ __forceinline__ int lmn_index(int l, int m, int n) { return l * (4 * l * l - 1) / 3 + (l + m) * (2 * l + 1) + (l + n); }
+
+// Workgroup -> (m, z tile).  Consecutive workgroups go round-robin over the 8 XCDs; all workgroups
+// of one XCD that run together share m (and so the table slab in that XCD's L2).  Small |m| (long
+// degree ranges) first.  Returns false for padding workgroups.
+__device__ __forceinline__ bool decode_block(int MW, int nb, int nzt, int& m, int& zt) {
+  const int wid = blockIdx.x;
+  const int xcd = wid & 7, slot = wid >> 3;
+  const int o = xcd + 8 * (slot / nzt);
+  zt = slot % nzt;
+  if (o >= MW) return false;
+  m = (o & 1) ? (o + 1) / 2 : -(o / 2);
+  return true;
+}
+
+inline int grid_size(int MW, long nbatch) {
+  const long nzt = (nbatch + ZT - 1) / ZT;
+  return (int)(8L * ((MW + 7) / 8) * nzt);
+}
+
+// ---------------------------------------------------------------------------------------------
+// analysis: 256 threads, thread = (zq = t % 8 -> z = 2 zq, 2 zq + 1 ; n = t / 8)
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void wigner_fwd_tiled(const float2* __restrict__ X, const float* __restrict__ T,
+                                                        float2* __restrict__ out, int n2, int nb, int nl, long nbatch) {
+  __shared__ __attribute__((aligned(16))) float2 Xs[KB * ZT * XLD];
+  __shared__ __attribute__((aligned(16))) float Ts[KB * 32 * TLD];
+  const int MW = 2 * nb - 1, NW = nb;
+  const int nzt = (int)((nbatch + ZT - 1) / ZT);
+  int m, zt;
+  if (!decode_block(MW, nb, nzt, m, zt)) return;
+  const int mi = m + nb - 1;
+  const long z0 = (long)zt * ZT;
+  const long nspec = (long)nl * (4L * nl * nl - 1) / 3;
+  const int am = abs(m);
+  const int l4start = am >> 2;
+
+  const int t = threadIdx.x;
+  const int zq = t & 7, n = t >> 3;
+  float2 acc[32][2];
+#pragma unroll
+  for (int l = 0; l < 32; ++l) { acc[l][0] = make_float2(0.f, 0.f); acc[l][1] = make_float2(0.f, 0.f); }
+
+  // loader roles
+  const int ln = t & 31;            // n for both loaders
+  const int lr = t >> 5;            // 0..7: z (X loader, + 8) / l (T loader, + 8 j)
+  const size_t plane = (size_t)MW * NW;
+
+  for (int b0 = 0; b0 < n2; b0 += KB) {
+    __syncthreads();
+    // X chunk: [KB][ZT][n]
+#pragma unroll
+    for (int i = 0; i < KB * 2; ++i) {
+      const int bt = i >> 1, z = lr + 8 * (i & 1);
+      float2 v = make_float2(0.f, 0.f);
+      if (ln < NW && z0 + z < nbatch && b0 + bt < n2)
+        v = X[(((size_t)(z0 + z) * n2 + (b0 + bt)) * MW + mi) * NW + ln];
+      Xs[(bt * ZT + z) * XLD + ln] = v;
+    }
+    // T chunk: [KB][n][l], zero outside the valid (l, n) range
+    for (int bt = 0; bt < KB; ++bt) {
+      const float* Tr = T + (size_t)(b0 + bt) * nspec;
+      const bool bok = b0 + bt < n2;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int l = lr + 8 * j;
+        float v = 0.f;
+        if (bok && ln < NW && l < nl && l >= am && l >= ln) v = Tr[lmn_index(l, m, ln)];
+        Ts[(bt * 32 + ln) * TLD + l] = v;
+      }
+    }
+    __syncthreads();
+#pragma unroll 2
+    for (int bt = 0; bt < KB; ++bt) {
+      const float2 x0 = Xs[(bt * ZT + 2 * zq) * XLD + n];
+      const float2 x1 = Xs[(bt * ZT + 2 * zq + 1) * XLD + n];
+      const float4* tr = reinterpret_cast<const float4*>(Ts + (bt * 32 + n) * TLD);
+#pragma unroll
+      for (int l4 = 0; l4 < 8; ++l4) {
+        if (l4 >= l4start) {
+          const float4 tv = tr[l4];
+          const float tt[4] = {tv.x, tv.y, tv.z, tv.w};
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            acc[4 * l4 + u][0].x += tt[u] * x0.x; acc[4 * l4 + u][0].y += tt[u] * x0.y;
+            acc[4 * l4 + u][1].x += tt[u] * x1.x; acc[4 * l4 + u][1].y += tt[u] * x1.y;
+          }
+        }
+      }
+    }
+  }
+
+  // ---- write out[lmn][z] and its mirror (-m,-n); (m < 0, n = 0) is written by the workgroup of -m
+  if (n >= NW || (n == 0 && m < 0)) return;
+  const long z = z0 + 2 * zq;
+  if (z >= nbatch) return;
+  const bool pair = (z + 1 < nbatch);
+  const bool vec = pair && ((nbatch & 1) == 0);
+  const bool mirror = (n > 0 || m > 0);
+  const float sgn = ((m - n) & 1) ? -1.f : 1.f;
+  const int lmin = am > n ? am : n;
+#pragma unroll
+  for (int l = 0; l < 32; ++l) {
+    if (l >= lmin && l < nl) {
+      const float2 a0 = acc[l][0], a1 = acc[l][1];
+      float2* p = out + (size_t)lmn_index(l, m, n) * nbatch + z;
+      if (vec) *reinterpret_cast<float4*>(p) = make_float4(a0.x, a0.y, a1.x, a1.y);
+      else { p[0] = a0; if (pair) p[1] = a1; }
+      if (mirror) {
+        float2* q = out + (size_t)lmn_index(l, -m, -n) * nbatch + z;
+        if (vec) *reinterpret_cast<float4*>(q) = make_float4(sgn * a0.x, -sgn * a0.y, sgn * a1.x, -sgn * a1.y);
+        else { q[0] = make_float2(sgn * a0.x, -sgn * a0.y); if (pair) q[1] = make_float2(sgn * a1.x, -sgn * a1.y); }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// synthesis: 512 threads, thread = (n = t % 32, zq = (t / 32) % 8, beta half = t / 256)
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(512) void wigner_inv_tiled(const float2* __restrict__ xh, const float* __restrict__ T,
+                                                        float2* __restrict__ S, int n2, int nb, int b_spec, long nbatch) {
+  __shared__ __attribute__((aligned(16))) float2 xs[LC * ZT * SLD];
+  __shared__ __attribute__((aligned(16))) float Tq[LC * 32 * QLD];
+  const int MW = 2 * nb - 1, NW = nb;
+  const int nzt = (int)((nbatch + ZT - 1) / ZT);
+  int m, zt;
+  if (!decode_block(MW, nb, nzt, m, zt)) return;
+  const int mi = m + nb - 1;
+  const long z0 = (long)zt * ZT;
+  const long nspec = (long)b_spec * (4L * b_spec * b_spec - 1) / 3;
+  const int am = abs(m);
+
+  const int t = threadIdx.x;
+  const int n = t & 31, zq = (t >> 5) & 7, bh = t >> 8;
+  float2 acc[32][2];
+#pragma unroll
+  for (int j = 0; j < 32; ++j) { acc[j][0] = make_float2(0.f, 0.f); acc[j][1] = make_float2(0.f, 0.f); }
+
+  const int xz = t & 15, xn = t >> 4;           // spectrum loader: z fastest (contiguous in memory), n = 0..31
+  const float hs = ((m & 1) ? -0.5f : 0.5f);    // (-1)^(m-n)/2 = hs * (-1)^n
+
+  for (int l0 = (am / LC) * LC; l0 < nb; l0 += LC) {
+    __syncthreads();
+    // symmetrised spectrum chunk: [LC][ZT][n]
+#pragma unroll
+    for (int i = 0; i < LC; ++i) {
+      const int l = l0 + i;
+      float2 v = make_float2(0.f, 0.f);
+      if (l < nb && l >= am && l >= xn && xn < NW && z0 + xz < nbatch) {
+        const float2 a = xh[(size_t)lmn_index(l, m, xn) * nbatch + z0 + xz];
+        const float2 b = xh[(size_t)lmn_index(l, -m, -xn) * nbatch + z0 + xz];
+        const float s = (xn & 1) ? -hs : hs;
+        v = make_float2(0.5f * a.x + s * b.x, 0.5f * a.y - s * b.y);
+      }
+      xs[(i * ZT + xz) * SLD + xn] = v;
+    }
+    // T chunk: [LC][n][beta]
+    for (int i = 0; i < LC; ++i) {
+      const int l = l0 + i;
+      const bool ok = (l < nb && l >= am && l >= n && n < NW);
+      const int idx = ok ? lmn_index(l, m, n) : 0;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int bt = (t >> 5) + 16 * j;
+        float v = 0.f;
+        if (ok && bt < n2) v = T[(size_t)bt * nspec + idx];
+        Tq[(i * 32 + n) * QLD + bt] = v;
+      }
+    }
+    __syncthreads();
+#pragma unroll 2
+    for (int i = 0; i < LC; ++i) {
+      if (l0 + i < am || l0 + i >= nb) continue;
+      const float2 x0 = xs[(i * ZT + 2 * zq) * SLD + n];
+      const float2 x1 = xs[(i * ZT + 2 * zq + 1) * SLD + n];
+      const float4* tr = reinterpret_cast<const float4*>(Tq + (i * 32 + n) * QLD + 32 * bh);
+#pragma unroll
+      for (int b4 = 0; b4 < 8; ++b4) {
+        const float4 tv = tr[b4];
+        const float tt[4] = {tv.x, tv.y, tv.z, tv.w};
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          acc[4 * b4 + u][0].x += tt[u] * x0.x; acc[4 * b4 + u][0].y += tt[u] * x0.y;
+          acc[4 * b4 + u][1].x += tt[u] * x1.x; acc[4 * b4 + u][1].y += tt[u] * x1.y;
+        }
+      }
+    }
+  }
+
+  if (n >= NW) return;
+  const size_t plane = (size_t)MW * NW;
+#pragma unroll
+  for (int zz = 0; zz < 2; ++zz) {
+    const long z = z0 + 2 * zq + zz;
+    if (z >= nbatch) continue;
+    float2* p = S + ((size_t)z * n2 * MW + mi) * NW + n;
+#pragma unroll
+    for (int j = 0; j < 32; ++j) {
+      const int bt = 32 * bh + j;
+      if (bt < n2) p[(size_t)bt * plane] = acc[j][zz];
+    }
+  }
+}
+
+}  // namespace wigner_tiled

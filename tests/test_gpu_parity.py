@@ -73,7 +73,7 @@ def test_s2_mm_forward_backward(hip, nl, B, Fi, Fo):
 
 
 # ------------------------------------------------------------------ SO(3) transforms
-SO3_PAIRS = [(2, 9), (6, 6), (9, 2), (10, 11), (11, 10), (7, 5), (4, 6), (16, 16)]   # first five: tests/so3_fft.py:102
+SO3_PAIRS = [(2, 9), (6, 6), (9, 2), (10, 11), (11, 10), (7, 5), (4, 6), (16, 16), (32, 32), (32, 12), (12, 32)]   # first five: tests/so3_fft.py:102
 
 
 @pytest.mark.parametrize("b_in,b_out", SO3_PAIRS)
