@@ -81,6 +81,8 @@ int s2cnn_s2_mm_grady(const float *gz, const float *x, float *gy,
  *       [nbatch, 2b_in, 2b_in, 2b_in, 2]   (complex_in = 1)
  * table [2b_in, nspec(b_out)]  row beta_j, entries scale * d^l_{mn}(beta_j); must satisfy
  *       table[j, l,-m,-n] = (-1)^(m-n) table[j, l,m,n] (true of Wigner small-d)
+ * packed_table  NULL, or the same table repacked once by s2cnn_so3_pack_table(..., synthesis = 0)
+ *       (skips a per-call repack on the fast path; ignored where the fast path does not apply)
  * out   [nspec(b_out), nbatch, 2]
  *       out[l,m,n,z] = sum_beta table[beta,lmn] sum_{alpha,gamma} x[z,beta,alpha,gamma]
  *                      exp(-i(m alpha + n gamma)),   0 where |m| or |n| >= b_in
@@ -89,13 +91,14 @@ int s2cnn_s2_mm_grady(const float *gz, const float *x, float *gy,
  * workspace: s2cnn_so3_analysis_workspace(...) bytes of device scratch, 256-byte aligned.
  */
 size_t s2cnn_so3_analysis_workspace(int b_in, int b_out, long nbatch, int complex_in);
-int s2cnn_so3_analysis(const float *x, const float *table, float *out,
+int s2cnn_so3_analysis(const float *x, const float *table, const float *packed_table, float *out,
                        void *workspace, size_t workspace_bytes,
                        int b_in, int b_out, long nbatch, int complex_in, void *stream);
 
 /* ---- SO(3) Fourier synthesis: spectrum -> grid -------------------------------------
  * xhat  [nspec(b_in), nbatch, 2]
  * table [2b_out, nspec(b_in)]   (same symmetry requirement as above)
+ * packed_table  NULL, or s2cnn_so3_pack_table(table, ..., synthesis = 1) of the same table
  * out   [nbatch, 2b_out, 2b_out, 2b_out]     (complex_out = 0): the REAL PART of
  *       [nbatch, 2b_out, 2b_out, 2b_out, 2]  (complex_out = 1):
  *       y[z,beta,alpha,gamma] = sum_{l < min(b_in,b_out)} sum_{m,n} xhat[l,m,n,z]
@@ -105,9 +108,21 @@ int s2cnn_so3_analysis(const float *x, const float *table, float *out,
  * (so3_fft.py:158-202, CPU-branch semantics) and so3_ifft (so3_fft.py:115-155).
  */
 size_t s2cnn_so3_synthesis_workspace(int b_in, int b_out, long nbatch, int complex_out);
-int s2cnn_so3_synthesis(const float *xhat, const float *table, float *out,
+int s2cnn_so3_synthesis(const float *xhat, const float *table, const float *packed_table, float *out,
                         void *workspace, size_t workspace_bytes,
                         int b_in, int b_out, long nbatch, int complex_out, void *stream);
+
+/* ---- table repacking for the real-signal fast path of the two transforms above ------
+ * The reference uploads its Wigner table once per (b, nl, weighted, device) and reuses it
+ * (soft/so3_fft.py:205-209); a caller of this library does the same with the packed copy:
+ *   bytes = s2cnn_so3_packed_table_bytes(b_in, b_out, synthesis)   (0: no fast path for these sizes)
+ *   s2cnn_so3_pack_table(table, packed, b_in, b_out, synthesis, stream)
+ * b_in / b_out have the meaning they have in the transform the table is for; `packed` must be
+ * 16-byte aligned.  Passing packed_table = NULL to a transform is always valid (it repacks into
+ * its workspace on every call).
+ */
+size_t s2cnn_so3_packed_table_bytes(int b_in, int b_out, int synthesis);
+int s2cnn_so3_pack_table(const float *table, float *packed, int b_in, int b_out, int synthesis, void *stream);
 
 /* ---- S^2 Fourier analysis / synthesis ----------------------------------------------
  * analysis : x [nbatch, 2b_in, 2b_in] (complex_in = 0) or [..., 2] (complex_in = 1),

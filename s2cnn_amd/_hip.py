@@ -18,6 +18,7 @@ _int, _long, _size_t, _vp = ctypes.c_int, ctypes.c_long, ctypes.c_size_t, ctypes
 
 _MM_SIG = [_c_float_p, _c_float_p, _c_float_p, _int, _int, _int, _int, _vp]
 _FT_SIG = [_c_float_p, _c_float_p, _c_float_p, _vp, _size_t, _int, _int, _long, _int, _vp]
+_FT3_SIG = [_c_float_p, _c_float_p, _c_float_p, _c_float_p, _vp, _size_t, _int, _int, _long, _int, _vp]
 _WS_SIG = [_int, _int, _long, _int]
 
 SIGNATURES = {
@@ -30,9 +31,11 @@ SIGNATURES = {
     "s2cnn_s2_mm_gradx": (_int, _MM_SIG),
     "s2cnn_s2_mm_grady": (_int, _MM_SIG),
     "s2cnn_so3_analysis_workspace": (_size_t, _WS_SIG),
-    "s2cnn_so3_analysis": (_int, _FT_SIG),
+    "s2cnn_so3_analysis": (_int, _FT3_SIG),
     "s2cnn_so3_synthesis_workspace": (_size_t, _WS_SIG),
-    "s2cnn_so3_synthesis": (_int, _FT_SIG),
+    "s2cnn_so3_synthesis": (_int, _FT3_SIG),
+    "s2cnn_so3_packed_table_bytes": (_size_t, [_int, _int, _int]),
+    "s2cnn_so3_pack_table": (_int, [_c_float_p, _c_float_p, _int, _int, _int, _vp]),
     "s2cnn_s2_analysis_workspace": (_size_t, _WS_SIG),
     "s2cnn_s2_analysis": (_int, _FT_SIG),
     "s2cnn_s2_synthesis_workspace": (_size_t, _WS_SIG),

@@ -43,7 +43,7 @@ __device__ inline void fill_twiddles(float2* w, int n2) {
 // ---------------------------------------------------------------------------------------
 template <bool CPLX>
 __global__ __launch_bounds__(256) void so3_plane_dft_fwd(const float* __restrict__ x, float2* __restrict__ X,
-                                                         int n2, int nb) {
+                                                         int n2, int nb, int ztile) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
   const int MW = 2 * nb - 1;
   const int NW = CPLX ? MW : nb;
@@ -82,7 +82,14 @@ __global__ __launch_bounds__(256) void so3_plane_dft_fwd(const float* __restrict
   __syncthreads();
 
   // X[mi][ni] = sum_alpha Y[alpha][ni] w^(m alpha)
+  // ztile = 0: X is [plane][mi][ni];  ztile = Z > 0: [z / Z][mi][beta][z % Z][ni] (plane = z * n2 + beta)
   float2* dst = X + pl * (size_t)(MW * NW);
+  size_t mstride = NW;
+  if (ztile > 0) {
+    const size_t z = pl / n2, beta = pl % n2;
+    dst = X + ((z / ztile) * MW * n2 + beta) * ztile * NW + (z % ztile) * NW;
+    mstride = (size_t)n2 * ztile * NW;
+  }
   for (int o = threadIdx.x; o < MW * NW; o += blockDim.x) {
     const int mi = o / NW, ni = o - mi * NW;
     const int m = mi - (nb - 1);
@@ -94,7 +101,7 @@ __global__ __launch_bounds__(256) void so3_plane_dft_fwd(const float* __restrict
       acc.x += pr.x; acc.y += pr.y;
       tw += step; if (tw >= n2) tw -= n2;
     }
-    dst[o] = acc;
+    dst[mi * mstride + ni] = acc;
   }
 }
 
@@ -271,11 +278,13 @@ __global__ __launch_bounds__(256) void so3_plane_dft_inv(const float2* __restric
   }
 }
 
+// batch items padded to the z tile of the tiled Wigner kernels
 size_t ws_bytes(int b_grid, int b_spec, long nbatch, int cplx) {
   if (b_grid < 1 || b_spec < 1 || nbatch < 1) return 0;
   const long nb = b_grid < b_spec ? b_grid : b_spec;
   const long MW = 2 * nb - 1, NW = cplx ? MW : nb;
-  return (size_t)nbatch * (2 * b_grid) * MW * NW * sizeof(float2);
+  const long zpad = (nbatch + wigner_tiled::ZT - 1) / wigner_tiled::ZT * wigner_tiled::ZT;
+  return (size_t)zpad * (2 * b_grid) * MW * NW * sizeof(float2);
 }
 
 bool sizes_ok(int b_grid, int b_spec, long nbatch) {
@@ -283,23 +292,54 @@ bool sizes_ok(int b_grid, int b_spec, long nbatch) {
          nbatch * 2L * b_grid < (1L << 31) && (nbatch + 15) / 16 <= 65535;
 }
 
+// Bytes of the packed table of the tiled fast path; 0 when that path does not apply.
+size_t packed_bytes(int b_grid, int b_spec, int cplx, bool synthesis) {
+  const int nb = b_grid < b_spec ? b_grid : b_spec;
+  if (cplx || nb > 32) return 0;
+  if (synthesis) return 2 * b_grid <= 64 ? wigner_tiled::packed_floats_synthesis(nb) * sizeof(float) : 0;
+  return b_spec <= 32 ? wigner_tiled::packed_floats_analysis(2 * b_grid, nb) * sizeof(float) : 0;
+}
+
+size_t round256(size_t n) { return (n + 255) & ~(size_t)255; }
+
 }  // namespace
 
+extern "C" size_t s2cnn_so3_packed_table_bytes(int b_in, int b_out, int synthesis) {
+  if (b_in < 1 || b_out < 1) return 0;
+  return synthesis ? packed_bytes(b_out, b_in, 0, true) : packed_bytes(b_in, b_out, 0, false);
+}
+
+extern "C" int s2cnn_so3_pack_table(const float* table, float* packed, int b_in, int b_out, int synthesis, void* stream) {
+  if (!table || !packed || b_in < 1 || b_out < 1 || b_in > 512 || b_out > 512) return S2CNN_EINVAL;
+  if (s2cnn_so3_packed_table_bytes(b_in, b_out, synthesis) == 0) return S2CNN_EINVAL;
+  if (!s2cnn::aligned16(packed)) return S2CNN_EALIGN;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int nb = b_in < b_out ? b_in : b_out;
+  if (synthesis)
+    hipLaunchKernelGGL(wigner_tiled::pack_table_synthesis, dim3(2048), dim3(256), 0, st, table, packed, 2 * b_out, nb, b_in);
+  else
+    hipLaunchKernelGGL(wigner_tiled::pack_table_analysis, dim3(2048), dim3(256), 0, st, table, packed, 2 * b_in, nb, b_out);
+  return s2cnn::launch_status();
+}
+
 extern "C" size_t s2cnn_so3_analysis_workspace(int b_in, int b_out, long nbatch, int complex_in) {
-  return ws_bytes(b_in, b_out, nbatch, complex_in);
+  const size_t w = ws_bytes(b_in, b_out, nbatch, complex_in);
+  return w ? round256(w) + packed_bytes(b_in, b_out, complex_in, false) : 0;
 }
 
 extern "C" size_t s2cnn_so3_synthesis_workspace(int b_in, int b_out, long nbatch, int complex_out) {
-  return ws_bytes(b_out, b_in, nbatch, complex_out);
+  const size_t w = ws_bytes(b_out, b_in, nbatch, complex_out);
+  return w ? round256(w) + packed_bytes(b_out, b_in, complex_out, true) : 0;
 }
 
-extern "C" int s2cnn_so3_analysis(const float* x, const float* table, float* out, void* workspace,
-                                  size_t workspace_bytes, int b_in, int b_out, long nbatch, int complex_in,
-                                  void* stream) {
+extern "C" int s2cnn_so3_analysis(const float* x, const float* table, const float* packed_table, float* out,
+                                  void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
+                                  int complex_in, void* stream) {
   if (!x || !table || !out || !sizes_ok(b_in, b_out, nbatch)) return S2CNN_EINVAL;
   if (!s2cnn::aligned8(out) || (complex_in && !s2cnn::aligned8(x))) return S2CNN_EALIGN;
-  const size_t need = ws_bytes(b_in, b_out, nbatch, complex_in);
-  if (!workspace || workspace_bytes < need || !s2cnn::aligned8(workspace)) return S2CNN_EWORKSPACE;
+  if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
+  const size_t need = s2cnn_so3_analysis_workspace(b_in, b_out, nbatch, complex_in);
+  if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int n2 = 2 * b_in, nb = b_in < b_out ? b_in : b_out;
   const int MW = 2 * nb - 1, NW = complex_in ? MW : nb;
@@ -307,16 +347,18 @@ extern "C" int s2cnn_so3_analysis(const float* x, const float* table, float* out
   const size_t lds = sizeof(float) * (2 * n2 + (complex_in ? 2 : 1) * n2 * n2 + 2 * n2 * NW);
   if (lds > 160 * 1024) return S2CNN_EINVAL;
   const unsigned planes = (unsigned)(nbatch * n2);
-  const bool tiled = !complex_in && nb <= 32 && b_out <= 32;
+  const bool tiled = packed_bytes(b_in, b_out, complex_in, false) != 0;
+  const bool x16 = s2cnn::aligned16(x);
   if (complex_in) {
     if (lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)so3_plane_dft_fwd<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    hipLaunchKernelGGL(so3_plane_dft_fwd<true>, dim3(planes), dim3(256), lds, st, x, X, n2, nb);
-  } else if (n2 == 64) {
+    hipLaunchKernelGGL(so3_plane_dft_fwd<true>, dim3(planes), dim3(256), lds, st, x, X, n2, nb, 0);
+  } else if (n2 == 64 && x16) {
     const long npairs = nbatch * 32;
-    hipLaunchKernelGGL(fft64::plane_fft64_fwd, dim3((unsigned)(npairs < 2048 ? npairs : 2048)), dim3(fft64::THREADS), 0, st, x, X, npairs, nb);
+    hipLaunchKernelGGL(fft64::plane_fft64_fwd, dim3((unsigned)(npairs < 2048 ? npairs : 2048)), dim3(fft64::THREADS), 0, st, x, X, npairs, nb,
+                       tiled ? wigner_tiled::ZT : 0);
   } else {
     if (lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)so3_plane_dft_fwd<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    hipLaunchKernelGGL(so3_plane_dft_fwd<false>, dim3(planes), dim3(256), lds, st, x, X, n2, nb);
+    hipLaunchKernelGGL(so3_plane_dft_fwd<false>, dim3(planes), dim3(256), lds, st, x, X, n2, nb, tiled ? wigner_tiled::ZT : 0);
   }
   int rc = s2cnn::launch_status();
   if (rc) return rc;
@@ -324,24 +366,33 @@ extern "C" int s2cnn_so3_analysis(const float* x, const float* table, float* out
     const size_t nfl = (size_t)s2cnn::so3_nspec(b_out) * nbatch * 2;
     hipLaunchKernelGGL(fill_zero, dim3(1024), dim3(256), 0, st, out, nfl);
   }
-  dim3 grid(s2cnn::ceil_div(NW, 16), MW, (unsigned)((nbatch + 15) / 16));
-  if (tiled)
-    hipLaunchKernelGGL(wigner_tiled::wigner_fwd_tiled, dim3(wigner_tiled::grid_size(MW, nbatch)), dim3(256), 0, st, X, table,
+  if (tiled) {
+    const float* Tp = packed_table;
+    if (!Tp) {  // pack on the fly behind the intermediate
+      float* dst = reinterpret_cast<float*>(static_cast<char*>(workspace) + round256(ws_bytes(b_in, b_out, nbatch, complex_in)));
+      hipLaunchKernelGGL(wigner_tiled::pack_table_analysis, dim3(2048), dim3(256), 0, st, table, dst, n2, nb, b_out);
+      Tp = dst;
+    }
+    hipLaunchKernelGGL(wigner_tiled::wigner_fwd_tiled, dim3(wigner_tiled::grid_size(MW, nbatch)), dim3(256), 0, st, X, Tp,
                        reinterpret_cast<float2*>(out), n2, nb, b_out, nbatch);
-  else if (complex_in)
+    return s2cnn::launch_status();
+  }
+  dim3 grid(s2cnn::ceil_div(NW, 16), MW, (unsigned)((nbatch + 15) / 16));
+  if (complex_in)
     hipLaunchKernelGGL(so3_wigner_fwd<true>, grid, dim3(16, 16), 0, st, X, table, reinterpret_cast<float2*>(out), n2, nb, b_out, nbatch);
   else
     hipLaunchKernelGGL(so3_wigner_fwd<false>, grid, dim3(16, 16), 0, st, X, table, reinterpret_cast<float2*>(out), n2, nb, b_out, nbatch);
   return s2cnn::launch_status();
 }
 
-extern "C" int s2cnn_so3_synthesis(const float* xhat, const float* table, float* out, void* workspace,
-                                   size_t workspace_bytes, int b_in, int b_out, long nbatch, int complex_out,
-                                   void* stream) {
+extern "C" int s2cnn_so3_synthesis(const float* xhat, const float* table, const float* packed_table, float* out,
+                                   void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
+                                   int complex_out, void* stream) {
   if (!xhat || !table || !out || !sizes_ok(b_out, b_in, nbatch)) return S2CNN_EINVAL;
   if (!s2cnn::aligned8(xhat) || (complex_out && !s2cnn::aligned8(out))) return S2CNN_EALIGN;
-  const size_t need = ws_bytes(b_out, b_in, nbatch, complex_out);
-  if (!workspace || workspace_bytes < need || !s2cnn::aligned8(workspace)) return S2CNN_EWORKSPACE;
+  if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
+  const size_t need = s2cnn_so3_synthesis_workspace(b_in, b_out, nbatch, complex_out);
+  if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int n2 = 2 * b_out, nb = b_in < b_out ? b_in : b_out;
   const int MW = 2 * nb - 1, NW = complex_out ? MW : nb;
@@ -350,20 +401,28 @@ extern "C" int s2cnn_so3_synthesis(const float* xhat, const float* table, float*
   if (lds > 160 * 1024) return S2CNN_EINVAL;
   dim3 grid(s2cnn::ceil_div(NW, 16), MW, (unsigned)((nbatch + 15) / 16));
   const float2* xh = reinterpret_cast<const float2*>(xhat);
-  if (complex_out)
-    hipLaunchKernelGGL(so3_wigner_inv<true>, grid, dim3(16, 16), 0, st, xh, table, S, n2, nb, b_in, nbatch);
-  else if (nb <= 32 && n2 <= 64)
-    hipLaunchKernelGGL(wigner_tiled::wigner_inv_tiled, dim3(wigner_tiled::grid_size(MW, nbatch)), dim3(512), 0, st, xh, table, S,
+  const bool tiled = packed_bytes(b_out, b_in, complex_out, true) != 0;
+  if (tiled) {
+    const float* Tq = packed_table;
+    if (!Tq) {
+      float* dst = reinterpret_cast<float*>(static_cast<char*>(workspace) + round256(ws_bytes(b_out, b_in, nbatch, complex_out)));
+      hipLaunchKernelGGL(wigner_tiled::pack_table_synthesis, dim3(2048), dim3(256), 0, st, table, dst, n2, nb, b_in);
+      Tq = dst;
+    }
+    hipLaunchKernelGGL(wigner_tiled::wigner_inv_tiled, dim3(wigner_tiled::grid_size(MW, nbatch)), dim3(512), 0, st, xh, Tq, S,
                        n2, nb, b_in, nbatch);
-  else
+  } else if (complex_out) {
+    hipLaunchKernelGGL(so3_wigner_inv<true>, grid, dim3(16, 16), 0, st, xh, table, S, n2, nb, b_in, nbatch);
+  } else {
     hipLaunchKernelGGL(so3_wigner_inv<false>, grid, dim3(16, 16), 0, st, xh, table, S, n2, nb, b_in, nbatch);
+  }
   int rc = s2cnn::launch_status();
   if (rc) return rc;
   const unsigned planes = (unsigned)(nbatch * n2);
   if (complex_out) {
     if (lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)so3_plane_dft_inv<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     hipLaunchKernelGGL(so3_plane_dft_inv<true>, dim3(planes), dim3(256), lds, st, S, out, n2, nb);
-  } else if (n2 == 64) {
+  } else if (n2 == 64 && s2cnn::aligned16(out)) {
     const long npairs = nbatch * 32;
     hipLaunchKernelGGL(fft64::plane_fft64_inv, dim3((unsigned)(npairs < 2048 ? npairs : 2048)), dim3(fft64::THREADS), 0, st, S, out, npairs, nb);
   } else {

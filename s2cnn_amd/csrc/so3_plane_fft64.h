@@ -119,8 +119,10 @@ __device__ __forceinline__ void make_twiddles(float2 (&tw)[8]) {
 
 // Forward: planes 2q, 2q+1 of x ([planes][64][64] real) -> X ([planes][mw][nb] complex), the bins
 // m = -(nb-1)..nb-1, n = 0..nb-1 of each plane's 2-D DFT.  Grid-stride over plane pairs.
+// ztile = 0: X is [plane][mi][n];  ztile = Z > 0: X is [z / Z][mi][beta][z % Z][n] (plane = z * 64 + beta),
+// the order in which the tiled Wigner contraction streams it.
 __global__ __launch_bounds__(THREADS) void plane_fft64_fwd(const float* __restrict__ x, float2* __restrict__ X,
-                                                           long npairs, int nb) {
+                                                           long npairs, int nb, int ztile) {
   __shared__ float2 buf[LDS_ELEMS];
   float2 tw[8];
   make_twiddles<false>(tw);
@@ -139,15 +141,28 @@ __global__ __launch_bounds__(THREADS) void plane_fft64_fwd(const float* __restri
     __syncthreads();
     transform_2d<false>(buf, tw);
     // Z = A + iB with A, B Hermitian:  A[m,n] = (Z[m,n] + conj Z[-m,-n]) / 2,  B[m,n] = (Z[m,n] - conj Z[-m,-n]) / (2i)
-    float2* Xa = X + pair * 2 * (size_t)(MW * nb);
-    float2* Xb = Xa + (size_t)MW * nb;
+    // element (mi, n) of plane a at Xa[mi * mstride + n]; plane b (the next beta) at + bstride
+    float2* Xa;
+    size_t mstride, bstride;
+    if (ztile > 0) {
+      const long z = pair >> 5;
+      const int beta = (int)(pair & 31) * 2;
+      Xa = X + ((size_t)(z / ztile) * MW * N + beta) * ztile * nb + (size_t)(z % ztile) * nb;
+      mstride = (size_t)N * ztile * nb;
+      bstride = (size_t)ztile * nb;
+    } else {
+      Xa = X + pair * 2 * (size_t)(MW * nb);
+      mstride = nb;
+      bstride = (size_t)MW * nb;
+    }
     for (int o = threadIdx.x; o < MW * nb; o += THREADS) {
       const int mi = o / nb, n = o - mi * nb;
       const int m = mi - (nb - 1);
       const float2 z1 = buf[sigma(m & 63) * PITCH + sigma(n)];
       const float2 z2 = buf[sigma((-m) & 63) * PITCH + sigma((-n) & 63)];
-      Xa[o] = make_float2(0.5f * (z1.x + z2.x), 0.5f * (z1.y - z2.y));
-      Xb[o] = make_float2(0.5f * (z1.y + z2.y), 0.5f * (z2.x - z1.x));
+      float2* d = Xa + mi * mstride + n;
+      d[0] = make_float2(0.5f * (z1.x + z2.x), 0.5f * (z1.y - z2.y));
+      d[bstride] = make_float2(0.5f * (z1.y + z2.y), 0.5f * (z2.x - z1.x));
     }
     __syncthreads();
   }

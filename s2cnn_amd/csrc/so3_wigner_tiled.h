@@ -6,9 +6,11 @@
 //   synthesis: S[z,beta,m,n] = sum_l   T[beta, lmn] xs[l,m,n,z]            (accumulators over beta)
 //              xs = (xhat[l,m,n] + (-1)^(m-n) conj xhat[l,-m,-n]) / 2
 //
-// The table is read in its public layout [2b][nspec]; for fixed (beta, l, m) the entries n = 0..l
-// are contiguous.  Requirements: nb = min(b_grid, b_spec) <= 32, degrees <= 32 (analysis),
-// 2 b_grid <= 64 (synthesis).
+// The table is consumed in a packed, zero-padded order that makes every chunk one contiguous block:
+//   analysis : Tp[mi][beta][n (32)][l (32)]        (pack_table_analysis)
+//   synthesis: Tq[mi][l (nb)][n (32)][beta (64)]   (pack_table_synthesis)
+// with zeros outside max(|m|, n) <= l < number of degrees, n < nb, beta < 2 b_grid.
+// Requirements: nb = min(b_grid, b_spec) <= 32, degrees <= 32 (analysis), 2 b_grid <= 64 (synthesis).
 #pragma once
 #include <hip/hip_runtime.h>
 
@@ -42,10 +44,42 @@ inline int grid_size(int MW, long nbatch) {
   return (int)(8L * ((MW + 7) / 8) * nzt);
 }
 
+__host__ __device__ inline size_t packed_floats_analysis(int n2, int nb) { return (size_t)(2 * nb - 1) * n2 * 1024; }
+__host__ __device__ inline size_t packed_floats_synthesis(int nb) { return (size_t)(2 * nb - 1) * nb * 32 * 64; }
+
+// one thread per packed element
+__global__ void pack_table_analysis(const float* __restrict__ T, float* __restrict__ Tp, int n2, int nb, int nl) {
+  const size_t total = packed_floats_analysis(n2, nb);
+  const long nspec = (long)nl * (4L * nl * nl - 1) / 3;
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+    const int l = i & 31, n = (i >> 5) & 31;
+    const size_t r = i >> 10;
+    const int bt = (int)(r % n2), m = (int)(r / n2) - (nb - 1);
+    const int am = m < 0 ? -m : m;
+    float v = 0.f;
+    if (n < nb && l < nl && l >= am && l >= n) v = T[(size_t)bt * nspec + lmn_index(l, m, n)];
+    Tp[i] = v;
+  }
+}
+
+__global__ void pack_table_synthesis(const float* __restrict__ T, float* __restrict__ Tq, int n2, int nb, int b_spec) {
+  const size_t total = packed_floats_synthesis(nb);
+  const long nspec = (long)b_spec * (4L * b_spec * b_spec - 1) / 3;
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+    const int bt = i & 63, n = (i >> 6) & 31;
+    const size_t r = i >> 11;
+    const int l = (int)(r % nb), m = (int)(r / nb) - (nb - 1);
+    const int am = m < 0 ? -m : m;
+    float v = 0.f;
+    if (n < nb && bt < n2 && l >= am && l >= n) v = T[(size_t)bt * nspec + lmn_index(l, m, n)];
+    Tq[i] = v;
+  }
+}
+
 // ---------------------------------------------------------------------------------------------
 // analysis: 256 threads, thread = (zq = t % 8 -> z = 2 zq, 2 zq + 1 ; n = t / 8)
 // ---------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void wigner_fwd_tiled(const float2* __restrict__ X, const float* __restrict__ T,
+__global__ __launch_bounds__(256) void wigner_fwd_tiled(const float2* __restrict__ X, const float* __restrict__ Tp,
                                                         float2* __restrict__ out, int n2, int nb, int nl, long nbatch) {
   __shared__ __attribute__((aligned(16))) float2 Xs[KB * ZT * XLD];
   __shared__ __attribute__((aligned(16))) float Ts[KB * 32 * TLD];
@@ -65,35 +99,53 @@ __global__ __launch_bounds__(256) void wigner_fwd_tiled(const float2* __restrict
 #pragma unroll
   for (int l = 0; l < 32; ++l) { acc[l][0] = make_float2(0.f, 0.f); acc[l][1] = make_float2(0.f, 0.f); }
 
-  // loader roles
-  const int ln = t & 31;            // n for both loaders
-  const int lr = t >> 5;            // 0..7: z (X loader, + 8) / l (T loader, + 8 j)
-  const size_t plane = (size_t)MW * NW;
+  // Loads are unconditional (clamped addresses, values zeroed by select) so that all of a chunk's
+  // loads are in flight together, and the next chunk is fetched while the current one is consumed.
+  float2 xr[KB * 2];
+  float4 tr_[KB];
+  // packed table: the chunk of KB betas is KB*1024 contiguous floats; slot i covers floats 4 (t + 256 i)..+3,
+  // i.e. beta_local = i, n = t / 8, l = 4 (t % 8)
+  const float4* tbase = reinterpret_cast<const float4*>(Tp + (size_t)mi * n2 * 1024);
+  const int tlds = (t >> 3) * TLD + 4 * (t & 7);
+  // X is laid out [z tile][mi][beta][z % 16][n]: one chunk (KB betas) is KB*16*NW contiguous complex
+  // numbers; thread slot i covers element e = t + 256 i of the chunk.
+  const int chunk_elems = KB * ZT * NW;
+  const float2* xbase = X + ((size_t)zt * MW + mi) * n2 * ZT * NW;
+  const int n2elems = n2 * ZT * NW;
+  int xlds[KB * 2];
+#pragma unroll
+  for (int i = 0; i < KB * 2; ++i) {
+    const int e = t + 256 * i;
+    const int row = e / NW;                     // beta_local * 16 + z
+    xlds[i] = e < chunk_elems ? row * XLD + (e - row * NW) : -1;
+  }
 
-  for (int b0 = 0; b0 < n2; b0 += KB) {
-    __syncthreads();
-    // X chunk: [KB][ZT][n]
+  auto load_chunk = [&](int b0) {
+    const int e0 = b0 * ZT * NW;
 #pragma unroll
     for (int i = 0; i < KB * 2; ++i) {
-      const int bt = i >> 1, z = lr + 8 * (i & 1);
-      float2 v = make_float2(0.f, 0.f);
-      if (ln < NW && z0 + z < nbatch && b0 + bt < n2)
-        v = X[(((size_t)(z0 + z) * n2 + (b0 + bt)) * MW + mi) * NW + ln];
-      Xs[(bt * ZT + z) * XLD + ln] = v;
+      const int e = e0 + t + 256 * i;
+      const float2 v = xbase[e < n2elems ? e : 0];
+      xr[i] = e < n2elems ? v : make_float2(0.f, 0.f);
     }
-    // T chunk: [KB][n][l], zero outside the valid (l, n) range
-    for (int bt = 0; bt < KB; ++bt) {
-      const float* Tr = T + (size_t)(b0 + bt) * nspec;
-      const bool bok = b0 + bt < n2;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int l = lr + 8 * j;
-        float v = 0.f;
-        if (bok && ln < NW && l < nl && l >= am && l >= ln) v = Tr[lmn_index(l, m, ln)];
-        Ts[(bt * 32 + ln) * TLD + l] = v;
-      }
+    for (int bt = 0; bt < KB; ++bt) {
+      const int bc = b0 + bt < n2 ? b0 + bt : n2 - 1;
+      const float4 v = tbase[(size_t)bc * 256 + t];
+      tr_[bt] = b0 + bt < n2 ? v : make_float4(0.f, 0.f, 0.f, 0.f);
     }
+  };
+
+  load_chunk(0);
+  for (int b0 = 0; b0 < n2; b0 += KB) {
     __syncthreads();
+#pragma unroll
+    for (int i = 0; i < KB * 2; ++i)
+      if (xlds[i] >= 0) Xs[xlds[i]] = xr[i];
+#pragma unroll
+    for (int bt = 0; bt < KB; ++bt) *reinterpret_cast<float4*>(Ts + bt * 32 * TLD + tlds) = tr_[bt];
+    __syncthreads();
+    if (b0 + KB < n2) load_chunk(b0 + KB);
 #pragma unroll 2
     for (int bt = 0; bt < KB; ++bt) {
       const float2 x0 = Xs[(bt * ZT + 2 * zq) * XLD + n];
@@ -142,7 +194,7 @@ __global__ __launch_bounds__(256) void wigner_fwd_tiled(const float2* __restrict
 // ---------------------------------------------------------------------------------------------
 // synthesis: 512 threads, thread = (n = t % 32, zq = (t / 32) % 8, beta half = t / 256)
 // ---------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(512) void wigner_inv_tiled(const float2* __restrict__ xh, const float* __restrict__ T,
+__global__ __launch_bounds__(512) void wigner_inv_tiled(const float2* __restrict__ xh, const float* __restrict__ Tq_g,
                                                         float2* __restrict__ S, int n2, int nb, int b_spec, long nbatch) {
   __shared__ __attribute__((aligned(16))) float2 xs[LC * ZT * SLD];
   __shared__ __attribute__((aligned(16))) float Tq[LC * 32 * QLD];
@@ -164,35 +216,43 @@ __global__ __launch_bounds__(512) void wigner_inv_tiled(const float2* __restrict
   const int xz = t & 15, xn = t >> 4;           // spectrum loader: z fastest (contiguous in memory), n = 0..31
   const float hs = ((m & 1) ? -0.5f : 0.5f);    // (-1)^(m-n)/2 = hs * (-1)^n
 
-  for (int l0 = (am / LC) * LC; l0 < nb; l0 += LC) {
-    __syncthreads();
-    // symmetrised spectrum chunk: [LC][ZT][n]
+  // Unconditional (clamped) loads, next chunk fetched while the current one is consumed.
+  float2 xa[LC], xb[LC];
+  float4 tq[LC];
+  // packed table: degree l of this m is 32*64 contiguous floats; slot i covers floats 4 t..+3 of degree l0 + i,
+  // i.e. n = t / 16, beta = 4 (t % 16)
+  const float4* tbase = reinterpret_cast<const float4*>(Tq_g + (size_t)mi * nb * 2048);
+  const int tlds = (t >> 4) * QLD + 4 * (t & 15);
+  const long zc = z0 + xz < nbatch ? z0 + xz : nbatch - 1;
+
+  auto load_chunk = [&](int l0) {
 #pragma unroll
     for (int i = 0; i < LC; ++i) {
       const int l = l0 + i;
-      float2 v = make_float2(0.f, 0.f);
-      if (l < nb && l >= am && l >= xn && xn < NW && z0 + xz < nbatch) {
-        const float2 a = xh[(size_t)lmn_index(l, m, xn) * nbatch + z0 + xz];
-        const float2 b = xh[(size_t)lmn_index(l, -m, -xn) * nbatch + z0 + xz];
-        const float s = (xn & 1) ? -hs : hs;
-        v = make_float2(0.5f * a.x + s * b.x, 0.5f * a.y - s * b.y);
-      }
-      xs[(i * ZT + xz) * SLD + xn] = v;
+      const bool okx = (l < nb && l >= am && l >= xn && xn < NW);
+      const int ia = okx ? lmn_index(l, m, xn) : 0, ib = okx ? lmn_index(l, -m, -xn) : 0;
+      xa[i] = xh[(size_t)ia * nbatch + zc];
+      xb[i] = xh[(size_t)ib * nbatch + zc];
+      const float4 v = tbase[(size_t)(l < nb ? l : nb - 1) * 512 + t];
+      tq[i] = l < nb ? v : make_float4(0.f, 0.f, 0.f, 0.f);
     }
-    // T chunk: [LC][n][beta]
+  };
+
+  const int lstart = (am / LC) * LC;
+  load_chunk(lstart);
+  for (int l0 = lstart; l0 < nb; l0 += LC) {
+    __syncthreads();
+#pragma unroll
     for (int i = 0; i < LC; ++i) {
       const int l = l0 + i;
-      const bool ok = (l < nb && l >= am && l >= n && n < NW);
-      const int idx = ok ? lmn_index(l, m, n) : 0;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int bt = (t >> 5) + 16 * j;
-        float v = 0.f;
-        if (ok && bt < n2) v = T[(size_t)bt * nspec + idx];
-        Tq[(i * 32 + n) * QLD + bt] = v;
-      }
+      const bool okx = (l < nb && l >= am && l >= xn && xn < NW && z0 + xz < nbatch);
+      const float sg = (xn & 1) ? -hs : hs;
+      const float2 a = xa[i], b = xb[i];
+      xs[(i * ZT + xz) * SLD + xn] = okx ? make_float2(0.5f * a.x + sg * b.x, 0.5f * a.y - sg * b.y) : make_float2(0.f, 0.f);
+      *reinterpret_cast<float4*>(Tq + i * 32 * QLD + tlds) = tq[i];
     }
     __syncthreads();
+    if (l0 + LC < nb) load_chunk(l0 + LC);
 #pragma unroll 2
     for (int i = 0; i < LC; ++i) {
       if (l0 + i < am || l0 + i >= nb) continue;

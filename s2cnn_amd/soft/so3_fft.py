@@ -19,13 +19,33 @@ def _setup_wigner(b, nl, weighted, device):
     return torch.tensor(dss, dtype=torch.float32, device=device).contiguous()
 
 
+@lru_cache(maxsize=32)
+def _setup_packed_wigner(b_in, b_out, weighted, synthesis, device):
+    """The table of `_setup_wigner` repacked once for the tiled kernels (None where they do not apply)."""
+    L = _hip.lib()
+    nbytes = L.s2cnn_so3_packed_table_bytes(b_in, b_out, int(synthesis))
+    if nbytes == 0:
+        return None
+    table = _setup_wigner(b_out, b_in, weighted, device) if synthesis else _setup_wigner(b_in, b_out, weighted, device)
+    packed = torch.empty(nbytes // 4, dtype=torch.float32, device=device)
+    with torch.cuda.device(device):
+        _hip.check(L.s2cnn_so3_pack_table(_hip.ptr(table), _hip.ptr(packed), b_in, b_out, int(synthesis), _hip.stream_ptr()))
+        torch.cuda.current_stream().synchronize()
+    return packed
+
+
+def _null_or_ptr(t):
+    return _hip.ptr(t) if t is not None else None
+
+
 def _analysis(x, b_in, b_out, nbatch, for_grad, complex_in):
     _hip.require_gpu_f32(x)
     L = _hip.lib()
     table = _setup_wigner(b_in, nl=b_out, weighted=not for_grad, device=x.device)
+    packed = None if complex_in else _setup_packed_wigner(b_in, b_out, not for_grad, False, x.device)
     out = x.new_empty((_nspec(b_out), nbatch, 2))
     ws = _hip.workspace(L.s2cnn_so3_analysis_workspace(b_in, b_out, nbatch, complex_in), x.device)
-    _hip.call("s2cnn_so3_analysis", _hip.ptr(x), _hip.ptr(table), _hip.ptr(out), _hip.ptr(ws), ws.numel(),
+    _hip.call("s2cnn_so3_analysis", _hip.ptr(x), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out), _hip.ptr(ws), ws.numel(),
                   b_in, b_out, nbatch, complex_in, _hip.stream_ptr())
     return out
 
@@ -34,10 +54,11 @@ def _synthesis(x, b_in, b_out, nbatch, for_grad, complex_out):
     _hip.require_gpu_f32(x)
     L = _hip.lib()
     table = _setup_wigner(b_out, nl=b_in, weighted=for_grad, device=x.device)
+    packed = None if complex_out else _setup_packed_wigner(b_in, b_out, for_grad, True, x.device)
     shape = (nbatch, 2 * b_out, 2 * b_out, 2 * b_out) + ((2,) if complex_out else ())
     out = x.new_empty(shape)
     ws = _hip.workspace(L.s2cnn_so3_synthesis_workspace(b_in, b_out, nbatch, complex_out), x.device)
-    _hip.call("s2cnn_so3_synthesis", _hip.ptr(x), _hip.ptr(table), _hip.ptr(out), _hip.ptr(ws), ws.numel(),
+    _hip.call("s2cnn_so3_synthesis", _hip.ptr(x), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out), _hip.ptr(ws), ws.numel(),
                   b_in, b_out, nbatch, complex_out, _hip.stream_ptr())
     return out
 

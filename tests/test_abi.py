@@ -19,7 +19,7 @@ def test_library_exports_every_declared_symbol():
     from s2cnn_amd import _hip
     lib = _hip.lib()
     names = _declared()
-    assert len(names) >= 18
+    assert len(names) >= 20
     for n in names:
         assert hasattr(lib, n), n
     assert sorted(_hip.SIGNATURES) == names
@@ -32,15 +32,19 @@ def test_argument_rejection_without_gpu():
     null = ctypes.c_void_p(0)
     assert lib.s2cnn_so3_mm_fwd(null, null, null, 4, 2, 3, 5, null) == -1
     assert lib.s2cnn_s2_mm_fwd(null, null, null, 4, 2, 3, 5, null) == -1
-    assert lib.s2cnn_so3_analysis(null, null, null, null, 0, 4, 4, 1, 0, null) == -1
+    assert lib.s2cnn_so3_analysis(null, null, null, null, null, 0, 4, 4, 1, 0, null) == -1
     assert lib.s2cnn_so3_integrate(null, null, null, 4, 1, null) == -1
     fake = ctypes.c_void_p(0x1000)
     assert lib.s2cnn_so3_mm_fwd(fake, fake, fake, 0, 2, 3, 5, null) == -1          # nl < 1
     assert lib.s2cnn_so3_mm_fwd(ctypes.c_void_p(0x1004), fake, fake, 2, 2, 3, 5, null) == -3
-    assert lib.s2cnn_so3_analysis(fake, fake, fake, null, 0, 4, 4, 1, 0, null) == -2  # no workspace
+    assert lib.s2cnn_so3_analysis(fake, fake, null, fake, null, 0, 4, 4, 1, 0, null) == -2  # no workspace
     assert lib.s2cnn_s2_analysis(fake, fake, fake, fake, 1 << 30, 4, 5, 1, 0, null) == -1  # b_out > b_in
-    assert lib.s2cnn_so3_analysis_workspace(32, 32, 256, 0) == 256 * 64 * 63 * 32 * 8
-    assert lib.s2cnn_so3_synthesis_workspace(4, 6, 3, 1) == 3 * 12 * 7 * 7 * 8
+    packed = lib.s2cnn_so3_packed_table_bytes(32, 32, 0)
+    assert packed == 63 * 64 * 1024 * 4
+    assert lib.s2cnn_so3_analysis_workspace(32, 32, 256, 0) == 256 * 64 * 63 * 32 * 8 + packed
+    assert lib.s2cnn_so3_synthesis_workspace(4, 6, 3, 1) == 16 * 12 * 7 * 7 * 8      # batch padded to the z tile, no fast path
+    assert lib.s2cnn_so3_packed_table_bytes(40, 40, 0) == 0 and lib.s2cnn_so3_packed_table_bytes(32, 40, 1) == 0
+    assert lib.s2cnn_so3_pack_table(fake, fake, 40, 40, 0, null) == -1
     assert b"workspace" in lib.s2cnn_strerror(-2)
 
 

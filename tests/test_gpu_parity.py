@@ -103,6 +103,29 @@ def test_so3_transform_batch_dims_and_ragged(hip):
     close(PSO3.so3_rfft(x0.cuda()), O.so3_rfft(x0.double()), "b=1")
 
 
+def test_so3_transforms_without_prepacked_table(hip):
+    """packed_table = NULL (the library repacks into its workspace) gives the same bits as the prepacked path."""
+    from s2cnn_amd import _hip
+    for b_in, b_out in [(32, 32), (10, 6)]:
+        nz = 5
+        x = rnd((nz, 2 * b_in, 2 * b_in, 2 * b_in), 17).cuda()
+        want = PSO3.so3_rfft(x, b_out=b_out)
+        table = PSO3._setup_wigner(b_in, b_out, True, x.device)
+        out = torch.empty_like(want)
+        ws = _hip.workspace(hip.s2cnn_so3_analysis_workspace(b_in, b_out, nz, 0), x.device)
+        _hip.check(hip.s2cnn_so3_analysis(_hip.ptr(x), _hip.ptr(table), None, _hip.ptr(out), _hip.ptr(ws), ws.numel(),
+                                          b_in, b_out, nz, 0, _hip.stream_ptr()))
+        assert torch.equal(out, want)
+        s = rnd((O.nspec_so3(b_out), nz, 2), 18).cuda()
+        want = PSO3.so3_rifft(s, b_out=b_in)
+        table = PSO3._setup_wigner(b_in, b_out, False, x.device)
+        out = torch.empty_like(want)
+        ws = _hip.workspace(hip.s2cnn_so3_synthesis_workspace(b_out, b_in, nz, 0), x.device)
+        _hip.check(hip.s2cnn_so3_synthesis(_hip.ptr(s), _hip.ptr(table), None, _hip.ptr(out), _hip.ptr(ws), ws.numel(),
+                                           b_out, b_in, nz, 0, _hip.stream_ptr()))
+        assert torch.equal(out, want)
+
+
 def test_so3_reference_identities_on_gpu(hip):
     """tests/so3_fft.py:8-24 and :34-91 of the reference, run on the HIP path."""
     b_in, b_out = 7, 5
