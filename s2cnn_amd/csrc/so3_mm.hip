@@ -20,6 +20,12 @@
 // accumulates ar*br + ai*bi (the real part of a*conj(b)), and with b'' = (-bi, br) the
 // imaginary part; without conjugation b' = (br, -bi), b'' = (bi, br).  Four real MACs per
 // complex MAC - the algorithmic minimum - and the A operand register is shared by both.
+//
+// Tiling.  A workgroup (4 waves) owns 128 rows x 128 columns = 4 x 4 blocks of 32.  Wave (wm, wn)
+// takes row blocks wm, wm+2 and column blocks wn, wn+2, so a ragged tile (fewer live blocks) still
+// splits evenly over the waves; blocks that lie wholly outside the matrix are skipped per wave.
+// The grid lists exactly the tiles of all degrees, heaviest degree first (no idle workgroups:
+// a workgroup that exits at once still waits for a full slot and stalls the in-order dispatch).
 #include <type_traits>
 #include "common.h"
 
@@ -27,13 +33,14 @@ namespace {
 
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-constexpr int TM = 128;           // tile rows   (flattened (spectral, feature) index)
-constexpr int TN = 128;           // tile cols
+constexpr int NRB = 2;            // 32-row blocks per wave
+constexpr int NCB = 2;            // 32-column blocks per wave
+constexpr int TM = 64 * NRB;      // tile rows   (flattened (spectral, feature) index): 2 waves x NRB blocks
+constexpr int TN = 64 * NCB;      // tile cols
+constexpr int BSTR = 64, WSTR = 32;   // a wave's blocks are 64 apart, the two waves of a dimension offset by 32
 constexpr int TK = 16;            // complex contraction steps per LDS stage
-constexpr int NT = 256;           // threads: 4 waves, each a 64x64 complex sub-tile
+constexpr int NT = 256;           // threads: 4 waves
 constexpr int KC_LD = TK + 2;     // leading dim (complex) of a K-contiguous LDS tile: 144 B rows
-constexpr int MN_LD = 128;        // leading dim of an MN-contiguous LDS tile
-constexpr int TILE_ELEMS = (TM * KC_LD > TK * MN_LD) ? TM * KC_LD : TK * MN_LD;
 
 enum Mode { FWD = 0, GRADX = 1, GRADY = 2 };
 
@@ -53,11 +60,19 @@ template <> struct Cfg<FWD>   { static constexpr bool A_KC = true,  B_KC = false
 template <> struct Cfg<GRADX> { static constexpr bool A_KC = true,  B_KC = true,  A_MNMAJ = true,  B_MNMAJ = false, C_RMAJ = true,  CONJ = false; };
 template <> struct Cfg<GRADY> { static constexpr bool A_KC = false, B_KC = false, A_MNMAJ = false, B_MNMAJ = false, C_RMAJ = false, CONJ = true;  };
 
-// One operand's tile loader: global -> registers -> LDS.  VEC = complex numbers per access.
-template <bool KC, bool MNMAJ, int VEC>
+template <bool KC, int EXT> struct TileShape {
+  static constexpr int LD = KC ? KC_LD : EXT;             // LDS leading dimension (complex)
+  static constexpr int ELEMS = KC ? EXT * KC_LD : TK * EXT;
+};
+
+// One operand's tile loader: global -> registers -> LDS.  EXT = tile extent along the free index,
+// VEC = complex numbers per access.
+template <bool KC, bool MNMAJ, int EXT, int VEC>
 struct TileLoader {
-  static constexpr int NSLOT = TM * TK / (NT * VEC);
+  static constexpr int NSLOT = EXT * TK / (NT * VEC);
+  static constexpr int LD = TileShape<KC, EXT>::LD;
   typedef typename std::conditional<VEC == 2, float4, float2>::type vec_t;
+  static_assert(NSLOT >= 1, "tile too small for the workgroup");
 
   const float2* base;   // start of degree l
   int off[KC ? NSLOT : 1];
@@ -79,7 +94,7 @@ struct TileLoader {
       constexpr int TPR = TK / VEC;          // threads per tile row
       kk = (t % TPR) * VEC;
       const int r0 = t / TPR;
-      lds_off = r0 * KC_LD + kk;
+      lds_off = r0 * LD + kk;
 #pragma unroll
       for (int q = 0; q < NSLOT; ++q) {
         const int row = tile0 + r0 + q * (NT / TPR);
@@ -88,34 +103,35 @@ struct TileLoader {
         if (row < L * MNI) valid_mn |= 1u << q;
       }
     } else {
-      constexpr int TPR = TM / VEC;          // threads per k-row of the tile
+      constexpr int TPR = EXT / VEC;         // threads per k-row of the tile
       const int mn = tile0 + (t % TPR) * VEC;
       kk = t / TPR;
-      lds_off = kk * MN_LD + (t % TPR) * VEC;
+      lds_off = kk * LD + (t % TPR) * VEC;
       const int mb = mn / MNI, mi = mn - mb * MNI;
       off[0] = mb * blk_mn_stride + mi;
       if (mn < L * MNI) valid_mn = 1u;
     }
   }
 
+  // clamped address + select instead of a predicated load: all loads of a stage are in flight together
   __device__ void load(int kb, int k0) {
     const float2* p = base + (size_t)kb * blk_k_stride;
     if (KC) {
       const bool kvalid = (k0 + kk) < KI;
 #pragma unroll
       for (int q = 0; q < NSLOT; ++q) {
-        vec_t v = {};
-        if (kvalid && ((valid_mn >> q) & 1u)) v = *reinterpret_cast<const vec_t*>(p + off[q] + k0);
-        reg[q] = v;
+        const bool ok = kvalid && ((valid_mn >> q) & 1u);
+        const vec_t v = *reinterpret_cast<const vec_t*>(p + (ok ? off[q] + k0 : 0));
+        reg[q] = ok ? v : vec_t{};
       }
     } else {
-      constexpr int KSTEP = NT * VEC / TM;
+      constexpr int KSTEP = NT * VEC / EXT;
 #pragma unroll
       for (int q = 0; q < NSLOT; ++q) {
         const int k = k0 + kk + q * KSTEP;
-        vec_t v = {};
-        if (valid_mn && k < KI) v = *reinterpret_cast<const vec_t*>(p + off[0] + (size_t)k * MNI);
-        reg[q] = v;
+        const bool ok = valid_mn && k < KI;
+        const vec_t v = *reinterpret_cast<const vec_t*>(p + (ok ? off[0] + k * MNI : 0));
+        reg[q] = ok ? v : vec_t{};
       }
     }
   }
@@ -125,71 +141,82 @@ struct TileLoader {
       constexpr int RSTEP = NT * VEC / TK;
 #pragma unroll
       for (int q = 0; q < NSLOT; ++q)
-        *reinterpret_cast<vec_t*>(tile + lds_off + q * RSTEP * KC_LD) = reg[q];
+        *reinterpret_cast<vec_t*>(tile + lds_off + q * RSTEP * LD) = reg[q];
     } else {
-      constexpr int KSTEP = NT * VEC / TM;
+      constexpr int KSTEP = NT * VEC / EXT;
 #pragma unroll
       for (int q = 0; q < NSLOT; ++q)
-        *reinterpret_cast<vec_t*>(tile + lds_off + q * KSTEP * MN_LD) = reg[q];
+        *reinterpret_cast<vec_t*>(tile + lds_off + q * KSTEP * LD) = reg[q];
     }
   }
 };
 
 // The four reals (re k0, im k0, re k0+1, im k0+1) one lane feeds to four consecutive MFMAs,
 // for tile row/col `idx` and the lane's pair of contraction steps k0 = 4s + 2h.
-template <bool KC>
-__device__ inline float4 fetch_operand(const float2* tile, int idx, int k0) {
+template <bool KC, int LD>
+__device__ __forceinline__ float4 fetch_operand(const float2* tile, int idx, int k0) {
   if (KC) {
-    return *reinterpret_cast<const float4*>(tile + idx * KC_LD + k0);
+    return *reinterpret_cast<const float4*>(tile + idx * LD + k0);
   } else {
-    const float2 a = tile[k0 * MN_LD + idx];
-    const float2 b = tile[(k0 + 1) * MN_LD + idx];
+    const float2 a = tile[k0 * LD + idx];
+    const float2 b = tile[(k0 + 1) * LD + idx];
     return make_float4(a.x, a.y, b.x, b.y);
   }
 }
 
-template <int MODE, int VEC>
-__global__ __launch_bounds__(NT) void so3_block_mm_kernel(MmParams p) {
-  typedef Cfg<MODE> C_;
-  __shared__ __attribute__((aligned(16))) float2 As[TILE_ELEMS];
-  __shared__ __attribute__((aligned(16))) float2 Bs[TILE_ELEMS];
-
-  // ---- which tile: degrees in descending order so the heaviest tiles are dispatched first
-  int t = blockIdx.x;
-  int l = p.nl - 1, tm = 0, tn = 0;
-  for (;; --l) {
-    const int L_ = 2 * l + 1;
-    tm = s2cnn::ceil_div(L_ * p.RI, TM);
-    tn = s2cnn::ceil_div(L_ * p.CI, TN);
-    if (t < tm * tn || l == 0) break;
-    t -= tm * tn;
+// All matrix-core work of one LDS stage for a wave with NI live row blocks (rows arow + 64 i) and NJ
+// live column blocks (columns bcol + 64 j).  Operand registers are double buffered: the LDS reads of
+// step s+1 are issued before the MFMAs of step s.
+template <typename C_, int NI, int NJ>
+__device__ __forceinline__ void stage_mma(const float2* As, const float2* Bs, v16f (&acc_re)[NRB][NCB], v16f (&acc_im)[NRB][NCB],
+                                          int arow, int bcol, int h) {
+  constexpr int ALD = TileShape<C_::A_KC, TM>::LD, BLD = TileShape<C_::B_KC, TN>::LD;
+  float4 a[2][NI], b[2][NJ];
+#pragma unroll
+  for (int i = 0; i < NI; ++i) a[0][i] = fetch_operand<C_::A_KC, ALD>(As, arow + BSTR * i, 2 * h);
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) b[0][j] = fetch_operand<C_::B_KC, BLD>(Bs, bcol + BSTR * j, 2 * h);
+#pragma unroll
+  for (int s = 0; s < TK / 4; ++s) {
+    const int cur = s & 1, nxt = cur ^ 1;
+    if (s + 1 < TK / 4) {
+#pragma unroll
+      for (int i = 0; i < NI; ++i) a[nxt][i] = fetch_operand<C_::A_KC, ALD>(As, arow + BSTR * i, 4 * (s + 1) + 2 * h);
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) b[nxt][j] = fetch_operand<C_::B_KC, BLD>(Bs, bcol + BSTR * j, 4 * (s + 1) + 2 * h);
+    }
+    __builtin_amdgcn_sched_barrier(0);   // keep the LDS reads of the next step ahead of this step's MFMAs
+    float4 bre[NJ], bim[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const float4 v = b[cur][j];
+      if (C_::CONJ) {
+        bre[j] = v;
+        bim[j] = make_float4(-v.y, v.x, -v.w, v.z);
+      } else {
+        bre[j] = make_float4(v.x, -v.y, v.z, -v.w);
+        bim[j] = make_float4(v.y, v.x, v.w, v.z);
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int i = 0; i < NI; ++i)
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+          const float av = t == 0 ? a[cur][i].x : t == 1 ? a[cur][i].y : t == 2 ? a[cur][i].z : a[cur][i].w;
+          const float br = t == 0 ? bre[j].x : t == 1 ? bre[j].y : t == 2 ? bre[j].z : bre[j].w;
+          const float bi = t == 0 ? bim[j].x : t == 1 ? bim[j].y : t == 2 ? bim[j].z : bim[j].w;
+          acc_re[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, br, acc_re[i][j], 0, 0, 0);
+          acc_im[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bi, acc_im[i][j], 0, 0, 0);
+        }
   }
-  const int L = 2 * l + 1;
-  const int tile_m = (t % tm) * TM;
-  const int tile_n = (t / tm) * TN;
-  const size_t L0 = (size_t)l * (4 * l * l - 1) / 3;
-  const int M = L * p.RI, N = L * p.CI;
+}
 
-  TileLoader<C_::A_KC, C_::A_MNMAJ, VEC> la;
-  TileLoader<C_::B_KC, C_::B_MNMAJ, VEC> lb;
-  la.init(p.A + L0 * p.RI * p.KI, L, p.RI, p.KI, tile_m);
-  lb.init(p.B + L0 * p.CI * p.KI, L, p.CI, p.KI, tile_n);
-
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int r32 = lane & 31, h = lane >> 5;
-  const int wrow = (wave >> 1) * 64, wcol = (wave & 1) * 64;
-
-  v16f acc_re[2][2], acc_im[2][2];
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) { acc_re[i][j][v] = 0.f; acc_im[i][j][v] = 0.f; }
-
-  const int nkc = s2cnn::ceil_div(p.KI, TK);
-  const int nstage = L * nkc;
+// The contraction loop of one tile: LDS stage s is consumed while the global loads of stage s+1 are in flight.
+template <typename C_, int NI, int NJ, typename LA, typename LB>
+__device__ __forceinline__ void contract(LA& la, LB& lb, float2* As, float2* Bs, v16f (&acc_re)[NRB][NCB], v16f (&acc_im)[NRB][NCB],
+                                         int nstage, int nkc, int arow, int bcol, int h) {
   la.load(0, 0);
   lb.load(0, 0);
   int kb = 0, kc = 0;
@@ -203,53 +230,102 @@ __global__ __launch_bounds__(NT) void so3_block_mm_kernel(MmParams p) {
       la.load(kb, kc * TK);
       lb.load(kb, kc * TK);
     }
+    if (NI > 0 && NJ > 0) stage_mma<C_, (NI > 0 ? NI : 1), (NJ > 0 ? NJ : 1)>(As, Bs, acc_re, acc_im, arow, bcol, h);
+  }
+}
+
+__host__ __device__ inline void tile_counts(int L, int RI, int CI, int& tm, int& tn, int& slots) {
+  tm = s2cnn::ceil_div(L * RI, TM);
+  tn = s2cnn::ceil_div(L * CI, TN);
+  slots = tm * tn;   // every workgroup of the grid has a tile: idle workgroups stall the dispatcher
+}
+
+template <int MODE, int VEC>
+__global__ __launch_bounds__(NT) void so3_block_mm_kernel(MmParams p) {
+  typedef Cfg<MODE> C_;
+  __shared__ __attribute__((aligned(16))) float2 As[TileShape<C_::A_KC, TM>::ELEMS];
+  __shared__ __attribute__((aligned(16))) float2 Bs[TileShape<C_::B_KC, TN>::ELEMS];
+
+  // ---- which tile: degrees in descending order so the heaviest tiles are dispatched first
+  int t = blockIdx.x;
+  int l = p.nl - 1, tm = 0, tn = 0, slots = 0;
+  for (;; --l) {
+    tile_counts(2 * l + 1, p.RI, p.CI, tm, tn, slots);
+    if (t < slots || l == 0) break;
+    t -= slots;
+  }
+  const int r = t;                                  // row tiles run fastest within a degree
+  const int tile_nq = r / tm;
+  const int L = 2 * l + 1;
+  const int tile_m = (r % tm) * TM;
+  const int tile_n = tile_nq * TN;
+  const size_t L0 = (size_t)l * (4 * l * l - 1) / 3;
+  const int M = L * p.RI, N = L * p.CI;
+
+  TileLoader<C_::A_KC, C_::A_MNMAJ, TM, VEC> la;
+  TileLoader<C_::B_KC, C_::B_MNMAJ, TN, VEC> lb;
+  la.init(p.A + L0 * p.RI * p.KI, L, p.RI, p.KI, tile_m);
+  lb.init(p.B + L0 * p.CI * p.KI, L, p.CI, p.KI, tile_n);
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r32 = lane & 31, h = lane >> 5;
+  const int wrow = (wave >> 1) * WSTR, wcol = (wave & 1) * WSTR;
+
+  v16f acc_re[NRB][NCB], acc_im[NRB][NCB];
 #pragma unroll
-    for (int s = 0; s < TK / 4; ++s) {
-      const int k0 = 4 * s + 2 * h;
-      float4 a[2], bre[2], bim[2];
+  for (int i = 0; i < NRB; ++i)
 #pragma unroll
-      for (int i = 0; i < 2; ++i) a[i] = fetch_operand<C_::A_KC>(As, wrow + 32 * i + r32, k0);
+    for (int j = 0; j < NCB; ++j)
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const float4 b = fetch_operand<C_::B_KC>(Bs, wcol + 32 * j + r32, k0);
-        if (C_::CONJ) {
-          bre[j] = b;
-          bim[j] = make_float4(-b.y, b.x, -b.w, b.z);
-        } else {
-          bre[j] = make_float4(b.x, -b.y, b.z, -b.w);
-          bim[j] = make_float4(b.y, b.x, b.w, b.z);
-        }
-      }
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          acc_re[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i].x, bre[j].x, acc_re[i][j], 0, 0, 0);
-          acc_im[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i].x, bim[j].x, acc_im[i][j], 0, 0, 0);
-          acc_re[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i].y, bre[j].y, acc_re[i][j], 0, 0, 0);
-          acc_im[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i].y, bim[j].y, acc_im[i][j], 0, 0, 0);
-          acc_re[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i].z, bre[j].z, acc_re[i][j], 0, 0, 0);
-          acc_im[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i].z, bim[j].z, acc_im[i][j], 0, 0, 0);
-          acc_re[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i].w, bre[j].w, acc_re[i][j], 0, 0, 0);
-          acc_im[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i].w, bim[j].w, acc_im[i][j], 0, 0, 0);
-        }
+      for (int v = 0; v < 16; ++v) { acc_re[i][j][v] = 0.f; acc_im[i][j][v] = 0.f; }
+
+  // live blocks of this wave: rows tile_m + wrow + 64 i < M, columns tile_n + wcol + 64 j < N (prefixes of i, j)
+  const int remr = M - tile_m - wrow, remc = N - tile_n - wcol;
+  int ni = remr <= 0 ? 0 : (remr + BSTR - 1) / BSTR, nj = remc <= 0 ? 0 : (remc + BSTR - 1) / BSTR;
+  ni = ni > NRB ? NRB : ni;
+  nj = nj > NCB ? NCB : nj;
+  if (ni == 0 || nj == 0) ni = nj = 0;
+
+  const int nkc = s2cnn::ceil_div(p.KI, TK);
+  const int nstage = L * nkc;
+  // one specialised copy of the whole contraction loop per count of live blocks (wave-uniform choice)
+#define S2CNN_CONTRACT(I, J) contract<C_, I, J>(la, lb, As, Bs, acc_re, acc_im, nstage, nkc, wrow + r32, wcol + r32, h)
+  if (nj == NCB) {
+    switch (ni) {
+      case 4: if (NRB >= 4) { S2CNN_CONTRACT((NRB >= 4 ? 4 : 1), NCB); } break;
+      case 3: if (NRB >= 3) { S2CNN_CONTRACT((NRB >= 3 ? 3 : 1), NCB); } break;
+      case 2: if (NRB >= 2) { S2CNN_CONTRACT((NRB >= 2 ? 2 : 1), NCB); } break;
+      case 1: S2CNN_CONTRACT(1, NCB); break;
+      default: S2CNN_CONTRACT(0, 0); break;
+    }
+  } else if (nj == 0) {
+    S2CNN_CONTRACT(0, 0);
+  } else {  // NCB == 2 and one live column block
+    switch (ni) {
+      case 4: if (NRB >= 4) { S2CNN_CONTRACT((NRB >= 4 ? 4 : 1), 1); } break;
+      case 3: if (NRB >= 3) { S2CNN_CONTRACT((NRB >= 3 ? 3 : 1), 1); } break;
+      case 2: if (NRB >= 2) { S2CNN_CONTRACT((NRB >= 2 ? 2 : 1), 1); } break;
+      default: S2CNN_CONTRACT(1, 1); break;
     }
   }
+#undef S2CNN_CONTRACT
 
-  // ---- write the 64x64 complex sub-tile.  Accumulator register v of lane (r32, h) holds
-  // row 8*(v/4) + 4*h + v%4 and column r32 of its 32x32 tile.
+  // ---- write the sub-tile.  Accumulator register v of lane (r32, h) holds row 8*(v/4) + 4*h + v%4
+  // and column r32 of its 32x32 block.
   float2* Cl = p.C + L0 * p.RI * p.CI;
   const int blk_elems = p.RI * p.CI;
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int col = tile_n + wcol + 32 * j + r32;
-    if (col >= N) continue;
+  for (int j = 0; j < NCB; ++j) {
+    const int col = tile_n + wcol + BSTR * j + r32;
+    if (j >= nj || col >= N) continue;
     const int cb = col / p.CI, ci = col - cb * p.CI;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < NRB; ++i) {
+      if (i >= ni) continue;
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const int row = tile_m + wrow + 32 * i + 8 * (v / 4) + 4 * h + (v % 4);
+        const int row = tile_m + wrow + BSTR * i + 8 * (v / 4) + 4 * h + (v % 4);
         if (row < M) {
           const int rb = row / p.RI, ri = row - rb * p.RI;
           const int blk = C_::C_RMAJ ? rb * L + cb : cb * L + rb;
@@ -260,11 +336,12 @@ __global__ __launch_bounds__(NT) void so3_block_mm_kernel(MmParams p) {
   }
 }
 
-int total_tiles(int nl, int RI, int CI) {
+int total_slots(int nl, int RI, int CI) {
   long n = 0;
   for (int l = 0; l < nl; ++l) {
-    const int L = 2 * l + 1;
-    n += (long)s2cnn::ceil_div(L * RI, TM) * s2cnn::ceil_div(L * CI, TN);
+    int tm, tn, slots;
+    tile_counts(2 * l + 1, RI, CI, tm, tn, slots);
+    n += slots;
   }
   return n > 0x7fffffffL ? -1 : (int)n;
 }
@@ -277,8 +354,8 @@ int run(const float* a, const float* b, float* c, int nl, int RI, int CI, int KI
   const long Lmax = 2L * nl - 1;
   if (Lmax * Lmax * RI * KI >= (1L << 31) || Lmax * Lmax * CI * KI >= (1L << 31)) return S2CNN_EINVAL;
   if (!s2cnn::aligned8(a) || !s2cnn::aligned8(b) || !s2cnn::aligned8(c)) return S2CNN_EALIGN;
-  const int tiles = total_tiles(nl, RI, CI);
-  if (tiles < 1) return S2CNN_EINVAL;
+  const int grid = total_slots(nl, RI, CI);
+  if (grid < 1) return S2CNN_EINVAL;
   MmParams p{reinterpret_cast<const float2*>(a), reinterpret_cast<const float2*>(b),
              reinterpret_cast<float2*>(c), nl, RI, CI, KI};
   typedef Cfg<MODE> C_;
@@ -288,9 +365,9 @@ int run(const float* a, const float* b, float* c, int nl, int RI, int CI, int KI
   const bool vec2 = a_even && b_even && s2cnn::aligned16(a) && s2cnn::aligned16(b);
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (vec2)
-    hipLaunchKernelGGL((so3_block_mm_kernel<MODE, 2>), dim3(tiles), dim3(NT), 0, st, p);
+    hipLaunchKernelGGL((so3_block_mm_kernel<MODE, 2>), dim3(grid), dim3(NT), 0, st, p);
   else
-    hipLaunchKernelGGL((so3_block_mm_kernel<MODE, 1>), dim3(tiles), dim3(NT), 0, st, p);
+    hipLaunchKernelGGL((so3_block_mm_kernel<MODE, 1>), dim3(grid), dim3(NT), 0, st, p);
   return s2cnn::launch_status();
 }
 
