@@ -96,7 +96,7 @@ def main():
 
     per_call = {k: sum(v) / len(v) for k, v in timer.summary().items()}
     flops = mm_flops(b, B, F, F)
-    mm_names = ["s2cnn_so3_mm_fwd", "s2cnn_so3_mm_gradx", "s2cnn_so3_mm_grady"]
+    mm_names = [n for n in per_call if n.startswith("s2cnn_so3_mm_")]   # fwd / gradx / grady (planar-y entry points in the layer)
     dominant = max(mm_names, key=lambda n: per_call[n])
     ach = flops / (per_call[dominant] * 1e-3) / 1e12
     roofline = {"bound": "mfma", "kernel": dominant, "achieved": round(ach, 2), "peak": PEAK_FP32_MFMA_TFLOPS,

@@ -38,24 +38,32 @@ def _null_or_ptr(t):
     return _hip.ptr(t) if t is not None else None
 
 
-def _analysis(x, b_in, b_out, nbatch, for_grad, complex_in):
+def _analysis(x, b_in, b_out, batch_size, for_grad, complex_in):
+    """x: contiguous grid tensor whose leading dims are `batch_size`; the result is allocated in its
+    final shape (never a view: autograd can then take ownership of it as a gradient without a copy)."""
     _hip.require_gpu_f32(x)
     L = _hip.lib()
+    nbatch = 1
+    for d in batch_size:
+        nbatch *= d
     table = _setup_wigner(b_in, nl=b_out, weighted=not for_grad, device=x.device)
     packed = None if complex_in else _setup_packed_wigner(b_in, b_out, not for_grad, False, x.device)
-    out = x.new_empty((_nspec(b_out), nbatch, 2))
+    out = x.new_empty((_nspec(b_out), *batch_size, 2))
     ws = _hip.workspace(L.s2cnn_so3_analysis_workspace(b_in, b_out, nbatch, complex_in), x.device)
     _hip.call("s2cnn_so3_analysis", _hip.ptr(x), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out), _hip.ptr(ws), ws.numel(),
                   b_in, b_out, nbatch, complex_in, _hip.stream_ptr())
     return out
 
 
-def _synthesis(x, b_in, b_out, nbatch, for_grad, complex_out):
+def _synthesis(x, b_in, b_out, batch_size, for_grad, complex_out):
     _hip.require_gpu_f32(x)
     L = _hip.lib()
+    nbatch = 1
+    for d in batch_size:
+        nbatch *= d
     table = _setup_wigner(b_out, nl=b_in, weighted=for_grad, device=x.device)
     packed = None if complex_out else _setup_packed_wigner(b_in, b_out, for_grad, True, x.device)
-    shape = (nbatch, 2 * b_out, 2 * b_out, 2 * b_out) + ((2,) if complex_out else ())
+    shape = (*batch_size, 2 * b_out, 2 * b_out, 2 * b_out) + ((2,) if complex_out else ())
     out = x.new_empty(shape)
     ws = _hip.workspace(L.s2cnn_so3_synthesis_workspace(b_in, b_out, nbatch, complex_out), x.device)
     _hip.call("s2cnn_so3_synthesis", _hip.ptr(x), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out), _hip.ptr(ws), ws.numel(),
@@ -76,9 +84,7 @@ def so3_fft(x, for_grad=False, b_out=None):
     if b_out is None:
         b_out = b_in
     batch_size = x.size()[:-4]
-    x = x.contiguous().view(-1, 2 * b_in, 2 * b_in, 2 * b_in, 2)
-    out = _analysis(x, b_in, b_out, x.size(0), for_grad, 1)
-    return out.view(-1, *batch_size, 2)
+    return _analysis(x.contiguous(), b_in, b_out, batch_size, for_grad, 1)
 
 
 def so3_rfft(x, for_grad=False, b_out=None):
@@ -93,9 +99,7 @@ def so3_rfft(x, for_grad=False, b_out=None):
     if b_out is None:
         b_out = b_in
     batch_size = x.size()[:-3]
-    x = x.contiguous().view(-1, 2 * b_in, 2 * b_in, 2 * b_in)
-    out = _analysis(x, b_in, b_out, x.size(0), for_grad, 0)
-    return out.view(-1, *batch_size, 2)
+    return _analysis(x.contiguous(), b_in, b_out, batch_size, for_grad, 0)
 
 
 def _spectrum_args(x, b_out):
@@ -106,8 +110,7 @@ def _spectrum_args(x, b_out):
     if b_out is None:
         b_out = b_in
     batch_size = x.size()[1:-1]
-    x = x.contiguous().view(nspec, -1, 2)
-    return x, b_in, b_out, batch_size
+    return x.contiguous(), b_in, b_out, batch_size
 
 
 def so3_ifft(x, for_grad=False, b_out=None):
@@ -116,8 +119,7 @@ def so3_ifft(x, for_grad=False, b_out=None):
     :return: [..., beta, alpha, gamma, complex]
     '''
     x, b_in, b_out, batch_size = _spectrum_args(x, b_out)
-    out = _synthesis(x, b_in, b_out, x.size(1), for_grad, 1)
-    return out.view(*batch_size, 2 * b_out, 2 * b_out, 2 * b_out, 2)
+    return _synthesis(x, b_in, b_out, batch_size, for_grad, 1)
 
 
 def so3_rifft(x, for_grad=False, b_out=None):
@@ -126,8 +128,7 @@ def so3_rifft(x, for_grad=False, b_out=None):
     :return: [..., beta, alpha, gamma]  (the real part of so3_ifft, whatever the symmetry of x)
     '''
     x, b_in, b_out, batch_size = _spectrum_args(x, b_out)
-    out = _synthesis(x, b_in, b_out, x.size(1), for_grad, 0)
-    return out.view(*batch_size, 2 * b_out, 2 * b_out, 2 * b_out)
+    return _synthesis(x, b_in, b_out, batch_size, for_grad, 0)
 
 
 class SO3_fft_real(torch.autograd.Function):
