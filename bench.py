@@ -23,6 +23,10 @@ if ROOT not in sys.path:
 
 PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X dense fp32 matrix
 PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
+# HBM-side bytes per launch of the three so3_mm kernels at this workload, from rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE scaled by a 1 GiB copy (profiles/so3_mm_b32_B16_F64_hbm_traffic.md); not re-measured at run time.
+MM_TRAFFIC_BYTES = {"s2cnn_so3_mm_fwd": 13.08e9 + 0.358e9, "s2cnn_so3_mm_gradx": 13.19e9 + 0.358e9,
+                    "s2cnn_so3_mm_grady": 11.07e9 + 1.431e9}
 
 
 def nspec(b):
@@ -100,7 +104,8 @@ def main():
     dominant = max(mm_names, key=lambda n: per_call[n])
     ach = flops / (per_call[dominant] * 1e-3) / 1e12
     roofline = {"bound": "mfma", "kernel": dominant, "achieved": round(ach, 2), "peak": PEAK_FP32_MFMA_TFLOPS,
-                "unit": "TFLOP/s", "frac": round(ach / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None,
+                "unit": "TFLOP/s", "frac": round(ach / PEAK_FP32_MFMA_TFLOPS, 4),
+                "traffic": MM_TRAFFIC_BYTES.get(dominant) if (B, F, b) == (16, 64, 32) else None,
                 "flop_per_launch": flops, "ms_per_launch": round(per_call[dominant], 3)}
     kernels = {n: {"ms": round(ms, 3)} for n, ms in per_call.items()}
     for n in mm_names:
