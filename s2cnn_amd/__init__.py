@@ -7,4 +7,4 @@ from .so3_grid import so3_near_identity_grid, so3_equatorial_grid, so3_soft_grid
 from .s2_mm import s2_mm
 from .so3_mm import so3_mm
 from .soft import *  # noqa: F401,F403
-from .soft import S2Convolution, SO3Convolution, SO3Shortcut, so3_integrate
+from .soft import S2Convolution, SO3Convolution, SO3Shortcut, so3_integrate, so3_rotation

@@ -254,6 +254,39 @@ def test_z_rotation_equivariance_on_gpu(hip):
     assert rel.item() < 1e-4
 
 
+def test_so3_rotation(hip):
+    """s2cnn/soft/so3_rotation.py of the reference: parity with the oracle, the group law, and the
+    arbitrary-rotation equivariance of a layer (examples/equivariance_plot/main.py:74-78 of the reference)."""
+    b = 6
+    x = rnd((2, 3, 2 * b, 2 * b, 2 * b), 90)
+    a, bt, g = 0.3, 1.1, -0.7
+    got = s2cnn_amd.so3_rotation(x.cuda(), a, bt, g)
+    close(got, O.so3_rotation(x.double(), a, bt, g), "so3_rotation")
+    # rotating by the z-axis angle 2 pi k / 2b is a roll of the alpha axis (band-limited part of x)
+    xb = PSO3.so3_rifft(PSO3.so3_rfft(x.cuda()))
+    rolled = s2cnn_amd.so3_rotation(xb, 2 * 3.141592653589793 * 2 / (2 * b), 0.0, 0.0)
+    assert (rolled - torch.roll(xb, 2, dims=-2)).abs().max().item() < 1e-4 * xb.abs().max().item() or \
+           (rolled - torch.roll(xb, -2, dims=-2)).abs().max().item() < 1e-4 * xb.abs().max().item()
+    # equivariance of an SO(3) convolution under an arbitrary rotation
+    torch.manual_seed(5)
+    conv = s2cnn_amd.SO3Convolution(3, 2, b, b, s2cnn_amd.so3_near_identity_grid(n_alpha=4, n_beta=2, n_gamma=3)).cuda()
+    with torch.no_grad():
+        y1 = s2cnn_amd.so3_rotation(conv(xb), a, bt, g)
+        y2 = conv(s2cnn_amd.so3_rotation(xb, a, bt, g))
+    rel = ((y1 - y2).std() / y1.std()).item()
+    print("rotation equivariance residual", rel, flush=True)
+    assert rel < 1e-3
+
+
+def test_so3_shortcut(hip):
+    sc = s2cnn_amd.SO3Shortcut(3, 3, 4, 4)
+    x = rnd((2, 3, 8, 8, 8), 91).cuda()
+    assert sc(x) is x
+    sc2 = s2cnn_amd.SO3Shortcut(3, 5, 4, 3).cuda()
+    want = O.so3_conv(x.cpu().double(), sc2.conv.kernel.detach().cpu().double(), sc2.conv.bias.detach().cpu().double(), 4, 3, ((0, 0, 0),))
+    close(sc2(x), want, "shortcut conv")
+
+
 def test_size_independent_properties_at_config_sizes(hip):
     """Config 2 (b = 32) at a reduced batch: fft -> ifft -> fft reproduces the spectrum (projector),
     linearity, and the Hermitian symmetry of the spectrum of a real signal."""
