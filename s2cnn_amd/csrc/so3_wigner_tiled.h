@@ -77,11 +77,18 @@ __global__ void pack_table_synthesis(const float* __restrict__ T, float* __restr
 }
 
 // ---------------------------------------------------------------------------------------------
-// analysis: 256 threads, thread = (zq = t % 8 -> z = 2 zq, 2 zq + 1 ; n = t / 8)
+// analysis: 256 threads = 4 waves; wave w owns n = 8w .. 8w+7.  For each n the contraction
+//   D_n[l, (z,c)] += sum_beta T[beta, n, l] * X[beta, z, n].c        (32 degrees x 16 z x (re,im))
+// is a 32x32 matrix-core tile with K = beta: v_mfma_f32_32x32x2_f32 takes two betas per instruction,
+// A = T (lane = l, half-wave = beta parity), B = X (lane = 2 z + c).  T is zero outside the valid
+// (l, n) range, so the padded rows cost matrix-core time but no correctness.
 // ---------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void wigner_fwd_tiled(const float2* __restrict__ X, const float* __restrict__ Tp,
-                                                        float2* __restrict__ out, int n2, int nb, int nl, long nbatch) {
-  __shared__ __attribute__((aligned(16))) float2 Xs[KB * ZT * XLD];
+typedef float v16f __attribute__((ext_vector_type(16)));
+constexpr int XLD_M = 33;     // z stride (complex) of the X chunk: (z, c) lanes hit 32 distinct banks
+
+__global__ __launch_bounds__(256, 2) void wigner_fwd_tiled(const float2* __restrict__ X, const float* __restrict__ Tp,
+                                                           float2* __restrict__ out, int n2, int nb, int nl, long nbatch) {
+  __shared__ __attribute__((aligned(16))) float2 Xs[KB * ZT * XLD_M];
   __shared__ __attribute__((aligned(16))) float Ts[KB * 32 * TLD];
   const int MW = 2 * nb - 1, NW = nb;
   const int nzt = (int)((nbatch + ZT - 1) / ZT);
@@ -89,15 +96,16 @@ __global__ __launch_bounds__(256) void wigner_fwd_tiled(const float2* __restrict
   if (!decode_block(MW, nb, nzt, m, zt)) return;
   const int mi = m + nb - 1;
   const long z0 = (long)zt * ZT;
-  const long nspec = (long)nl * (4L * nl * nl - 1) / 3;
   const int am = abs(m);
-  const int l4start = am >> 2;
 
   const int t = threadIdx.x;
-  const int zq = t & 7, n = t >> 3;
-  float2 acc[32][2];
+  const int lane = t & 63, wave = t >> 6;
+  const int l32 = lane & 31, h = lane >> 5;
+  v16f acc[8];
 #pragma unroll
-  for (int l = 0; l < 32; ++l) { acc[l][0] = make_float2(0.f, 0.f); acc[l][1] = make_float2(0.f, 0.f); }
+  for (int j = 0; j < 8; ++j)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
 
   // Loads are unconditional (clamped addresses, values zeroed by select) so that all of a chunk's
   // loads are in flight together, and the next chunk is fetched while the current one is consumed.
@@ -112,13 +120,9 @@ __global__ __launch_bounds__(256) void wigner_fwd_tiled(const float2* __restrict
   const int chunk_elems = KB * ZT * NW;
   const float2* xbase = X + ((size_t)zt * MW + mi) * n2 * ZT * NW;
   const int n2elems = n2 * ZT * NW;
-  int xlds[KB * 2];
-#pragma unroll
-  for (int i = 0; i < KB * 2; ++i) {
-    const int e = t + 256 * i;
-    const int row = e / NW;                     // beta_local * 16 + z
-    xlds[i] = e < chunk_elems ? row * XLD + (e - row * NW) : -1;
-  }
+  const float inv_nw = 1.0f / (float)NW;         // e / NW for e < 4096, NW <= 32: (e + 0.5) * inv_nw truncates exactly
+  // columns n >= NW of the X chunk are never loaded: clear them once (T is zero there, but 0 * NaN is not)
+  for (int i = t; i < KB * ZT * XLD_M; i += 256) Xs[i] = make_float2(0.f, 0.f);
 
   auto load_chunk = [&](int b0) {
     const int e0 = b0 * ZT * NW;
@@ -136,56 +140,64 @@ __global__ __launch_bounds__(256) void wigner_fwd_tiled(const float2* __restrict
     }
   };
 
+  // operand addresses of this lane: A = Ts[(beta_local * 32 + n) * TLD + l], B = Xs[(beta_local * 16 + z) * XLD_M + n].c
+  const float* Xf = reinterpret_cast<const float*>(Xs);
+  const int a_off = (h * 32 + 8 * wave) * TLD + l32;
+  const int b_off = ((h * ZT + (l32 >> 1)) * XLD_M + 8 * wave) * 2 + (l32 & 1);
+
   load_chunk(0);
   for (int b0 = 0; b0 < n2; b0 += KB) {
     __syncthreads();
 #pragma unroll
-    for (int i = 0; i < KB * 2; ++i)
-      if (xlds[i] >= 0) Xs[xlds[i]] = xr[i];
+    for (int i = 0; i < KB * 2; ++i) {
+      const int e = t + 256 * i;
+      const int row = (int)(((float)e + 0.5f) * inv_nw);     // beta_local * 16 + z
+      if (e < chunk_elems) Xs[row * XLD_M + (e - row * NW)] = xr[i];
+    }
 #pragma unroll
     for (int bt = 0; bt < KB; ++bt) *reinterpret_cast<float4*>(Ts + bt * 32 * TLD + tlds) = tr_[bt];
     __syncthreads();
     if (b0 + KB < n2) load_chunk(b0 + KB);
-#pragma unroll 2
-    for (int bt = 0; bt < KB; ++bt) {
-      const float2 x0 = Xs[(bt * ZT + 2 * zq) * XLD + n];
-      const float2 x1 = Xs[(bt * ZT + 2 * zq + 1) * XLD + n];
-      const float4* tr = reinterpret_cast<const float4*>(Ts + (bt * 32 + n) * TLD);
 #pragma unroll
-      for (int l4 = 0; l4 < 8; ++l4) {
-        if (l4 >= l4start) {
-          const float4 tv = tr[l4];
-          const float tt[4] = {tv.x, tv.y, tv.z, tv.w};
+    for (int q = 0; q < KB / 2; ++q) {          // beta pair (2q, 2q+1) of the chunk
 #pragma unroll
-          for (int u = 0; u < 4; ++u) {
-            acc[4 * l4 + u][0].x += tt[u] * x0.x; acc[4 * l4 + u][0].y += tt[u] * x0.y;
-            acc[4 * l4 + u][1].x += tt[u] * x1.x; acc[4 * l4 + u][1].y += tt[u] * x1.y;
-          }
-        }
+      for (int j = 0; j < 8; ++j) {
+        const float a = Ts[a_off + (2 * q * 32 + j) * TLD];
+        const float b = Xf[b_off + (2 * q * ZT * XLD_M + j) * 2];
+        acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[j], 0, 0, 0);
       }
     }
   }
 
-  // ---- write out[lmn][z] and its mirror (-m,-n); (m < 0, n = 0) is written by the workgroup of -m
-  if (n >= NW || (n == 0 && m < 0)) return;
-  const long z = z0 + 2 * zq;
+  // ---- write out[lmn][z].c and its mirror (-m,-n); (m < 0, n = 0) is written by the workgroup of -m.
+  // Accumulator register v of lane (l32 = 2 z + c, h) holds degree l = 8 (v / 4) + 4 h + v % 4.
+  const long z = z0 + (l32 >> 1);
   if (z >= nbatch) return;
-  const bool pair = (z + 1 < nbatch);
-  const bool vec = pair && ((nbatch & 1) == 0);
-  const bool mirror = (n > 0 || m > 0);
-  const float sgn = ((m - n) & 1) ? -1.f : 1.f;
-  const int lmin = am > n ? am : n;
+  const int c = l32 & 1;
+  float* outf = reinterpret_cast<float*>(out) + z * 2 + c;
+  const size_t rowf = (size_t)nbatch * 2;        // floats per spectral row
+  // lmn(l, m, n) = lbase[l] + m (2l+1) + n with lbase[l] = l(4l^2-1)/3 + l(2l+1) + l; the mirror is lbase[l] - m(2l+1) - n
+  int lbase[16], lcoef[16];
 #pragma unroll
-  for (int l = 0; l < 32; ++l) {
-    if (l >= lmin && l < nl) {
-      const float2 a0 = acc[l][0], a1 = acc[l][1];
-      float2* p = out + (size_t)lmn_index(l, m, n) * nbatch + z;
-      if (vec) *reinterpret_cast<float4*>(p) = make_float4(a0.x, a0.y, a1.x, a1.y);
-      else { p[0] = a0; if (pair) p[1] = a1; }
-      if (mirror) {
-        float2* q = out + (size_t)lmn_index(l, -m, -n) * nbatch + z;
-        if (vec) *reinterpret_cast<float4*>(q) = make_float4(sgn * a0.x, -sgn * a0.y, sgn * a1.x, -sgn * a1.y);
-        else { q[0] = make_float2(sgn * a0.x, -sgn * a0.y); if (pair) q[1] = make_float2(sgn * a1.x, -sgn * a1.y); }
+  for (int v = 0; v < 16; ++v) {
+    const int l = 8 * (v / 4) + 4 * h + (v % 4);
+    lcoef[v] = 2 * l + 1;
+    lbase[v] = l * (4 * l * l - 1) / 3 + l * (2 * l + 1) + l;
+  }
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int n = 8 * wave + j;
+    if (n >= NW || (n == 0 && m < 0)) continue;
+    const bool mirror = (n > 0 || m > 0);
+    const float sg = (((m - n) & 1) ? -1.f : 1.f) * (c ? -1.f : 1.f);
+    const int lmin = am > n ? am : n;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int l = 8 * (v / 4) + 4 * h + (v % 4);
+      if (l >= lmin && l < nl) {
+        const int d = m * lcoef[v] + n;
+        outf[(size_t)(lbase[v] + d) * rowf] = acc[j][v];
+        if (mirror) outf[(size_t)(lbase[v] - d) * rowf] = sg * acc[j][v];
       }
     }
   }

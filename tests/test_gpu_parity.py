@@ -235,6 +235,48 @@ def test_config1_shaped_network(hip):
     close(got, want, "config-1 features")
 
 
+def _config5_layers(seed=8):
+    """BASELINE config 5 (SHREC17-shaped): S2Conv 6->100 b128->32, SO3Conv 100->100 b32->22, SO3Conv 100->55 b22->7,
+    near-identity grids with max_beta scaled by the bandwidth ratio (examples/shrec17/model_original.py:12-40)."""
+    import math
+    g1 = s2cnn_amd.s2_near_identity_grid(max_beta=math.pi / 8 * 30 / 128, n_alpha=8, n_beta=3)
+    g2 = s2cnn_amd.so3_near_identity_grid(max_beta=math.pi / 8 * 30 / 32, max_gamma=2 * math.pi, n_alpha=8, n_beta=3, n_gamma=8)
+    g3 = s2cnn_amd.so3_near_identity_grid(max_beta=math.pi / 8 * 30 / 22, max_gamma=2 * math.pi, n_alpha=8, n_beta=3, n_gamma=8)
+    torch.manual_seed(seed)
+    return (s2cnn_amd.S2Convolution(6, 100, 128, 32, g1), s2cnn_amd.SO3Convolution(100, 100, 32, 22, g2),
+            s2cnn_amd.SO3Convolution(100, 55, 22, 7, g3)), (g1, g2, g3)
+
+
+def test_config5_shaped_network(hip):
+    """Forward parity against the oracle at batch 1; forward + backward at batch 4 on the GPU must reproduce the
+    batch-1 result for its first sample (batch independence) and give finite gradients."""
+    (c1, c2, c3), (g1, g2, g3) = _config5_layers()
+    x = torch.rand(4, 6, 256, 256, generator=torch.Generator().manual_seed(9))
+    x1 = x[:1].double()
+
+    def kb(c):
+        return c.kernel.detach().double(), c.bias.detach().double()
+
+    y = O.s2_conv(x1, *kb(c1), 128, 32, g1)
+    y = O.so3_conv(torch.relu(y), *kb(c2), 32, 22, g2)
+    y = O.so3_conv(torch.relu(y), *kb(c3), 22, 7, g3)
+    want = O.so3_integrate(y)
+    c1, c2, c3 = c1.cuda(), c2.cuda(), c3.cuda()
+
+    def net(t):
+        return s2cnn_amd.so3_integrate(c3(torch.relu(c2(torch.relu(c1(t))))))
+
+    with torch.no_grad():
+        got1 = net(x[:1].cuda())
+    close(got1, want, "config-5 features, batch 1")
+    xg = x.cuda().requires_grad_()
+    out = net(xg)
+    (out ** 2).sum().backward()
+    assert (out[:1] - got1).abs().max().item() < 1e-4 * got1.abs().max().item()
+    for t in (xg.grad, c1.kernel.grad, c2.kernel.grad, c3.kernel.grad, c3.bias.grad):
+        assert torch.isfinite(t).all() and t.abs().max().item() > 0
+
+
 def test_z_rotation_equivariance_on_gpu(hip):
     """examples/equivariance_error/main.py:18-46 of the reference at reduced sizes."""
     torch.manual_seed(2)
