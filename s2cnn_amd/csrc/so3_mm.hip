@@ -213,24 +213,39 @@ __device__ __forceinline__ void stage_mma(const float2* As, const float2* Bs, v1
   }
 }
 
-// The contraction loop of one tile: LDS stage s is consumed while the global loads of stage s+1 are in flight.
+// The contraction loop of one tile.  LDS is double buffered: while the matrix cores consume stage s from one
+// buffer, the operands of stage s+1 (fetched during stage s-1) are written to the other and the global loads
+// of stage s+2 are issued; one barrier per stage.
 template <typename C_, int NI, int NJ, typename LA, typename LB>
 __device__ __forceinline__ void contract(LA& la, LB& lb, float2* As, float2* Bs, v16f (&acc_re)[NRB][NCB], v16f (&acc_im)[NRB][NCB],
                                          int nstage, int nkc, int arow, int bcol, int h) {
+  constexpr int AEL = TileShape<C_::A_KC, TM>::ELEMS, BEL = TileShape<C_::B_KC, TN>::ELEMS;
+  int kb = 0, kc = 0;
+  auto advance = [&]() { if (++kc == nkc) { kc = 0; ++kb; } };
   la.load(0, 0);
   lb.load(0, 0);
-  int kb = 0, kc = 0;
+  la.store(As);
+  lb.store(Bs);
+  advance();
+  if (nstage > 1) {
+    la.load(kb, kc * TK);
+    lb.load(kb, kc * TK);
+  }
+  __syncthreads();
   for (int stage = 0; stage < nstage; ++stage) {
-    __syncthreads();
-    la.store(As);
-    lb.store(Bs);
-    __syncthreads();
-    if (++kc == nkc) { kc = 0; ++kb; }
+    const int cur = stage & 1;
     if (stage + 1 < nstage) {
-      la.load(kb, kc * TK);
-      lb.load(kb, kc * TK);
+      la.store(As + (cur ^ 1) * AEL);       // that buffer was last read in stage - 1, which every wave has left
+      lb.store(Bs + (cur ^ 1) * BEL);
+      advance();
+      if (stage + 2 < nstage) {
+        la.load(kb, kc * TK);
+        lb.load(kb, kc * TK);
+      }
     }
-    if (NI > 0 && NJ > 0) stage_mma<C_, (NI > 0 ? NI : 1), (NJ > 0 ? NJ : 1)>(As, Bs, acc_re, acc_im, arow, bcol, h);
+    if (NI > 0 && NJ > 0)
+      stage_mma<C_, (NI > 0 ? NI : 1), (NJ > 0 ? NJ : 1)>(As + cur * AEL, Bs + cur * BEL, acc_re, acc_im, arow, bcol, h);
+    __syncthreads();
   }
 }
 
@@ -243,8 +258,8 @@ __host__ __device__ inline void tile_counts(int L, int RI, int CI, int& tm, int&
 template <int MODE, int VEC>
 __global__ __launch_bounds__(NT) void so3_block_mm_kernel(MmParams p) {
   typedef Cfg<MODE> C_;
-  __shared__ __attribute__((aligned(16))) float2 As[TileShape<C_::A_KC, TM>::ELEMS];
-  __shared__ __attribute__((aligned(16))) float2 Bs[TileShape<C_::B_KC, TN>::ELEMS];
+  __shared__ __attribute__((aligned(16))) float2 As[2 * TileShape<C_::A_KC, TM>::ELEMS];
+  __shared__ __attribute__((aligned(16))) float2 Bs[2 * TileShape<C_::B_KC, TN>::ELEMS];
 
   // ---- which tile: degrees in descending order so the heaviest tiles are dispatched first
   int t = blockIdx.x;
