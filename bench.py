@@ -43,6 +43,96 @@ def so3_fft_bytes(b_in, b_out, n):
     return 4.0 * n * (2 * b_in) ** 3 + 8.0 * n * nspec(b_out)
 
 
+def measure_rows(torch, dev, with_cpu):
+    """Every other op of the path at its BASELINE-config size: GPU time (events on the launch stream), the
+    algorithmic bytes or flops, the roofline fraction, and the CPU oracle on a bounded sample beside it."""
+    import s2cnn_amd
+    from s2cnn_amd import _hip
+    from s2cnn_amd.soft import s2_fft as PS2
+    from s2cnn_amd.soft import so3_fft as PSO3
+    from oracle import cpu_path as O
+
+    def gpu_ms(fn, reps=5):
+        for _ in range(2):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps
+
+    def cpu_s(fn):
+        if not with_cpu:
+            return None
+        t0 = time.perf_counter()
+        fn()
+        return time.perf_counter() - t0
+
+    rows = {}
+
+    def add(name, ms, work, unit, cpu_t, cpu_frac, note):
+        rate = work / (ms * 1e-3)
+        if unit == "B":
+            ent = {"ms": round(ms, 4), "bound": "hbm", "achieved_GBs": round(rate / 1e9, 1), "frac": round(rate / 1e9 / PEAK_HBM_GBS, 4)}
+        else:
+            ent = {"ms": round(ms, 4), "bound": "mfma", "achieved_TFLOPs": round(rate / 1e12, 2),
+                   "frac": round(rate / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4)}
+        if cpu_t is not None:
+            ent["cpu_s_full_size_estimate"] = round(cpu_t / cpu_frac, 3)
+            ent["cpu_sample"] = note
+        rows[name] = ent
+
+    g = torch.Generator().manual_seed(11)
+    # --- S^2 ops at config-5 sizes: x [32, 6, 256, 256] -> [1024, 192, 2]; s2_mm 6 -> 100 features at nl = 32
+    B5, Fi5, Fo5, b5i, b5o = 32, 6, 100, 128, 32
+    xs2 = torch.rand(B5, Fi5, 2 * b5i, 2 * b5i, generator=g)
+    xs2g = xs2.to(dev)
+    s2spec = PS2.s2_rfft(xs2g, b_out=b5o)
+    by = 4.0 * xs2.numel() + 8.0 * s2spec.numel() / 2
+    t = cpu_s(lambda: O.s2_fft(O.as_complex(xs2[:4]), b_out=b5o))
+    add("s2_analysis [32,6,256,256]->b32", gpu_ms(lambda: PS2.s2_rfft(xs2g, b_out=b5o)), by, "B", t, 4 / B5, "batch 4 of 32")
+    gspec = torch.randn_like(s2spec)
+    t = cpu_s(lambda: O.s2_ifft(gspec[:, :4].cpu(), for_grad=True, b_out=b5i))
+    add("s2_synthesis b32->[32,6,256,256]", gpu_ms(lambda: PS2.s2_rifft(gspec, for_grad=True, b_out=b5i)), by, "B", t, 4 / B5, "batch 4 of 32")
+    xk = torch.randn(b5o * b5o, B5, Fi5, 2, generator=g)
+    yk = torch.randn(b5o * b5o, Fi5, Fo5, 2, generator=g)
+    xkg, ykg = xk.to(dev).requires_grad_(), yk.to(dev).requires_grad_()
+    zk = s2cnn_amd.s2_mm(xkg, ykg)
+    gzk = torch.randn_like(zk)
+    zbytes = 4.0 * zk.numel()
+    t = cpu_s(lambda: O.s2_mm(xk[:, :2], yk))
+    add("s2_mm fwd nl=32 B=32 6->100", gpu_ms(lambda: s2cnn_amd.s2_mm(xkg, ykg)), zbytes + 4.0 * (xk.numel() + yk.numel()), "B", t, 2 / B5, "batch 2 of 32")
+    add("s2_mm grad (x and y)", gpu_ms(lambda: torch.autograd.grad(zk, (xkg, ykg), gzk, retain_graph=True)),
+        2 * zbytes + 4.0 * 2 * (xk.numel() + yk.numel()), "B", None, 1, "")
+    del zk, gzk, xkg, ykg, s2spec, gspec, xs2g
+    # --- Haar integral at config-4 output size [16, 64, 64, 64, 64]
+    xi = torch.randn(16, 64, 64, 64, 64, device=dev)
+    t = cpu_s(lambda: O.so3_integrate(xi[:2].cpu()))
+    add("so3_integrate [16,64,64^3]", gpu_ms(lambda: s2cnn_amd.so3_integrate(xi)), 4.0 * xi.numel(), "B", t, 2 / 16, "batch 2 of 16")
+    del xi
+    # --- complex SO(3) transforms (so3_fft / so3_ifft) at b = 32, 16 volumes
+    xc = torch.randn(16, 64, 64, 64, 2, device=dev)
+    sc = PSO3.so3_fft(xc)
+    byc = 4.0 * xc.numel() + 4.0 * sc.numel()
+    t = cpu_s(lambda: O.so3_fft(xc[:1].cpu()))
+    add("so3_fft complex b=32 N=16", gpu_ms(lambda: PSO3.so3_fft(xc)), byc, "B", t, 1 / 16, "1 volume of 16")
+    t = cpu_s(lambda: O.so3_ifft(sc[:, :1].cpu()))
+    add("so3_ifft complex b=32 N=16", gpu_ms(lambda: PSO3.so3_ifft(sc)), byc, "B", t, 1 / 16, "1 volume of 16")
+    del xc, sc
+    # --- kernel -> spectrum (library GEMM) at config-4 size: [64, 64, 192] -> [43680, 64, 64, 2]
+    grid = s2cnn_amd.so3_near_identity_grid()
+    kk = torch.randn(64, 64, len(grid), device=dev)
+    s2cnn_amd.so3_rft(kk, 32, grid)
+    t = cpu_s(lambda: O.so3_rft(kk[:8].cpu(), 32, grid))
+    add("so3_rft [64,64,192]->b32", gpu_ms(lambda: s2cnn_amd.so3_rft(kk, 32, grid)), 2.0 * 64 * 64 * 192 * nspec(32) * 2, "F", t, 8 / 64,
+        "8 of 64 input features")
+    torch.cuda.empty_cache()
+    return rows
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -50,6 +140,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-fft", action="store_true", help="skip the standalone FFT round trip")
+    ap.add_argument("--rows", action="store_true", help="also time every other op of the path (adds a `rows` object)")
     ap.add_argument("--batch", type=int, default=16)
     ap.add_argument("--b", type=int, default=32)
     ap.add_argument("--features", type=int, default=64)
@@ -147,6 +238,9 @@ def main():
                              "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4)}
         del xf
         torch.cuda.empty_cache()
+
+    if args.rows:
+        result["rows"] = measure_rows(torch, dev, not args.no_cpu)
 
     # ---- CPU baseline: the oracle (a restatement of the reference's CPU branches) on a bounded sample
     if not args.no_cpu:
