@@ -33,9 +33,10 @@ def nspec(b):
     return b * (4 * b * b - 1) // 3
 
 
-def mm_flops(nl, B, Fi, Fo):
-    """Algorithmic flops of one so3_mm pass: 8 B Fi Fo sum_l (2l+1)^3 = 8 B Fi Fo nl^2 (2 nl^2 - 1)."""
-    return 8.0 * B * Fi * Fo * nl * nl * (2 * nl * nl - 1)
+def mm_flops(nl, B, Fi, Fo, real=True):
+    """Algorithmic flops of one block product: B Fi Fo sum_l (2l+1)^3 = B Fi Fo nl^2 (2 nl^2 - 1) multiply-adds,
+    real (2 flops each) in the real basis the layer uses, complex (8 flops each) in so3_mm proper."""
+    return (2.0 if real else 8.0) * B * Fi * Fo * nl * nl * (2 * nl * nl - 1)
 
 
 def so3_fft_bytes(b_in, b_out, n):
@@ -140,6 +141,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-fft", action="store_true", help="skip the standalone FFT round trip")
+    ap.add_argument("--complex-product", action="store_true",
+                    help="multiply complex spectra as the reference does instead of real-basis ones")
     ap.add_argument("--rows", action="store_true", help="also time every other op of the path (adds a `rows` object)")
     ap.add_argument("--batch", type=int, default=16)
     ap.add_argument("--b", type=int, default=32)
@@ -165,6 +168,7 @@ def main():
     x_cpu = torch.randn(B, F, 2 * b, 2 * b, 2 * b, generator=gen)
     k_cpu = torch.randn(F, F, len(grid), generator=torch.Generator().manual_seed(7)) * math.sqrt(2.0 / (F * len(grid)))
     layer = s2cnn_amd.SO3Convolution(F, F, b, b, grid)
+    layer.real_basis = not args.complex_product
     with torch.no_grad():
         layer.kernel.copy_(k_cpu)
     layer = layer.to(dev)
@@ -190,9 +194,10 @@ def main():
     value = B / (ms_per_step * 1e-3)
 
     per_call = {k: sum(v) / len(v) for k, v in timer.summary().items()}
-    flops = mm_flops(b, B, F, F)
-    mm_names = [n for n in per_call if n.startswith("s2cnn_so3_mm_")]   # fwd / gradx / grady (planar-y entry points in the layer)
+    mm_names = [n for n in per_call if n.startswith("s2cnn_so3_mm_")]   # fwd / gradx / grady of the product the layer ran
     dominant = max(mm_names, key=lambda n: per_call[n])
+    flops_of = {n: mm_flops(b, B, F, F, real="_real_" in n) for n in mm_names}
+    flops = flops_of[dominant]
     ach = flops / (per_call[dominant] * 1e-3) / 1e12
     roofline = {"bound": "mfma", "kernel": dominant, "achieved": round(ach, 2), "peak": PEAK_FP32_MFMA_TFLOPS,
                 "unit": "TFLOP/s", "frac": round(ach / PEAK_FP32_MFMA_TFLOPS, 4),
@@ -200,7 +205,7 @@ def main():
                 "flop_per_launch": flops, "ms_per_launch": round(per_call[dominant], 3)}
     kernels = {n: {"ms": round(ms, 3)} for n, ms in per_call.items()}
     for n in mm_names:
-        kernels[n]["tflops"] = round(flops / (per_call[n] * 1e-3) / 1e12, 2)
+        kernels[n]["tflops"] = round(flops_of[n] / (per_call[n] * 1e-3) / 1e12, 2)
     for n in ("s2cnn_so3_analysis", "s2cnn_so3_synthesis"):
         kernels[n]["gbs"] = round(so3_fft_bytes(b, b, B * F) / (per_call[n] * 1e-3) / 1e9, 1)
 

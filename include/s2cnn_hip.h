@@ -60,6 +60,35 @@ int s2cnn_so3_mm_gradx(const float *gz, const float *y, float *gx,
 int s2cnn_so3_mm_grady(const float *gz, const float *x, float *gy,
                        int nl, int nbatch, int f_in, int f_out, void *stream);
 
+/* ---- the same products for spectra of REAL signals, in the real basis -----------------
+ * The spectrum of a real signal on SO(3) obeys X[l,-m,-n] = (-1)^(m-n) conj(X[l,m,n]), and so do the
+ * kernel spectrum of so3_ft.py:4-25 (real kernel) and every product and gradient the convolution
+ * layer soft/so3_conv.py:36-56 forms from them.  A fixed unitary U_l per degree,
+ *     U[0,0] = 1,  U[+m,m] = 1/sqrt2,  U[+m,-m] = (-1)^m/sqrt2,  U[-m,m] = -i/sqrt2,  U[-m,-m] = i(-1)^m/sqrt2
+ * (rows r = -l..l stored at l + r), makes every block R = U X U^H real, and  U (X Y^H) U^H = R_x R_y^T:
+ * the complex products above become real ones with a quarter of the multiply-adds.  The reference
+ * does not exploit this; the entries below have no counterpart there and are used by the convolution
+ * layer only, where the symmetry is guaranteed.
+ *
+ * to_real    : x [nspec(nl), ncols, 2] -> r [nspec(nl), ncols],  r = Re(U x U^H) per column (any x)
+ * to_complex : r [nspec(nl), ncols] -> x [nspec(nl), ncols, 2],  x = U^H r U  (inverse on real-signal
+ *              spectra, and the adjoint of to_real)
+ * mm_real    : x [nspec, nbatch, f_in], y [nspec, f_in, f_out], z [nspec, nbatch, f_out]
+ *   fwd   : z [l,m,n,i,j] = sum_{p,k} x [l,m,p,i,k] * y[l,n,p,k,j]
+ *   gradx : gx[l,m,p,i,k] = sum_{n,j} gz[l,m,n,i,j] * y[l,n,p,k,j]
+ *   grady : gy[l,n,p,k,j] = sum_{m,i} gz[l,m,n,i,j] * x[l,m,p,i,k]
+ * Pointers of mm_real need 4-byte alignment only (16-byte and feature counts divisible by 4 for the
+ * fast path).
+ */
+int s2cnn_so3_spectrum_to_real(const float *x, float *r, int nl, long ncols, void *stream);
+int s2cnn_so3_spectrum_to_complex(const float *r, float *x, int nl, long ncols, void *stream);
+int s2cnn_so3_mm_real_fwd(const float *x, const float *y, float *z,
+                          int nl, int nbatch, int f_in, int f_out, void *stream);
+int s2cnn_so3_mm_real_gradx(const float *gz, const float *y, float *gx,
+                            int nl, int nbatch, int f_in, int f_out, void *stream);
+int s2cnn_so3_mm_real_grady(const float *gz, const float *x, float *gy,
+                            int nl, int nbatch, int f_in, int f_out, void *stream);
+
 /* ---- S^2 x S^2 -> SO(3) spectral outer products -------------------------------------
  * x  [nl^2, nbatch, f_in , 2]
  * y  [nl^2, f_in  , f_out, 2]

@@ -138,6 +138,39 @@ def so3_ft_matrix(b, grid):
     return out
 
 
+def real_basis_matrix(l):
+    """Unitary U_l [2l+1, 2l+1] (complex128) that makes the degree-l block of a real signal's SO(3)
+    spectrum real: for X[-m,-n] = (-1)^(m-n) conj(X[m,n]) the matrix U X U^H has no imaginary part.
+    Rows are the real index r = -l..l (r > 0 cosine-like, r < 0 sine-like), columns m = -l..l."""
+    L = 2 * l + 1
+    U = np.zeros((L, L), dtype=np.complex128)
+    U[l, l] = 1.0
+    s = 1.0 / np.sqrt(2.0)
+    for m in range(1, l + 1):
+        sg = -1.0 if m & 1 else 1.0
+        U[l + m, l + m] = s
+        U[l + m, l - m] = sg * s
+        U[l - m, l + m] = -1j * s
+        U[l - m, l - m] = 1j * sg * s
+    return U
+
+
+def so3_ft_matrix_real(b, grid):
+    """The matrix of so3_ft_matrix in the real basis: Re(U_l F[a, l] U_l^H) per grid point and degree,
+    float64 [len(grid), nspec(b)].  The imaginary part that is dropped vanishes identically because
+    Wigner D-functions obey D^l_{-m,-n} = (-1)^(m-n) conj(D^l_{mn})."""
+    F = so3_ft_matrix(b, grid)
+    out = np.empty(F.shape, dtype=np.float64)
+    pos = 0
+    for l in range(b):
+        L = 2 * l + 1
+        U = real_basis_matrix(l)
+        blk = F[:, pos:pos + L * L].reshape(-1, L, L)
+        out[:, pos:pos + L * L] = np.einsum("rm,amn,sn->ars", U, blk, U.conj()).real.reshape(-1, L * L)
+        pos += L * L
+    return out
+
+
 def s2_ft_matrix(b, grid):
     """F[a, lm] = 2b conj(D^l_{m0}(alpha_a, beta_a, 0)) for grid points given as
     (beta, alpha) tuples: complex128 [len(grid), b^2] (s2cnn/s2_ft.py:28-50)."""

@@ -1,0 +1,205 @@
+"""The real basis of SO(3) spectra of real signals (no counterpart in the reference, so pinned by
+mathematics and by the oracle's complex path): unitarity, reality of transformed spectra that the
+oracle computes from real signals, the product identity U (X Y^H) U^H = X_r Y_r^T against the oracle's
+complex so3_mm, and the real-basis kernel matrix against the complex one."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import cpu_path as O
+from s2cnn_amd import wigner
+
+
+def dense_to_real(x):
+    """x [nspec, ...] complex128 ndarray -> U x U^H per degree (complex; caller checks / takes the real part)."""
+    out = np.empty_like(x)
+    pos, l = 0, 0
+    while pos < x.shape[0]:
+        L = 2 * l + 1
+        U = wigner.real_basis_matrix(l)
+        blk = x[pos:pos + L * L].reshape(L, L, -1)
+        out[pos:pos + L * L] = np.einsum("rm,mnc,sn->rsc", U, blk, U.conj()).reshape(L * L, *x.shape[1:])
+        pos += L * L
+        l += 1
+    return out
+
+
+def dense_to_complex(r):
+    out = np.empty(r.shape, dtype=np.complex128)
+    pos, l = 0, 0
+    while pos < r.shape[0]:
+        L = 2 * l + 1
+        U = wigner.real_basis_matrix(l)
+        blk = r[pos:pos + L * L].reshape(L, L, -1)
+        out[pos:pos + L * L] = np.einsum("rm,rsc,sn->mnc", U.conj(), blk, U).reshape(L * L, *r.shape[1:])
+        pos += L * L
+        l += 1
+    return out
+
+
+def as_np(t):
+    t = t.detach().double().numpy()
+    return t[..., 0] + 1j * t[..., 1]
+
+
+@pytest.mark.parametrize("l", [0, 1, 2, 5, 8])
+def test_unitary(l):
+    U = wigner.real_basis_matrix(l)
+    assert np.allclose(U @ U.conj().T, np.eye(2 * l + 1), atol=1e-14)
+
+
+@pytest.mark.parametrize("b", [3, 6])
+def test_spectrum_of_real_signal_becomes_real(b):
+    x = torch.randn(2, 2 * b, 2 * b, 2 * b, dtype=torch.float64, generator=torch.Generator().manual_seed(b))
+    X = as_np(O.so3_rfft(x))
+    R = dense_to_real(X)
+    assert np.abs(R.imag).max() < 1e-12 * np.abs(R).max()
+    assert np.allclose(dense_to_complex(R.real), X, atol=1e-12)
+    # an asymmetric spectrum does NOT become real: the test above is not vacuous
+    Y = X.copy()
+    Y[4] += 1.0          # (l, m, n) = (1, 0, -1) alone
+    assert np.abs(dense_to_real(Y).imag).max() > 0.1
+
+
+def test_product_identity_against_oracle_so3_mm():
+    b, B, Fi, Fo = 4, 2, 3, 2
+    g = torch.Generator().manual_seed(1)
+    x = O.so3_rfft(torch.randn(B * Fi, 2 * b, 2 * b, 2 * b, dtype=torch.float64, generator=g))
+    y = O.so3_rfft(torch.randn(Fi * Fo, 2 * b, 2 * b, 2 * b, dtype=torch.float64, generator=g))
+    ns = x.shape[0]
+    x = x.reshape(ns, B, Fi, 2)
+    y = y.reshape(ns, Fi, Fo, 2)
+    z = as_np(O.so3_mm(x, y))
+    xr, yr = dense_to_real(as_np(x)).real, dense_to_real(as_np(y)).real
+    zr = np.empty((ns, B, Fo))
+    pos = 0
+    for l in range(b):
+        L = 2 * l + 1
+        xa = xr[pos:pos + L * L].reshape(L, L, B, Fi)
+        ya = yr[pos:pos + L * L].reshape(L, L, Fi, Fo)
+        zr[pos:pos + L * L] = np.einsum("mpik,npkj->mnij", xa, ya).reshape(L * L, B, Fo)
+        pos += L * L
+    assert np.allclose(dense_to_complex(zr), z, atol=1e-10 * np.abs(z).max())
+
+
+def test_real_kernel_matrix_matches_complex_one():
+    b = 5
+    grid = tuple((0.1 * i + 0.05, 0.3 * i, -0.2 * i + 1.0) for i in range(7))
+    F = wigner.so3_ft_matrix(b, grid)
+    Fr = wigner.so3_ft_matrix_real(b, grid)
+    assert np.allclose(dense_to_complex(Fr.T.copy()).T, F, atol=1e-12)
+    # and against the oracle's so3_rft of a real kernel
+    k = torch.randn(3, len(grid), dtype=torch.float64, generator=torch.Generator().manual_seed(2))
+    Y = as_np(O.so3_rft(k, b, grid))                       # [nspec, 3]
+    Yr = (k.numpy() @ Fr).T
+    assert np.allclose(dense_to_real(Y).real, Yr, atol=1e-12)
+    assert np.abs(dense_to_real(Y).imag).max() < 1e-12
+
+
+# ------------------------------------------------------------------ GPU kernels
+def _close(got, want, tol=1e-4):
+    got = got.detach().double().cpu().numpy()
+    scale = max(want.std(), 1e-30)
+    q = np.abs(got - want).max() / scale
+    print(f"max|d|/std={q:.2e}", flush=True)
+    assert got.shape == want.shape and q < tol, q
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("nl,cols", [(1, (3,)), (4, (2, 3)), (7, (5, 1)), (12, (16, 20))])
+def test_basis_kernels_against_dense(hip, nl, cols):
+    import s2cnn_amd
+    print(f"real basis kernels nl={nl} cols={cols}", flush=True)
+    ns = O.nspec_so3(nl)
+    g = torch.Generator().manual_seed(nl)
+    x = torch.randn(ns, *cols, 2, generator=g)          # arbitrary, not symmetric: to_real is Re(U x U^H)
+    r = torch.randn(ns, *cols, generator=g)
+    xr = s2cnn_amd.so3_spectrum_to_real(x.cuda())
+    _close(xr, dense_to_real(as_np(x).reshape(ns, -1)).real.reshape(ns, *cols))
+    xc = s2cnn_amd.so3_spectrum_to_complex(r.cuda())
+    want = dense_to_complex(r.double().numpy().reshape(ns, -1)).reshape(ns, *cols)
+    _close(xc, np.stack((want.real, want.imag), -1))
+    # adjoint pair: <to_real x, r> = <x, to_complex r>
+    lhs = (xr.double().cpu() * r.double()).sum().item()
+    rhs = (x.double() * xc.double().cpu()).sum().item()
+    assert abs(lhs - rhs) < 1e-4 * max(abs(lhs), 1.0)
+    # autograd wiring
+    xg = x.cuda().requires_grad_()
+    (s2cnn_amd.so3_spectrum_to_real(xg) * r.cuda()).sum().backward()
+    _close(xg.grad, np.stack((want.real, want.imag), -1))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("nl,B,Fi,Fo", [(4, 2, 3, 5), (3, 32, 20, 40), (6, 3, 7, 55), (8, 16, 64, 64), (5, 1, 1, 1),
+                                        (12, 16, 32, 48), (9, 4, 100, 36)])
+def test_so3_mm_real_forward_backward(hip, nl, B, Fi, Fo):
+    import s2cnn_amd
+    print(f"so3_mm_real nl={nl} B={B} Fi={Fi} Fo={Fo}", flush=True)
+    ns = O.nspec_so3(nl)
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(ns, B, Fi, generator=g)
+    y = torch.randn(ns, Fi, Fo, generator=g) * Fi ** -0.5
+    gz = torch.randn(ns, B, Fo, generator=g)
+    xd, yd, gd = x.double().numpy(), y.double().numpy(), gz.double().numpy()
+    z = np.empty((ns, B, Fo)); gx = np.empty((ns, B, Fi)); gy = np.empty((ns, Fi, Fo))
+    pos = 0
+    for l in range(nl):
+        L = 2 * l + 1
+        sl = slice(pos, pos + L * L)
+        xa, ya, ga = xd[sl].reshape(L, L, B, Fi), yd[sl].reshape(L, L, Fi, Fo), gd[sl].reshape(L, L, B, Fo)
+        z[sl] = np.einsum("mpik,npkj->mnij", xa, ya).reshape(L * L, B, Fo)
+        gx[sl] = np.einsum("mnij,npkj->mpik", ga, ya).reshape(L * L, B, Fi)
+        gy[sl] = np.einsum("mnij,mpik->npkj", ga, xa).reshape(L * L, Fi, Fo)
+        pos += L * L
+    xg, yg = x.cuda().requires_grad_(), y.cuda().requires_grad_()
+    zg = s2cnn_amd.so3_mm_real(xg, yg)
+    gxg, gyg = torch.autograd.grad(zg, (xg, yg), gz.cuda())
+    _close(zg, z)
+    _close(gxg, gx)
+    _close(gyg, gy)
+
+
+@pytest.mark.gpu
+def test_real_product_equals_oracle_complex_product(hip):
+    """to_complex(mm_real(to_real x, to_real y)) against the oracle's so3_mm on spectra of real signals."""
+    import s2cnn_amd
+    b, B, Fi, Fo = 6, 3, 4, 5
+    g = torch.Generator().manual_seed(3)
+    x = O.so3_rfft(torch.randn(B * Fi, 2 * b, 2 * b, 2 * b, generator=g))
+    y = O.so3_rfft(torch.randn(Fi * Fo, 2 * b, 2 * b, 2 * b, generator=g))
+    ns = x.shape[0]
+    x, y = x.reshape(ns, B, Fi, 2), y.reshape(ns, Fi, Fo, 2)
+    want = O.so3_mm(x.double(), y.double()).numpy()
+    got = s2cnn_amd.so3_spectrum_to_complex(
+        s2cnn_amd.so3_mm_real(s2cnn_amd.so3_spectrum_to_real(x.cuda()), s2cnn_amd.so3_spectrum_to_real(y.cuda())))
+    _close(got, want)
+
+
+@pytest.mark.gpu
+def test_so3_rft_real_matches_complex(hip):
+    import s2cnn_amd
+    b = 6
+    grid = s2cnn_amd.so3_near_identity_grid()
+    k = torch.randn(3, 4, len(grid), generator=torch.Generator().manual_seed(5))
+    want = O.so3_rft(k.double(), b, grid).numpy()
+    got = s2cnn_amd.so3_spectrum_to_complex(s2cnn_amd.so3_rft_real(k.cuda(), b, grid))
+    _close(got, want)
+
+
+@pytest.mark.gpu
+def test_convolution_real_and_complex_paths_agree(hip):
+    import s2cnn_amd
+    from s2cnn_amd.soft.so3_conv import SO3Convolution
+    torch.manual_seed(0)
+    conv = SO3Convolution(3, 4, 6, 4, s2cnn_amd.so3_near_identity_grid()).cuda()
+    x = torch.randn(2, 3, 12, 12, 12, device="cuda", requires_grad=True)
+    out = {}
+    for flag in (True, False):
+        conv.real_basis = flag
+        conv.zero_grad()
+        x.grad = None
+        z = conv(x)
+        z.pow(2).sum().backward()
+        out[flag] = (z.detach(), x.grad.clone(), conv.kernel.grad.clone())
+    for a, c in zip(out[True], out[False]):
+        _close(a, c.double().cpu().numpy())
