@@ -63,30 +63,35 @@ template <int VEC> struct VecT { typedef float type; };
 template <> struct VecT<4> { typedef float4 type; };
 
 // One operand's tile loader: global -> registers -> LDS.  EXT = tile extent along the free index,
-// VEC = floats per access.
+// VEC = floats per access.  The contraction index is the flattened pair (block kb, feature kin): a stage
+// takes the next TK values of it whatever the block size, so small blocks (a batch of 16 in grad y) fill
+// whole stages and odd block sizes pad only the very last stage.  load() fetches the current stage and
+// steps to the next one.
 template <bool KC, bool MNMAJ, int EXT, int VEC>
 struct TileLoader {
   static constexpr int NSLOT = EXT * TK / (NT * VEC);
   static constexpr int LD = TileShape<KC, EXT>::LD;
+  static constexpr int KSTEP = NT * VEC / EXT;     // MN-contiguous: contraction steps between slots
   typedef typename VecT<VEC>::type vec_t;
   static_assert(NSLOT >= 1 && NSLOT <= 32, "tile does not fit the workgroup");
 
   const float* base;    // start of degree l
   int off[KC ? NSLOT : 1];
   unsigned valid_mn;    // bit q: slot q's row is inside the matrix (KC) / bit 0 (MN-contiguous)
-  int kk;               // KC: this thread's k inside the stage; else k of slot 0
+  int kb, kin;          // block and feature of this thread's first contraction step in the current stage
   int lds_off;
   int blk_k_stride;
-  int MNI, KI;
+  int MNI, KI, L;
   vec_t reg[NSLOT];
 
-  __device__ void init(const float* base_l, int L, int MNI_, int KI_, int tile0) {
-    base = base_l; MNI = MNI_; KI = KI_;
+  __device__ void init(const float* base_l, int L_, int MNI_, int KI_, int tile0) {
+    base = base_l; MNI = MNI_; KI = KI_; L = L_;
     const int t = threadIdx.x;
     const int blk_elems = MNI * KI;
     const int blk_mn_stride = (MNMAJ ? L : 1) * blk_elems;
     blk_k_stride = (MNMAJ ? 1 : L) * blk_elems;
     valid_mn = 0;
+    int kk;
     if (KC) {
       constexpr int TPR = TK / VEC;
       kk = (t % TPR) * VEC;
@@ -96,7 +101,7 @@ struct TileLoader {
       for (int q = 0; q < NSLOT; ++q) {
         const int row = tile0 + r0 + q * (NT / TPR);
         const int mb = row / MNI, mi = row - mb * MNI;
-        off[q] = mb * blk_mn_stride + mi * KI + kk;
+        off[q] = mb * blk_mn_stride + mi * KI;
         if (row < L * MNI) valid_mn |= 1u << q;
       }
     } else {
@@ -108,33 +113,40 @@ struct TileLoader {
       off[0] = mb * blk_mn_stride + mi;
       if (mn < L * MNI) valid_mn = 1u;
     }
+    kb = kk / KI;
+    kin = kk - kb * KI;
   }
 
   // clamped address + select instead of a predicated load: all loads of a stage are in flight together
-  __device__ void load(int kb, int k0) {
-    const float* p = base + (size_t)kb * blk_k_stride;
+  __device__ __forceinline__ void load() {
     if (KC) {
-      const bool kvalid = (k0 + kk) < KI;
+      const bool kvalid = kb < L;
+      const int koff = kb * blk_k_stride + kin;
 #pragma unroll
       for (int q = 0; q < NSLOT; ++q) {
         const bool ok = kvalid && ((valid_mn >> q) & 1u);
-        const vec_t v = *reinterpret_cast<const vec_t*>(p + (ok ? off[q] + k0 : 0));
+        const vec_t v = *reinterpret_cast<const vec_t*>(base + (ok ? off[q] + koff : 0));
         reg[q] = ok ? v : vec_t{};
       }
     } else {
-      constexpr int KSTEP = NT * VEC / EXT;
+      int b = kb, k = kin;
 #pragma unroll
       for (int q = 0; q < NSLOT; ++q) {
-        const int k = k0 + kk + q * KSTEP;
-        const bool ok = valid_mn && k < KI;
-        const vec_t v = *reinterpret_cast<const vec_t*>(p + (ok ? off[0] + k * MNI : 0));
+        const bool ok = valid_mn && b < L;
+        const vec_t v = *reinterpret_cast<const vec_t*>(base + (ok ? b * blk_k_stride + off[0] + k * MNI : 0));
         reg[q] = ok ? v : vec_t{};
+        k += KSTEP;
+        if (KI >= KSTEP) { if (k >= KI) { k -= KI; ++b; } }
+        else { const int w = k / KI; b += w; k -= w * KI; }
       }
     }
+    kin += TK;
+    if (KI >= TK) { if (kin >= KI) { kin -= KI; ++kb; } }
+    else { const int w = kin / KI; kb += w; kin -= w * KI; }
   }
 
-  __device__ void store(float* tile) const {
-    constexpr int QSTEP = KC ? NT * VEC / TK : NT * VEC / EXT;   // rows (KC) or k-rows between slots
+  __device__ __forceinline__ void store(float* tile) const {
+    constexpr int QSTEP = KC ? NT * VEC / TK : KSTEP;   // rows (KC) or k-rows between slots
 #pragma unroll
     for (int q = 0; q < NSLOT; ++q)
       *reinterpret_cast<vec_t*>(tile + lds_off + q * QSTEP * LD) = reg[q];
@@ -185,32 +197,29 @@ __device__ __forceinline__ void stage_mma(const float* As, const float* Bs, v16f
 }
 
 // Double-buffered LDS: while the matrix cores consume stage s from one buffer, the operands of stage s+1
-// are written to the other and the global loads of stage s+2 are issued; one barrier per stage.
+// (fetched during stage s-1) are written to the other and the global loads of stage s+2 are issued; one
+// barrier per stage.
 template <typename C_, int NI, int NJ, typename LA, typename LB>
 __device__ __forceinline__ void contract(LA& la, LB& lb, float* As, float* Bs, v16f (&acc)[NRB][NCB],
-                                         int nstage, int nkc, int arow, int bcol, int h) {
+                                         int nstage, int arow, int bcol, int h) {
   constexpr int AEL = TileShape<C_::A_KC, TM>::ELEMS, BEL = TileShape<C_::B_KC, TN>::ELEMS;
-  int kb = 0, kc = 0;
-  auto advance = [&]() { if (++kc == nkc) { kc = 0; ++kb; } };
-  la.load(0, 0);
-  lb.load(0, 0);
+  la.load();
+  lb.load();
   la.store(As);
   lb.store(Bs);
-  advance();
   if (nstage > 1) {
-    la.load(kb, kc * TK);
-    lb.load(kb, kc * TK);
+    la.load();
+    lb.load();
   }
   __syncthreads();
   for (int stage = 0; stage < nstage; ++stage) {
     const int cur = stage & 1;
     if (stage + 1 < nstage) {
-      la.store(As + (cur ^ 1) * AEL);
+      la.store(As + (cur ^ 1) * AEL);       // that buffer was last read in stage - 1, which every wave has left
       lb.store(Bs + (cur ^ 1) * BEL);
-      advance();
       if (stage + 2 < nstage) {
-        la.load(kb, kc * TK);
-        lb.load(kb, kc * TK);
+        la.load();
+        lb.load();
       }
     }
     if (NI > 0 && NJ > 0)
@@ -228,6 +237,7 @@ __host__ __device__ inline void tile_counts(int L, int RI, int CI, int& tm, int&
 template <int MODE, int VEC>
 __global__ __launch_bounds__(NT) void so3_block_mm_real_kernel(MmParams p) {
   typedef Cfg<MODE> C_;
+
   __shared__ __attribute__((aligned(16))) float As[2 * TileShape<C_::A_KC, TM>::ELEMS];
   __shared__ __attribute__((aligned(16))) float Bs[2 * TileShape<C_::B_KC, TN>::ELEMS];
 
@@ -269,9 +279,8 @@ __global__ __launch_bounds__(NT) void so3_block_mm_real_kernel(MmParams p) {
   nj = nj > NCB ? NCB : nj;
   if (ni == 0 || nj == 0) ni = nj = 0;
 
-  const int nkc = s2cnn::ceil_div(p.KI, TK);
-  const int nstage = L * nkc;
-#define S2CNN_CONTRACT(I, J) contract<C_, I, J>(la, lb, As, Bs, acc, nstage, nkc, wrow + r32, wcol + r32, h)
+  const int nstage = s2cnn::ceil_div(L * p.KI, TK);
+#define S2CNN_CONTRACT(I, J) contract<C_, I, J>(la, lb, As, Bs, acc, nstage, wrow + r32, wcol + r32, h)
   if (nj == NCB) {
     switch (ni) {
       case 4: if (NRB >= 4) { S2CNN_CONTRACT((NRB >= 4 ? 4 : 1), NCB); } break;
