@@ -23,10 +23,11 @@ if ROOT not in sys.path:
 
 PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X dense fp32 matrix
 PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
-# HBM-side bytes per launch of the three so3_mm kernels at this workload, from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE scaled by a 1 GiB copy (profiles/so3_mm_b32_B16_F64_hbm_traffic.md); not re-measured at run time.
-MM_TRAFFIC_BYTES = {"s2cnn_so3_mm_fwd": 13.08e9 + 0.358e9, "s2cnn_so3_mm_gradx": 13.19e9 + 0.358e9,
-                    "s2cnn_so3_mm_grady": 11.07e9 + 1.431e9}
+# HBM-side bytes per launch of the three product kernels at this workload, from rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE scaled by a 1 GiB elementwise kernel of the same run (profiles/so3_mm_real_b32_B16_F64_hbm_traffic.md);
+# not re-measured at run time.
+MM_TRAFFIC_BYTES = {"s2cnn_so3_mm_real_fwd": 6.37e9 + 0.179e9, "s2cnn_so3_mm_real_gradx": 6.42e9 + 0.179e9,
+                    "s2cnn_so3_mm_real_grady": 4.78e9 + 0.716e9}
 
 
 def nspec(b):
