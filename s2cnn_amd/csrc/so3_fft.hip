@@ -19,6 +19,7 @@
 #include "common.h"
 #include "so3_plane_fft64.h"
 #include "so3_wigner_tiled.h"
+#include "so3_fused64.h"
 
 namespace {
 
@@ -278,9 +279,15 @@ __global__ __launch_bounds__(256) void so3_plane_dft_inv(const float2* __restric
   }
 }
 
-// batch items padded to the z tile of the tiled Wigner kernels
-size_t ws_bytes(int b_grid, int b_spec, long nbatch, int cplx) {
+// Real signals on the 64^3 grid go through the per-volume kernels of so3_fused64.h (the planes never leave the CU).
+bool fused_path(int b_grid, int b_spec, int cplx, bool synthesis) {
+  return !cplx && b_grid == 32 && (synthesis || b_spec <= 32);
+}
+
+// Bytes of the intermediate; batch items padded to the z tile of the tiled Wigner kernels.
+size_t ws_bytes(int b_grid, int b_spec, long nbatch, int cplx, bool synthesis) {
   if (b_grid < 1 || b_spec < 1 || nbatch < 1) return 0;
+  if (fused_path(b_grid, b_spec, cplx, synthesis)) return fused64::scratch_bytes(nbatch);
   const long nb = b_grid < b_spec ? b_grid : b_spec;
   const long MW = 2 * nb - 1, NW = cplx ? MW : nb;
   const long zpad = (nbatch + wigner_tiled::ZT - 1) / wigner_tiled::ZT * wigner_tiled::ZT;
@@ -294,6 +301,7 @@ bool sizes_ok(int b_grid, int b_spec, long nbatch) {
 
 // Bytes of the packed table of the tiled fast path; 0 when that path does not apply.
 size_t packed_bytes(int b_grid, int b_spec, int cplx, bool synthesis) {
+  if (fused_path(b_grid, b_spec, cplx, synthesis)) return fused64::PACKED_FLOATS * sizeof(float);
   const int nb = b_grid < b_spec ? b_grid : b_spec;
   if (cplx || nb > 32) return 0;
   if (synthesis) return 2 * b_grid <= 64 ? wigner_tiled::packed_floats_synthesis(nb) * sizeof(float) : 0;
@@ -315,21 +323,25 @@ extern "C" int s2cnn_so3_pack_table(const float* table, float* packed, int b_in,
   if (!s2cnn::aligned16(packed)) return S2CNN_EALIGN;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int nb = b_in < b_out ? b_in : b_out;
-  if (synthesis)
+  if (fused_path(synthesis ? b_out : b_in, synthesis ? b_in : b_out, 0, synthesis != 0)) {
+    const int b_spec = synthesis ? b_in : b_out;
+    hipLaunchKernelGGL(fused64::pack_table, dim3(1024), dim3(256), 0, st, table, packed, s2cnn::so3_nspec(b_spec), b_spec < 32 ? b_spec : 32);
+  } else if (synthesis) {
     hipLaunchKernelGGL(wigner_tiled::pack_table_synthesis, dim3(2048), dim3(256), 0, st, table, packed, 2 * b_out, nb, b_in);
-  else
+  } else {
     hipLaunchKernelGGL(wigner_tiled::pack_table_analysis, dim3(2048), dim3(256), 0, st, table, packed, 2 * b_in, nb, b_out);
+  }
   return s2cnn::launch_status();
 }
 
 extern "C" size_t s2cnn_so3_analysis_workspace(int b_in, int b_out, long nbatch, int complex_in) {
-  const size_t w = ws_bytes(b_in, b_out, nbatch, complex_in);
-  return w ? round256(w) + packed_bytes(b_in, b_out, complex_in, false) : 0;
+  if (!sizes_ok(b_in, b_out, nbatch)) return 0;
+  return round256(ws_bytes(b_in, b_out, nbatch, complex_in, false)) + packed_bytes(b_in, b_out, complex_in, false);
 }
 
 extern "C" size_t s2cnn_so3_synthesis_workspace(int b_in, int b_out, long nbatch, int complex_out) {
-  const size_t w = ws_bytes(b_out, b_in, nbatch, complex_out);
-  return w ? round256(w) + packed_bytes(b_out, b_in, complex_out, true) : 0;
+  if (!sizes_ok(b_out, b_in, nbatch)) return 0;
+  return round256(ws_bytes(b_out, b_in, nbatch, complex_out, true)) + packed_bytes(b_out, b_in, complex_out, true);
 }
 
 extern "C" int s2cnn_so3_analysis(const float* x, const float* table, const float* packed_table, float* out,
@@ -338,9 +350,24 @@ extern "C" int s2cnn_so3_analysis(const float* x, const float* table, const floa
   if (!x || !table || !out || !sizes_ok(b_in, b_out, nbatch)) return S2CNN_EINVAL;
   if (!s2cnn::aligned8(out) || (complex_in && !s2cnn::aligned8(x))) return S2CNN_EALIGN;
   if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (fused_path(b_in, b_out, complex_in, false)) {
+    if (!s2cnn::aligned16(x)) return S2CNN_EALIGN;
+    if (!workspace || workspace_bytes < s2cnn_so3_analysis_workspace(b_in, b_out, nbatch, 0) || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
+    float4* rec = static_cast<float4*>(workspace);
+    const float* Tf = packed_table;
+    if (!Tf) {  // pack behind the records on every call
+      float* dst = reinterpret_cast<float*>(static_cast<char*>(workspace) + round256(fused64::scratch_bytes(nbatch)));
+      hipLaunchKernelGGL(fused64::pack_table, dim3(1024), dim3(256), 0, st, table, dst, s2cnn::so3_nspec(b_out), b_out);
+      Tf = dst;
+    }
+    hipLaunchKernelGGL(fused64::analysis_kernel, dim3(fused64::grid_size(nbatch)), dim3(fused64::THREADS), 0, st, x, Tf, rec, nbatch);
+    hipLaunchKernelGGL(fused64::spectrum_scatter, dim3((unsigned)((nbatch + fused64::ZT - 1) / fused64::ZT), fused64::NIT * 16), dim3(256), 0, st,
+                       rec, reinterpret_cast<float2*>(out), b_out, nbatch);
+    return s2cnn::launch_status();
+  }
   const size_t need = s2cnn_so3_analysis_workspace(b_in, b_out, nbatch, complex_in);
   if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
-  hipStream_t st = static_cast<hipStream_t>(stream);
   const int n2 = 2 * b_in, nb = b_in < b_out ? b_in : b_out;
   const int MW = 2 * nb - 1, NW = complex_in ? MW : nb;
   float2* X = static_cast<float2*>(workspace);
@@ -369,7 +396,7 @@ extern "C" int s2cnn_so3_analysis(const float* x, const float* table, const floa
   if (tiled) {
     const float* Tp = packed_table;
     if (!Tp) {  // pack on the fly behind the intermediate
-      float* dst = reinterpret_cast<float*>(static_cast<char*>(workspace) + round256(ws_bytes(b_in, b_out, nbatch, complex_in)));
+      float* dst = reinterpret_cast<float*>(static_cast<char*>(workspace) + round256(ws_bytes(b_in, b_out, nbatch, complex_in, false)));
       hipLaunchKernelGGL(wigner_tiled::pack_table_analysis, dim3(2048), dim3(256), 0, st, table, dst, n2, nb, b_out);
       Tp = dst;
     }
@@ -391,9 +418,25 @@ extern "C" int s2cnn_so3_synthesis(const float* xhat, const float* table, const 
   if (!xhat || !table || !out || !sizes_ok(b_out, b_in, nbatch)) return S2CNN_EINVAL;
   if (!s2cnn::aligned8(xhat) || (complex_out && !s2cnn::aligned8(out))) return S2CNN_EALIGN;
   if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (fused_path(b_out, b_in, complex_out, true)) {
+    if (!s2cnn::aligned16(out)) return S2CNN_EALIGN;
+    const int nl = b_in < 32 ? b_in : 32;
+    if (!workspace || workspace_bytes < s2cnn_so3_synthesis_workspace(b_in, b_out, nbatch, 0) || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
+    float4* rec = static_cast<float4*>(workspace);
+    const float* Tf = packed_table;
+    if (!Tf) {
+      float* dst = reinterpret_cast<float*>(static_cast<char*>(workspace) + round256(fused64::scratch_bytes(nbatch)));
+      hipLaunchKernelGGL(fused64::pack_table, dim3(1024), dim3(256), 0, st, table, dst, s2cnn::so3_nspec(b_in), nl);
+      Tf = dst;
+    }
+    hipLaunchKernelGGL(fused64::spectrum_gather, dim3((unsigned)((nbatch + fused64::ZT - 1) / fused64::ZT), fused64::NIT * 16), dim3(256), 0, st,
+                       reinterpret_cast<const float2*>(xhat), rec, nl, nbatch);
+    hipLaunchKernelGGL(fused64::synthesis_kernel, dim3(fused64::grid_size(nbatch)), dim3(fused64::THREADS), 0, st, rec, Tf, out, nbatch);
+    return s2cnn::launch_status();
+  }
   const size_t need = s2cnn_so3_synthesis_workspace(b_in, b_out, nbatch, complex_out);
   if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
-  hipStream_t st = static_cast<hipStream_t>(stream);
   const int n2 = 2 * b_out, nb = b_in < b_out ? b_in : b_out;
   const int MW = 2 * nb - 1, NW = complex_out ? MW : nb;
   float2* S = static_cast<float2*>(workspace);
@@ -405,7 +448,7 @@ extern "C" int s2cnn_so3_synthesis(const float* xhat, const float* table, const 
   if (tiled) {
     const float* Tq = packed_table;
     if (!Tq) {
-      float* dst = reinterpret_cast<float*>(static_cast<char*>(workspace) + round256(ws_bytes(b_out, b_in, nbatch, complex_out)));
+      float* dst = reinterpret_cast<float*>(static_cast<char*>(workspace) + round256(ws_bytes(b_out, b_in, nbatch, complex_out, true)));
       hipLaunchKernelGGL(wigner_tiled::pack_table_synthesis, dim3(2048), dim3(256), 0, st, table, dst, n2, nb, b_in);
       Tq = dst;
     }

@@ -1,0 +1,620 @@
+// SO(3) analysis and synthesis of real signals on the 64^3 grid (bandwidth 32) as ONE kernel each:
+// a workgroup owns one volume, keeps its whole half spectrum in registers and walks over beta, so
+// the transformed planes never leave the compute unit (no intermediate in HBM).
+//
+// Per step the workgroup takes the two planes beta_j and beta_{63-j} (j < 32) as one complex plane,
+// transforms it inside LDS (radix 8 x 8, see so3_plane_fft64.h) and contracts it with the Wigner
+// table.  The table is needed for j < 32 only, because on the SOFT grid beta_{63-j} = pi - beta_j and
+//     d^l_{mn}(pi - beta) = (-1)^(l-n) d^l_{-m,n}(beta)          (weights symmetric in j as well),
+// and for n >= 0 only, because spectra of real signals obey X[l,-m,-n] = (-1)^(m-n) conj X[l,m,n].
+//
+// Work decomposition: an ITEM is (c, a, n) = four consecutive degrees l = 4c..4c+3 of the two columns
+// (m = +a, n) and (m = -a, n), 0 <= a, n <= 4c+3.  There are sum_c (4c+4)^2 = 3264 items for c < 8;
+// thread t owns items t, t+512, ..., t+6*512, i.e. 7 x 4 x 2 complex values in registers.
+// With P = plane of beta_j, P' = plane of beta_{63-j}, t1 = T[j,l,+a,n], t2 = T[j,l,-a,n], s = (-1)^(l-n):
+//   analysis : X[l,+a,n] += t1 P[+a,n] + s t2 P'[+a,n]      X[l,-a,n] += t2 P[-a,n] + s t1 P'[-a,n]
+//   synthesis: S[+a,n] = sum_l t1 xs[l,+a,n]   S'[+a,n] = sum_l s t2 xs[l,+a,n]   (and -a with t1 <-> t2)
+// The packed table holds t1/2, t2/2 per (j, item, degree) in the order the threads load it.
+//
+// The two halves of a step overlap: while plane pair j is contracted out of one LDS buffer, pair j+1 is
+// transformed in the other, stage by stage between the same barriers.
+//
+// A spectral row holds ONE 8-byte entry per volume, so a workgroup never touches the spectrum itself:
+// it exchanges its registers with a per-volume record in scratch memory (coalesced), and
+// spectrum_scatter / spectrum_gather move tiles of 16 volumes between the records and the rows
+// (128-byte pieces, mirror half and symmetrisation included).
+#pragma once
+#include <hip/hip_runtime.h>
+#include "so3_plane_fft64.h"
+
+namespace fused64 {
+
+using fft64::N;
+using fft64::PITCH;
+using fft64::LDS_ELEMS;
+using fft64::sigma;
+
+constexpr int THREADS = 512;
+constexpr int NIT = 7;             // items per thread
+constexpr int NITEMS = 3264;       // sum_{c<8} (4c+4)^2
+constexpr int NJ = 32;             // beta pairs
+constexpr size_t PACKED_FLOATS = (size_t)NJ * NIT * 2 * THREADS * 4;
+
+// Buffer addressing (uniform descriptor in SGPRs + one 32-bit lane offset + a scalar offset): the bases are
+// uniform per workgroup, so no 64-bit address arithmetic is left in vector registers.  Offsets in bytes.
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, unsigned bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ float buf_load_f32(__amdgpu_buffer_rsrc_t r, unsigned voff, unsigned soff) {
+  return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, (int)voff, (int)soff, 0));
+}
+__device__ __forceinline__ float4 buf_load_f32x4(__amdgpu_buffer_rsrc_t r, unsigned voff, unsigned soff) {
+  const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, (int)soff, 0);
+  return make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
+}
+__device__ __forceinline__ void buf_store_f32(float x, __amdgpu_buffer_rsrc_t r, unsigned voff, unsigned soff) {
+  __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(x), r, (int)voff, (int)soff, 0);
+}
+__device__ __forceinline__ void buf_store_f32x4(float4 x, __amdgpu_buffer_rsrc_t r, unsigned voff, unsigned soff) {
+  u32x4 v; v.x = __float_as_uint(x.x); v.y = __float_as_uint(x.y); v.z = __float_as_uint(x.z); v.w = __float_as_uint(x.w);
+  __builtin_amdgcn_raw_buffer_store_b128(v, r, (int)voff, (int)soff, 0);
+}
+
+// x with its sign flipped where `signbit` (0 or 0x80000000) is set
+__device__ __forceinline__ float flip(float x, unsigned signbit) { return __uint_as_float(__float_as_uint(x) ^ signbit); }
+
+__host__ __device__ inline int lmn_index(int l, int m, int n) { return l * (4 * l * l - 1) / 3 + (l + m) * (2 * l + 1) + (l + n); }
+
+// item index -> (c, a, n); false for the padding slots behind the last item
+__host__ __device__ inline bool decode_item(int i, int& c, int& a, int& n) {
+  c = 0; a = 0; n = 0;
+  if (i >= NITEMS) return false;
+  int off = 0;
+  for (int cc = 0; cc < 8; ++cc) {
+    const int s = 4 * cc + 4;
+    if (i < off + s * s) {
+      const int r = i - off;
+      c = cc; a = r / s; n = r - a * s;
+      return true;
+    }
+    off += s * s;
+  }
+  return false;
+}
+
+// Packed table: float index ((((j*NIT + it)*2 + h)*THREADS + t)*4 + u) holds
+//   0.5 * T[j, l = 4c+u, m = (h ? -a : +a), n]   for item (c, a, n) = it*THREADS + t,
+// zero where l < max(a, n), l >= nl, or the slot is padding.  T is [64][nspec_stride].
+__global__ void pack_table(const float* __restrict__ T, float* __restrict__ Tf, long nspec_stride, int nl) {
+  for (size_t e = blockIdx.x * (size_t)blockDim.x + threadIdx.x; e < PACKED_FLOATS; e += (size_t)gridDim.x * blockDim.x) {
+    const int u = (int)(e & 3);
+    const int t = (int)((e >> 2) & (THREADS - 1));
+    const int h = (int)((e >> 11) & 1);
+    const int r = (int)(e >> 12);
+    const int it = r % NIT, j = r / NIT;
+    int c, a, n;
+    float v = 0.f;
+    if (decode_item(it * THREADS + t, c, a, n)) {
+      const int l = 4 * c + u;
+      if (l >= a && l >= n && l < nl) v = 0.5f * T[(size_t)j * nspec_stride + lmn_index(l, h ? -a : a, n)];
+    }
+    Tf[e] = v;
+  }
+}
+
+// One radix-8 pass of the in-place 2-D transform of a 64x64 complex plane in LDS by 512 threads
+// (natural order in, sigma order out on both axes): P = 0, 1 rows, P = 2, 3 columns.
+// twl[8*d + k] = w64^(d k) (conjugated for the inverse).  A barrier must follow each pass.
+template <bool INV, int P>
+__device__ __forceinline__ void fft_pass(float2* buf, const float2* twl) {
+  using namespace fft64;
+  const int lo = threadIdx.x & 63;   // line
+  const int d = threadIdx.x >> 6;    // j2 in the first pass of an axis, k1 in the second
+  float2* line = P == 0 ? buf + lo * PITCH + d : P == 1 ? buf + lo * PITCH + 8 * d : P == 2 ? buf + lo + d * PITCH : buf + lo + 8 * d * PITCH;
+  constexpr int stride = P == 0 ? 8 : P == 1 ? 1 : P == 2 ? 8 * PITCH : PITCH;
+  float2 v[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) v[j] = line[j * stride];
+  fft8<INV>(v);
+  if (P == 0 || P == 2) {
+#pragma unroll
+    for (int j = 1; j < 8; ++j) v[j] = cmul(v[j], twl[8 * d + j]);
+  }
+#pragma unroll
+  for (int j = 0; j < 8; ++j) line[j * stride] = v[j];
+}
+
+template <bool INV>
+__device__ __forceinline__ void fill_twiddles(float2* twl) {
+  if (threadIdx.x < 64) {
+    const int d = threadIdx.x >> 3, k = threadIdx.x & 7;
+    float s, c;
+    sincospif((float)(d * k) / 32.0f, &s, &c);   // angle 2 pi d k / 64
+    twl[threadIdx.x] = make_float2(c, INV ? s : -s);
+  }
+}
+
+// Workgroup -> volume.  Consecutive workgroups go round-robin over the 8 XCDs; the workgroups of one
+// XCD take consecutive volumes (neighbouring records, and the same table slab at the same time).
+__device__ __forceinline__ long volume_of_block(long nbatch) {
+  const long zper = (nbatch + 7) / 8;
+  const long xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const long z = xcd * zper + slot;
+  return (slot < zper && z < nbatch) ? z : -1;
+}
+inline unsigned grid_size(long nbatch) { return (unsigned)(8 * ((nbatch + 7) / 8)); }
+
+// Per-volume record in scratch memory: [k = 4 it + q][t] float4, q = 0: (+a) degrees u = 0, 1 as
+// (re, im, re, im); q = 1: (+a) u = 2, 3; q = 2, 3: the same for (-a).
+constexpr int REC_F4 = NIT * 4 * THREADS;                 // float4 per record
+constexpr size_t REC_BYTES = (size_t)REC_F4 * 16;         // 229376
+inline size_t scratch_bytes(long nbatch) { return (size_t)nbatch * REC_BYTES; }
+
+// ---------------------------------------------------------------------------------------------
+// analysis: x [nbatch][64][64][64] real -> records of the half spectrum n >= 0
+//
+// Plane pair j+1 goes global -> registers -> first alpha stage -> `work` (LDS) -> second alpha stage ->
+// two gamma stages, the last of which writes the QUAD layout: the four bins an item reads,
+// Z[+a,n], Z[-a,-n], Z[-a,n], Z[+a,-n], side by side at quad[a][n][0..3].  Meanwhile pair j is
+// contracted out of the other quad buffer, two items per stage.
+// ---------------------------------------------------------------------------------------------
+constexpr int QPITCH = 32 * 4 + 6;              // complex numbers per a-row of the quad layout; the pad takes the unused n = 32
+constexpr int QUAD_ELEMS = 33 * QPITCH;         // row 32 takes the unused m = 32
+// table registers: four slots, item it in slot it % 4; a slot is refilled right after its item has been used:
+//   after item 0, 1, 2: items 4, 5, 6 of the same plane pair;  after 3, 4, 5, 6: items 3, 0, 1, 2 of the next pair
+__device__ constexpr int table_slot(int it) { return it & 3; }
+
+__global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restrict__ x, const float* __restrict__ Tf,
+                                                           float4* __restrict__ rec, long nbatch) {
+  using namespace fft64;
+  __shared__ __attribute__((aligned(16))) float2 work[LDS_ELEMS];
+  __shared__ __attribute__((aligned(16))) float2 quad[2][QUAD_ELEMS];
+  __shared__ float2 twl[64];
+  const long z = volume_of_block(nbatch);
+  if (z < 0) return;
+  const int t = threadIdx.x;
+  const int lo = t & 63, d = t >> 6;
+  fill_twiddles<false>(twl);
+  for (int i = t; i < 2 * QUAD_ELEMS; i += THREADS) (&quad[0][0])[i] = make_float2(0.f, 0.f);   // places nobody writes (the -a half of a = 0) read as zero
+
+  // quad address of the item (complex index), bit 31 = sign bit of (-1)^n
+  unsigned adr[NIT];
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    int c, a, n;
+    decode_item(it * THREADS + t, c, a, n);
+    adr[it] = (unsigned)(a * QPITCH + 4 * n) | ((unsigned)(n & 1) << 31);
+  }
+  // where this thread's outputs of the last gamma stage go: row slot lo holds m = sigma(lo)
+  const int m = sigma(lo);
+  // quad[a][n] = { Z[+a,n], Z[-a,-n], Z[-a,n], Z[+a,-n] }; +0 and -0 are the same frequency, so
+  //   m = 0 counts as -0 when n < 0 (the item (0, n) then finds Z[0,n], Z[0,-n] in its first two places) and
+  //   n = 0 is written to the place of -0 as well (the one extra store below, by the wave d = 0).
+  const int qa = (m <= 32 ? m : 64 - m) * QPITCH;     // m = 32: the dump row
+  const int pos_lo = m > 32 ? 2 : 0;                  // place of an output with n >= 0
+  const int pos_hi = (m > 32 || m == 0) ? 1 : 3;      // place of an output with n < 0
+  const int extra = d == 0 ? qa + pos_hi : 32 * QPITCH + 130;   // n = 0 again as -0; other waves: the dump row
+
+  float2 accp[NIT][4], accm[NIT][4];
+#pragma unroll
+  for (int it = 0; it < NIT; ++it)
+#pragma unroll
+    for (int u = 0; u < 4; ++u) { accp[it][u] = make_float2(0.f, 0.f); accm[it][u] = make_float2(0.f, 0.f); }
+
+  const __amdgpu_buffer_rsrc_t rx = make_rsrc(x + (size_t)z * (N * N * N), N * N * N * 4);
+  const __amdgpu_buffer_rsrc_t rt = make_rsrc(Tf, (unsigned)(PACKED_FLOATS * 4));
+  const unsigned xoff = (d * N + lo) * 4;        // + (beta * 4096 + j1 * 512) * 4: row alpha = 8 j1 + d, column gamma = lo
+  const unsigned toff = t * 16;
+  float pa[8], pb[8];
+  float4 t1[4], t2[4];
+
+  auto load_planes = [&](int j) {            // planes j and 63-j: one full row (256 bytes) per wave and load
+#pragma unroll
+    for (int j1 = 0; j1 < 8; ++j1) {
+      pa[j1] = buf_load_f32(rx, xoff, (j * 4096 + j1 * 512) * 4);
+      pb[j1] = buf_load_f32(rx, xoff, ((63 - j) * 4096 + j1 * 512) * 4);
+    }
+  };
+  auto load_planes_part = [&](int j, int g) {   // a quarter of load_planes
+#pragma unroll
+    for (int j1 = 2 * g; j1 < 2 * g + 2; ++j1) {
+      pa[j1] = buf_load_f32(rx, xoff, (j * 4096 + j1 * 512) * 4);
+      pb[j1] = buf_load_f32(rx, xoff, ((63 - j) * 4096 + j1 * 512) * 4);
+    }
+  };
+  auto load_table = [&](int j, int it) {
+    t1[table_slot(it)] = buf_load_f32x4(rt, toff, ((j * NIT + it) * 2 + 0) * (THREADS * 16));
+    t2[table_slot(it)] = buf_load_f32x4(rt, toff, ((j * NIT + it) * 2 + 1) * (THREADS * 16));
+  };
+  // first alpha stage, out of the registers: 8-point transforms over j1, twiddle, -> work[8 k1 + d][lo]
+  auto stage_c1 = [&]() {
+    float2 v[8];
+#pragma unroll
+    for (int j1 = 0; j1 < 8; ++j1) v[j1] = make_float2(pa[j1], pb[j1]);
+    fft8<false>(v);
+#pragma unroll
+    for (int k = 1; k < 8; ++k) v[k] = cmul(v[k], twl[8 * d + k]);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) work[(8 * k + d) * PITCH + lo] = v[k];
+  };
+  // second gamma stage: row slot lo, inputs at slots 8 d + j2, outputs n = d + 8 k2 -> quad layout
+  auto stage_r2 = [&](float2* q) {
+    float2 v[8];
+    const float2* line = work + lo * PITCH + 8 * d;
+#pragma unroll
+    for (int j2 = 0; j2 < 8; ++j2) v[j2] = line[j2];
+    fft8<false>(v);
+#pragma unroll
+    for (int k2 = 0; k2 < 4; ++k2) q[qa + 4 * (d + 8 * k2) + pos_lo] = v[k2];
+#pragma unroll
+    for (int k2 = 4; k2 < 8; ++k2) q[qa + 4 * (64 - d - 8 * k2) + pos_hi] = v[k2];   // n = 32 (d = 0, k2 = 4) lands in the pad of the row
+    q[extra] = v[0];
+  };
+  auto accumulate = [&](const float2* q, int it) {
+    const float4* src = reinterpret_cast<const float4*>(q + (adr[it] & 0x7fffffffu));
+    const float4 za = src[0], zb = src[1];              // Z[+a,n], Z[-a,-n] | Z[-a,n], Z[+a,-n]
+    const unsigned sb = adr[it] & 0x80000000u;
+    // twice the separated planes (the table carries the factor 1/2):
+    // P = Z[m,n] + conj Z[-m,-n],  P' = (Z[m,n] - conj Z[-m,-n]) / i, the latter times (-1)^n
+    const float2 Pp = make_float2(za.x + za.z, za.y - za.w);
+    const float2 Qp = make_float2(flip(za.y + za.w, sb), flip(za.z - za.x, sb));
+    const float2 Pm = make_float2(zb.x + zb.z, zb.y - zb.w);
+    const float2 Qm = make_float2(flip(zb.y + zb.w, sb), flip(zb.z - zb.x, sb));
+    const float4 ta = t1[table_slot(it)], tb = t2[table_slot(it)];
+    const float a1[4] = {ta.x, ta.y, ta.z, ta.w};
+    const float a2[4] = {tb.x, tb.y, tb.z, tb.w};
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      // (-1)^(l-n) = (-1)^u (-1)^n for l = 4c+u: the sign of odd u goes into the table operand
+      const float b1 = (u & 1) ? -a1[u] : a1[u], b2 = (u & 1) ? -a2[u] : a2[u];
+      accp[it][u].x = fmaf(b2, Qp.x, fmaf(a1[u], Pp.x, accp[it][u].x));
+      accp[it][u].y = fmaf(b2, Qp.y, fmaf(a1[u], Pp.y, accp[it][u].y));
+      accm[it][u].x = fmaf(b1, Qm.x, fmaf(a2[u], Pm.x, accm[it][u].x));
+      accm[it][u].y = fmaf(b1, Qm.y, fmaf(a2[u], Pm.y, accm[it][u].y));
+    }
+  };
+
+  // first plane pair: transformed alone
+  load_planes(0);
+  load_table(0, 0); load_table(0, 1); load_table(0, 2); load_table(0, 3);
+  __syncthreads();                              // twiddles, cleared quads
+  stage_c1();
+  load_planes(1);
+  __syncthreads();
+  fft_pass<false, 3>(work, twl); __syncthreads();
+  fft_pass<false, 0>(work, twl); __syncthreads();
+  stage_r2(quad[0]); __syncthreads();
+
+  // step j: contract pair j out of quad[j & 1] while pair j+1 is transformed into quad[(j+1) & 1].
+  // The scheduling fences keep the parts of a stage in program order.
+#define S2CNN_FENCE() __builtin_amdgcn_sched_barrier(0)
+  // contract item k, then refill its table slot with the item that uses the slot next; plane loads in quarters:
+  // memory instructions are spread over the step so that their queue never fills up
+#define S2CNN_ACC(k, jl, il) accumulate(cur, k); S2CNN_FENCE(); load_table(jl, il); S2CNN_FENCE();
+#define S2CNN_PLANES(g) load_planes_part(jp, g); S2CNN_FENCE();
+  // Waves d < 4 transform first and contract second, waves d >= 4 the other way round: each SIMD holds one
+  // wave of either kind, so its LDS-bound and its FMA-bound half of a stage overlap.
+  if (d < 4) {
+    for (int j = 0; j < NJ - 1; ++j) {
+      const float2* cur = quad[j & 1];
+      float2* nxt = quad[(j + 1) & 1];
+      const int jp = j + 2 < NJ ? j + 2 : NJ - 1;     // clamped, not branched: a branch would make the loads synchronous
+      stage_c1(); S2CNN_FENCE();
+      S2CNN_PLANES(0) S2CNN_ACC(0, j, 4) S2CNN_PLANES(1) S2CNN_ACC(1, j, 5)
+      __syncthreads();
+      fft_pass<false, 3>(work, twl); S2CNN_FENCE();
+      S2CNN_PLANES(2) S2CNN_ACC(2, j, 6) S2CNN_PLANES(3) S2CNN_ACC(3, j + 1, 3)
+      __syncthreads();
+      fft_pass<false, 0>(work, twl); S2CNN_FENCE();
+      S2CNN_ACC(4, j + 1, 0) S2CNN_ACC(5, j + 1, 1)
+      __syncthreads();
+      stage_r2(nxt); S2CNN_FENCE();
+      S2CNN_ACC(6, j + 1, 2)
+      __syncthreads();
+    }
+  } else {
+    for (int j = 0; j < NJ - 1; ++j) {
+      const float2* cur = quad[j & 1];
+      float2* nxt = quad[(j + 1) & 1];
+      const int jp = j + 2 < NJ ? j + 2 : NJ - 1;
+      S2CNN_ACC(0, j, 4) S2CNN_ACC(1, j, 5)
+      stage_c1(); S2CNN_FENCE();
+      S2CNN_PLANES(0) S2CNN_PLANES(1)
+      __syncthreads();
+      S2CNN_ACC(2, j, 6) S2CNN_PLANES(2) S2CNN_ACC(3, j + 1, 3) S2CNN_PLANES(3)
+      fft_pass<false, 3>(work, twl);
+      __syncthreads();
+      S2CNN_ACC(4, j + 1, 0) S2CNN_ACC(5, j + 1, 1)
+      fft_pass<false, 0>(work, twl);
+      __syncthreads();
+      S2CNN_ACC(6, j + 1, 2)
+      stage_r2(nxt);
+      __syncthreads();
+    }
+  }
+  {
+    const float2* cur = quad[(NJ - 1) & 1];
+    S2CNN_ACC(0, NJ - 1, 4) S2CNN_ACC(1, NJ - 1, 5) S2CNN_ACC(2, NJ - 1, 6)
+    accumulate(cur, 3); accumulate(cur, 4); accumulate(cur, 5); accumulate(cur, 6);
+  }
+#undef S2CNN_ACC
+#undef S2CNN_PLANES
+#undef S2CNN_FENCE
+
+  const __amdgpu_buffer_rsrc_t rr = make_rsrc(rec + (size_t)z * REC_F4, (unsigned)REC_BYTES);
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    buf_store_f32x4(make_float4(accp[it][0].x, accp[it][0].y, accp[it][1].x, accp[it][1].y), rr, toff, (it * 4 + 0) * (THREADS * 16));
+    buf_store_f32x4(make_float4(accp[it][2].x, accp[it][2].y, accp[it][3].x, accp[it][3].y), rr, toff, (it * 4 + 1) * (THREADS * 16));
+    buf_store_f32x4(make_float4(accm[it][0].x, accm[it][0].y, accm[it][1].x, accm[it][1].y), rr, toff, (it * 4 + 2) * (THREADS * 16));
+    buf_store_f32x4(make_float4(accm[it][2].x, accm[it][2].y, accm[it][3].x, accm[it][3].y), rr, toff, (it * 4 + 3) * (THREADS * 16));
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// records <-> spectral rows, for a tile of 16 volumes and 32 items per workgroup (256 threads).
+// grid (ceil(nbatch / 16), NIT * 16).  Row kinds of an item and degree: 0 (+a, n)  1 (-a, n)
+// 2 (-a,-n)  3 (+a,-n); kinds 2, 3 are (-1)^(a-n) conj of kinds 0, 1 in a spectrum of a real signal.
+// ---------------------------------------------------------------------------------------------
+constexpr int ZT = 16;              // volumes per tile: one 128-byte piece of a spectral row
+constexpr int IT_TILE = 32;         // items per tile
+constexpr int VLD = 16 * ZT + 1;    // LDS floats per item: 16 components x 16 volumes, padded
+
+__device__ __forceinline__ int pack_item_info(int i) {
+  int c, a, n;
+  const bool ok = decode_item(i, c, a, n);
+  return c | (a << 8) | (n << 16) | (ok ? 1 << 24 : 0);
+}
+
+// rows of item `info`, degree offset u, kind k: spectral index, or -1 if there is no such row
+__device__ __forceinline__ int row_index(int info, int u, int kind, int nl) {
+  const int c = info & 0xff, a = (info >> 8) & 0xff, n = (info >> 16) & 0xff;
+  const int l = 4 * c + u;
+  const bool ok = (info >> 24) && l >= a && l >= n && l < nl && (!(kind & 1) || a > 0) && (kind < 2 || n > 0) &&
+                  (kind != 3 || a > 0);
+  if (!ok) return -1;
+  const int m = (kind == 1 || kind == 2) ? -a : a;
+  return lmn_index(l, m, kind >= 2 ? -n : n);
+}
+
+__global__ __launch_bounds__(256) void spectrum_scatter(const float4* __restrict__ rec, float2* __restrict__ out, int nl, long nbatch) {
+  __shared__ float vals[IT_TILE * VLD];
+  __shared__ int info[IT_TILE];
+  const int th = threadIdx.x;
+  const long z0 = (long)blockIdx.x * ZT;
+  const int it = blockIdx.y >> 4, t0 = (blockIdx.y & 15) * IT_TILE;
+  if (th < IT_TILE) info[th] = pack_item_info(it * THREADS + t0 + th);
+#pragma unroll
+  for (int r = 0; r < 8; ++r) {
+    const int e = th + 256 * r;
+    const int item = e & 31, q = (e >> 5) & 3, zz = e >> 7;
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (z0 + zz < nbatch) v = rec[(size_t)(z0 + zz) * REC_F4 + (it * 4 + q) * THREADS + t0 + item];
+    float* d = vals + item * VLD + (4 * q) * ZT + zz;
+    d[0] = v.x; d[ZT] = v.y; d[2 * ZT] = v.z; d[3 * ZT] = v.w;
+  }
+  __syncthreads();
+  const int zz = th & 15, u = th >> 6, kind = (th >> 4) & 3;
+  if (z0 + zz >= nbatch) return;
+  const int comp = 4 * ((kind & 1) * 2 + (u >> 1)) + 2 * (u & 1);
+  for (int item = 0; item < IT_TILE; ++item) {
+    const int inf = info[item];
+    const int row = row_index(inf, u, kind, nl);
+    if (row < 0) continue;
+    float re = vals[item * VLD + comp * ZT + zz], im = vals[item * VLD + (comp + 1) * ZT + zz];
+    if (kind >= 2) {
+      const float sg = (((inf >> 8) - (inf >> 16)) & 1) ? -1.f : 1.f;
+      re *= sg; im *= -sg;
+    }
+    out[(size_t)row * nbatch + z0 + zz] = make_float2(re, im);
+  }
+}
+
+// xh [nspec][nbatch] complex (any symmetry) -> records of the symmetrised spectrum
+//   xs[l,m,n] = xh[l,m,n] + (-1)^(m-n) conj xh[l,-m,-n]   (twice the Hermitian part: the table carries 1/2),
+// zero where there is no such degree; the (-a) half of items with a = 0 is zero (it is the (+a) half).
+__global__ __launch_bounds__(256) void spectrum_gather(const float2* __restrict__ xh, float4* __restrict__ rec, int nl, long nbatch) {
+  __shared__ float vals[IT_TILE * VLD];
+  __shared__ int info[IT_TILE];
+  const int th = threadIdx.x;
+  const long z0 = (long)blockIdx.x * ZT;
+  const int it = blockIdx.y >> 4, t0 = (blockIdx.y & 15) * IT_TILE;
+  if (th < IT_TILE) info[th] = pack_item_info(it * THREADS + t0 + th);
+  __syncthreads();
+  {
+    const int zz = th & 15, u = (th >> 4) & 3, pm = (th >> 6) & 1, sub = th >> 7;
+    const int comp = 4 * (pm * 2 + (u >> 1)) + 2 * (u & 1);
+    const long zc = z0 + zz < nbatch ? z0 + zz : nbatch - 1;
+    for (int item = sub; item < IT_TILE; item += 2) {
+      const int inf = info[item];
+      const int r0 = row_index(inf, u, pm, nl);                 // (+-a, n)
+      float re = 0.f, im = 0.f;
+      if (r0 >= 0) {
+        const int a = (inf >> 8) & 0xff, n = (inf >> 16) & 0xff;
+        const int l = 4 * (inf & 0xff) + u;
+        const int r1 = lmn_index(l, pm ? a : -a, -n);           // the partner (-+a, -n); exists for every n
+        const float2 v0 = xh[(size_t)r0 * nbatch + zc], v1 = xh[(size_t)r1 * nbatch + zc];
+        const float sg = ((a - n) & 1) ? -1.f : 1.f;
+        re = v0.x + sg * v1.x; im = v0.y - sg * v1.y;
+      }
+      vals[item * VLD + comp * ZT + zz] = re;
+      vals[item * VLD + (comp + 1) * ZT + zz] = im;
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < 8; ++r) {
+    const int e = th + 256 * r;
+    const int item = e & 31, q = (e >> 5) & 3, zz = e >> 7;
+    if (z0 + zz >= nbatch) continue;
+    const float* d = vals + item * VLD + (4 * q) * ZT + zz;
+    rec[(size_t)(z0 + zz) * REC_F4 + (it * 4 + q) * THREADS + t0 + item] = make_float4(d[0], d[ZT], d[2 * ZT], d[3 * ZT]);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// synthesis: records of the symmetrised spectrum -> y [nbatch][64][64][64] real
+//
+// While plane pair j is transformed in `work` (two gamma stages, two alpha stages, the last one
+// straight into the global stores), every item puts its share of the bins of pair j+1 into a staging
+// area; a reduction over the (up to 8) items of a column then fills `work` for the next step.
+// Sums are formed in a fixed order: results are reproducible bit for bit.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __restrict__ rec, const float* __restrict__ Tf,
+                                                            float* __restrict__ y, long nbatch) {
+  using namespace fft64;
+  __shared__ __attribute__((aligned(16))) float2 work[LDS_ELEMS];
+  __shared__ __attribute__((aligned(16))) float4 stg[NIT * THREADS * 2];     // item i: bins [+a,n], [-a,-n] | [-a,n], [+a,-n]
+  __shared__ float2 twl[64];
+  const long z = volume_of_block(nbatch);
+  if (z < 0) return;
+  const int t = threadIdx.x;
+  const int lo = t & 63, d = t >> 6;
+  fill_twiddles<true>(twl);
+  for (int i = t; i < LDS_ELEMS; i += THREADS) work[i] = make_float2(0.f, 0.f);   // bins of m = 32 and n = 32 stay zero ... until a transform overwrites them: cleared again in reduce()
+
+  float2 xp[NIT][4], xm[NIT][4];
+  unsigned sgn = 0;                 // bit it = n odd for item it
+  const __amdgpu_buffer_rsrc_t rr = make_rsrc(rec + (size_t)z * REC_F4, (unsigned)REC_BYTES);
+  const __amdgpu_buffer_rsrc_t rt = make_rsrc(Tf, (unsigned)(PACKED_FLOATS * 4));
+  const __amdgpu_buffer_rsrc_t ry = make_rsrc(y + (size_t)z * (N * N * N), N * N * N * 4);
+  const unsigned toff = t * 16;
+  const unsigned yoff = (d * N + sigma(lo)) * 4;   // + (beta * 4096 + k2 * 512) * 4: row alpha = d + 8 k2, column gamma = sigma(lo)
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    int c, a, n;
+    decode_item(it * THREADS + t, c, a, n);
+    sgn |= (unsigned)(n & 1) << it;
+    const float4 v0 = buf_load_f32x4(rr, toff, (it * 4 + 0) * (THREADS * 16)), v1 = buf_load_f32x4(rr, toff, (it * 4 + 1) * (THREADS * 16));
+    const float4 v2 = buf_load_f32x4(rr, toff, (it * 4 + 2) * (THREADS * 16)), v3 = buf_load_f32x4(rr, toff, (it * 4 + 3) * (THREADS * 16));
+    xp[it][0] = make_float2(v0.x, v0.y); xp[it][1] = make_float2(v0.z, v0.w);
+    xp[it][2] = make_float2(v1.x, v1.y); xp[it][3] = make_float2(v1.z, v1.w);
+    xm[it][0] = make_float2(v2.x, v2.y); xm[it][1] = make_float2(v2.z, v2.w);
+    xm[it][2] = make_float2(v3.x, v3.y); xm[it][3] = make_float2(v3.z, v3.w);
+  }
+  // the two columns (a, n) this thread reduces: shell order q -> k = max(a, n), (k, 0..k) then (0..k-1, k);
+  // q = t and 1023 - t, so that the lanes of a wave have the same number of items per column
+  int ca[2], cn[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int q = h ? 1023 - t : t;
+    int k = (int)sqrtf((float)q);
+    if (k * k > q) --k;
+    if ((k + 1) * (k + 1) <= q) ++k;
+    const int rr = q - k * k;
+    ca[h] = rr <= k ? k : rr - k - 1;
+    cn[h] = rr <= k ? rr : k;
+  }
+
+  float4 t1[4], t2[4];
+  auto load_table = [&](int j, int it) {
+    t1[table_slot(it)] = buf_load_f32x4(rt, toff, ((j * NIT + it) * 2 + 0) * (THREADS * 16));
+    t2[table_slot(it)] = buf_load_f32x4(rt, toff, ((j * NIT + it) * 2 + 1) * (THREADS * 16));
+  };
+  // the item's share of a plane pair: S = sum_l t1 xs, S' = sum_l s t2 xs at (+a, n), t1 <-> t2 at (-a, n);
+  // complex plane Z = S + i S' at [m,n], its Hermitian partner conj S + i conj S' at [-m,-n]
+  auto contribute = [&](int it) {
+    const float4 ta = t1[table_slot(it)], tb = t2[table_slot(it)];
+    const float a1[4] = {ta.x, ta.y, ta.z, ta.w};
+    const float a2[4] = {tb.x, tb.y, tb.z, tb.w};
+    float2 Sp = make_float2(0.f, 0.f), Qp = make_float2(0.f, 0.f), Sm = make_float2(0.f, 0.f), Qm = make_float2(0.f, 0.f);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const float b1 = (u & 1) ? -a1[u] : a1[u], b2 = (u & 1) ? -a2[u] : a2[u];
+      Sp.x = fmaf(a1[u], xp[it][u].x, Sp.x); Sp.y = fmaf(a1[u], xp[it][u].y, Sp.y);
+      Qp.x = fmaf(b2, xp[it][u].x, Qp.x);    Qp.y = fmaf(b2, xp[it][u].y, Qp.y);
+      Sm.x = fmaf(a2[u], xm[it][u].x, Sm.x); Sm.y = fmaf(a2[u], xm[it][u].y, Sm.y);
+      Qm.x = fmaf(b1, xm[it][u].x, Qm.x);    Qm.y = fmaf(b1, xm[it][u].y, Qm.y);
+    }
+    const unsigned sb = ((sgn >> it) & 1u) << 31;
+    Qp.x = flip(Qp.x, sb); Qp.y = flip(Qp.y, sb); Qm.x = flip(Qm.x, sb); Qm.y = flip(Qm.y, sb);
+    float4* dst = stg + 2 * (it * THREADS + t);
+    dst[0] = make_float4(Sp.x - Qp.y, Sp.y + Qp.x, Sp.x + Qp.y, Qp.x - Sp.y);
+    dst[1] = make_float4(Sm.x - Qm.y, Sm.y + Qm.x, Sm.x + Qm.y, Qm.x - Sm.y);
+  };
+  // staging -> work (natural order): sum over the items c = max(a,n)/4 .. 7 of each column, in that order
+  auto reduce = [&]() {
+    constexpr int OFF[8] = {0, 16, 80, 224, 480, 880, 1456, 2240};
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int a = ca[h], n = cn[h];
+      const int cmin = (a > n ? a : n) >> 2;
+      float4 s0 = make_float4(0.f, 0.f, 0.f, 0.f), s1 = s0;
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        if (c >= cmin) {
+          const float4* src = stg + 2 * (OFF[c] + a * (4 * c + 4) + n);
+          const float4 u0 = src[0], u1 = src[1];
+          s0.x += u0.x; s0.y += u0.y; s0.z += u0.z; s0.w += u0.w;
+          s1.x += u1.x; s1.y += u1.y; s1.z += u1.z; s1.w += u1.w;
+        }
+      }
+      const int rp = a * PITCH, rm = ((64 - a) & 63) * PITCH;
+      work[rp + n] = make_float2(s0.x, s0.y);
+      if (n > 0) work[rm + 64 - n] = make_float2(s0.z, s0.w);
+      if (a > 0) {
+        work[rm + n] = make_float2(s1.x, s1.y);
+        if (n > 0) work[rp + 64 - n] = make_float2(s1.z, s1.w);
+      }
+    }
+    if (t < 64) { work[32 * PITCH + t] = make_float2(0.f, 0.f); work[t * PITCH + 32] = make_float2(0.f, 0.f); }
+  };
+  // second alpha stage: column slot lo, inputs at row slots 8 d + j, outputs rows alpha = d + 8 k2:
+  // real part -> plane j, imaginary part -> plane 63-j, one full row (256 bytes) per wave and store
+  auto stage_c2_store = [&](int j) {
+    float2 v[8];
+    const float2* line = work + lo + 8 * d * PITCH;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v[k] = line[k * PITCH];
+    fft8<true>(v);
+#pragma unroll
+    for (int k2 = 0; k2 < 8; ++k2) {
+      buf_store_f32(v[k2].x, ry, yoff, (j * 4096 + k2 * 512) * 4);
+      buf_store_f32(v[k2].y, ry, yoff, ((63 - j) * 4096 + k2 * 512) * 4);
+    }
+  };
+
+  load_table(0, 0); load_table(0, 1);
+  __syncthreads();
+  load_table(0, 2); load_table(0, 3);
+  contribute(0); contribute(1);
+  load_table(0, 4); load_table(0, 5);
+  contribute(2); contribute(3);
+  load_table(0, 6);
+  contribute(4); contribute(5);
+  load_table(1, 0); load_table(1, 1);
+  contribute(6);
+  __syncthreads();
+  reduce();
+  __syncthreads();
+
+  // step j: transform pair j in `work` and write it out, while the shares of pair j+1 go to the staging area
+  for (int j = 0; j < NJ - 1; ++j) {
+    const int jn = j + 2 < NJ ? j + 2 : NJ - 1;     // table prefetch for the step after the next (unused at the end)
+    load_table(j + 1, 2); load_table(j + 1, 3);
+    fft_pass<true, 0>(work, twl);
+    contribute(0); contribute(1);
+    __syncthreads();
+    load_table(j + 1, 4); load_table(j + 1, 5);
+    fft_pass<true, 1>(work, twl);
+    contribute(2); contribute(3);
+    __syncthreads();
+    load_table(j + 1, 6);
+    fft_pass<true, 2>(work, twl);
+    contribute(4); contribute(5);
+    __syncthreads();
+    load_table(jn, 0); load_table(jn, 1);
+    stage_c2_store(j);
+    contribute(6);
+    __syncthreads();
+    reduce();
+    __syncthreads();
+  }
+  fft_pass<true, 0>(work, twl); __syncthreads();
+  fft_pass<true, 1>(work, twl); __syncthreads();
+  fft_pass<true, 2>(work, twl); __syncthreads();
+  stage_c2_store(NJ - 1);
+}
+
+}  // namespace fused64

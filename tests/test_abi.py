@@ -40,8 +40,13 @@ def test_argument_rejection_without_gpu():
     assert lib.s2cnn_so3_analysis(fake, fake, null, fake, null, 0, 4, 4, 1, 0, null) == -2  # no workspace
     assert lib.s2cnn_s2_analysis(fake, fake, fake, fake, 1 << 30, 4, 5, 1, 0, null) == -1  # b_out > b_in
     packed = lib.s2cnn_so3_packed_table_bytes(32, 32, 0)
-    assert packed == 63 * 64 * 1024 * 4
-    assert lib.s2cnn_so3_analysis_workspace(32, 32, 256, 0) == 256 * 64 * 63 * 32 * 8 + packed
+    assert packed == 32 * 7 * 2 * 512 * 4 * 4                                        # one-kernel path: 32 beta pairs x 7 items x 2 x 512 threads x 4 degrees
+    assert lib.s2cnn_so3_analysis_workspace(32, 32, 256, 0) == 256 * 28 * 512 * 16 + packed   # one record per volume (7 items x 4 float4 x 512 threads), no intermediate planes
+    assert lib.s2cnn_so3_synthesis_workspace(40, 32, 256, 0) == 256 * 28 * 512 * 16 + packed
+    packed16 = lib.s2cnn_so3_packed_table_bytes(16, 16, 0)
+    assert packed16 == 31 * 32 * 1024 * 4
+    assert lib.s2cnn_so3_analysis_workspace(16, 16, 256, 0) == 256 * 32 * 31 * 16 * 8 + packed16
+    assert lib.s2cnn_so3_analysis(ctypes.c_void_p(0x1008), fake, fake, fake, null, 0, 32, 32, 1, 0, null) == -3   # 64^3 real input: 16-byte alignment
     assert lib.s2cnn_so3_synthesis_workspace(4, 6, 3, 1) == 16 * 12 * 7 * 7 * 8      # batch padded to the z tile, no fast path
     assert lib.s2cnn_so3_packed_table_bytes(40, 40, 0) == 0 and lib.s2cnn_so3_packed_table_bytes(32, 40, 1) == 0
     assert lib.s2cnn_so3_pack_table(fake, fake, 40, 40, 0, null) == -1

@@ -103,6 +103,20 @@ def test_so3_transform_batch_dims_and_ragged(hip):
     close(PSO3.so3_rfft(x0.cuda()), O.so3_rfft(x0.double()), "b=1")
 
 
+@pytest.mark.parametrize("nz", [1, 9, 20])
+def test_so3_one_kernel_path_batches(hip, nz):
+    """Real signals on the 64^3 grid take the one-kernel path (one workgroup per volume): batch sizes that
+    leave XCD slots empty, truncated and over-long spectra, weighted and unweighted tables."""
+    print(f"so3 one-kernel path nz={nz}", flush=True)
+    x = rnd((nz, 64, 64, 64), 50 + nz)
+    for for_grad in (False, True):
+        for b_out in (32, 20, 1):
+            close(PSO3.so3_rfft(x.cuda(), for_grad, b_out), O.so3_rfft(x.double(), for_grad, b_out), f"rfft 32->{b_out} for_grad={for_grad}")
+        for b_spec in (32, 20, 36, 1):
+            s = rnd((O.nspec_so3(b_spec), nz, 2), 60 + b_spec)
+            close(PSO3.so3_rifft(s.cuda(), for_grad, 32), O.so3_rifft(s.double(), for_grad, 32), f"rifft {b_spec}->32 for_grad={for_grad}")
+
+
 def test_so3_transforms_without_prepacked_table(hip):
     """packed_table = NULL (the library repacks into its workspace) gives the same bits as the prepacked path."""
     from s2cnn_amd import _hip
@@ -123,7 +137,8 @@ def test_so3_transforms_without_prepacked_table(hip):
         ws = _hip.workspace(hip.s2cnn_so3_synthesis_workspace(b_out, b_in, nz, 0), x.device)
         _hip.check(hip.s2cnn_so3_synthesis(_hip.ptr(s), _hip.ptr(table), None, _hip.ptr(out), _hip.ptr(ws), ws.numel(),
                                            b_out, b_in, nz, 0, _hip.stream_ptr()))
-        assert torch.equal(out, want)
+        # the one-kernel synthesis sums its plane bins with LDS atomics: equal up to the order of additions
+        assert (out - want).abs().max().item() <= 1e-5 * want.abs().max().item()
 
 
 def test_so3_reference_identities_on_gpu(hip):
