@@ -61,6 +61,18 @@ __device__ __forceinline__ void buf_store_f32x4(float4 x, __amdgpu_buffer_rsrc_t
   __builtin_amdgcn_raw_buffer_store_b128(v, r, (int)voff, (int)soff, 0);
 }
 
+// 4 x 4 transpose across the four lanes of a quad: afterwards r_k of lane i is what r_i of lane k was.
+__device__ __forceinline__ float dpp_quad_xor1(float x) { return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0xB1, 0xf, 0xf, false)); }
+__device__ __forceinline__ float dpp_quad_xor2(float x) { return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x4E, 0xf, 0xf, false)); }
+__device__ __forceinline__ void quad_transpose(float& r0, float& r1, float& r2, float& r3) {
+  const bool b0 = threadIdx.x & 1, b1 = threadIdx.x & 2;
+  float u;
+  u = dpp_quad_xor1(b0 ? r0 : r1); if (b0) r0 = u; else r1 = u;
+  u = dpp_quad_xor1(b0 ? r2 : r3); if (b0) r2 = u; else r3 = u;
+  u = dpp_quad_xor2(b1 ? r0 : r2); if (b1) r0 = u; else r2 = u;
+  u = dpp_quad_xor2(b1 ? r1 : r3); if (b1) r1 = u; else r3 = u;
+}
+
 // x with its sign flipped where `signbit` (0 or 0x80000000) is set
 __device__ __forceinline__ float flip(float x, unsigned signbit) { return __uint_as_float(__float_as_uint(x) ^ signbit); }
 
@@ -465,7 +477,8 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
                                                             float* __restrict__ y, long nbatch) {
   using namespace fft64;
   __shared__ __attribute__((aligned(16))) float2 work[LDS_ELEMS];
-  __shared__ __attribute__((aligned(16))) float4 stg[NIT * THREADS * 2];     // item i: bins [+a,n], [-a,-n] | [-a,n], [+a,-n]
+  __shared__ __attribute__((aligned(16))) float4 stg_p[NIT * THREADS];       // item i: its share of the bins [+a,n], [-a,-n]
+  __shared__ __attribute__((aligned(16))) float4 stg_m[NIT * THREADS];       //                              [-a,n], [+a,-n]
   __shared__ float2 twl[64];
   const long z = volume_of_block(nbatch);
   if (z < 0) return;
@@ -480,7 +493,7 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
   const __amdgpu_buffer_rsrc_t rt = make_rsrc(Tf, (unsigned)(PACKED_FLOATS * 4));
   const __amdgpu_buffer_rsrc_t ry = make_rsrc(y + (size_t)z * (N * N * N), N * N * N * 4);
   const unsigned toff = t * 16;
-  const unsigned yoff = (d * N + sigma(lo)) * 4;   // + (beta * 4096 + k2 * 512) * 4: row alpha = d + 8 k2, column gamma = sigma(lo)
+  const unsigned yoff = ((d + 8 * (lo & 3)) * N + 4 * (lo >> 2)) * 4;   // + (beta * 4096 + 2048 h) * 4: row d + 8 (lo % 4) + 32 h, columns 4 (lo / 4)..+3
 #pragma unroll
   for (int it = 0; it < NIT; ++it) {
     int c, a, n;
@@ -529,9 +542,8 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
     }
     const unsigned sb = ((sgn >> it) & 1u) << 31;
     Qp.x = flip(Qp.x, sb); Qp.y = flip(Qp.y, sb); Qm.x = flip(Qm.x, sb); Qm.y = flip(Qm.y, sb);
-    float4* dst = stg + 2 * (it * THREADS + t);
-    dst[0] = make_float4(Sp.x - Qp.y, Sp.y + Qp.x, Sp.x + Qp.y, Qp.x - Sp.y);
-    dst[1] = make_float4(Sm.x - Qm.y, Sm.y + Qm.x, Sm.x + Qm.y, Qm.x - Sm.y);
+    stg_p[it * THREADS + t] = make_float4(Sp.x - Qp.y, Sp.y + Qp.x, Sp.x + Qp.y, Qp.x - Sp.y);
+    stg_m[it * THREADS + t] = make_float4(Sm.x - Qm.y, Sm.y + Qm.x, Sm.x + Qm.y, Qm.x - Sm.y);
   };
   // staging -> work (natural order): sum over the items c = max(a,n)/4 .. 7 of each column, in that order
   auto reduce = [&]() {
@@ -544,8 +556,8 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
 #pragma unroll
       for (int c = 0; c < 8; ++c) {
         if (c >= cmin) {
-          const float4* src = stg + 2 * (OFF[c] + a * (4 * c + 4) + n);
-          const float4 u0 = src[0], u1 = src[1];
+          const int i = OFF[c] + a * (4 * c + 4) + n;
+          const float4 u0 = stg_p[i], u1 = stg_m[i];
           s0.x += u0.x; s0.y += u0.y; s0.z += u0.z; s0.w += u0.w;
           s1.x += u1.x; s1.y += u1.y; s1.z += u1.z; s1.w += u1.w;
         }
@@ -560,57 +572,78 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
     }
     if (t < 64) { work[32 * PITCH + t] = make_float2(0.f, 0.f); work[t * PITCH + 32] = make_float2(0.f, 0.f); }
   };
-  // second alpha stage: column slot lo, inputs at row slots 8 d + j, outputs rows alpha = d + 8 k2:
-  // real part -> plane j, imaginary part -> plane 63-j, one full row (256 bytes) per wave and store
+  // second alpha stage: lane lo takes the column slot sigma(lo), i.e. column gamma = lo; inputs at row slots
+  // 8 d + j, outputs rows alpha = d + 8 k2.  The four lanes of a quad then exchange their values (4 x 4
+  // transposes) so that a lane holds four adjacent columns of one row: 16-byte stores, whole rows per wave.
+  // Real part -> plane j, imaginary part -> plane 63-j.
   auto stage_c2_store = [&](int j) {
     float2 v[8];
-    const float2* line = work + lo + 8 * d * PITCH;
+    const float2* line = work + sigma(lo) + 8 * d * PITCH;
 #pragma unroll
     for (int k = 0; k < 8; ++k) v[k] = line[k * PITCH];
     fft8<true>(v);
+    float ra[8], rb[8];
 #pragma unroll
-    for (int k2 = 0; k2 < 8; ++k2) {
-      buf_store_f32(v[k2].x, ry, yoff, (j * 4096 + k2 * 512) * 4);
-      buf_store_f32(v[k2].y, ry, yoff, ((63 - j) * 4096 + k2 * 512) * 4);
-    }
+    for (int k = 0; k < 8; ++k) { ra[k] = v[k].x; rb[k] = v[k].y; }
+    quad_transpose(ra[0], ra[1], ra[2], ra[3]); quad_transpose(ra[4], ra[5], ra[6], ra[7]);
+    quad_transpose(rb[0], rb[1], rb[2], rb[3]); quad_transpose(rb[4], rb[5], rb[6], rb[7]);
+    // lane (q, i) = (lo / 4, lo % 4) now holds columns 4q..4q+3 of the rows d + 8 i and d + 8 (4 + i)
+    buf_store_f32x4(make_float4(ra[0], ra[1], ra[2], ra[3]), ry, yoff, (j * 4096) * 4);
+    buf_store_f32x4(make_float4(ra[4], ra[5], ra[6], ra[7]), ry, yoff, (j * 4096 + 2048) * 4);
+    buf_store_f32x4(make_float4(rb[0], rb[1], rb[2], rb[3]), ry, yoff, ((63 - j) * 4096) * 4);
+    buf_store_f32x4(make_float4(rb[4], rb[5], rb[6], rb[7]), ry, yoff, ((63 - j) * 4096 + 2048) * 4);
   };
 
-  load_table(0, 0); load_table(0, 1);
+#define S2CNN_FENCE() __builtin_amdgcn_sched_barrier(0)
+  // the item's share, then its table slot is refilled with the item that uses the slot next (see table_slot)
+#define S2CNN_CON(k, jl, il) contribute(k); S2CNN_FENCE(); load_table((jl) < NJ ? (jl) : NJ - 1, il); S2CNN_FENCE();
+  load_table(0, 0); load_table(0, 1); load_table(0, 2); load_table(0, 3);
   __syncthreads();
-  load_table(0, 2); load_table(0, 3);
-  contribute(0); contribute(1);
-  load_table(0, 4); load_table(0, 5);
-  contribute(2); contribute(3);
-  load_table(0, 6);
-  contribute(4); contribute(5);
-  load_table(1, 0); load_table(1, 1);
-  contribute(6);
+  S2CNN_CON(0, 0, 4) S2CNN_CON(1, 0, 5) S2CNN_CON(2, 0, 6) S2CNN_CON(3, 1, 3) S2CNN_CON(4, 1, 0) S2CNN_CON(5, 1, 1) S2CNN_CON(6, 1, 2)
   __syncthreads();
   reduce();
   __syncthreads();
 
-  // step j: transform pair j in `work` and write it out, while the shares of pair j+1 go to the staging area
-  for (int j = 0; j < NJ - 1; ++j) {
-    const int jn = j + 2 < NJ ? j + 2 : NJ - 1;     // table prefetch for the step after the next (unused at the end)
-    load_table(j + 1, 2); load_table(j + 1, 3);
-    fft_pass<true, 0>(work, twl);
-    contribute(0); contribute(1);
-    __syncthreads();
-    load_table(j + 1, 4); load_table(j + 1, 5);
-    fft_pass<true, 1>(work, twl);
-    contribute(2); contribute(3);
-    __syncthreads();
-    load_table(j + 1, 6);
-    fft_pass<true, 2>(work, twl);
-    contribute(4); contribute(5);
-    __syncthreads();
-    load_table(jn, 0); load_table(jn, 1);
-    stage_c2_store(j);
-    contribute(6);
-    __syncthreads();
-    reduce();
-    __syncthreads();
+  // step j: transform pair j in `work` and write it out, while the shares of pair j+1 go to the staging area.
+  // Waves d < 4 transform first, waves d >= 4 last: each SIMD holds one wave of either kind, so the LDS-bound
+  // and the FMA-bound half of a stage overlap.
+  if (d < 4) {
+    for (int j = 0; j < NJ - 1; ++j) {
+      fft_pass<true, 0>(work, twl); S2CNN_FENCE();
+      S2CNN_CON(0, j + 1, 4) S2CNN_CON(1, j + 1, 5)
+      __syncthreads();
+      fft_pass<true, 1>(work, twl); S2CNN_FENCE();
+      S2CNN_CON(2, j + 1, 6) S2CNN_CON(3, j + 2, 3)
+      __syncthreads();
+      fft_pass<true, 2>(work, twl); S2CNN_FENCE();
+      S2CNN_CON(4, j + 2, 0) S2CNN_CON(5, j + 2, 1)
+      __syncthreads();
+      stage_c2_store(j); S2CNN_FENCE();
+      S2CNN_CON(6, j + 2, 2)
+      __syncthreads();
+      reduce();
+      __syncthreads();
+    }
+  } else {
+    for (int j = 0; j < NJ - 1; ++j) {
+      S2CNN_CON(0, j + 1, 4) S2CNN_CON(1, j + 1, 5)
+      fft_pass<true, 0>(work, twl);
+      __syncthreads();
+      S2CNN_CON(2, j + 1, 6) S2CNN_CON(3, j + 2, 3)
+      fft_pass<true, 1>(work, twl);
+      __syncthreads();
+      S2CNN_CON(4, j + 2, 0) S2CNN_CON(5, j + 2, 1)
+      fft_pass<true, 2>(work, twl);
+      __syncthreads();
+      S2CNN_CON(6, j + 2, 2)
+      stage_c2_store(j);
+      __syncthreads();
+      reduce();
+      __syncthreads();
+    }
   }
+#undef S2CNN_CON
+#undef S2CNN_FENCE
   fft_pass<true, 0>(work, twl); __syncthreads();
   fft_pass<true, 1>(work, twl); __syncthreads();
   fft_pass<true, 2>(work, twl); __syncthreads();
