@@ -207,8 +207,10 @@ def main():
     kernels = {n: {"ms": round(ms, 3)} for n, ms in per_call.items()}
     for n in mm_names:
         kernels[n]["tflops"] = round(flops_of[n] / (per_call[n] * 1e-3) / 1e12, 2)
-    for n in ("s2cnn_so3_analysis", "s2cnn_so3_synthesis"):
-        kernels[n]["gbs"] = round(so3_fft_bytes(b, b, B * F) / (per_call[n] * 1e-3) / 1e9, 1)
+    for n in per_call:   # transforms of the step: grid bytes + spectrum bytes (half of them in the real basis)
+        if n.startswith(("s2cnn_so3_analysis", "s2cnn_so3_synthesis")):
+            nbytes = so3_fft_bytes(b, b, B * F) - (4 * nspec(b) * B * F if n.endswith("_real_basis") else 0)
+            kernels[n]["gbs"] = round(nbytes / (per_call[n] * 1e-3) / 1e9, 1)
 
     result = {
         "metric": "SO3Conv fwd+bwd samples/s (b=32, 64->64 ch); SO(3) FFT achieved HBM GB/s",

@@ -110,6 +110,9 @@ int s2cnn_s2_mm_grady(const float *gz, const float *x, float *gy,
  *       [nbatch, 2b_in, 2b_in, 2b_in, 2]   (complex_in = 1)
  * table [2b_in, nspec(b_out)]  row beta_j, entries scale * d^l_{mn}(beta_j); must satisfy
  *       table[j, l,-m,-n] = (-1)^(m-n) table[j, l,m,n] (true of Wigner small-d)
+ *       and, for real input on the 64^3 grid (b_in = 32), table[2b-1-j, l,m,n] = (-1)^(l-n) table[j, l,-m,n]
+ *       (true of Wigner small-d on the SOFT grid, whose weights are symmetric in j); x then needs
+ *       16-byte alignment
  * packed_table  NULL, or the same table repacked once by s2cnn_so3_pack_table(..., synthesis = 0)
  *       (skips a per-call repack on the fast path; ignored where the fast path does not apply)
  * out   [nspec(b_out), nbatch, 2]
@@ -152,6 +155,26 @@ int s2cnn_so3_synthesis(const float *xhat, const float *table, const float *pack
  */
 size_t s2cnn_so3_packed_table_bytes(int b_in, int b_out, int synthesis);
 int s2cnn_so3_pack_table(const float *table, float *packed, int b_in, int b_out, int synthesis, void *stream);
+
+/* ---- the two transforms with the spectrum in the real basis ------------------------------
+ * For real signals the spectrum side of the transforms above can be read or written directly in the
+ * real basis of s2cnn_so3_spectrum_to_real (one float per entry):
+ *   analysis_real_basis (x)  = spectrum_to_real(analysis(x))          out [nspec(b_out), nbatch]
+ *   synthesis_real_basis(r)  = synthesis(spectrum_to_complex(r))      r   [nspec(b_in),  nbatch]
+ * which saves the conversion pass and half of the spectrum traffic inside the convolution layer
+ * (soft/so3_conv.py:36-56 has no such step: the reference keeps complex spectra throughout).
+ * Available where s2cnn_so3_real_basis_transform_available(b_in, b_out, synthesis) returns 1
+ * (a 64^3 grid on the signal side; S2CNN_EINVAL otherwise: compose the two calls instead).
+ * Tables, packed tables and workspace exactly as for s2cnn_so3_analysis / s2cnn_so3_synthesis with
+ * complex_in / complex_out = 0.
+ */
+int s2cnn_so3_real_basis_transform_available(int b_in, int b_out, int synthesis);
+int s2cnn_so3_analysis_real_basis(const float *x, const float *table, const float *packed_table, float *out,
+                                  void *workspace, size_t workspace_bytes,
+                                  int b_in, int b_out, long nbatch, void *stream);
+int s2cnn_so3_synthesis_real_basis(const float *r, const float *table, const float *packed_table, float *out,
+                                   void *workspace, size_t workspace_bytes,
+                                   int b_in, int b_out, long nbatch, void *stream);
 
 /* ---- S^2 Fourier analysis / synthesis ----------------------------------------------
  * analysis : x [nbatch, 2b_in, 2b_in] (complex_in = 0) or [..., 2] (complex_in = 1),

@@ -19,6 +19,7 @@ _int, _long, _size_t, _vp = ctypes.c_int, ctypes.c_long, ctypes.c_size_t, ctypes
 _MM_SIG = [_c_float_p, _c_float_p, _c_float_p, _int, _int, _int, _int, _vp]
 _FT_SIG = [_c_float_p, _c_float_p, _c_float_p, _vp, _size_t, _int, _int, _long, _int, _vp]
 _FT3_SIG = [_c_float_p, _c_float_p, _c_float_p, _c_float_p, _vp, _size_t, _int, _int, _long, _int, _vp]
+_FT3R_SIG = [_c_float_p, _c_float_p, _c_float_p, _c_float_p, _vp, _size_t, _int, _int, _long, _vp]
 _WS_SIG = [_int, _int, _long, _int]
 
 SIGNATURES = {
@@ -39,6 +40,9 @@ SIGNATURES = {
     "s2cnn_so3_analysis": (_int, _FT3_SIG),
     "s2cnn_so3_synthesis_workspace": (_size_t, _WS_SIG),
     "s2cnn_so3_synthesis": (_int, _FT3_SIG),
+    "s2cnn_so3_real_basis_transform_available": (_int, [_int, _int, _int]),
+    "s2cnn_so3_analysis_real_basis": (_int, _FT3R_SIG),
+    "s2cnn_so3_synthesis_real_basis": (_int, _FT3R_SIG),
     "s2cnn_so3_packed_table_bytes": (_size_t, [_int, _int, _int]),
     "s2cnn_so3_pack_table": (_int, [_c_float_p, _c_float_p, _int, _int, _int, _vp]),
     "s2cnn_s2_analysis_workspace": (_size_t, _WS_SIG),

@@ -310,7 +310,75 @@ size_t packed_bytes(int b_grid, int b_spec, int cplx, bool synthesis) {
 
 size_t round256(size_t n) { return (n + 255) & ~(size_t)255; }
 
+// Real signals on the 64^3 grid: per-volume kernel + the pass between its records and the spectral rows.
+// real_basis: the spectrum is stored in the real basis (one float per entry) instead of complex pairs.
+int fused_analysis(const float* x, const float* table, const float* packed_table, float* out, void* workspace,
+                   size_t workspace_bytes, int b_out, long nbatch, bool real_basis, hipStream_t st) {
+  if (!s2cnn::aligned16(x)) return S2CNN_EALIGN;
+  const size_t need = round256(fused64::scratch_bytes(nbatch)) + fused64::PACKED_FLOATS * sizeof(float);
+  if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
+  float4* rec = static_cast<float4*>(workspace);
+  const float* Tf = packed_table;
+  if (!Tf) {  // pack behind the records on every call
+    float* dst = reinterpret_cast<float*>(static_cast<char*>(workspace) + round256(fused64::scratch_bytes(nbatch)));
+    hipLaunchKernelGGL(fused64::pack_table, dim3(1024), dim3(256), 0, st, table, dst, s2cnn::so3_nspec(b_out), b_out);
+    Tf = dst;
+  }
+  hipLaunchKernelGGL(fused64::analysis_kernel, dim3(fused64::grid_size(nbatch)), dim3(fused64::THREADS), 0, st, x, Tf, rec, nbatch);
+  if (real_basis)
+    hipLaunchKernelGGL(fused64::spectrum_scatter_real, dim3((unsigned)((nbatch + fused64::ZR - 1) / fused64::ZR), fused64::NIT * 32), dim3(256), 0, st,
+                       rec, out, b_out, nbatch);
+  else
+    hipLaunchKernelGGL(fused64::spectrum_scatter, dim3((unsigned)((nbatch + fused64::ZT - 1) / fused64::ZT), fused64::NIT * 16), dim3(256), 0, st,
+                       rec, reinterpret_cast<float2*>(out), b_out, nbatch);
+  return s2cnn::launch_status();
+}
+
+int fused_synthesis(const float* xhat, const float* table, const float* packed_table, float* out, void* workspace,
+                    size_t workspace_bytes, int b_in, long nbatch, bool real_basis, hipStream_t st) {
+  if (!s2cnn::aligned16(out)) return S2CNN_EALIGN;
+  const int nl = b_in < 32 ? b_in : 32;
+  const size_t need = round256(fused64::scratch_bytes(nbatch)) + fused64::PACKED_FLOATS * sizeof(float);
+  if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
+  float4* rec = static_cast<float4*>(workspace);
+  const float* Tf = packed_table;
+  if (!Tf) {
+    float* dst = reinterpret_cast<float*>(static_cast<char*>(workspace) + round256(fused64::scratch_bytes(nbatch)));
+    hipLaunchKernelGGL(fused64::pack_table, dim3(1024), dim3(256), 0, st, table, dst, s2cnn::so3_nspec(b_in), nl);
+    Tf = dst;
+  }
+  if (real_basis)
+    hipLaunchKernelGGL(fused64::spectrum_gather_real, dim3((unsigned)((nbatch + fused64::ZR - 1) / fused64::ZR), fused64::NIT * 32), dim3(256), 0, st,
+                       xhat, rec, nl, nbatch);
+  else
+    hipLaunchKernelGGL(fused64::spectrum_gather, dim3((unsigned)((nbatch + fused64::ZT - 1) / fused64::ZT), fused64::NIT * 16), dim3(256), 0, st,
+                       reinterpret_cast<const float2*>(xhat), rec, nl, nbatch);
+  hipLaunchKernelGGL(fused64::synthesis_kernel, dim3(fused64::grid_size(nbatch)), dim3(fused64::THREADS), 0, st, rec, Tf, out, nbatch);
+  return s2cnn::launch_status();
+}
+
 }  // namespace
+
+extern "C" int s2cnn_so3_real_basis_transform_available(int b_in, int b_out, int synthesis) {
+  if (b_in < 1 || b_out < 1) return 0;
+  return synthesis ? fused_path(b_out, b_in, 0, true) : fused_path(b_in, b_out, 0, false);
+}
+
+extern "C" int s2cnn_so3_analysis_real_basis(const float* x, const float* table, const float* packed_table, float* out,
+                                             void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch, void* stream) {
+  if (!x || !table || !out || !sizes_ok(b_in, b_out, nbatch)) return S2CNN_EINVAL;
+  if (!fused_path(b_in, b_out, 0, false)) return S2CNN_EINVAL;
+  if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
+  return fused_analysis(x, table, packed_table, out, workspace, workspace_bytes, b_out, nbatch, true, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int s2cnn_so3_synthesis_real_basis(const float* r, const float* table, const float* packed_table, float* out,
+                                              void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch, void* stream) {
+  if (!r || !table || !out || !sizes_ok(b_out, b_in, nbatch)) return S2CNN_EINVAL;
+  if (!fused_path(b_out, b_in, 0, true)) return S2CNN_EINVAL;
+  if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
+  return fused_synthesis(r, table, packed_table, out, workspace, workspace_bytes, b_in, nbatch, true, static_cast<hipStream_t>(stream));
+}
 
 extern "C" size_t s2cnn_so3_packed_table_bytes(int b_in, int b_out, int synthesis) {
   if (b_in < 1 || b_out < 1) return 0;
@@ -351,21 +419,8 @@ extern "C" int s2cnn_so3_analysis(const float* x, const float* table, const floa
   if (!s2cnn::aligned8(out) || (complex_in && !s2cnn::aligned8(x))) return S2CNN_EALIGN;
   if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (fused_path(b_in, b_out, complex_in, false)) {
-    if (!s2cnn::aligned16(x)) return S2CNN_EALIGN;
-    if (!workspace || workspace_bytes < s2cnn_so3_analysis_workspace(b_in, b_out, nbatch, 0) || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
-    float4* rec = static_cast<float4*>(workspace);
-    const float* Tf = packed_table;
-    if (!Tf) {  // pack behind the records on every call
-      float* dst = reinterpret_cast<float*>(static_cast<char*>(workspace) + round256(fused64::scratch_bytes(nbatch)));
-      hipLaunchKernelGGL(fused64::pack_table, dim3(1024), dim3(256), 0, st, table, dst, s2cnn::so3_nspec(b_out), b_out);
-      Tf = dst;
-    }
-    hipLaunchKernelGGL(fused64::analysis_kernel, dim3(fused64::grid_size(nbatch)), dim3(fused64::THREADS), 0, st, x, Tf, rec, nbatch);
-    hipLaunchKernelGGL(fused64::spectrum_scatter, dim3((unsigned)((nbatch + fused64::ZT - 1) / fused64::ZT), fused64::NIT * 16), dim3(256), 0, st,
-                       rec, reinterpret_cast<float2*>(out), b_out, nbatch);
-    return s2cnn::launch_status();
-  }
+  if (fused_path(b_in, b_out, complex_in, false))
+    return fused_analysis(x, table, packed_table, out, workspace, workspace_bytes, b_out, nbatch, false, st);
   const size_t need = s2cnn_so3_analysis_workspace(b_in, b_out, nbatch, complex_in);
   if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
   const int n2 = 2 * b_in, nb = b_in < b_out ? b_in : b_out;
@@ -419,22 +474,8 @@ extern "C" int s2cnn_so3_synthesis(const float* xhat, const float* table, const 
   if (!s2cnn::aligned8(xhat) || (complex_out && !s2cnn::aligned8(out))) return S2CNN_EALIGN;
   if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (fused_path(b_out, b_in, complex_out, true)) {
-    if (!s2cnn::aligned16(out)) return S2CNN_EALIGN;
-    const int nl = b_in < 32 ? b_in : 32;
-    if (!workspace || workspace_bytes < s2cnn_so3_synthesis_workspace(b_in, b_out, nbatch, 0) || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
-    float4* rec = static_cast<float4*>(workspace);
-    const float* Tf = packed_table;
-    if (!Tf) {
-      float* dst = reinterpret_cast<float*>(static_cast<char*>(workspace) + round256(fused64::scratch_bytes(nbatch)));
-      hipLaunchKernelGGL(fused64::pack_table, dim3(1024), dim3(256), 0, st, table, dst, s2cnn::so3_nspec(b_in), nl);
-      Tf = dst;
-    }
-    hipLaunchKernelGGL(fused64::spectrum_gather, dim3((unsigned)((nbatch + fused64::ZT - 1) / fused64::ZT), fused64::NIT * 16), dim3(256), 0, st,
-                       reinterpret_cast<const float2*>(xhat), rec, nl, nbatch);
-    hipLaunchKernelGGL(fused64::synthesis_kernel, dim3(fused64::grid_size(nbatch)), dim3(fused64::THREADS), 0, st, rec, Tf, out, nbatch);
-    return s2cnn::launch_status();
-  }
+  if (fused_path(b_out, b_in, complex_out, true))
+    return fused_synthesis(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, nbatch, false, st);
   const size_t need = s2cnn_so3_synthesis_workspace(b_in, b_out, nbatch, complex_out);
   if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
   const int n2 = 2 * b_out, nb = b_in < b_out ? b_in : b_out;

@@ -466,6 +466,105 @@ __global__ __launch_bounds__(256) void spectrum_gather(const float2* __restrict_
 }
 
 // ---------------------------------------------------------------------------------------------
+// The same two passes for a spectrum kept in the REAL basis (see so3_real_basis.hip: R = Re(U X U^H),
+// one float per entry).  With A = X[l,+a,n], C = X[l,-a,n] of a real signal, s = (-1)^a:
+//     R[+a,+n] = A.re + s C.re     R[+a,-n] = -A.im - s C.im
+//     R[-a,+n] = A.im - s C.im     R[-a,-n] =  A.re - s C.re          (a, n > 0)
+//     a = 0: sqrt2 A.re, -sqrt2 A.im      n = 0: (A.re + s C.re)/sqrt2, (A.im - s C.im)/sqrt2      a = n = 0: A.re
+// and backwards (records hold twice the complex value, the table carries 1/2):
+//     2 A = (cc + ss, sc - cs)   2 C = s (cc - ss, -(cs + sc))   with cc, cs, sc, ss = R[+a,+n], R[+a,-n], R[-a,+n], R[-a,-n]
+//     a = 0: sqrt2 (cc, -cs), C unused     n = 0: sqrt2 (cc, sc), s sqrt2 (cc, -sc)     a = n = 0: (2 cc, 0)
+// Tiles of 32 volumes (128-byte pieces of a row) and 16 items; grid (ceil(nbatch / 32), NIT * 32).
+// ---------------------------------------------------------------------------------------------
+constexpr int ZR = 32;
+constexpr int IT_TILE_R = 16;
+constexpr int VLD_R = 16 * ZR + 1;
+constexpr float SQRT2 = 1.41421356237309504880f, RSQRT2 = 0.70710678118654752440f;
+
+__global__ __launch_bounds__(256) void spectrum_scatter_real(const float4* __restrict__ rec, float* __restrict__ out, int nl, long nbatch) {
+  __shared__ float vals[IT_TILE_R * VLD_R];
+  __shared__ int info[IT_TILE_R];
+  const int th = threadIdx.x;
+  const long z0 = (long)blockIdx.x * ZR;
+  const int it = blockIdx.y >> 5, t0 = (blockIdx.y & 31) * IT_TILE_R;
+  if (th < IT_TILE_R) info[th] = pack_item_info(it * THREADS + t0 + th);
+#pragma unroll
+  for (int r = 0; r < 8; ++r) {
+    const int e = th + 256 * r;
+    const int item = e & 15, q = (e >> 4) & 3, zz = e >> 6;
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (z0 + zz < nbatch) v = rec[(size_t)(z0 + zz) * REC_F4 + (it * 4 + q) * THREADS + t0 + item];
+    float* d = vals + item * VLD_R + (4 * q) * ZR + zz;
+    d[0] = v.x; d[ZR] = v.y; d[2 * ZR] = v.z; d[3 * ZR] = v.w;
+  }
+  __syncthreads();
+  const int zz = th & 31, sub = th >> 5;       // sub = 0..7: row slots 2 p + (0, 1) -> (u, kind) = ((sub & 1) * 2 + p / 2 ... see below)
+  if (z0 + zz >= nbatch) return;
+  for (int p = 0; p < 2 * IT_TILE_R; ++p) {    // 16 rows per item (4 degrees x 4 kinds), 8 at a time
+    const int item = p >> 1;
+    const int rs = (p & 1) * 8 + sub;          // 0..15
+    const int u = rs >> 2, kind = rs & 3;      // kind: 0 (+a,+n)  1 (+a,-n)  2 (-a,+n)  3 (-a,-n)
+    const int inf = info[item];
+    const int c = inf & 0xff, a = (inf >> 8) & 0xff, n = (inf >> 16) & 0xff;
+    const int l = 4 * c + u;
+    if (!(inf >> 24) || l < a || l < n || l >= nl || ((kind & 1) && n == 0) || ((kind & 2) && a == 0)) continue;
+    const int row = lmn_index(l, (kind & 2) ? -a : a, (kind & 1) ? -n : n);
+    // A = (+a) half: components 4 (u / 2) + 2 (u % 2) + (0 re, 1 im);  C = (-a) half: the same + 8
+    const int comp = 4 * (u >> 1) + 2 * (u & 1) + ((kind == 1 || kind == 2) ? 1 : 0);
+    const float av = vals[item * VLD_R + comp * ZR + zz], cv = vals[item * VLD_R + (comp + 8) * ZR + zz];
+    const float s = (a & 1) ? -1.f : 1.f;
+    float alpha = kind == 1 ? -1.f : 1.f;
+    float beta = (kind == 0) ? s : -s;
+    if (a == 0) { alpha *= SQRT2; beta = 0.f; if (n == 0) alpha = 1.f; }
+    else if (n == 0) { alpha *= RSQRT2; beta *= RSQRT2; }
+    out[(size_t)row * nbatch + z0 + zz] = alpha * av + beta * cv;
+  }
+}
+
+__global__ __launch_bounds__(256) void spectrum_gather_real(const float* __restrict__ rr, float4* __restrict__ rec, int nl, long nbatch) {
+  __shared__ float vals[IT_TILE_R * VLD_R];
+  __shared__ int info[IT_TILE_R];
+  const int th = threadIdx.x;
+  const long z0 = (long)blockIdx.x * ZR;
+  const int it = blockIdx.y >> 5, t0 = (blockIdx.y & 31) * IT_TILE_R;
+  if (th < IT_TILE_R) info[th] = pack_item_info(it * THREADS + t0 + th);
+  __syncthreads();
+  {
+    const int zz = th & 31, u = (th >> 5) & 3, sub = th >> 7;
+    const long zc = z0 + zz < nbatch ? z0 + zz : nbatch - 1;
+    for (int item = sub; item < IT_TILE_R; item += 2) {
+      const int inf = info[item];
+      const int c = inf & 0xff, a = (inf >> 8) & 0xff, n = (inf >> 16) & 0xff;
+      const int l = 4 * c + u;
+      float2 A = make_float2(0.f, 0.f), C = A;
+      if ((inf >> 24) && l >= a && l >= n && l < nl) {
+        const float cc = rr[(size_t)lmn_index(l, a, n) * nbatch + zc];
+        const float cs = n > 0 ? rr[(size_t)lmn_index(l, a, -n) * nbatch + zc] : 0.f;
+        const float sc = a > 0 ? rr[(size_t)lmn_index(l, -a, n) * nbatch + zc] : 0.f;
+        const float ss = (a > 0 && n > 0) ? rr[(size_t)lmn_index(l, -a, -n) * nbatch + zc] : 0.f;
+        const float s = (a & 1) ? -1.f : 1.f;
+        if (a > 0 && n > 0) { A = make_float2(cc + ss, sc - cs); C = make_float2(s * (cc - ss), -s * (cs + sc)); }
+        else if (a > 0)     { A = make_float2(SQRT2 * cc, SQRT2 * sc); C = make_float2(s * SQRT2 * cc, -s * SQRT2 * sc); }
+        else if (n > 0)     { A = make_float2(SQRT2 * cc, -SQRT2 * cs); }
+        else                { A = make_float2(2.f * cc, 0.f); }
+      }
+      const int comp = 4 * (u >> 1) + 2 * (u & 1);
+      float* d = vals + item * VLD_R + comp * ZR + zz;
+      d[0] = A.x; d[ZR] = A.y; d[8 * ZR] = C.x; d[9 * ZR] = C.y;
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < 8; ++r) {
+    const int e = th + 256 * r;
+    const int item = e & 15, q = (e >> 4) & 3, zz = e >> 6;
+    if (z0 + zz >= nbatch) continue;
+    const float* d = vals + item * VLD_R + (4 * q) * ZR + zz;
+    rec[(size_t)(z0 + zz) * REC_F4 + (it * 4 + q) * THREADS + t0 + item] = make_float4(d[0], d[ZR], d[2 * ZR], d[3 * ZR]);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
 // synthesis: records of the symmetrised spectrum -> y [nbatch][64][64][64] real
 //
 // While plane pair j is transformed in `work` (two gamma stages, two alpha stages, the last one

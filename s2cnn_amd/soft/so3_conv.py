@@ -8,8 +8,8 @@ from torch.nn.parameter import Parameter
 
 from ..so3_ft import so3_rft
 from ..so3_mm import so3_mm
-from ..so3_real import so3_mm_real, so3_rft_real, so3_spectrum_to_complex, so3_spectrum_to_real
-from .so3_fft import SO3_fft_real, SO3_ifft_real
+from ..so3_real import so3_mm_real, so3_rft_real
+from .so3_fft import SO3_fft_real, SO3_fft_real_basis, SO3_ifft_real, SO3_ifft_real_basis
 
 
 class SO3Convolution(Module):
@@ -48,15 +48,15 @@ class SO3Convolution(Module):
         assert x.size(3) == 2 * self.b_in
         assert x.size(4) == 2 * self.b_in
 
-        x = SO3_fft_real.apply(x, self.b_out)  # [l * m * n, batch, feature_in, complex]
         if self.real_basis:
-            x = so3_spectrum_to_real(x)  # [l * m * n, batch, feature_in]
+            x = SO3_fft_real_basis.apply(x, self.b_out)  # [l * m * n, batch, feature_in]
             y = so3_rft_real(self.kernel * self.scaling, self.b_out, self.grid)  # [l * m * n, feature_in, feature_out]
             assert x.size(0) == y.size(0)
             assert x.size(2) == y.size(1)
-            z = so3_spectrum_to_complex(so3_mm_real(x, y))  # [l * m * n, batch, feature_out, complex]
-            z = SO3_ifft_real.apply(z)  # [batch, feature_out, beta, alpha, gamma]
+            z = so3_mm_real(x, y)  # [l * m * n, batch, feature_out]
+            z = SO3_ifft_real_basis.apply(z)  # [batch, feature_out, beta, alpha, gamma]
             return z + self.bias
+        x = SO3_fft_real.apply(x, self.b_out)  # [l * m * n, batch, feature_in, complex]
         y = so3_rft(self.kernel * self.scaling, self.b_out, self.grid)  # [l * m * n, feature_in, feature_out, complex]
         assert x.size(0) == y.size(0)
         assert x.size(2) == y.size(1)

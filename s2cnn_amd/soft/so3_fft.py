@@ -42,6 +42,8 @@ def _analysis(x, b_in, b_out, batch_size, for_grad, complex_in):
     """x: contiguous grid tensor whose leading dims are `batch_size`; the result is allocated in its
     final shape (never a view: autograd can then take ownership of it as a gradient without a copy)."""
     _hip.require_gpu_f32(x)
+    if x.data_ptr() % 16:
+        x = x.clone()
     L = _hip.lib()
     nbatch = 1
     for d in batch_size:
@@ -156,3 +158,98 @@ class SO3_ifft_real(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output):  # pylint: disable=W
         return so3_rfft(grad_output, for_grad=True, b_out=ctx.b_in), None
+
+
+# ---------------------------------------------------------------------------------------------------
+# The two real transforms with the spectrum in the real basis of s2cnn_amd.so3_real (one float per
+# entry).  No counterpart in the reference; used by SO3Convolution, whose spectra are those of real
+# signals throughout.  Where the library has no direct kernel for the sizes, the two steps are composed.
+# ---------------------------------------------------------------------------------------------------
+def _real_basis_direct(b_in, b_out, synthesis):
+    return bool(_hip.lib().s2cnn_so3_real_basis_transform_available(b_in, b_out, int(synthesis)))
+
+
+def so3_rfft_real_basis(x, for_grad=False, b_out=None):
+    '''
+    :param x: [..., beta, alpha, gamma]
+    :return: [l * m * n, ...]  = so3_spectrum_to_real(so3_rfft(x))
+    '''
+    b_in = x.size(-1) // 2
+    assert x.size(-1) == 2 * b_in and x.size(-2) == 2 * b_in and x.size(-3) == 2 * b_in
+    if b_out is None:
+        b_out = b_in
+    if not (x.is_cuda and _real_basis_direct(b_in, b_out, False)):
+        from ..so3_real import _convert
+        y = so3_rfft(x, for_grad, b_out)
+        return _convert("s2cnn_so3_spectrum_to_real", y, y.shape[:-1])
+    _hip.require_gpu_f32(x)
+    x = x.contiguous()
+    if x.data_ptr() % 16:
+        x = x.clone()
+    batch_size = x.size()[:-3]
+    nbatch = 1
+    for d in batch_size:
+        nbatch *= d
+    L = _hip.lib()
+    table = _setup_wigner(b_in, nl=b_out, weighted=not for_grad, device=x.device)
+    packed = _setup_packed_wigner(b_in, b_out, not for_grad, False, x.device)
+    out = x.new_empty((_nspec(b_out), *batch_size))
+    ws = _hip.workspace(L.s2cnn_so3_analysis_workspace(b_in, b_out, nbatch, 0), x.device)
+    _hip.call("s2cnn_so3_analysis_real_basis", _hip.ptr(x), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out), _hip.ptr(ws),
+              ws.numel(), b_in, b_out, nbatch, _hip.stream_ptr())
+    return out
+
+
+def so3_rifft_real_basis(r, for_grad=False, b_out=None):
+    '''
+    :param r: [l * m * n, ...]  real-basis spectrum
+    :return: [..., beta, alpha, gamma]  = so3_rifft(so3_spectrum_to_complex(r))
+    '''
+    nspec = r.size(0)
+    b_in = round((3 / 4 * nspec) ** (1 / 3))
+    assert nspec == b_in * (4 * b_in ** 2 - 1) // 3
+    if b_out is None:
+        b_out = b_in
+    if not (r.is_cuda and _real_basis_direct(b_in, b_out, True)):
+        from ..so3_real import _convert
+        return so3_rifft(_convert("s2cnn_so3_spectrum_to_complex", r.contiguous(), (*r.shape, 2)), for_grad, b_out)
+    _hip.require_gpu_f32(r)
+    r = r.contiguous()
+    batch_size = r.size()[1:]
+    nbatch = 1
+    for d in batch_size:
+        nbatch *= d
+    L = _hip.lib()
+    table = _setup_wigner(b_out, nl=b_in, weighted=for_grad, device=r.device)
+    packed = _setup_packed_wigner(b_in, b_out, for_grad, True, r.device)
+    out = r.new_empty((*batch_size, 2 * b_out, 2 * b_out, 2 * b_out))
+    ws = _hip.workspace(L.s2cnn_so3_synthesis_workspace(b_in, b_out, nbatch, 0), r.device)
+    _hip.call("s2cnn_so3_synthesis_real_basis", _hip.ptr(r), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out), _hip.ptr(ws),
+              ws.numel(), b_in, b_out, nbatch, _hip.stream_ptr())
+    return out
+
+
+class SO3_fft_real_basis(torch.autograd.Function):
+    """SO3_fft_real followed by the change to the real basis; the backward is the adjoint pair of
+    SO3_fft_real.backward and so3_spectrum_to_complex."""
+    @staticmethod
+    def forward(ctx, x, b_out=None):  # pylint: disable=W
+        ctx.b_in = x.size(-1) // 2
+        return so3_rfft_real_basis(x, b_out=b_out)
+
+    @staticmethod
+    def backward(ctx, grad_output):  # pylint: disable=W
+        return so3_rifft_real_basis(grad_output, for_grad=True, b_out=ctx.b_in), None
+
+
+class SO3_ifft_real_basis(torch.autograd.Function):
+    """The change from the real basis followed by SO3_ifft_real."""
+    @staticmethod
+    def forward(ctx, r, b_out=None):  # pylint: disable=W
+        nspec = r.size(0)
+        ctx.b_in = round((3 / 4 * nspec) ** (1 / 3))
+        return so3_rifft_real_basis(r, b_out=b_out)
+
+    @staticmethod
+    def backward(ctx, grad_output):  # pylint: disable=W
+        return so3_rfft_real_basis(grad_output, for_grad=True, b_out=ctx.b_in), None

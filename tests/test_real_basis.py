@@ -203,3 +203,69 @@ def test_convolution_real_and_complex_paths_agree(hip):
         out[flag] = (z.detach(), x.grad.clone(), conv.kernel.grad.clone())
     for a, c in zip(out[True], out[False]):
         _close(a, c.double().cpu().numpy())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("b_in,b_out,nz", [(32, 32, 3), (32, 20, 33), (20, 32, 5), (6, 4, 2), (4, 6, 3)])
+def test_transforms_in_the_real_basis(hip, b_in, b_out, nz):
+    """so3_rfft_real_basis / so3_rifft_real_basis against the two-step compositions they replace (direct
+    kernels on the 64^3 grid, composed elsewhere), for both tables, and the autograd pair by a dot-product test."""
+    from s2cnn_amd.soft import so3_fft as P
+    from s2cnn_amd.so3_real import so3_spectrum_to_complex, so3_spectrum_to_real
+    g = torch.Generator().manual_seed(b_in * 100 + b_out)
+    x = torch.randn(nz, 2 * b_in, 2 * b_in, 2 * b_in, generator=g).cuda()
+    ns = b_in * (4 * b_in ** 2 - 1) // 3
+    r = torch.randn(ns, nz, generator=g).cuda()
+    for for_grad in (False, True):
+        got = P.so3_rfft_real_basis(x, for_grad, b_out)
+        want = so3_spectrum_to_real(P.so3_rfft(x, for_grad, b_out))
+        assert got.shape == want.shape
+        assert (got - want).abs().max().item() < 1e-5 * want.abs().max().item(), (b_in, b_out, for_grad)
+        got = P.so3_rifft_real_basis(r, for_grad, b_out)
+        want = P.so3_rifft(so3_spectrum_to_complex(r), for_grad, b_out)
+        assert got.shape == want.shape
+        assert (got - want).abs().max().item() < 1e-5 * want.abs().max().item(), (b_in, b_out, for_grad)
+    # <fft(x), r'> = <x, fft.backward(r')> and the same for ifft
+    xg = x.clone().requires_grad_()
+    y = P.SO3_fft_real_basis.apply(xg, b_out)
+    w = torch.randn(y.shape, generator=g).cuda()
+    (gx,) = torch.autograd.grad(y, xg, w)
+    lhs, rhs = (y.double() * w.double()).sum().item(), (x.double() * gx.double()).sum().item()
+    if b_out <= b_in:   # the reference's backward is the exact adjoint only when no frequencies are cut off
+        assert abs(lhs - rhs) < 1e-4 * abs(lhs), (lhs, rhs)
+    rg = r.clone().requires_grad_()
+    y = P.SO3_ifft_real_basis.apply(rg, b_out)
+    w = torch.randn(y.shape, generator=g).cuda()
+    (gr,) = torch.autograd.grad(y, rg, w)
+    lhs, rhs = (y.double() * w.double()).sum().item(), (r.double() * gr.double()).sum().item()
+    if b_out >= b_in:
+        assert abs(lhs - rhs) < 1e-4 * abs(lhs), (lhs, rhs)
+
+
+@pytest.mark.gpu
+def test_convolution_on_the_64_grid_matches_oracle(hip):
+    """SO3Convolution with b_in = b_out = 32 (direct real-basis transforms on both sides) against the oracle,
+    forward and all gradients, at a small batch and few features."""
+    import s2cnn_amd
+    from oracle import cpu_path as O
+    B, Fi, Fo, b = 2, 2, 3, 32
+    grid = s2cnn_amd.so3_near_identity_grid()
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(B, Fi, 64, 64, 64, generator=g)
+    layer = s2cnn_amd.SO3Convolution(Fi, Fo, b, b, grid)
+    k = torch.rand(Fi, Fo, len(grid), generator=g) * 2 - 1
+    bias = torch.randn(1, Fo, 1, 1, 1, generator=g) * 0.1
+    with torch.no_grad():
+        layer.kernel.copy_(k)
+        layer.bias.copy_(bias)
+    layer = layer.cuda()
+    xg = x.cuda().requires_grad_()
+    out = layer(xg)
+    (out * out).sum().backward()
+    xo, ko, bo = x.requires_grad_(), k.requires_grad_(), bias.requires_grad_()   # float32 oracle: b = 32 in float64 takes minutes
+    outo = O.so3_conv(xo, ko, bo, b, b, grid)
+    (outo * outo).sum().backward()
+    for name, a, c in (("out", out, outo), ("grad_x", xg.grad, xo.grad), ("grad_kernel", layer.kernel.grad, ko.grad), ("grad_bias", layer.bias.grad, bo.grad)):
+        q = (a.detach().cpu().double() - c.detach().double()).abs().max().item() / c.detach().double().std().item()
+        print(name, q, flush=True)
+        assert q < 1e-4, (name, q)
