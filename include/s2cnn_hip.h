@@ -167,6 +167,9 @@ int s2cnn_so3_pack_table(const float *table, float *packed, int b_in, int b_out,
  * (a 64^3 grid on the signal side; S2CNN_EINVAL otherwise: compose the two calls instead).
  * Tables, packed tables and workspace exactly as for s2cnn_so3_analysis / s2cnn_so3_synthesis with
  * complex_in / complex_out = 0.
+ * bias: NULL, or nfeature values; with the batch laid out [..., nfeature] (nbatch a multiple of nfeature),
+ *       bias[z % nfeature] is added to every sample of volume z: the "+ self.bias" of soft/so3_conv.py:56
+ *       in the epilogue of the transform instead of a pass of its own.
  */
 int s2cnn_so3_real_basis_transform_available(int b_in, int b_out, int synthesis);
 int s2cnn_so3_analysis_real_basis(const float *x, const float *table, const float *packed_table, float *out,
@@ -174,7 +177,8 @@ int s2cnn_so3_analysis_real_basis(const float *x, const float *table, const floa
                                   int b_in, int b_out, long nbatch, void *stream);
 int s2cnn_so3_synthesis_real_basis(const float *r, const float *table, const float *packed_table, float *out,
                                    void *workspace, size_t workspace_bytes,
-                                   int b_in, int b_out, long nbatch, void *stream);
+                                   int b_in, int b_out, long nbatch,
+                                   const float *bias, int nfeature, void *stream);
 
 /* ---- S^2 Fourier analysis / synthesis ----------------------------------------------
  * analysis : x [nbatch, 2b_in, 2b_in] (complex_in = 0) or [..., 2] (complex_in = 1),

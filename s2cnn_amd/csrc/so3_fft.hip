@@ -335,7 +335,7 @@ int fused_analysis(const float* x, const float* table, const float* packed_table
 }
 
 int fused_synthesis(const float* xhat, const float* table, const float* packed_table, float* out, void* workspace,
-                    size_t workspace_bytes, int b_in, long nbatch, bool real_basis, hipStream_t st) {
+                    size_t workspace_bytes, int b_in, long nbatch, bool real_basis, const float* bias, int nfeature, hipStream_t st) {
   if (!s2cnn::aligned16(out)) return S2CNN_EALIGN;
   const int nl = b_in < 32 ? b_in : 32;
   const size_t need = round256(fused64::scratch_bytes(nbatch)) + fused64::PACKED_FLOATS * sizeof(float);
@@ -353,7 +353,7 @@ int fused_synthesis(const float* xhat, const float* table, const float* packed_t
   else
     hipLaunchKernelGGL(fused64::spectrum_gather, dim3((unsigned)((nbatch + fused64::ZT - 1) / fused64::ZT), fused64::NIT * 16), dim3(256), 0, st,
                        reinterpret_cast<const float2*>(xhat), rec, nl, nbatch);
-  hipLaunchKernelGGL(fused64::synthesis_kernel, dim3(fused64::grid_size(nbatch)), dim3(fused64::THREADS), 0, st, rec, Tf, out, nbatch);
+  hipLaunchKernelGGL(fused64::synthesis_kernel, dim3(fused64::grid_size(nbatch)), dim3(fused64::THREADS), 0, st, rec, Tf, out, nbatch, bias, nfeature);
   return s2cnn::launch_status();
 }
 
@@ -373,11 +373,14 @@ extern "C" int s2cnn_so3_analysis_real_basis(const float* x, const float* table,
 }
 
 extern "C" int s2cnn_so3_synthesis_real_basis(const float* r, const float* table, const float* packed_table, float* out,
-                                              void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch, void* stream) {
+                                              void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
+                                              const float* bias, int nfeature, void* stream) {
   if (!r || !table || !out || !sizes_ok(b_out, b_in, nbatch)) return S2CNN_EINVAL;
+  if (bias && (nfeature < 1 || nbatch % nfeature != 0)) return S2CNN_EINVAL;
   if (!fused_path(b_out, b_in, 0, true)) return S2CNN_EINVAL;
   if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
-  return fused_synthesis(r, table, packed_table, out, workspace, workspace_bytes, b_in, nbatch, true, static_cast<hipStream_t>(stream));
+  return fused_synthesis(r, table, packed_table, out, workspace, workspace_bytes, b_in, nbatch, true, bias, bias ? nfeature : 1,
+                         static_cast<hipStream_t>(stream));
 }
 
 extern "C" size_t s2cnn_so3_packed_table_bytes(int b_in, int b_out, int synthesis) {
@@ -475,7 +478,7 @@ extern "C" int s2cnn_so3_synthesis(const float* xhat, const float* table, const 
   if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (fused_path(b_out, b_in, complex_out, true))
-    return fused_synthesis(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, nbatch, false, st);
+    return fused_synthesis(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, nbatch, false, nullptr, 1, st);
   const size_t need = s2cnn_so3_synthesis_workspace(b_in, b_out, nbatch, complex_out);
   if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
   const int n2 = 2 * b_out, nb = b_in < b_out ? b_in : b_out;

@@ -572,8 +572,9 @@ __global__ __launch_bounds__(256) void spectrum_gather_real(const float* __restr
 // area; a reduction over the (up to 8) items of a column then fills `work` for the next step.
 // Sums are formed in a fixed order: results are reproducible bit for bit.
 // ---------------------------------------------------------------------------------------------
+// bias: NULL, or one value per feature added to every sample of volume z (feature = z % nfeature)
 __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __restrict__ rec, const float* __restrict__ Tf,
-                                                            float* __restrict__ y, long nbatch) {
+                                                            float* __restrict__ y, long nbatch, const float* __restrict__ bias, int nfeature) {
   using namespace fft64;
   __shared__ __attribute__((aligned(16))) float2 work[LDS_ELEMS];
   __shared__ __attribute__((aligned(16))) float4 stg_p[NIT * THREADS];       // item i: its share of the bins [+a,n], [-a,-n]
@@ -583,6 +584,7 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
   if (z < 0) return;
   const int t = threadIdx.x;
   const int lo = t & 63, d = t >> 6;
+  const float bz = bias ? bias[z % nfeature] : 0.f;
   fill_twiddles<true>(twl);
   for (int i = t; i < LDS_ELEMS; i += THREADS) work[i] = make_float2(0.f, 0.f);   // bins of m = 32 and n = 32 stay zero ... until a transform overwrites them: cleared again in reduce()
 
@@ -683,14 +685,25 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
     fft8<true>(v);
     float ra[8], rb[8];
 #pragma unroll
-    for (int k = 0; k < 8; ++k) { ra[k] = v[k].x; rb[k] = v[k].y; }
+    for (int k = 0; k < 8; ++k) { ra[k] = v[k].x + bz; rb[k] = v[k].y + bz; }
     quad_transpose(ra[0], ra[1], ra[2], ra[3]); quad_transpose(ra[4], ra[5], ra[6], ra[7]);
     quad_transpose(rb[0], rb[1], rb[2], rb[3]); quad_transpose(rb[4], rb[5], rb[6], rb[7]);
     // lane (q, i) = (lo / 4, lo % 4) now holds columns 4q..4q+3 of the rows d + 8 i and d + 8 (4 + i)
-    buf_store_f32x4(make_float4(ra[0], ra[1], ra[2], ra[3]), ry, yoff, (j * 4096) * 4);
-    buf_store_f32x4(make_float4(ra[4], ra[5], ra[6], ra[7]), ry, yoff, (j * 4096 + 2048) * 4);
-    buf_store_f32x4(make_float4(rb[0], rb[1], rb[2], rb[3]), ry, yoff, ((63 - j) * 4096) * 4);
-    buf_store_f32x4(make_float4(rb[4], rb[5], rb[6], rb[7]), ry, yoff, ((63 - j) * 4096 + 2048) * 4);
+    // Four 16-byte stores.  Observed on gfx950: when such stores follow each other within a few cycles (or their
+    // data registers are refilled for the next store), the first component of the earlier store can come out
+    // holding the later store's value in lanes 12-15 of each 16-lane row - run-to-run varying, and only when loads
+    // had just been queued.  Hence: 16 distinct data registers, idle cycles between and after the stores, and the
+    // plane offset in the lane offset (an integer add between the stores) instead of the scalar offset.
+    __builtin_amdgcn_sched_barrier(0);
+    buf_store_f32x4(make_float4(ra[0], ra[1], ra[2], ra[3]), ry, yoff + (j * 4096) * 4, 0);
+    asm volatile("s_nop 7" ::: "memory");
+    buf_store_f32x4(make_float4(ra[4], ra[5], ra[6], ra[7]), ry, yoff + (j * 4096 + 2048) * 4, 0);
+    asm volatile("s_nop 7" ::: "memory");
+    buf_store_f32x4(make_float4(rb[0], rb[1], rb[2], rb[3]), ry, yoff + ((63 - j) * 4096) * 4, 0);
+    asm volatile("s_nop 7" ::: "memory");
+    buf_store_f32x4(make_float4(rb[4], rb[5], rb[6], rb[7]), ry, yoff + ((63 - j) * 4096 + 2048) * 4, 0);
+    asm volatile("s_nop 7\n\ts_nop 7" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
   };
 
 #define S2CNN_FENCE() __builtin_amdgcn_sched_barrier(0)

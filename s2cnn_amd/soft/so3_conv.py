@@ -54,8 +54,7 @@ class SO3Convolution(Module):
             assert x.size(0) == y.size(0)
             assert x.size(2) == y.size(1)
             z = so3_mm_real(x, y)  # [l * m * n, batch, feature_out]
-            z = SO3_ifft_real_basis.apply(z)  # [batch, feature_out, beta, alpha, gamma]
-            return z + self.bias
+            return SO3_ifft_real_basis.apply(z, None, self.bias)  # [batch, feature_out, beta, alpha, gamma], bias added
         x = SO3_fft_real.apply(x, self.b_out)  # [l * m * n, batch, feature_in, complex]
         y = so3_rft(self.kernel * self.scaling, self.b_out, self.grid)  # [l * m * n, feature_in, feature_out, complex]
         assert x.size(0) == y.size(0)

@@ -200,10 +200,11 @@ def so3_rfft_real_basis(x, for_grad=False, b_out=None):
     return out
 
 
-def so3_rifft_real_basis(r, for_grad=False, b_out=None):
+def so3_rifft_real_basis(r, for_grad=False, b_out=None, bias=None):
     '''
     :param r: [l * m * n, ...]  real-basis spectrum
-    :return: [..., beta, alpha, gamma]  = so3_rifft(so3_spectrum_to_complex(r))
+    :param bias: None, or one value per entry of the last batch dimension, added to every sample of its volumes
+    :return: [..., beta, alpha, gamma]  = so3_rifft(so3_spectrum_to_complex(r)) (+ bias)
     '''
     nspec = r.size(0)
     b_in = round((3 / 4 * nspec) ** (1 / 3))
@@ -212,7 +213,10 @@ def so3_rifft_real_basis(r, for_grad=False, b_out=None):
         b_out = b_in
     if not (r.is_cuda and _real_basis_direct(b_in, b_out, True)):
         from ..so3_real import _convert
-        return so3_rifft(_convert("s2cnn_so3_spectrum_to_complex", r.contiguous(), (*r.shape, 2)), for_grad, b_out)
+        out = so3_rifft(_convert("s2cnn_so3_spectrum_to_complex", r.contiguous(), (*r.shape, 2)), for_grad, b_out)
+        if bias is not None:
+            out.add_(bias.reshape(*([1] * (r.dim() - 2)), -1, 1, 1, 1))
+        return out
     _hip.require_gpu_f32(r)
     r = r.contiguous()
     batch_size = r.size()[1:]
@@ -224,8 +228,14 @@ def so3_rifft_real_basis(r, for_grad=False, b_out=None):
     packed = _setup_packed_wigner(b_in, b_out, for_grad, True, r.device)
     out = r.new_empty((*batch_size, 2 * b_out, 2 * b_out, 2 * b_out))
     ws = _hip.workspace(L.s2cnn_so3_synthesis_workspace(b_in, b_out, nbatch, 0), r.device)
+    nfeature = 1
+    if bias is not None:
+        _hip.require_gpu_f32(bias)
+        bias = bias.reshape(-1).contiguous()
+        nfeature = bias.numel()
+        assert r.dim() >= 2 and r.size(-1) == nfeature
     _hip.call("s2cnn_so3_synthesis_real_basis", _hip.ptr(r), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out), _hip.ptr(ws),
-              ws.numel(), b_in, b_out, nbatch, _hip.stream_ptr())
+              ws.numel(), b_in, b_out, nbatch, _null_or_ptr(bias), nfeature, _hip.stream_ptr())
     return out
 
 
@@ -243,13 +253,20 @@ class SO3_fft_real_basis(torch.autograd.Function):
 
 
 class SO3_ifft_real_basis(torch.autograd.Function):
-    """The change from the real basis followed by SO3_ifft_real."""
+    """The change from the real basis followed by SO3_ifft_real and, optionally, the bias of the convolution
+    layer (r [l * m * n, batch, feature], bias with `feature` entries in any shape).  The gradient of the bias
+    costs nothing: the degree-0 coefficient of the unweighted analysis of grad_output IS its sum over the grid."""
     @staticmethod
-    def forward(ctx, r, b_out=None):  # pylint: disable=W
+    def forward(ctx, r, b_out=None, bias=None):  # pylint: disable=W
         nspec = r.size(0)
         ctx.b_in = round((3 / 4 * nspec) ** (1 / 3))
-        return so3_rifft_real_basis(r, b_out=b_out)
+        ctx.bias_shape = None if bias is None else bias.shape
+        return so3_rifft_real_basis(r, b_out=b_out, bias=bias)
 
     @staticmethod
     def backward(ctx, grad_output):  # pylint: disable=W
-        return so3_rfft_real_basis(grad_output, for_grad=True, b_out=ctx.b_in), None
+        g = so3_rfft_real_basis(grad_output, for_grad=True, b_out=ctx.b_in)
+        gb = None
+        if ctx.bias_shape is not None and ctx.needs_input_grad[2]:
+            gb = g[0].reshape(-1, g.size(-1)).sum(0).reshape(ctx.bias_shape)
+        return g, None, gb
