@@ -89,6 +89,21 @@ int s2cnn_so3_mm_real_gradx(const float *gz, const float *y, float *gx,
 int s2cnn_so3_mm_real_grady(const float *gz, const float *x, float *gy,
                             int nl, int nbatch, int f_in, int f_out, void *stream);
 
+/* ---- kernel spectrum of the SO(3) layer for grids with few distinct beta values ------------
+ * The reference computes y[l,m,n] = sum_a x_a conj(D^l_{mn}(alpha_a, beta_a, gamma_a)) as one dense product with a
+ * [len(grid), nspec] matrix (so3_ft.py:8-24).  For the grid points A_i that share beta_i,
+ * conj D^l_{mn} = d^l_{mn}(beta_i) exp(-i(m alpha_a + n gamma_a)), hence
+ *     y[l,m,n] = sum_i d^l_{mn}(beta_i) G_i[m,n],    G_i[m,n] = sum_{a in A_i} x_a exp(-i(m alpha_a + n gamma_a)):
+ * a small GEMM (caller's library) for G, then the pass below, linear in the size of y.  Real x only.
+ *   G    [nbeta, (2b-1) * b, 2, ncols]   row (m + b-1) * b + n, m in -(b-1)..b-1, n in 0..b-1; (re, im) planes
+ *   dtab [nbeta, nspec(b)]               d^l_{mn}(beta_i), degree-major then m then n
+ *   y    [nspec(b), ncols]               in the real basis of s2cnn_so3_spectrum_to_real
+ * expand_real      : y from G              expand_real_grad : gG from gy (the adjoint)
+ * nbeta <= 4, ncols a multiple of 4, G / y / gy / gG 16-byte aligned.
+ */
+int s2cnn_so3_rft_expand_real(const float *G, const float *dtab, float *y, int b, int nbeta, long ncols, void *stream);
+int s2cnn_so3_rft_expand_real_grad(const float *gy, const float *dtab, float *gG, int b, int nbeta, long ncols, void *stream);
+
 /* ---- S^2 x S^2 -> SO(3) spectral outer products -------------------------------------
  * x  [nl^2, nbatch, f_in , 2]
  * y  [nl^2, f_in  , f_out, 2]

@@ -110,14 +110,64 @@ def _setup_so3_ft_real(b, grid, device):
     return torch.tensor(F.astype(np.float32), dtype=torch.float32, device=device)
 
 
+@lru_cache(maxsize=32)
+def _setup_so3_rft_plan(b, grid, device):
+    """Factorised form of the matrix of `_setup_so3_ft_real` for grids with few distinct beta values
+    (wigner.so3_rft_plan); None where it does not apply."""
+    plan = wigner.so3_rft_plan(b, grid)
+    if plan is None:
+        return None
+    idx, E, dtab = plan
+    valid = torch.tensor(idx >= 0, device=device)
+    return (torch.tensor(np.maximum(idx, 0), dtype=torch.long, device=device), valid,
+            torch.tensor(E.astype(np.float32), device=device).contiguous(),
+            torch.tensor(dtab.astype(np.float32), device=device).contiguous())
+
+
+class _SO3RftRealFactorised(torch.autograd.Function):
+    """x [ncols, n_grid] -> y [nspec, ncols]: plane coefficients per beta group by a batched GEMM, then the
+    expansion over the degrees (s2cnn_so3_rft_expand_real) and its adjoint."""
+    @staticmethod
+    def forward(ctx, x2, b, plan):
+        idx, valid, E, dtab = plan
+        ncols = x2.size(0)
+        xg = x2.t()[idx] * valid.unsqueeze(-1)                    # [nbeta, P, ncols]
+        G = torch.bmm(E.transpose(1, 2), xg).contiguous()        # [nbeta, R, ncols]
+        y = x2.new_empty((b * (4 * b * b - 1) // 3, ncols))
+        _hip.call("s2cnn_so3_rft_expand_real", _hip.ptr(G), _hip.ptr(dtab), _hip.ptr(y), b, idx.size(0), ncols, _hip.stream_ptr())
+        ctx.plan, ctx.b, ctx.n_grid = plan, b, x2.size(1)
+        return y
+
+    @staticmethod
+    def backward(ctx, gy):
+        idx, valid, E, dtab = ctx.plan
+        gy = gy.contiguous()
+        ncols = gy.size(1)
+        gG = gy.new_empty((idx.size(0), E.size(2), ncols))
+        _hip.call("s2cnn_so3_rft_expand_real_grad", _hip.ptr(gy), _hip.ptr(dtab), _hip.ptr(gG), ctx.b, idx.size(0), ncols, _hip.stream_ptr())
+        gxg = torch.bmm(E, gG)                                    # [nbeta, P, ncols]
+        gx = gy.new_zeros((ctx.n_grid, ncols))
+        gx.index_add_(0, idx[valid], gxg[valid])
+        return gx.t(), None, None
+
+
 def so3_rft_real(x, b, grid):
     """
     so3_rft followed by so3_spectrum_to_real, as one real GEMM with the transformed matrix
     :param x: [..., beta_alpha_gamma]
     :return: [l * m * n, ...]
     """
+    sz = x.size()
+    ncols = x.numel() // sz[-1]
+    plan = _setup_so3_rft_plan(b, tuple(grid), x.device) if (x.is_cuda and ncols % 4 == 0 and so3_rft_real.factorised) else None
+    if plan is not None:
+        assert sz[-1] == len(grid)
+        out = _SO3RftRealFactorised.apply(x.reshape(-1, sz[-1]), b, plan)
+        return out.view(-1, *sz[:-1])
     F = _setup_so3_ft_real(b, grid, x.device)  # [beta_alpha_gamma, l * m * n]
     assert x.size(-1) == F.size(0)
-    sz = x.size()
     out = torch.matmul(F.t(), x.reshape(-1, sz[-1]).t())
     return out.view(-1, *sz[:-1])
+
+
+so3_rft_real.factorised = True   # False: always the dense product with the [len(grid), nspec] matrix

@@ -182,3 +182,43 @@ def s2_ft_matrix(b, grid):
         D = wigner_D(l, alpha, beta, zero).conj()
         out[:, l * l:l * l + 2 * l + 1] = (2 * b) * D[:, :, l]
     return out
+
+
+def so3_rft_plan(b, grid, max_betas=4):
+    """Factorisation of so3_ft_matrix for grids with few distinct beta values (every grid of
+    s2cnn/so3_grid.py:6-37 is of that kind): with A_i the points whose beta is beta_i,
+
+        F[a, (l,m,n)] = d^l_{mn}(beta_i) * E_a[m, n],   E_a[m, n] = exp(-i (m alpha_a + n gamma_a)),   a in A_i,
+
+    so the transform of x is  y[l,m,n] = sum_i d^l_{mn}(beta_i) G_i[m,n],  G_i = sum_{a in A_i} x_a E_a:
+    a small GEMM per beta_i followed by a pass that is linear in the size of the result.
+
+    Returns None when the grid has more than `max_betas` distinct betas, else (idx, E, dtab), float64:
+      idx  [nbeta, P] int64   grid index of each group member (-1: padding)
+      E    [nbeta, P, R]      R = (2b-1) * b * 2; column ((m + b-1) * b + n) * 2 + (0: re, 1: im), m in -(b-1)..b-1,
+                              n in 0..b-1 (the half n >= 0 suffices for real x)
+      dtab [nbeta, nspec(b)]  d^l_{mn}(beta_i), degree-major then m then n
+    """
+    g = np.asarray(grid, dtype=np.float64).reshape(-1, 3)
+    ub, inv = np.unique(np.round(g[:, 0], 12), return_inverse=True)
+    if len(ub) > max_betas:
+        return None
+    groups = [np.nonzero(inv == i)[0] for i in range(len(ub))]
+    P = max(len(q) for q in groups)
+    idx = -np.ones((len(ub), P), dtype=np.int64)
+    m = np.arange(-(b - 1), b)[:, None]
+    n = np.arange(b)[None, :]
+    E = np.zeros((len(ub), P, (2 * b - 1) * b * 2), dtype=np.float64)
+    for i, q in enumerate(groups):
+        idx[i, :len(q)] = q
+        for p, a in enumerate(q):
+            ang = m * g[a, 1] + n * g[a, 2]
+            E[i, p, 0::2] = np.cos(ang).reshape(-1)
+            E[i, p, 1::2] = -np.sin(ang).reshape(-1)
+    dtab = np.empty((len(ub), so3_nspec(b)), dtype=np.float64)
+    pos = 0
+    for l in range(b):
+        cnt = (2 * l + 1) ** 2
+        dtab[:, pos:pos + cnt] = wigner_d(l, g[[q[0] for q in groups], 0]).reshape(len(ub), cnt)
+        pos += cnt
+    return idx, E, dtab

@@ -269,3 +269,67 @@ def test_convolution_on_the_64_grid_matches_oracle(hip):
         q = (a.detach().cpu().double() - c.detach().double()).abs().max().item() / c.detach().double().std().item()
         print(name, q, flush=True)
         assert q < 1e-4, (name, q)
+
+
+def test_factorised_kernel_transform_plan():
+    """wigner.so3_rft_plan: plane coefficients per beta group, expanded with the real-basis formulas of
+    csrc/so3_rft.hip in numpy, reproduce the dense real-basis matrix (itself pinned against the oracle above)."""
+    import s2cnn_amd
+    from s2cnn_amd import wigner
+    b = 5
+    for grid in (s2cnn_amd.so3_near_identity_grid(n_alpha=4, n_beta=3, n_gamma=5), s2cnn_amd.so3_equatorial_grid(n_alpha=6, n_gamma=3), ((0, 0, 0),)):
+        idx, E, dtab = wigner.so3_rft_plan(b, grid)
+        rng = np.random.default_rng(1)
+        x = rng.standard_normal((3, len(grid)))
+        want = wigner.so3_ft_matrix_real(b, grid).T @ x.T
+        xg = np.where((idx >= 0)[..., None], x.T[np.maximum(idx, 0)], 0.0)
+        G = np.einsum("ipr,ipc->irc", E, xg)
+
+        def lmn(l, m, n):
+            return l * (4 * l * l - 1) // 3 + (l + m) * (2 * l + 1) + (l + n)
+
+        def row(i, m, n):
+            r = ((m + b - 1) * b + n) * 2
+            return G[i, r] + 1j * G[i, r + 1]
+        got = np.zeros_like(want)
+        for a in range(b):
+            for n in range(b):
+                s = -1.0 if a & 1 else 1.0
+                for l in range(max(a, n), b):
+                    A = sum(dtab[i, lmn(l, a, n)] * row(i, a, n) for i in range(len(idx)))
+                    C = sum(dtab[i, lmn(l, -a, n)] * row(i, -a, n) for i in range(len(idx)))
+                    if a > 0 and n > 0:
+                        got[lmn(l, a, n)], got[lmn(l, a, -n)] = A.real + s * C.real, -A.imag - s * C.imag
+                        got[lmn(l, -a, n)], got[lmn(l, -a, -n)] = A.imag - s * C.imag, A.real - s * C.real
+                    elif a > 0:
+                        got[lmn(l, a, 0)], got[lmn(l, -a, 0)] = (A.real + s * C.real) / np.sqrt(2), (A.imag - s * C.imag) / np.sqrt(2)
+                    elif n > 0:
+                        got[lmn(l, 0, n)], got[lmn(l, 0, -n)] = np.sqrt(2) * A.real, -np.sqrt(2) * A.imag
+                    else:
+                        got[lmn(l, 0, 0)] = A.real
+        assert np.abs(got - want).max() < 1e-12 * max(1.0, np.abs(want).max())
+    assert wigner.so3_rft_plan(3, s2cnn_amd.so3_soft_grid(3)) is None        # 6 distinct betas: dense product
+
+
+@pytest.mark.gpu
+def test_factorised_kernel_transform_matches_dense(hip):
+    """so3_rft_real through the factorised path against the dense product, forward and gradient."""
+    import s2cnn_amd
+    from s2cnn_amd.so3_real import so3_rft_real
+    for b, grid, shape in ((32, s2cnn_amd.so3_near_identity_grid(), (8, 12)), (7, s2cnn_amd.so3_equatorial_grid(n_alpha=8), (4, 5)),
+                           (6, ((0, 0, 0),), (2, 2))):
+        g = torch.Generator().manual_seed(b)
+        x = torch.randn(*shape, len(grid), generator=g).cuda().requires_grad_()
+        w = None
+        res = {}
+        for flag in (True, False):
+            so3_rft_real.factorised = flag
+            y = so3_rft_real(x, b, grid)
+            if w is None:
+                w = torch.randn(y.shape, generator=g).cuda()
+            (gx,) = torch.autograd.grad(y, x, w)
+            res[flag] = (y.detach(), gx)
+        so3_rft_real.factorised = True
+        for got, want in zip(res[True], res[False]):
+            assert got.shape == want.shape
+            assert (got - want).abs().max().item() < 2e-5 * want.abs().max().item(), (b, (got - want).abs().max().item(), want.abs().max().item())
