@@ -190,7 +190,7 @@ def test_s2_transforms(hip, b_in, b_out, for_grad):
 
 
 def test_so3_integrate(hip):
-    for b in (1, 3, 6, 16):
+    for b in (1, 3, 6, 16, 32):                     # 32: the 16-byte-load path (planes of 4096 samples)
         x = rnd((2, 5, 2 * b, 2 * b, 2 * b), 40 + b)
         xg = x.cuda().requires_grad_()
         out = s2cnn_amd.so3_integrate(xg)
