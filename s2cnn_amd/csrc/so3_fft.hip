@@ -20,6 +20,7 @@
 #include "so3_plane_fft64.h"
 #include "so3_wigner_tiled.h"
 #include "so3_fused64.h"
+#include "so3_plane_dft_real.h"
 
 namespace {
 
@@ -430,10 +431,11 @@ extern "C" int s2cnn_so3_analysis(const float* x, const float* table, const floa
   const int MW = 2 * nb - 1, NW = complex_in ? MW : nb;
   float2* X = static_cast<float2*>(workspace);
   const size_t lds = sizeof(float) * (2 * n2 + (complex_in ? 2 : 1) * n2 * n2 + 2 * n2 * NW);
-  if (lds > 160 * 1024) return S2CNN_EINVAL;
   const unsigned planes = (unsigned)(nbatch * n2);
   const bool tiled = packed_bytes(b_in, b_out, complex_in, false) != 0;
   const bool x16 = s2cnn::aligned16(x);
+  const plane_real::Plan plan = complex_in ? plane_real::Plan{0, 0, 0, 0} : plane_real::plan_fwd(n2, nb, planes);
+  if (lds > 160 * 1024 && plan.pl == 0) return S2CNN_EINVAL;
   if (complex_in) {
     if (lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)so3_plane_dft_fwd<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     hipLaunchKernelGGL(so3_plane_dft_fwd<true>, dim3(planes), dim3(256), lds, st, x, X, n2, nb, 0);
@@ -441,6 +443,10 @@ extern "C" int s2cnn_so3_analysis(const float* x, const float* table, const floa
     const long npairs = nbatch * 32;
     hipLaunchKernelGGL(fft64::plane_fft64_fwd, dim3((unsigned)(npairs < 2048 ? npairs : 2048)), dim3(fft64::THREADS), 0, st, x, X, npairs, nb,
                        tiled ? wigner_tiled::ZT : 0);
+  } else if (plan.pl > 0) {
+    if (plan.lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)plane_real::plane_dft_fwd, hipFuncAttributeMaxDynamicSharedMemorySize, (int)plan.lds);
+    hipLaunchKernelGGL(plane_real::plane_dft_fwd, dim3((planes + plan.pl - 1) / plan.pl), dim3(plan.nt), plan.lds, st, x, X, n2, nb,
+                       tiled ? wigner_tiled::ZT : 0, (long)planes, plan.pl, plan.alias);
   } else {
     if (lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)so3_plane_dft_fwd<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     hipLaunchKernelGGL(so3_plane_dft_fwd<false>, dim3(planes), dim3(256), lds, st, x, X, n2, nb, tiled ? wigner_tiled::ZT : 0);
@@ -485,7 +491,8 @@ extern "C" int s2cnn_so3_synthesis(const float* xhat, const float* table, const 
   const int MW = 2 * nb - 1, NW = complex_out ? MW : nb;
   float2* S = static_cast<float2*>(workspace);
   const size_t lds = sizeof(float2) * (n2 + MW * NW + n2 * NW);
-  if (lds > 160 * 1024) return S2CNN_EINVAL;
+  const plane_real::Plan plan = complex_out ? plane_real::Plan{0, 0, 0, 0} : plane_real::plan_inv(n2, nb, nbatch * n2);
+  if (lds > 160 * 1024 && plan.pl == 0) return S2CNN_EINVAL;
   dim3 grid(s2cnn::ceil_div(NW, 16), MW, (unsigned)((nbatch + 15) / 16));
   const float2* xh = reinterpret_cast<const float2*>(xhat);
   const bool tiled = packed_bytes(b_out, b_in, complex_out, true) != 0;
@@ -512,6 +519,10 @@ extern "C" int s2cnn_so3_synthesis(const float* xhat, const float* table, const 
   } else if (n2 == 64 && s2cnn::aligned16(out)) {
     const long npairs = nbatch * 32;
     hipLaunchKernelGGL(fft64::plane_fft64_inv, dim3((unsigned)(npairs < 2048 ? npairs : 2048)), dim3(fft64::THREADS), 0, st, S, out, npairs, nb);
+  } else if (plan.pl > 0) {
+    if (plan.lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)plane_real::plane_dft_inv, hipFuncAttributeMaxDynamicSharedMemorySize, (int)plan.lds);
+    hipLaunchKernelGGL(plane_real::plane_dft_inv, dim3((planes + plan.pl - 1) / plan.pl), dim3(plan.nt), plan.lds, st, S, out, n2, nb,
+                       (long)planes, plan.pl, plan.alias);
   } else {
     if (lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)so3_plane_dft_inv<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     hipLaunchKernelGGL(so3_plane_dft_inv<false>, dim3(planes), dim3(256), lds, st, S, out, n2, nb);

@@ -1,0 +1,436 @@
+// (alpha, gamma) transform of the planes of REAL signals for any grid size: a DFT pruned to the
+// frequencies |m|, n < nb, folded over both mirror symmetries of the trigonometric matrix and
+// register-blocked so that the inner loops are fused multiply-adds fed by 16-byte LDS reads.
+//
+// With h = n2/2, c[jk] = cos(2 pi j k / n2) and s[jk] = sin(2 pi j k / n2):
+//
+//   analysis   X[m][n] = sum_{a,g} x[a][g] e^{-i(m a + n g) 2 pi / n2}
+//     gamma:   E[a][g] = x[a][g] + x[a][n2-g],  O[a][g] = x[a][g] - x[a][n2-g]   (g = 0 and g = h stand alone)
+//              Y[a][n] = sum_{g<=h} E[a][g] c[gn]  -  i sum_{g<=h} O[a][g] s[gn]
+//     alpha:   Ye[a] = Y[a] + Y[n2-a],  Yo[a] = Y[a] - Y[n2-a]                      (a = 0 and a = h stand alone)
+//              P[m][n] = sum_{a<=h} Ye[a][n] c[am],   Q[m][n] = sum_{a<=h} Yo[a][n] s[am]
+//              X[+m] = P - iQ,  X[-m] = P + iQ
+//
+//   synthesis  y[a][g] = sum_n w_n Re( U[a][n] e^{+i n g 2 pi / n2} ),  U[a][n] = sum_m S[m][n] e^{+i m a 2 pi / n2},
+//              w_0 = 1, w_n = 2 (the half plane n >= 0 of a Hermitian spectrum)
+//     alpha:   A[m] = S[m] + S[-m],  B[m] = i (S[m] - S[-m])  (A[0] = S[0], B[0] = 0)
+//              Uc[a][n] = sum_m A[m][n] c[ma],  Us[a][n] = sum_m B[m][n] s[ma];   U[a] = Uc + Us,  U[n2-a] = Uc - Us
+//     gamma:   for the row pair (a, n2-a) and g <= h four sums over n,
+//              CC = w Re Uc c[ng], SC = w Re Us c[ng], CS = w Im Uc s[ng], SS = w Im Us s[ng], give
+//              y[a][g] = (CC+SC) - (CS+SS),        y[a][n2-g] = (CC+SC) + (CS+SS),
+//              y[n2-a][g] = (CC-SC) - (CS-SS),     y[n2-a][n2-g] = (CC-SC) + (CS-SS).
+//
+// A workgroup takes PL planes at once (small planes have too few 4x4 register blocks to fill it otherwise);
+// every thread owns 32 accumulators and reads four 16-byte LDS words per 32 FMAs.  When one round of the
+// workgroup covers all blocks of its planes, the output of each pass overwrites its input (after a barrier,
+// out of the accumulators): half the LDS per plane and twice the workgroups per CU, and the planes of the
+// synthesis leave the LDS as one contiguous run of 16-byte stores instead of four-byte scatters.
+#pragma once
+#include <hip/hip_runtime.h>
+
+namespace plane_real {
+
+constexpr int NT_MAX = 1024;
+constexpr int PL_MAX = 64;                  // planes per workgroup
+constexpr unsigned LDS_SOFT = 32 * 1024;    // five workgroups per CU when the planes allow it
+constexpr unsigned LDS_HARD = 160 * 1024;
+
+__host__ __device__ inline int pad(int v, int q) { return (v + q - 1) / q * q; }
+
+struct Plan {
+  int pl;         // planes per workgroup; 0: the plane does not fit the LDS
+  int nt;         // threads per workgroup
+  int alias;      // the first pass writes over its input
+  unsigned lds;   // bytes of dynamic LDS
+};
+
+// analysis: table [h+1][nbp] float2 | per plane: EO [h+1][ns] float2, Yf [h+1][nbp] float4
+// synthesis: table [nb][hp] float2  | per plane: AB [nb][nb2] float4, UU [nb][npp] float4
+inline Plan make_plan(unsigned table_bytes, unsigned in_bytes, unsigned mid_bytes, unsigned out_bytes, int items1, int items2,
+                      long nplanes) {
+  Plan p{0, 0, 0, 0};
+  const int items = items1 > items2 ? items1 : items2;
+  p.nt = items <= 256 ? 256 : items <= 512 ? 512 : NT_MAX;
+  p.alias = items <= p.nt;     // one round per pass: folded input, intermediate and staged output share one region
+  unsigned plane_bytes = in_bytes + mid_bytes;
+  if (p.alias) {
+    plane_bytes = in_bytes > mid_bytes ? in_bytes : mid_bytes;
+    if (out_bytes > plane_bytes) plane_bytes = out_bytes;
+    plane_bytes = (plane_bytes + 15u) & ~15u;
+  }
+  if (table_bytes + plane_bytes > LDS_HARD) return p;
+  int pl = p.nt / (items > 0 ? items : 1);
+  if (pl < 1) pl = 1;
+  if (table_bytes + plane_bytes > LDS_SOFT) pl = 1;
+  else if (table_bytes + (unsigned long)pl * plane_bytes > LDS_SOFT) pl = (int)((LDS_SOFT - table_bytes) / plane_bytes);
+  if (pl > nplanes) pl = (int)nplanes;
+  if (pl > PL_MAX) pl = PL_MAX;
+  // among the counts that fit, the one that fills its wavefronts best (the larger on a tie)
+  int best = 1;
+  float best_fill = 0.f;
+  for (int c = 1; c <= pl; ++c) {
+    const float fill = (float)(c * items) / (float)(64 * ((c * items + 63) / 64));
+    if (fill >= best_fill) { best_fill = fill; best = c; }
+  }
+  pl = best;
+  p.pl = pl;
+  p.lds = table_bytes + (unsigned)pl * plane_bytes;
+  return p;
+}
+
+inline Plan plan_fwd(int n2, int nb, long nplanes) {
+  const int hg = n2 / 2 + 1, ns = pad(n2, 4), nbp = pad(nb, 4);
+  return make_plan(hg * nbp * 8, hg * ns * 8, hg * nbp * 16, 0, ns / 4 * (nbp / 4), nbp / 4 * (nbp / 2), nplanes);
+}
+
+inline Plan plan_inv(int n2, int nb, long nplanes) {
+  const int hp = pad(n2 / 2 + 1, 4), npp = pad(n2 / 2 + 1, 2), nb2 = pad(nb, 2);
+  return make_plan(nb * hp * 8, nb * nb2 * 16, nb * npp * 16, n2 * n2 * 4, hp / 4 * (nb2 / 2), npp / 2 * (hp / 4), nplanes);
+}
+
+__device__ __forceinline__ float2 cs_entry(int j, int k, int n2) {
+  float s, c;
+  sincospif(2.0f * (float)((j * k) % n2) / (float)n2, &s, &c);
+  return make_float2(c, s);
+}
+
+struct F2x4 { float2 v[4]; };
+
+constexpr int LOADS = 8;   // global loads a thread has in flight while it stages planes
+
+// e -> (row, col) = (e / w, e % w) for e = e0, e0 + stride, e0 + 2 stride, ... without a division per step
+struct Walk2 {
+  int row, col, drow, dcol, w;
+  __device__ __forceinline__ void init(int e0, int stride, int width) {
+    w = width; row = e0 / w; col = e0 - row * w; drow = stride / w; dcol = stride - drow * w;
+  }
+  __device__ __forceinline__ void step() {
+    row += drow; col += dcol;
+    if (col >= w) { col -= w; ++row; }
+  }
+};
+
+__device__ __forceinline__ F2x4 lds_read_f2x4(const float2* p) {
+  const float4 lo = reinterpret_cast<const float4*>(p)[0], hi = reinterpret_cast<const float4*>(p)[1];
+  F2x4 r;
+  r.v[0] = make_float2(lo.x, lo.y); r.v[1] = make_float2(lo.z, lo.w);
+  r.v[2] = make_float2(hi.x, hi.y); r.v[3] = make_float2(hi.z, hi.w);
+  return r;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// analysis: x [nplanes][n2][n2] -> X, laid out [plane][mi][ni] (ztile = 0) or
+// [z / Z][mi][beta][z % Z][ni] (ztile = Z, plane = z n2 + beta); mi = m + nb-1, ni = n.
+// ---------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(NT_MAX) void plane_dft_fwd(const float* __restrict__ x, float2* __restrict__ X, int n2, int nb,
+                                                        int ztile, long nplanes, int PL, int alias) {
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  const int h = n2 / 2, nbp = pad(nb, 4), ns = pad(n2, 4);
+  float2* tab = reinterpret_cast<float2*>(smem);                      // [h+1][nbp]
+  float2* EO = tab + (h + 1) * nbp;                                   // [PL][h+1][ns]
+  float4* Yf = reinterpret_cast<float4*>(alias ? EO : EO + (size_t)PL * (h + 1) * ns);   // [PL][h+1][nbp]
+  const long plane0 = (long)blockIdx.x * PL;
+  const int t = threadIdx.x, NT = blockDim.x;
+
+  for (int i = t; i < (h + 1) * nbp; i += NT) {
+    const int j = i / nbp, k = i - j * nbp;
+    tab[i] = k < nb ? cs_entry(j, k, n2) : make_float2(0.f, 0.f);
+  }
+  // fold gamma; rows go to slots so that the pair (a, n2-a) is adjacent: 0 -> 0, h -> 1, a -> 2a, n2-a -> 2a+1.
+  // The planes of a workgroup are one contiguous run of rows; LOADS of them are issued before the first is used.
+  {
+    const int hg = h + 1, total = PL * n2 * hg;
+    const long rows_valid = (nplanes - plane0) * n2;
+    const float* src = x + (size_t)plane0 * n2 * n2;
+    const float inv_n2 = 1.0f / (float)n2;
+    Walk2 wk;
+    wk.init(t, NT, hg);
+    for (int e = t; e < total; e += LOADS * NT) {
+      float v1[LOADS], v2[LOADS];
+      int dst[LOADS];
+      unsigned pmask = 0;
+#pragma unroll
+      for (int u = 0; u < LOADS; ++u) {
+        const int R = wk.row, g = wk.col;
+        const bool live = e + u * NT < total;
+        const bool valid = live && R < rows_valid;
+        const bool paired = g > 0 && g < h;
+        const int o1 = valid ? R * n2 + g : 0;
+        v1[u] = src[o1];
+        v2[u] = src[valid && paired ? R * n2 + n2 - g : o1];
+        if (!valid) v1[u] = v2[u] = 0.f;
+        if (!paired) v2[u] = 0.f;
+        else pmask |= 1u << u;
+        const int q = (int)(((float)R + 0.5f) * inv_n2), a = R - q * n2;
+        const int slot = a == 0 ? 0 : a == h ? 1 : a < h ? 2 * a : 2 * (n2 - a) + 1;
+        dst[u] = live ? (q * hg + g) * ns + slot : -1;
+        wk.step();
+      }
+#pragma unroll
+      for (int u = 0; u < LOADS; ++u)
+        if (dst[u] >= 0) EO[dst[u]] = make_float2(v1[u] + v2[u], (pmask >> u) & 1u ? v1[u] - v2[u] : 0.f);
+    }
+    if (ns > n2)   // n2 = 2 mod 4: two empty slots
+      for (int i = t; i < PL * hg * (ns - n2); i += NT) EO[(i / (ns - n2)) * ns + n2 + i % (ns - n2)] = make_float2(0.f, 0.f);
+  }
+  __syncthreads();
+
+  // gamma pass: 4 row slots x 4 frequencies per thread
+  const int nkb = nbp / 4, i1 = ns / 4 * nkb;
+  for (int it = t; it - t < PL * i1; it += NT) {      // the same number of rounds for every thread
+    const bool active = it < PL * i1;
+    const int q = it / i1, r = it - q * i1;
+    const int sb = r / nkb, kb = r - sb * nkb;
+    const float2* eo = EO + (size_t)q * (h + 1) * ns + 4 * sb;
+    const float2* tb = tab + 4 * kb;
+    float yr[4][4], yi[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int k = 0; k < 4; ++k) yr[i][k] = yi[i][k] = 0.f;
+    if (active)
+      for (int g = 0; g <= h; ++g) {
+        const F2x4 e = lds_read_f2x4(eo + g * ns), w = lds_read_f2x4(tb + g * nbp);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            yr[i][k] = fmaf(e.v[i].x, w.v[k].x, yr[i][k]);
+            yi[i][k] = fmaf(e.v[i].y, w.v[k].y, yi[i][k]);
+          }
+      }
+    if (alias) __syncthreads();                        // one round only: every read of EO is done
+    float4* yf = Yf + (size_t)q * (h + 1) * nbp + 4 * kb;
+#pragma unroll
+    for (int pi = 0; pi < 2; ++pi) {
+      const int p = 2 * sb + pi;
+      if (p >= h || !active) continue;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const float r1 = yr[2 * pi][k], m1 = -yi[2 * pi][k], r2 = yr[2 * pi + 1][k], m2 = -yi[2 * pi + 1][k];
+        if (p == 0) {
+          yf[k] = make_float4(r1, m1, 0.f, 0.f);
+          yf[h * nbp + k] = make_float4(r2, m2, 0.f, 0.f);
+        } else {
+          yf[p * nbp + k] = make_float4(r1 + r2, m1 + m2, r1 - r2, m1 - m2);
+        }
+      }
+    }
+  }
+  __syncthreads();
+
+  // alpha pass: 4 frequencies m >= 0 x 2 frequencies n per thread
+  const int nnb = nbp / 2, i2 = nkb * nnb;
+  // X leaves straight from the accumulators: its rows lie far apart in the tiled layout, staging them does not pay
+  for (int it = t; it < PL * i2; it += NT) {
+    const int q = it / i2, r = it - q * i2;
+    const int mb = r / nnb, nk = r - mb * nnb;
+    const long pl = plane0 + q;
+    const float4* yf = Yf + (size_t)q * (h + 1) * nbp + 2 * nk;
+    const float2* tb = tab + 4 * mb;
+    float pr[4][2], pi_[4][2], qr[4][2], qi[4][2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int k = 0; k < 2; ++k) pr[i][k] = pi_[i][k] = qr[i][k] = qi[i][k] = 0.f;
+    for (int a = 0; a <= h; ++a) {
+      const float4 y0 = yf[a * nbp], y1 = yf[a * nbp + 1];
+      const F2x4 w = lds_read_f2x4(tb + a * nbp);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        pr[i][0] = fmaf(y0.x, w.v[i].x, pr[i][0]); pi_[i][0] = fmaf(y0.y, w.v[i].x, pi_[i][0]);
+        qr[i][0] = fmaf(y0.z, w.v[i].y, qr[i][0]); qi[i][0] = fmaf(y0.w, w.v[i].y, qi[i][0]);
+        pr[i][1] = fmaf(y1.x, w.v[i].x, pr[i][1]); pi_[i][1] = fmaf(y1.y, w.v[i].x, pi_[i][1]);
+        qr[i][1] = fmaf(y1.z, w.v[i].y, qr[i][1]); qi[i][1] = fmaf(y1.w, w.v[i].y, qi[i][1]);
+      }
+    }
+    if (pl >= nplanes) continue;
+    float2* dst = X + (size_t)pl * ((2 * nb - 1) * nb);
+    size_t mstride = nb;
+    if (ztile > 0) {
+      const size_t z = pl / n2, beta = pl % n2;
+      dst = X + ((z / ztile) * (2 * nb - 1) * n2 + beta) * ztile * nb + (z % ztile) * nb;
+      mstride = (size_t)n2 * ztile * nb;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = 4 * mb + i;
+      if (m >= nb) continue;
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+        const int n = 2 * nk + k;
+        if (n >= nb) continue;
+        dst[(size_t)(nb - 1 + m) * mstride + n] = make_float2(pr[i][k] + qi[i][k], pi_[i][k] - qr[i][k]);
+        if (m > 0) dst[(size_t)(nb - 1 - m) * mstride + n] = make_float2(pr[i][k] - qi[i][k], pi_[i][k] + qr[i][k]);
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// synthesis: S [nplanes][2nb-1][nb] -> y [nplanes][n2][n2]
+// ---------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(NT_MAX) void plane_dft_inv(const float2* __restrict__ S, float* __restrict__ y, int n2, int nb,
+                                                        long nplanes, int PL, int alias) {
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  const int h = n2 / 2, hp = pad(h + 1, 4), nb2 = pad(nb, 2), npp = pad(h + 1, 2);
+  float2* tab = reinterpret_cast<float2*>(smem);                          // [nb][hp]
+  float4* AB = reinterpret_cast<float4*>(tab + nb * hp);                  // [PL][nb][nb2]
+  float4* UU = alias ? AB : AB + (size_t)PL * nb * nb2;                   // [PL][nb][npp]
+  const long plane0 = (long)blockIdx.x * PL;
+  const int t = threadIdx.x, NT = blockDim.x;
+
+  for (int i = t; i < nb * hp; i += NT) {
+    const int k = i / hp, j = i - k * hp;
+    tab[i] = j <= h ? cs_entry(j, k, n2) : make_float2(0.f, 0.f);
+  }
+  // A, B from the rows +m and -m of S; LOADS pairs of rows are in flight per thread
+  {
+    const int total = PL * nb * nb2, srow = (2 * nb - 1) * nb;
+    const float2* src = S + (size_t)plane0 * srow;
+    const long planes_valid = nplanes - plane0;
+    const float inv_nb = 1.0f / (float)nb;
+    Walk2 wk;
+    wk.init(t, NT, nb2);
+    for (int e = t; e < total; e += LOADS * NT) {
+      float2 sp[LOADS], sm[LOADS];
+      unsigned keep = 0, both = 0;
+#pragma unroll
+      for (int u = 0; u < LOADS; ++u) {
+        const int R = wk.row, n = wk.col;                      // R = q nb + m
+        const int q = (int)(((float)R + 0.5f) * inv_nb), m = R - q * nb;
+        const bool live = e + u * NT < total;
+        const bool valid = live && n < nb && q < planes_valid;
+        const int o1 = valid ? q * srow + (nb - 1 + m) * nb + n : 0;
+        sp[u] = src[o1];
+        sm[u] = src[valid ? q * srow + (nb - 1 - m) * nb + n : 0];
+        if (valid) keep |= 1u << u;
+        if (m > 0) both |= 1u << u;
+        wk.step();
+      }
+#pragma unroll
+      for (int u = 0; u < LOADS; ++u) {
+        const int i = e + u * NT;
+        if (i >= total) continue;
+        float4 ab = make_float4(0.f, 0.f, 0.f, 0.f);
+        if ((keep >> u) & 1u)
+          ab = (both >> u) & 1u ? make_float4(sp[u].x + sm[u].x, sp[u].y + sm[u].y, sm[u].y - sp[u].y, sp[u].x - sm[u].x)
+                                : make_float4(sp[u].x, sp[u].y, 0.f, 0.f);
+        AB[i] = ab;
+      }
+    }
+  }
+  __syncthreads();
+
+  // alpha pass: 4 angles a <= h x 2 frequencies n per thread
+  const int njb = hp / 4, nnb = nb2 / 2, i1 = njb * nnb;
+  for (int it = t; it - t < PL * i1; it += NT) {      // the same number of rounds for every thread
+    const bool active = it < PL * i1;
+    const int q = it / i1, r = it - q * i1;
+    const int jb = r / nnb, nk = r - jb * nnb;
+    const float4* ab = AB + (size_t)q * nb * nb2 + 2 * nk;
+    const float2* tb = tab + 4 * jb;
+    float cr[4][2], ci[4][2], sr[4][2], si[4][2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int k = 0; k < 2; ++k) cr[i][k] = ci[i][k] = sr[i][k] = si[i][k] = 0.f;
+    for (int m = 0; m < (active ? nb : 0); ++m) {
+      const float4 a0 = ab[m * nb2], a1 = ab[m * nb2 + 1];
+      const F2x4 w = lds_read_f2x4(tb + m * hp);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        cr[i][0] = fmaf(a0.x, w.v[i].x, cr[i][0]); ci[i][0] = fmaf(a0.y, w.v[i].x, ci[i][0]);
+        sr[i][0] = fmaf(a0.z, w.v[i].y, sr[i][0]); si[i][0] = fmaf(a0.w, w.v[i].y, si[i][0]);
+        cr[i][1] = fmaf(a1.x, w.v[i].x, cr[i][1]); ci[i][1] = fmaf(a1.y, w.v[i].x, ci[i][1]);
+        sr[i][1] = fmaf(a1.z, w.v[i].y, sr[i][1]); si[i][1] = fmaf(a1.w, w.v[i].y, si[i][1]);
+      }
+    }
+    if (alias) __syncthreads();                        // one round only: every read of AB is done
+    float4* uu = UU + (size_t)q * nb * npp;
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const int n = 2 * nk + k;
+      if (n >= nb || !active) continue;
+      const float wn = n == 0 ? 1.f : 2.f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int a = 4 * jb + i;
+        if (a < npp) uu[n * npp + a] = make_float4(wn * cr[i][k], wn * ci[i][k], wn * sr[i][k], wn * si[i][k]);
+      }
+    }
+  }
+  __syncthreads();
+
+  // gamma pass: 2 row pairs (a, n2-a) x 4 angles g <= h per thread
+  const int npb = npp / 2, i2 = npb * njb;
+  float* Ys = reinterpret_cast<float*>(AB);            // staged mode: the planes of y
+  for (int it = t; it - t < PL * i2; it += NT) {
+    const bool active = it < PL * i2;
+    const int q = it / i2, r = it - q * i2;
+    const int pb = r / njb, gb = r - pb * njb;
+    const long pl = plane0 + q;
+    const float4* uu = UU + (size_t)q * nb * npp + 2 * pb;
+    const float2* tb = tab + 4 * gb;
+    float cc[2][4], sc[2][4], cs[2][4], ss[2][4];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int k = 0; k < 4; ++k) cc[i][k] = sc[i][k] = cs[i][k] = ss[i][k] = 0.f;
+    for (int n = 0; n < (active ? nb : 0); ++n) {
+      const float4 u0 = uu[n * npp], u1 = uu[n * npp + 1];
+      const F2x4 w = lds_read_f2x4(tb + n * hp);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        cc[0][k] = fmaf(u0.x, w.v[k].x, cc[0][k]); cs[0][k] = fmaf(u0.y, w.v[k].y, cs[0][k]);
+        sc[0][k] = fmaf(u0.z, w.v[k].x, sc[0][k]); ss[0][k] = fmaf(u0.w, w.v[k].y, ss[0][k]);
+        cc[1][k] = fmaf(u1.x, w.v[k].x, cc[1][k]); cs[1][k] = fmaf(u1.y, w.v[k].y, cs[1][k]);
+        sc[1][k] = fmaf(u1.z, w.v[k].x, sc[1][k]); ss[1][k] = fmaf(u1.w, w.v[k].y, ss[1][k]);
+      }
+    }
+    // staged mode (one round): y goes to LDS over the consumed spectra and leaves as one contiguous run below
+    float* dst;
+    if (alias) {
+      __syncthreads();
+      dst = Ys + (size_t)q * n2 * n2;
+    } else {
+      dst = y + (size_t)pl * n2 * n2;
+    }
+    if (!active || (!alias && pl >= nplanes)) continue;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int a = 2 * pb + i;
+      if (a > h) continue;
+      const bool mirror_a = a > 0 && a < h;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const int g = 4 * gb + k;
+        if (g > h) continue;
+        const bool mirror_g = g > 0 && g < h;
+        const float yc = cc[i][k] + sc[i][k], ys = cs[i][k] + ss[i][k];
+        dst[a * n2 + g] = yc - ys;
+        if (mirror_g) dst[a * n2 + n2 - g] = yc + ys;
+        if (mirror_a) {
+          const float zc = cc[i][k] - sc[i][k], zs = cs[i][k] - ss[i][k];
+          dst[(n2 - a) * n2 + g] = zc - zs;
+          if (mirror_g) dst[(n2 - a) * n2 + n2 - g] = zc + zs;
+        }
+      }
+    }
+  }
+  if (!alias) return;
+  __syncthreads();
+  {
+    long pv = nplanes - plane0;
+    if (pv > PL) pv = PL;
+    const int total = (int)pv * n2 * n2;                 // a multiple of 4
+    float* dst = y + (size_t)plane0 * n2 * n2;
+    if ((reinterpret_cast<uintptr_t>(y) & 15u) == 0) {
+      for (int i = t; i < total / 4; i += NT) reinterpret_cast<float4*>(dst)[i] = reinterpret_cast<const float4*>(Ys)[i];
+    } else {
+      for (int i = t; i < total; i += NT) dst[i] = Ys[i];
+    }
+  }
+}
+
+}  // namespace plane_real

@@ -392,3 +392,15 @@ def test_so3_mm_at_config3_features_linearity(hip):
         assert (got - want).abs().max().item() < 1e-4 * want.abs().std().item(), l
     z2 = s2cnn_amd.so3_mm(2 * x, y) - 2 * z
     assert z2.abs().max().item() < 1e-4 * z.std().item()
+
+
+@pytest.mark.parametrize("b_grid,b_spec,nz", [(22, 22, 2), (22, 7, 5), (40, 8, 1), (5, 5, 60), (1, 1, 300)])
+def test_so3_real_transforms_on_other_grids(hip, b_grid, b_spec, nz):
+    """Real signals on grids other than 64^3: the folded plane transform takes several planes per workgroup
+    (ragged last workgroup included) or one large plane; analysis truncates, synthesis zero-extends."""
+    print(f"so3 real transforms b_grid={b_grid} b_spec={b_spec} nz={nz}", flush=True)
+    x = rnd((nz, 2 * b_grid, 2 * b_grid, 2 * b_grid), 70)
+    for for_grad in (False, True):
+        close(PSO3.so3_rfft(x.cuda(), for_grad, b_spec), O.so3_rfft(x.double(), for_grad, b_spec), "so3_rfft")
+        s = rnd((O.nspec_so3(b_spec), nz, 2), 71)
+        close(PSO3.so3_rifft(s.cuda(), for_grad, b_grid), O.so3_rifft(s.double(), for_grad, b_grid), "so3_rifft")
