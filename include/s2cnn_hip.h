@@ -158,6 +158,15 @@ size_t s2cnn_so3_synthesis_workspace(int b_in, int b_out, long nbatch, int compl
 int s2cnn_so3_synthesis(const float *xhat, const float *table, const float *packed_table, float *out,
                         void *workspace, size_t workspace_bytes,
                         int b_in, int b_out, long nbatch, int complex_out, void *stream);
+/* The same with complex_out = 0 and a bias in the epilogue: bias has nfeature values and, with the batch laid
+ * out [..., nfeature] (nbatch a multiple of nfeature), bias[z % nfeature] is added to every sample of volume z.
+ * Replaces SO3_ifft_real followed by "z + self.bias" (soft/s2_conv.py:50-53, soft/so3_conv.py:54-56) without
+ * the extra pass over the output.  bias = NULL gives s2cnn_so3_synthesis(..., complex_out = 0, ...).
+ */
+int s2cnn_so3_synthesis_real_bias(const float *xhat, const float *table, const float *packed_table, float *out,
+                                  void *workspace, size_t workspace_bytes,
+                                  int b_in, int b_out, long nbatch,
+                                  const float *bias, int nfeature, void *stream);
 
 /* ---- table repacking for the real-signal fast path of the two transforms above ------
  * The reference uploads its Wigner table once per (b, nl, weighted, device) and reuses it

@@ -280,6 +280,12 @@ __global__ __launch_bounds__(256) void so3_plane_dft_inv(const float2* __restric
   }
 }
 
+// y[z, :] += bias[z % nfeature] for volumes of `vol` samples (only behind the plane kernel above, which has no epilogue)
+__global__ void add_bias_kernel(float* __restrict__ y, const float* __restrict__ bias, size_t vol, int nfeature, size_t total) {
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x)
+    y[i] += bias[(i / vol) % nfeature];
+}
+
 // Real signals on the 64^3 grid go through the per-volume kernels of so3_fused64.h (the planes never leave the CU).
 bool fused_path(int b_grid, int b_spec, int cplx, bool synthesis) {
   return !cplx && b_grid == 32 && (synthesis || b_spec <= 32);
@@ -476,15 +482,17 @@ extern "C" int s2cnn_so3_analysis(const float* x, const float* table, const floa
   return s2cnn::launch_status();
 }
 
-extern "C" int s2cnn_so3_synthesis(const float* xhat, const float* table, const float* packed_table, float* out,
-                                   void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
-                                   int complex_out, void* stream) {
+namespace {
+int synthesis_impl(const float* xhat, const float* table, const float* packed_table, float* out, void* workspace,
+                   size_t workspace_bytes, int b_in, int b_out, long nbatch, int complex_out, const float* bias, int nfeature,
+                   void* stream) {
   if (!xhat || !table || !out || !sizes_ok(b_out, b_in, nbatch)) return S2CNN_EINVAL;
+  if (bias && (complex_out || nfeature < 1 || nbatch % nfeature != 0)) return S2CNN_EINVAL;
   if (!s2cnn::aligned8(xhat) || (complex_out && !s2cnn::aligned8(out))) return S2CNN_EALIGN;
   if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (fused_path(b_out, b_in, complex_out, true))
-    return fused_synthesis(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, nbatch, false, nullptr, 1, st);
+    return fused_synthesis(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, nbatch, false, bias, bias ? nfeature : 1, st);
   const size_t need = s2cnn_so3_synthesis_workspace(b_in, b_out, nbatch, complex_out);
   if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
   const int n2 = 2 * b_out, nb = b_in < b_out ? b_in : b_out;
@@ -522,10 +530,28 @@ extern "C" int s2cnn_so3_synthesis(const float* xhat, const float* table, const 
   } else if (plan.pl > 0) {
     if (plan.lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)plane_real::plane_dft_inv, hipFuncAttributeMaxDynamicSharedMemorySize, (int)plan.lds);
     hipLaunchKernelGGL(plane_real::plane_dft_inv, dim3((planes + plan.pl - 1) / plan.pl), dim3(plan.nt), plan.lds, st, S, out, n2, nb,
-                       (long)planes, plan.pl, plan.alias);
+                       (long)planes, plan.pl, plan.alias, bias, bias ? nfeature : 1);
+    return s2cnn::launch_status();
   } else {
     if (lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)so3_plane_dft_inv<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     hipLaunchKernelGGL(so3_plane_dft_inv<false>, dim3(planes), dim3(256), lds, st, S, out, n2, nb);
   }
+  if (bias) {
+    const size_t vol = (size_t)n2 * n2 * n2;
+    hipLaunchKernelGGL(add_bias_kernel, dim3(2048), dim3(256), 0, st, out, bias, vol, nfeature, vol * nbatch);
+  }
   return s2cnn::launch_status();
+}
+}  // namespace
+
+extern "C" int s2cnn_so3_synthesis(const float* xhat, const float* table, const float* packed_table, float* out,
+                                   void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
+                                   int complex_out, void* stream) {
+  return synthesis_impl(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, complex_out, nullptr, 1, stream);
+}
+
+extern "C" int s2cnn_so3_synthesis_real_bias(const float* xhat, const float* table, const float* packed_table, float* out,
+                                             void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
+                                             const float* bias, int nfeature, void* stream) {
+  return synthesis_impl(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, 0, bias, nfeature, stream);
 }

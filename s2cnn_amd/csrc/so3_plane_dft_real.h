@@ -270,8 +270,10 @@ __global__ __launch_bounds__(NT_MAX) void plane_dft_fwd(const float* __restrict_
 // ---------------------------------------------------------------------------------------------------
 // synthesis: S [nplanes][2nb-1][nb] -> y [nplanes][n2][n2]
 // ---------------------------------------------------------------------------------------------------
+// bias: NULL, or nfeature values; bias[z % nfeature] is added to every sample of volume z = plane / n2
 __global__ __launch_bounds__(NT_MAX) void plane_dft_inv(const float2* __restrict__ S, float* __restrict__ y, int n2, int nb,
-                                                        long nplanes, int PL, int alias) {
+                                                        long nplanes, int PL, int alias, const float* __restrict__ bias,
+                                                        int nfeature) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
   const int h = n2 / 2, hp = pad(h + 1, 4), nb2 = pad(nb, 2), npp = pad(h + 1, 2);
   float2* tab = reinterpret_cast<float2*>(smem);                          // [nb][hp]
@@ -396,7 +398,8 @@ __global__ __launch_bounds__(NT_MAX) void plane_dft_inv(const float2* __restrict
     } else {
       dst = y + (size_t)pl * n2 * n2;
     }
-    if (!active || (!alias && pl >= nplanes)) continue;
+    if (!active || pl >= nplanes) continue;
+    const float bz = bias ? bias[(int)(pl / n2) % nfeature] : 0.f;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int a = 2 * pb + i;
@@ -407,6 +410,7 @@ __global__ __launch_bounds__(NT_MAX) void plane_dft_inv(const float2* __restrict
         const int g = 4 * gb + k;
         if (g > h) continue;
         const bool mirror_g = g > 0 && g < h;
+        cc[i][k] += bz;
         const float yc = cc[i][k] + sc[i][k], ys = cs[i][k] + ss[i][k];
         dst[a * n2 + g] = yc - ys;
         if (mirror_g) dst[a * n2 + n2 - g] = yc + ys;

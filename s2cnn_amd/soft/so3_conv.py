@@ -63,8 +63,7 @@ class SO3Convolution(Module):
         assert z.size(0) == x.size(0)
         assert z.size(1) == x.size(1)
         assert z.size(2) == y.size(2)
-        z = SO3_ifft_real.apply(z)  # [batch, feature_out, beta, alpha, gamma]
-        return z + self.bias
+        return SO3_ifft_real.apply(z, None, self.bias)  # [batch, feature_out, beta, alpha, gamma], bias added in the transform
 
 
 class SO3Shortcut(Module):

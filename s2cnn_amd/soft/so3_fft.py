@@ -57,7 +57,7 @@ def _analysis(x, b_in, b_out, batch_size, for_grad, complex_in):
     return out
 
 
-def _synthesis(x, b_in, b_out, batch_size, for_grad, complex_out):
+def _synthesis(x, b_in, b_out, batch_size, for_grad, complex_out, bias=None):
     _hip.require_gpu_f32(x)
     L = _hip.lib()
     nbatch = 1
@@ -68,6 +68,14 @@ def _synthesis(x, b_in, b_out, batch_size, for_grad, complex_out):
     shape = (*batch_size, 2 * b_out, 2 * b_out, 2 * b_out) + ((2,) if complex_out else ())
     out = x.new_empty(shape)
     ws = _hip.workspace(L.s2cnn_so3_synthesis_workspace(b_in, b_out, nbatch, complex_out), x.device)
+    if bias is not None:
+        assert not complex_out
+        _hip.require_gpu_f32(bias)
+        bias = bias.reshape(-1).contiguous()
+        assert len(batch_size) >= 1 and batch_size[-1] == bias.numel()
+        _hip.call("s2cnn_so3_synthesis_real_bias", _hip.ptr(x), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out), _hip.ptr(ws),
+                  ws.numel(), b_in, b_out, nbatch, _hip.ptr(bias), bias.numel(), _hip.stream_ptr())
+        return out
     _hip.call("s2cnn_so3_synthesis", _hip.ptr(x), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out), _hip.ptr(ws), ws.numel(),
                   b_in, b_out, nbatch, complex_out, _hip.stream_ptr())
     return out
@@ -124,13 +132,14 @@ def so3_ifft(x, for_grad=False, b_out=None):
     return _synthesis(x, b_in, b_out, batch_size, for_grad, 1)
 
 
-def so3_rifft(x, for_grad=False, b_out=None):
+def so3_rifft(x, for_grad=False, b_out=None, bias=None):
     '''
     :param x: [l * m * n, ..., complex]
+    :param bias: None, or one value per entry of the last batch dimension, added to every sample of its volumes
     :return: [..., beta, alpha, gamma]  (the real part of so3_ifft, whatever the symmetry of x)
     '''
     x, b_in, b_out, batch_size = _spectrum_args(x, b_out)
-    return _synthesis(x, b_in, b_out, batch_size, for_grad, 0)
+    return _synthesis(x, b_in, b_out, batch_size, for_grad, 0, bias)
 
 
 class SO3_fft_real(torch.autograd.Function):
@@ -148,16 +157,25 @@ class SO3_fft_real(torch.autograd.Function):
 
 
 class SO3_ifft_real(torch.autograd.Function):
+    """s2cnn/soft/so3_fft.py:224-236, with the bias of the convolution layers as an optional third argument
+    (x [l * m * n, batch, feature, complex], bias with `feature` entries in any shape): it is added in the
+    epilogue of the transform, and its gradient is read off the degree-0 coefficient of the unweighted analysis
+    of grad_output, which IS the sum of grad_output over the grid."""
     @staticmethod
-    def forward(ctx, x, b_out=None):  # pylint: disable=W
+    def forward(ctx, x, b_out=None, bias=None):  # pylint: disable=W
         nspec = x.size(0)
         ctx.b_out = b_out
         ctx.b_in = round((3 / 4 * nspec) ** (1 / 3))
-        return so3_rifft(x, b_out=ctx.b_out)
+        ctx.bias_shape = None if bias is None else bias.shape
+        return so3_rifft(x, b_out=ctx.b_out, bias=bias)
 
     @staticmethod
     def backward(ctx, grad_output):  # pylint: disable=W
-        return so3_rfft(grad_output, for_grad=True, b_out=ctx.b_in), None
+        g = so3_rfft(grad_output, for_grad=True, b_out=ctx.b_in)
+        gb = None
+        if ctx.bias_shape is not None and ctx.needs_input_grad[2]:
+            gb = g[0, ..., 0].reshape(-1, g.size(-2)).sum(0).reshape(ctx.bias_shape)
+        return g, None, gb
 
 
 # ---------------------------------------------------------------------------------------------------
@@ -213,10 +231,7 @@ def so3_rifft_real_basis(r, for_grad=False, b_out=None, bias=None):
         b_out = b_in
     if not (r.is_cuda and _real_basis_direct(b_in, b_out, True)):
         from ..so3_real import _convert
-        out = so3_rifft(_convert("s2cnn_so3_spectrum_to_complex", r.contiguous(), (*r.shape, 2)), for_grad, b_out)
-        if bias is not None:
-            out.add_(bias.reshape(*([1] * (r.dim() - 2)), -1, 1, 1, 1))
-        return out
+        return so3_rifft(_convert("s2cnn_so3_spectrum_to_complex", r.contiguous(), (*r.shape, 2)), for_grad, b_out, bias)
     _hip.require_gpu_f32(r)
     r = r.contiguous()
     batch_size = r.size()[1:]

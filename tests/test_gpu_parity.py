@@ -404,3 +404,22 @@ def test_so3_real_transforms_on_other_grids(hip, b_grid, b_spec, nz):
         close(PSO3.so3_rfft(x.cuda(), for_grad, b_spec), O.so3_rfft(x.double(), for_grad, b_spec), "so3_rfft")
         s = rnd((O.nspec_so3(b_spec), nz, 2), 71)
         close(PSO3.so3_rifft(s.cuda(), for_grad, b_grid), O.so3_rifft(s.double(), for_grad, b_grid), "so3_rifft")
+
+
+@pytest.mark.parametrize("b_spec,b_grid", [(5, 7), (7, 22), (12, 32), (3, 2)])
+def test_so3_synthesis_with_bias(hip, b_spec, b_grid):
+    """The bias argument of so3_rifft / SO3_ifft_real (the "+ self.bias" of s2_conv.py:53 and so3_conv.py:56 inside the
+    transform): same values as the separate addition, and the gradients autograd gives for that addition."""
+    print(f"so3 synthesis with bias b_spec={b_spec} b_grid={b_grid}", flush=True)
+    from s2cnn_amd.soft.so3_fft import SO3_ifft_real
+    s = rnd((O.nspec_so3(b_spec), 3, 4, 2), 80).cuda().requires_grad_()
+    bias = rnd((1, 4, 1, 1, 1), 81).cuda().requires_grad_()
+    w = rnd((3, 4, 2 * b_grid, 2 * b_grid, 2 * b_grid), 82).cuda()
+    out = SO3_ifft_real.apply(s, b_grid, bias)
+    (out * w).sum().backward()
+    got = (out.detach(), s.grad.clone(), bias.grad.clone())
+    s.grad = bias.grad = None
+    ref = SO3_ifft_real.apply(s, b_grid) + bias
+    (ref * w).sum().backward()
+    for name, a, c in zip(("out", "grad spectrum", "grad bias"), got, (ref.detach(), s.grad, bias.grad)):
+        close(a, c.double().cpu(), name)
