@@ -67,7 +67,13 @@ template <> struct VecT<4> { typedef float4 type; };
 // takes the next TK values of it whatever the block size, so small blocks (a batch of 16 in grad y) fill
 // whole stages and odd block sizes pad only the very last stage.  load() fetches the current stage and
 // steps to the next one.
-template <bool KC, bool MNMAJ, int EXT, int VEC>
+//
+// FAST: the block size KI along the contraction and the stage length TK divide one another, so every stage
+// starts at the same position inside a block for every thread.  Then the per-thread offsets are fixed at
+// init, the stage advances by a wave-uniform step (scalar arithmetic), rows outside the matrix are clamped
+// to a valid row (their products land in accumulators that are never stored) and only a ragged LAST stage
+// (TK a multiple of KI, odd number of blocks) is masked: the loop body is loads and LDS writes, nothing else.
+template <bool KC, bool MNMAJ, int EXT, int VEC, bool FAST>
 struct TileLoader {
   static constexpr int NSLOT = EXT * TK / (NT * VEC);
   static constexpr int LD = TileShape<KC, EXT>::LD;
@@ -83,6 +89,23 @@ struct TileLoader {
   int blk_k_stride;
   int MNI, KI, L;
   vec_t reg[NSLOT];
+  // FAST only
+  unsigned foff[FAST ? NSLOT : 1];   // per-slot BYTE offset: row/column block, row inside it, position inside the stage
+  __amdgpu_buffer_rsrc_t rsrc;  // the operand of this degree as a buffer: scalar base, per-slot offsets in VGPRs
+  unsigned soff;                // uniform: byte offset of the current stage (scalar offset of the loads)
+  int sub, nsub, step_in, step_cross;
+  int stage_i, last_ragged;     // last_ragged: index of the one masked stage, or -1
+  unsigned tail_ok;             // bit q: slot q lies inside the matrix in that stage
+
+  typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+  static __device__ __forceinline__ vec_t buffer_load(__amdgpu_buffer_rsrc_t r, unsigned voff, unsigned so) {
+    if constexpr (VEC == 4) {
+      const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, (int)so, 0);
+      return make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
+    } else {
+      return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, (int)voff, (int)so, 0));
+    }
+  }
 
   __device__ void init(const float* base_l, int L_, int MNI_, int KI_, int tile0) {
     base = base_l; MNI = MNI_; KI = KI_; L = L_;
@@ -90,6 +113,46 @@ struct TileLoader {
     const int blk_elems = MNI * KI;
     const int blk_mn_stride = (MNMAJ ? L : 1) * blk_elems;
     blk_k_stride = (MNMAJ ? 1 : L) * blk_elems;
+    if (FAST) {
+      const int unit = KC ? 1 : MNI;                       // stride of one contraction step inside a block
+      const int K = L * KI, nstage = (K + TK - 1) / TK, ktail = K - (nstage - 1) * TK;
+      rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base_l), 0, 4 * L * L * MNI * KI, 0x00020000);
+      soff = 0; sub = 0; stage_i = 0;
+      if (KI >= TK) { nsub = KI / TK; step_in = TK * unit; step_cross = blk_k_stride - (KI - TK) * unit; }
+      else { nsub = 1; step_in = 0; step_cross = (TK / KI) * blk_k_stride; }
+      last_ragged = ktail < TK ? nstage - 1 : -1;
+      tail_ok = 0;
+      const int last = L * MNI - 1;
+      if (KC) {
+        constexpr int TPR = TK / VEC;
+        const int kk = (t % TPR) * VEC, r0 = t / TPR;
+        const int kbl = KI >= TK ? 0 : kk / KI, kin = kk - kbl * KI;
+        lds_off = r0 * LD + kk;
+#pragma unroll
+        for (int q = 0; q < NSLOT; ++q) {
+          int row = tile0 + r0 + q * (NT / TPR);
+          row = row > last ? last : row;
+          const int mb = row / MNI, mi = row - mb * MNI;
+          foff[q] = 4u * (unsigned)(mb * blk_mn_stride + mi * KI + kbl * blk_k_stride + kin);
+          if (kk < ktail) tail_ok |= 1u << q;
+        }
+      } else {
+        constexpr int TPR = EXT / VEC;
+        int mn = tile0 + (t % TPR) * VEC;
+        mn = mn > last ? 0 : mn;
+        const int kk = t / TPR;
+        lds_off = kk * LD + (t % TPR) * VEC;
+        const int mb = mn / MNI, mi = mn - mb * MNI;
+#pragma unroll
+        for (int q = 0; q < NSLOT; ++q) {
+          const int k = kk + q * KSTEP;
+          const int kbl = KI >= TK ? 0 : k / KI, kin = k - kbl * KI;
+          foff[q] = 4u * (unsigned)(mb * blk_mn_stride + mi + kbl * blk_k_stride + kin * MNI);
+          if (k < ktail) tail_ok |= 1u << q;
+        }
+      }
+      return;
+    }
     valid_mn = 0;
     int kk;
     if (KC) {
@@ -119,6 +182,23 @@ struct TileLoader {
 
   // clamped address + select instead of a predicated load: all loads of a stage are in flight together
   __device__ __forceinline__ void load() {
+    if (FAST) {
+      if (stage_i == last_ragged) {
+#pragma unroll
+        for (int q = 0; q < NSLOT; ++q) {
+          const bool ok = (tail_ok >> q) & 1u;
+          const vec_t v = buffer_load(rsrc, foff[q], soff);
+          reg[q] = ok ? v : vec_t{};
+        }
+      } else {
+#pragma unroll
+        for (int q = 0; q < NSLOT; ++q) reg[q] = buffer_load(rsrc, foff[q], soff);
+      }
+      ++stage_i;
+      if (++sub == nsub) { sub = 0; soff += 4u * (unsigned)step_cross; }
+      else soff += 4u * (unsigned)step_in;
+      return;
+    }
     if (KC) {
       const bool kvalid = kb < L;
       const int koff = kb * blk_k_stride + kin;
@@ -234,7 +314,7 @@ __host__ __device__ inline void tile_counts(int L, int RI, int CI, int& tm, int&
   slots = tm * tn;
 }
 
-template <int MODE, int VEC>
+template <int MODE, int VEC, bool FAST>
 __global__ __launch_bounds__(NT) void so3_block_mm_real_kernel(MmParams p) {
   typedef Cfg<MODE> C_;
 
@@ -255,8 +335,8 @@ __global__ __launch_bounds__(NT) void so3_block_mm_real_kernel(MmParams p) {
   const size_t L0 = (size_t)l * (4 * l * l - 1) / 3;
   const int M = L * p.RI, N = L * p.CI;
 
-  TileLoader<C_::A_KC, C_::A_MNMAJ, TM, VEC> la;
-  TileLoader<C_::B_KC, C_::B_MNMAJ, TN, VEC> lb;
+  TileLoader<C_::A_KC, C_::A_MNMAJ, TM, VEC, FAST> la;
+  TileLoader<C_::B_KC, C_::B_MNMAJ, TN, VEC, FAST> lb;
   la.init(p.A + L0 * p.RI * p.KI, L, p.RI, p.KI, tile_m);
   lb.init(p.B + L0 * p.CI * p.KI, L, p.CI, p.KI, tile_n);
 
@@ -353,10 +433,14 @@ int run(const float* a, const float* b, float* c, int nl, int RI, int CI, int KI
   const bool b4 = (C_::B_KC ? KI : CI) % 4 == 0;
   const bool vec4 = a4 && b4 && s2cnn::aligned16(a) && s2cnn::aligned16(b);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (vec4)
-    hipLaunchKernelGGL((so3_block_mm_real_kernel<MODE, 4>), dim3(grid), dim3(NT), 0, st, p);
+  // the fast loaders address a degree with 32-bit byte offsets
+  const bool fast = vec4 && (KI % TK == 0 || TK % KI == 0) && Lmax * Lmax * RI * KI < (1L << 30) && Lmax * Lmax * CI * KI < (1L << 30);
+  if (fast)
+    hipLaunchKernelGGL((so3_block_mm_real_kernel<MODE, 4, true>), dim3(grid), dim3(NT), 0, st, p);
+  else if (vec4)
+    hipLaunchKernelGGL((so3_block_mm_real_kernel<MODE, 4, false>), dim3(grid), dim3(NT), 0, st, p);
   else
-    hipLaunchKernelGGL((so3_block_mm_real_kernel<MODE, 1>), dim3(grid), dim3(NT), 0, st, p);
+    hipLaunchKernelGGL((so3_block_mm_real_kernel<MODE, 1, false>), dim3(grid), dim3(NT), 0, st, p);
   return s2cnn::launch_status();
 }
 
