@@ -119,9 +119,12 @@ def _setup_so3_rft_plan(b, grid, device):
         return None
     idx, E, dtab = plan
     valid = torch.tensor(idx >= 0, device=device)
+    sel = np.flatnonzero(idx.reshape(-1) >= 0)       # positions of the grid points in the padded [nbeta * P] layout
     return (torch.tensor(np.maximum(idx, 0), dtype=torch.long, device=device), valid,
             torch.tensor(E.astype(np.float32), device=device).contiguous(),
-            torch.tensor(dtab.astype(np.float32), device=device).contiguous())
+            torch.tensor(dtab.astype(np.float32), device=device).contiguous(),
+            torch.tensor(sel, dtype=torch.long, device=device),
+            torch.tensor(idx.reshape(-1)[sel], dtype=torch.long, device=device))
 
 
 class _SO3RftRealFactorised(torch.autograd.Function):
@@ -129,7 +132,7 @@ class _SO3RftRealFactorised(torch.autograd.Function):
     expansion over the degrees (s2cnn_so3_rft_expand_real) and its adjoint."""
     @staticmethod
     def forward(ctx, x2, b, plan):
-        idx, valid, E, dtab = plan
+        idx, valid, E, dtab = plan[:4]
         ncols = x2.size(0)
         xg = x2.t()[idx] * valid.unsqueeze(-1)                    # [nbeta, P, ncols]
         G = torch.bmm(E.transpose(1, 2), xg).contiguous()        # [nbeta, R, ncols]
@@ -140,14 +143,14 @@ class _SO3RftRealFactorised(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, gy):
-        idx, valid, E, dtab = ctx.plan
+        idx, valid, E, dtab, sel, idx_sel = ctx.plan
         gy = gy.contiguous()
         ncols = gy.size(1)
         gG = gy.new_empty((idx.size(0), E.size(2), ncols))
         _hip.call("s2cnn_so3_rft_expand_real_grad", _hip.ptr(gy), _hip.ptr(dtab), _hip.ptr(gG), ctx.b, idx.size(0), ncols, _hip.stream_ptr())
         gxg = torch.bmm(E, gG)                                    # [nbeta, P, ncols]
         gx = gy.new_zeros((ctx.n_grid, ncols))
-        gx.index_add_(0, idx[valid], gxg[valid])
+        gx.index_add_(0, idx_sel, gxg.reshape(-1, ncols).index_select(0, sel))   # no boolean masks: they would sync with the host
         return gx.t(), None, None
 
 
