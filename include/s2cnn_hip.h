@@ -120,6 +120,24 @@ int s2cnn_s2_mm_gradx(const float *gz, const float *y, float *gx,
 int s2cnn_s2_mm_grady(const float *gz, const float *x, float *gy,
                       int nl, int nbatch, int f_in, int f_out, void *stream);
 
+/* ---- the same products for spectra of REAL signals, in the real basis --------------------
+ * The S^2 spectrum of a real signal (and of the real kernel of soft/s2_conv.py:47) obeys
+ * x[l,-m] = (-1)^m conj(x[l,m]); in the basis of s2cnn_so3_spectrum_to_real it is the real vector
+ * (row +m: sqrt2 Re x[l,m], row -m: sqrt2 Im x[l,m], row 0: x[l,0]) and the product above becomes
+ *   fwd   : z [l,r,s,i,j] = sum_k x[l,r,i,k] * y[l,s,k,j]
+ *   gradx : gx[l,r,i,k]   = sum_{s,j} gz[l,r,s,i,j] * y[l,s,k,j]
+ *   grady : gy[l,s,k,j]   = sum_{r,i} gz[l,r,s,i,j] * x[l,r,i,k]
+ * with x [nl^2, nbatch, f_in], y [nl^2, f_in, f_out], z [nspec_so3(nl), nbatch, f_out] (one float per entry):
+ * z is the real-basis SO(3) spectrum that s2cnn_so3_synthesis_real_basis takes.  Replaces s2_mm inside
+ * S2Convolution (soft/s2_conv.py:45-53) at half the bytes; the reference has no such step.
+ */
+int s2cnn_s2_mm_real_fwd(const float *x, const float *y, float *z,
+                         int nl, int nbatch, int f_in, int f_out, void *stream);
+int s2cnn_s2_mm_real_gradx(const float *gz, const float *y, float *gx,
+                           int nl, int nbatch, int f_in, int f_out, void *stream);
+int s2cnn_s2_mm_real_grady(const float *gz, const float *x, float *gy,
+                           int nl, int nbatch, int f_in, int f_out, void *stream);
+
 /* ---- SO(3) Fourier analysis: grid -> spectrum --------------------------------------
  * x     [nbatch, 2b_in, 2b_in, 2b_in]      (complex_in = 0)
  *       [nbatch, 2b_in, 2b_in, 2b_in, 2]   (complex_in = 1)

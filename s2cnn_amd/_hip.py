@@ -38,6 +38,9 @@ SIGNATURES = {
     "s2cnn_s2_mm_fwd": (_int, _MM_SIG),
     "s2cnn_s2_mm_gradx": (_int, _MM_SIG),
     "s2cnn_s2_mm_grady": (_int, _MM_SIG),
+    "s2cnn_s2_mm_real_fwd": (_int, _MM_SIG),
+    "s2cnn_s2_mm_real_gradx": (_int, _MM_SIG),
+    "s2cnn_s2_mm_real_grady": (_int, _MM_SIG),
     "s2cnn_so3_analysis_workspace": (_size_t, _WS_SIG),
     "s2cnn_so3_analysis": (_int, _FT3_SIG),
     "s2cnn_so3_synthesis_workspace": (_size_t, _WS_SIG),

@@ -8,7 +8,7 @@ import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(os.path.dirname(HERE))
-SOURCES = ["so3_mm.hip", "so3_mm_real.hip", "so3_real_basis.hip", "so3_rft.hip", "so3_fft.hip", "s2_fft.hip", "s2_mm.hip", "so3_integrate.hip"]
+SOURCES = ["so3_mm.hip", "so3_mm_real.hip", "so3_real_basis.hip", "so3_rft.hip", "so3_fft.hip", "s2_fft.hip", "s2_mm.hip", "s2_mm_real.hip", "so3_integrate.hip"]
 LIB = os.path.join(HERE, "libs2cnn_hip.so")
 
 

@@ -205,7 +205,7 @@ def test_so3_integrate(hip):
 
 
 # ------------------------------------------------------------------ layers, forward and gradients
-def _conv_case(kind, B, Fi, Fo, b_in, b_out, grid, seed):
+def _conv_case(kind, B, Fi, Fo, b_in, b_out, grid, seed, real_basis=None):
     if kind == "so3":
         x = rnd((B, Fi, 2 * b_in, 2 * b_in, 2 * b_in), seed)
         layer = s2cnn_amd.SO3Convolution(Fi, Fo, b_in, b_out, grid)
@@ -219,6 +219,8 @@ def _conv_case(kind, B, Fi, Fo, b_in, b_out, grid, seed):
     with torch.no_grad():
         layer.kernel.copy_(k)
         layer.bias.copy_(bias)
+    if real_basis is not None:
+        layer.real_basis = real_basis
     layer = layer.cuda()
     xg = x.cuda().requires_grad_()
     out = layer(xg)
@@ -238,9 +240,12 @@ def test_so3_convolution_parity(hip):
     _conv_case("so3", 2, 4, 6, 4, 4, s2cnn_amd.so3_equatorial_grid(n_alpha=8), 56)
 
 
-def test_s2_convolution_parity(hip):
-    _conv_case("s2", 2, 1, 4, 8, 4, s2cnn_amd.s2_near_identity_grid(), 60)
-    _conv_case("s2", 3, 6, 5, 10, 5, s2cnn_amd.s2_equatorial_grid(n_alpha=16), 63)
+@pytest.mark.parametrize("real_basis", [True, False])
+def test_s2_convolution_parity(hip, real_basis):
+    """Both paths of the layer: real-basis spectra (the default) and the reference's complex ones."""
+    _conv_case("s2", 2, 1, 4, 8, 4, s2cnn_amd.s2_near_identity_grid(), 60, real_basis)
+    _conv_case("s2", 3, 6, 5, 10, 5, s2cnn_amd.s2_equatorial_grid(n_alpha=16), 63, real_basis)
+    _conv_case("s2", 3, 10, 8, 6, 6, s2cnn_amd.s2_near_identity_grid(), 66, real_basis)      # two feature passes, 16-byte rows
 
 
 def test_config1_shaped_network(hip):

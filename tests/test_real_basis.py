@@ -336,3 +336,56 @@ def test_factorised_kernel_transform_matches_dense(hip):
         for got, want in zip(res[True], res[False]):
             assert got.shape == want.shape
             assert (got - want).abs().max().item() < 2e-5 * want.abs().max().item(), (b, (got - want).abs().max().item(), want.abs().max().item())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("nl,B,Fi,Fo", [(4, 2, 3, 5), (10, 32, 1, 20), (7, 5, 6, 9), (6, 16, 12, 16), (5, 3, 6, 100), (3, 1, 1, 1),
+                                        (4, 7, 20, 8), (2, 2, 3, 1028)])
+def test_s2_mm_real_forward_backward(hip, nl, B, Fi, Fo):
+    """The real outer product against numpy: odd sizes (4-byte accesses), multiples of four (16-byte accesses), more
+    input features than one register pass, an odd batch, rows longer than a workgroup."""
+    import s2cnn_amd
+    print(f"s2_mm_real nl={nl} B={B} Fi={Fi} Fo={Fo}", flush=True)
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(nl * nl, B, Fi, generator=g)
+    y = torch.randn(nl * nl, Fi, Fo, generator=g) * Fi ** -0.5
+    ns = O.nspec_so3(nl)
+    gz = torch.randn(ns, B, Fo, generator=g)
+    xd, yd, gd = x.double().numpy(), y.double().numpy(), gz.double().numpy()
+    z = np.empty((ns, B, Fo)); gx = np.empty((nl * nl, B, Fi)); gy = np.empty((nl * nl, Fi, Fo))
+    pos = 0
+    for l in range(nl):
+        L = 2 * l + 1
+        xa, ya = xd[l * l:l * l + L], yd[l * l:l * l + L]
+        ga = gd[pos:pos + L * L].reshape(L, L, B, Fo)
+        z[pos:pos + L * L] = np.einsum("rik,skj->rsij", xa, ya).reshape(L * L, B, Fo)
+        gx[l * l:l * l + L] = np.einsum("rsij,skj->rik", ga, ya)
+        gy[l * l:l * l + L] = np.einsum("rsij,rik->skj", ga, xa)
+        pos += L * L
+    xg, yg = x.cuda().requires_grad_(), y.cuda().requires_grad_()
+    zg = s2cnn_amd.s2_mm_real(xg, yg)
+    gxg, gyg = torch.autograd.grad(zg, (xg, yg), gz.cuda())
+    _close(zg, z)
+    _close(gxg, gx)
+    _close(gyg, gy)
+
+
+@pytest.mark.gpu
+def test_s2_real_product_equals_oracle_complex_product(hip):
+    """to_complex(s2_mm_real(to_real x, to_real y)) against the oracle's s2_mm on spectra of real signals, and the
+    real-basis kernel spectrum against the complex one."""
+    import s2cnn_amd
+    b, B, Fi, Fo = 6, 3, 4, 5
+    g = torch.Generator().manual_seed(5)
+    sig = torch.randn(B * Fi, 2 * b, 2 * b, generator=g).double()
+    x = O.s2_fft(torch.stack((sig, torch.zeros_like(sig)), -1))
+    grid = s2cnn_amd.s2_near_identity_grid()
+    k = torch.randn(Fi, Fo, len(grid), generator=g)
+    y = O.s2_rft(k.double(), b, grid)
+    x = x.reshape(b * b, B, Fi, 2)
+    want = O.s2_mm(x, y).numpy()
+    xr = s2cnn_amd.s2_spectrum_to_real(x.float().cuda())
+    yr = s2cnn_amd.s2_rft_real(k.cuda(), b, grid)
+    _close(yr, s2cnn_amd.s2_spectrum_to_real(y.float().cuda()).cpu().double().numpy())
+    got = s2cnn_amd.so3_spectrum_to_complex(s2cnn_amd.s2_mm_real(xr, yr))
+    _close(got, want)
