@@ -129,7 +129,14 @@ def measure_rows(torch, dev, with_cpu):
     add("s2_mm fwd nl=32 B=32 6->100", gpu_ms(lambda: s2cnn_amd.s2_mm(xkg, ykg)), zbytes + 4.0 * (xk.numel() + yk.numel()), "B", t, 2 / B5, "batch 2 of 32")
     add("s2_mm grad (x and y)", gpu_ms(lambda: torch.autograd.grad(zk, (xkg, ykg), gzk, retain_graph=True)),
         2 * zbytes + 4.0 * 2 * (xk.numel() + yk.numel()), "B", None, 1, "")
-    del zk, gzk, xkg, ykg, s2spec, gspec, xs2g
+    # the same product on real-basis spectra (what S2Convolution runs): half the bytes
+    xr, yr = torch.randn(b5o * b5o, B5, Fi5, device=dev).requires_grad_(), torch.randn(b5o * b5o, Fi5, Fo5, device=dev).requires_grad_()
+    zr = s2cnn_amd.s2_mm_real(xr, yr)
+    gzr = torch.randn_like(zr)
+    add("s2_mm_real fwd nl=32 B=32 6->100", gpu_ms(lambda: s2cnn_amd.s2_mm_real(xr, yr)), 4.0 * (zr.numel() + xr.numel() + yr.numel()), "B", None, 1, "")
+    add("s2_mm_real grad (x and y)", gpu_ms(lambda: torch.autograd.grad(zr, (xr, yr), gzr, retain_graph=True)),
+        4.0 * 2 * (zr.numel() + xr.numel() + yr.numel()), "B", None, 1, "")
+    del zk, gzk, xkg, ykg, s2spec, gspec, xs2g, xr, yr, zr, gzr
     # --- Haar integral at config-4 output size [16, 64, 64, 64, 64]
     xi = torch.randn(16, 64, 64, 64, 64, device=dev)
     t = cpu_s(lambda: O.so3_integrate(xi[:2].cpu()))
