@@ -7,6 +7,7 @@
 // is consumed, so the alpha transform is a DFT pruned to 2nb-1 bins; the intermediate lives in a
 // workspace [z][beta][mi], mi = m + nb - 1.
 #include "common.h"
+#include "s2_fft_real.h"
 
 namespace {
 
@@ -139,6 +140,15 @@ extern "C" int s2cnn_s2_analysis(const float* x, const float* table, float* out,
   if (!workspace || workspace_bytes < ws_bytes(b_in, b_out, nbatch) || !s2cnn::aligned8(workspace)) return S2CNN_EWORKSPACE;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int n2 = 2 * b_in, nb = b_out;
+  if (!complex_in) {   // real signals, b_out <= 32: one kernel, one workgroup per signal
+    const s2_real::Plan plan = s2_real::plan_fwd(n2, nb);
+    if (plan.rb > 0) {
+      if (plan.lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)s2_real::analysis_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)plan.lds);
+      hipLaunchKernelGGL(s2_real::analysis_kernel, dim3((unsigned)nbatch), dim3(s2_real::NT), plan.lds, st, x, table,
+                         reinterpret_cast<float2*>(out), n2, nb, nbatch, plan.rb);
+      return s2cnn::launch_status();
+    }
+  }
   float2* X = static_cast<float2*>(workspace);
   const size_t lds = sizeof(float) * (2 * n2 + (complex_in ? 2 : 1) * n2);
   const unsigned rows = (unsigned)(nbatch * n2);
@@ -158,6 +168,15 @@ extern "C" int s2cnn_s2_synthesis(const float* xhat, const float* table, float* 
   if (!workspace || workspace_bytes < ws_bytes(b_out, b_in, nbatch) || !s2cnn::aligned8(workspace)) return S2CNN_EWORKSPACE;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int n2 = 2 * b_out, nb = b_in;
+  if (!complex_out) {
+    const s2_real::Plan plan = s2_real::plan_inv(n2, nb);
+    if (plan.rb > 0) {
+      if (plan.lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)s2_real::synthesis_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)plan.lds);
+      hipLaunchKernelGGL(s2_real::synthesis_kernel, dim3((unsigned)nbatch), dim3(s2_real::NT), plan.lds, st,
+                         reinterpret_cast<const float2*>(xhat), table, out, n2, nb, nbatch);
+      return s2cnn::launch_status();
+    }
+  }
   const int MW = 2 * nb - 1;
   float2* S = static_cast<float2*>(workspace);
   dim3 grid((unsigned)((nbatch + 63) / 64), n2 * MW);

@@ -27,15 +27,19 @@
 // synthesis leave the LDS as one contiguous run of 16-byte stores instead of four-byte scatters.
 #pragma once
 #include <hip/hip_runtime.h>
+#include "dft_common.h"
 
 namespace plane_real {
+
+using dft_common::pad;
+using dft_common::cs_entry;
+using dft_common::Walk2;
 
 constexpr int NT_MAX = 1024;
 constexpr int PL_MAX = 64;                  // planes per workgroup
 constexpr unsigned LDS_SOFT = 32 * 1024;    // five workgroups per CU when the planes allow it
 constexpr unsigned LDS_HARD = 160 * 1024;
 
-__host__ __device__ inline int pad(int v, int q) { return (v + q - 1) / q * q; }
 
 struct Plan {
   int pl;         // planes per workgroup; 0: the plane does not fit the LDS
@@ -88,27 +92,7 @@ inline Plan plan_inv(int n2, int nb, long nplanes) {
   return make_plan(nb * hp * 8, nb * nb2 * 16, nb * npp * 16, n2 * n2 * 4, hp / 4 * (nb2 / 2), npp / 2 * (hp / 4), nplanes);
 }
 
-__device__ __forceinline__ float2 cs_entry(int j, int k, int n2) {
-  float s, c;
-  sincospif(2.0f * (float)((j * k) % n2) / (float)n2, &s, &c);
-  return make_float2(c, s);
-}
-
 struct F2x4 { float2 v[4]; };
-
-constexpr int LOADS = 8;   // global loads a thread has in flight while it stages planes
-
-// e -> (row, col) = (e / w, e % w) for e = e0, e0 + stride, e0 + 2 stride, ... without a division per step
-struct Walk2 {
-  int row, col, drow, dcol, w;
-  __device__ __forceinline__ void init(int e0, int stride, int width) {
-    w = width; row = e0 / w; col = e0 - row * w; drow = stride / w; dcol = stride - drow * w;
-  }
-  __device__ __forceinline__ void step() {
-    row += drow; col += dcol;
-    if (col >= w) { col -= w; ++row; }
-  }
-};
 
 __device__ __forceinline__ F2x4 lds_read_f2x4(const float2* p) {
   const float4 lo = reinterpret_cast<const float4*>(p)[0], hi = reinterpret_cast<const float4*>(p)[1];
@@ -117,6 +101,9 @@ __device__ __forceinline__ F2x4 lds_read_f2x4(const float2* p) {
   r.v[2] = make_float2(hi.x, hi.y); r.v[3] = make_float2(hi.z, hi.w);
   return r;
 }
+
+
+constexpr int LOADS = 8;   // global loads a thread has in flight while it stages planes
 
 // ---------------------------------------------------------------------------------------------------
 // analysis: x [nplanes][n2][n2] -> X, laid out [plane][mi][ni] (ztile = 0) or
