@@ -34,6 +34,11 @@ def _setup_packed_wigner(b_in, b_out, weighted, synthesis, device):
     return packed
 
 
+# Complex signals (so3_fft / so3_ifft; no layer uses them) run as two transforms of real signals.  False: the
+# library's own kernels for complex signals (s2cnn_so3_analysis / s2cnn_so3_synthesis with complex = 1).
+complex_via_real = True
+
+
 def _null_or_ptr(t):
     return _hip.ptr(t) if t is not None else None
 
@@ -42,6 +47,12 @@ def _analysis(x, b_in, b_out, batch_size, for_grad, complex_in):
     """x: contiguous grid tensor whose leading dims are `batch_size`; the result is allocated in its
     final shape (never a view: autograd can then take ownership of it as a gradient without a copy)."""
     _hip.require_gpu_f32(x)
+    if complex_in and complex_via_real:
+        # the transform is linear over the complex numbers: analysis(x) = analysis(Re x) + i analysis(Im x), and the
+        # kernels for real signals are the tuned ones
+        A = _analysis(x[..., 0].contiguous(), b_in, b_out, batch_size, for_grad, 0)
+        B = _analysis(x[..., 1].contiguous(), b_in, b_out, batch_size, for_grad, 0)
+        return torch.stack((A[..., 0] - B[..., 1], A[..., 1] + B[..., 0]), -1)
     if x.data_ptr() % 16:
         x = x.clone()
     L = _hip.lib()
@@ -59,6 +70,12 @@ def _analysis(x, b_in, b_out, batch_size, for_grad, complex_in):
 
 def _synthesis(x, b_in, b_out, batch_size, for_grad, complex_out, bias=None):
     _hip.require_gpu_f32(x)
+    if complex_out and complex_via_real:
+        # y = synthesis(x) is complex-linear in x and the real-output kernels return Re y for ANY spectrum:
+        # Re y = real_synthesis(x), Im y = Re(-i y) = real_synthesis(-i x)
+        re = _synthesis(x, b_in, b_out, batch_size, for_grad, 0)
+        im = _synthesis(torch.stack((x[..., 1], -x[..., 0]), -1), b_in, b_out, batch_size, for_grad, 0)
+        return torch.stack((re, im), -1)
     L = _hip.lib()
     nbatch = 1
     for d in batch_size:

@@ -92,6 +92,16 @@ def test_so3_transforms(hip, b_in, b_out, for_grad):
     close(PSO3.so3_rifft(sh.cuda(), for_grad, b_out), O.so3_rifft(sh.double(), for_grad, b_out), "so3_rifft (real signal)")
 
 
+@pytest.mark.parametrize("b_in,b_out", [(6, 6), (9, 2), (4, 6), (32, 12)])
+def test_so3_complex_transforms_library_kernels(hip, b_in, b_out, monkeypatch):
+    """so3_fft / so3_ifft through the library's kernels for complex signals (the default composes two real transforms)."""
+    monkeypatch.setattr(PSO3, "complex_via_real", False)
+    x = rnd((2, 2 * b_in, 2 * b_in, 2 * b_in, 2), 17)
+    close(PSO3.so3_fft(x.cuda(), False, b_out), O.so3_fft(x.double(), False, b_out), "so3_fft")
+    s = rnd((O.nspec_so3(b_in), 2, 2), 18)
+    close(PSO3.so3_ifft(s.cuda(), True, b_out), O.so3_ifft(s.double(), True, b_out), "so3_ifft")
+
+
 def test_so3_transform_batch_dims_and_ragged(hip):
     x = rnd((2, 3, 8, 8, 8), 13)
     close(PSO3.so3_rfft(x.cuda(), b_out=3), O.so3_rfft(x.double(), b_out=3), "lead dims")
