@@ -1,46 +1,33 @@
-"""Sampling grids on SO(3) for convolution kernels: mirrors s2cnn/so3_grid.py of the reference.
-Every grid is a tuple of (beta, alpha, gamma) tuples of Python floats (hashable: it keys caches)."""
+"""Kernel grids on SO(3): tuples of (beta, alpha, gamma) Euler-angle points (same functions, defaults and point
+order as s2cnn/so3_grid.py)."""
 import warnings
 
 import numpy as np
 
+from . import _grid_util as G
 
-def _pack(B, A, C):
-    grid = np.stack((B.flatten(), A.flatten(), C.flatten()), axis=1)
-    if sum(grid[:, 0] == 0) > 1:
+
+def _checked(beta, alpha, gamma):
+    pts = G.points(beta, alpha, gamma)
+    if sum(1 for p in pts if p[0] == 0) > 1:     # at beta = 0 only alpha + gamma matters: such points may coincide
         warnings.warn("Gimbal lock: beta take value 0 in the grid")
-    return tuple(tuple(float(v) for v in bac) for bac in grid)
+    return pts
 
 
 def so3_near_identity_grid(max_beta=np.pi / 8, max_gamma=2 * np.pi, n_alpha=8, n_beta=3, n_gamma=None):
-    '''
-    :return: rings of rotations around the identity, all points (rotations) in
-    a ring are at the same distance from the identity
-    size of the kernel = n_alpha * n_beta * n_gamma
-    '''
-    if n_gamma is None:
-        n_gamma = n_alpha  # similar to regular representations
-    beta = np.arange(start=1, stop=n_beta + 1, dtype=float) * max_beta / n_beta
-    alpha = np.linspace(start=0, stop=2 * np.pi, num=n_alpha, endpoint=False)
-    pre_gamma = np.linspace(start=-max_gamma, stop=max_gamma, num=n_gamma, endpoint=True)
-    B, A, preC = np.meshgrid(beta, alpha, pre_gamma, indexing='ij')
-    return _pack(B, A, preC - A)
+    """Rotations close to the identity: n_beta rings (every rotation of a ring is equally far from the identity) of
+    n_alpha directions, and n_gamma (default n_alpha) in-plane angles with alpha + gamma in [-max_gamma, max_gamma]."""
+    n_gamma = n_alpha if n_gamma is None else n_gamma
+    beta, alpha, twist = G.mesh(G.polar_rings(max_beta, n_beta), G.circle(n_alpha), G.band(0.0, max_gamma, n_gamma))
+    return _checked(beta, alpha, twist - alpha)
 
 
 def so3_equatorial_grid(max_beta=0, max_gamma=np.pi / 8, n_alpha=32, n_beta=1, n_gamma=2):
-    '''
-    :return: rings of rotations around the equator.
-    size of the kernel = n_alpha * n_beta * n_gamma
-    '''
-    beta = np.linspace(start=np.pi / 2 - max_beta, stop=np.pi / 2 + max_beta, num=n_beta, endpoint=True)
-    alpha = np.linspace(start=0, stop=2 * np.pi, num=n_alpha, endpoint=False)
-    gamma = np.linspace(start=-max_gamma, stop=max_gamma, num=n_gamma, endpoint=True)
-    return _pack(*np.meshgrid(beta, alpha, gamma, indexing='ij'))
+    """Rotations that take the north pole into the band of half-width max_beta around the equator, with
+    n_gamma in-plane angles in [-max_gamma, max_gamma]."""
+    return _checked(*G.mesh(G.band(np.pi / 2, max_beta, n_beta), G.circle(n_alpha), G.band(0.0, max_gamma, n_gamma)))
 
 
 def so3_soft_grid(b):
-    beta = (np.arange(2 * b) + 0.5) / (2 * b) * np.pi
-    alpha = gamma = np.linspace(start=0, stop=2 * np.pi, num=2 * b, endpoint=False)
-    B, A, C = np.meshgrid(beta, alpha, gamma, indexing='ij')
-    grid = np.stack((B.flatten(), A.flatten(), C.flatten()), axis=1)
-    return tuple(tuple(float(v) for v in bac) for bac in grid)
+    """Every point of the (2b)^3 SOFT grid."""
+    return G.points(*G.mesh(G.soft_colatitudes(b), G.circle(2 * b), G.circle(2 * b)))
