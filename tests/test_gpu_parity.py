@@ -438,3 +438,40 @@ def test_so3_synthesis_with_bias(hip, b_spec, b_grid):
     (ref * w).sum().backward()
     for name, a, c in zip(("out", "grad spectrum", "grad bias"), got, (ref.detach(), s.grad, bias.grad)):
         close(a, c.double().cpu(), name)
+
+
+def test_network_forward_replays_from_a_hip_graph(hip):
+    """Nothing on the path allocates through HIP, synchronises or clears memory with a memset node, so a forward pass
+    captures into a HIP graph (the launch-bound small configurations gain from it).  Each replay, with eager work and
+    synchronisations between the replays, must reproduce the eager result bit for bit."""
+    pi = 3.141592653589793
+    g1 = s2cnn_amd.s2_near_identity_grid(max_beta=pi / 8, n_alpha=8, n_beta=3)
+    g2 = s2cnn_amd.so3_near_identity_grid(max_beta=pi / 8, max_gamma=2 * pi, n_alpha=8, n_beta=3, n_gamma=8)
+    torch.manual_seed(3)
+    c1 = s2cnn_amd.S2Convolution(1, 20, 30, 10, g1).cuda()
+    c2 = s2cnn_amd.SO3Convolution(20, 40, 10, 6, g2).cuda()
+
+    def net(x):
+        return s2cnn_amd.so3_integrate(torch.relu(c2(torch.relu(c1(x)))))
+
+    gen = torch.Generator().manual_seed(4)
+    xs = [torch.rand(8, 1, 60, 60, generator=gen).cuda() for _ in range(3)]
+    static_x = xs[0].clone()
+    with torch.no_grad():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                net(static_x)                      # tables, workspaces and allocator pools exist before the capture
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            static_y = net(static_x)
+        for i, x in enumerate(xs):
+            static_x.copy_(x)
+            graph.replay()
+            torch.cuda.synchronize()
+            want = net(x)                          # eager work between the replays
+            torch.cuda.synchronize()
+            assert torch.equal(static_y, want), f"replay {i} differs from the eager pass"
