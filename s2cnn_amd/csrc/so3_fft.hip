@@ -331,7 +331,7 @@ int fused_analysis(const float* x, const float* table, const float* packed_table
     hipLaunchKernelGGL(fused64::pack_table, dim3(1024), dim3(256), 0, st, table, dst, s2cnn::so3_nspec(b_out), b_out);
     Tf = dst;
   }
-  hipLaunchKernelGGL(fused64::analysis_kernel, dim3(fused64::grid_size(nbatch)), dim3(fused64::THREADS), 0, st, x, Tf, rec, nbatch);
+  fused64::launch_analysis(b_out, st, x, Tf, rec, nbatch);
   if (real_basis)
     hipLaunchKernelGGL(fused64::spectrum_scatter_real, dim3((unsigned)((nbatch + fused64::ZR - 1) / fused64::ZR), fused64::NIT * 32), dim3(256), 0, st,
                        rec, out, b_out, nbatch);
@@ -360,7 +360,7 @@ int fused_synthesis(const float* xhat, const float* table, const float* packed_t
   else
     hipLaunchKernelGGL(fused64::spectrum_gather, dim3((unsigned)((nbatch + fused64::ZT - 1) / fused64::ZT), fused64::NIT * 16), dim3(256), 0, st,
                        reinterpret_cast<const float2*>(xhat), rec, nl, nbatch);
-  hipLaunchKernelGGL(fused64::synthesis_kernel, dim3(fused64::grid_size(nbatch)), dim3(fused64::THREADS), 0, st, rec, Tf, out, nbatch, bias, nfeature);
+  fused64::launch_synthesis(nl, st, rec, Tf, out, nbatch, bias, nfeature);
   return s2cnn::launch_status();
 }
 

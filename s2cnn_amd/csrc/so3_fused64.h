@@ -177,6 +177,9 @@ constexpr int QUAD_ELEMS = 33 * QPITCH;         // row 32 takes the unused m = 3
 //   after item 0, 1, 2: items 4, 5, 6 of the same plane pair;  after 3, 4, 5, 6: items 3, 0, 1, 2 of the next pair
 __device__ constexpr int table_slot(int it) { return it & 3; }
 
+// NA: item rounds that carry degrees below the output bandwidth (items are ordered by degree group, so a truncated
+// spectrum leaves the later rounds without work: NA = 3 covers l < 24, 5 covers l < 28, 7 everything).
+template <int NA>
 __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restrict__ x, const float* __restrict__ Tf,
                                                            float4* __restrict__ rec, long nbatch) {
   using namespace fft64;
@@ -289,7 +292,10 @@ __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restri
 
   // first plane pair: transformed alone
   load_planes(0);
-  load_table(0, 0); load_table(0, 1); load_table(0, 2); load_table(0, 3);
+  load_table(0, 0);
+  if constexpr (NA > 1) load_table(0, 1);
+  if constexpr (NA > 2) load_table(0, 2);
+  if constexpr (NA > 3) load_table(0, 3);
   __syncthreads();                              // twiddles, cleared quads
   stage_c1();
   load_planes(1);
@@ -303,7 +309,12 @@ __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restri
 #define S2CNN_FENCE() __builtin_amdgcn_sched_barrier(0)
   // contract item k, then refill its table slot with the item that uses the slot next; plane loads in quarters:
   // memory instructions are spread over the step so that their queue never fills up
-#define S2CNN_ACC(k, jl, il) accumulate(cur, k); S2CNN_FENCE(); load_table(jl, il); S2CNN_FENCE();
+#define S2CNN_ACC(k, jl, il)                                                                             \
+  if constexpr ((k) < NA) {                                                                              \
+    accumulate(cur, k); S2CNN_FENCE();                                                                   \
+    if constexpr ((k) + 4 < NA) load_table(j, (k) + 4); else load_table(j + 1, (k) & 3);                 \
+    S2CNN_FENCE();                                                                                       \
+  }
 #define S2CNN_PLANES(g) load_planes_part(jp, g); S2CNN_FENCE();
   // Waves d < 4 transform first and contract second, waves d >= 4 the other way round: each SIMD holds one
   // wave of either kind, so its LDS-bound and its FMA-bound half of a stage overlap.
@@ -347,8 +358,13 @@ __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restri
   }
   {
     const float2* cur = quad[(NJ - 1) & 1];
-    S2CNN_ACC(0, NJ - 1, 4) S2CNN_ACC(1, NJ - 1, 5) S2CNN_ACC(2, NJ - 1, 6)
-    accumulate(cur, 3); accumulate(cur, 4); accumulate(cur, 5); accumulate(cur, 6);
+#define S2CNN_LAST(k)                                                                                    \
+  if constexpr ((k) < NA) {                                                                              \
+    accumulate(cur, k);                                                                                  \
+    if constexpr ((k) + 4 < NA) { S2CNN_FENCE(); load_table(NJ - 1, (k) + 4); S2CNN_FENCE(); }           \
+  }
+    S2CNN_LAST(0) S2CNN_LAST(1) S2CNN_LAST(2) S2CNN_LAST(3) S2CNN_LAST(4) S2CNN_LAST(5) S2CNN_LAST(6)
+#undef S2CNN_LAST
   }
 #undef S2CNN_ACC
 #undef S2CNN_PLANES
@@ -573,6 +589,8 @@ __global__ __launch_bounds__(256) void spectrum_gather_real(const float* __restr
 // Sums are formed in a fixed order: results are reproducible bit for bit.
 // ---------------------------------------------------------------------------------------------
 // bias: NULL, or one value per feature added to every sample of volume z (feature = z % nfeature)
+// NA as in analysis_kernel; CMAX: degree groups c < CMAX carry degrees of the input (6 for NA = 3, 7 for 5, 8 for 7)
+template <int NA, int CMAX>
 __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __restrict__ rec, const float* __restrict__ Tf,
                                                             float* __restrict__ y, long nbatch, const float* __restrict__ bias, int nfeature) {
   using namespace fft64;
@@ -596,7 +614,7 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
   const unsigned toff = t * 16;
   const unsigned yoff = ((d + 8 * (lo & 3)) * N + 4 * (lo >> 2)) * 4;   // + (beta * 4096 + 2048 h) * 4: row d + 8 (lo % 4) + 32 h, columns 4 (lo / 4)..+3
 #pragma unroll
-  for (int it = 0; it < NIT; ++it) {
+  for (int it = 0; it < NA; ++it) {
     int c, a, n;
     decode_item(it * THREADS + t, c, a, n);
     sgn |= (unsigned)(n & 1) << it;
@@ -656,7 +674,7 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
       float4 s0 = make_float4(0.f, 0.f, 0.f, 0.f), s1 = s0;
 #pragma unroll
       for (int c = 0; c < 8; ++c) {
-        if (c >= cmin) {
+        if (c >= cmin && c < CMAX) {
           const int i = OFF[c] + a * (4 * c + 4) + n;
           const float4 u0 = stg_p[i], u1 = stg_m[i];
           s0.x += u0.x; s0.y += u0.y; s0.z += u0.z; s0.w += u0.w;
@@ -708,10 +726,20 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
 
 #define S2CNN_FENCE() __builtin_amdgcn_sched_barrier(0)
   // the item's share, then its table slot is refilled with the item that uses the slot next (see table_slot)
-#define S2CNN_CON(k, jl, il) contribute(k); S2CNN_FENCE(); load_table((jl) < NJ ? (jl) : NJ - 1, il); S2CNN_FENCE();
-  load_table(0, 0); load_table(0, 1); load_table(0, 2); load_table(0, 3);
+  // (pair P being contributed; the slot then takes item k + 4 of the same pair or item k % 4 of the next one)
+#define S2CNN_CON(k, P)                                                                                  \
+  if constexpr ((k) < NA) {                                                                              \
+    contribute(k); S2CNN_FENCE();                                                                        \
+    if constexpr ((k) + 4 < NA) load_table((P) < NJ ? (P) : NJ - 1, (k) + 4);                            \
+    else load_table((P) + 1 < NJ ? (P) + 1 : NJ - 1, (k) & 3);                                           \
+    S2CNN_FENCE();                                                                                       \
+  }
+  load_table(0, 0);
+  if constexpr (NA > 1) load_table(0, 1);
+  if constexpr (NA > 2) load_table(0, 2);
+  if constexpr (NA > 3) load_table(0, 3);
   __syncthreads();
-  S2CNN_CON(0, 0, 4) S2CNN_CON(1, 0, 5) S2CNN_CON(2, 0, 6) S2CNN_CON(3, 1, 3) S2CNN_CON(4, 1, 0) S2CNN_CON(5, 1, 1) S2CNN_CON(6, 1, 2)
+  S2CNN_CON(0, 0) S2CNN_CON(1, 0) S2CNN_CON(2, 0) S2CNN_CON(3, 0) S2CNN_CON(4, 0) S2CNN_CON(5, 0) S2CNN_CON(6, 0)
   __syncthreads();
   reduce();
   __syncthreads();
@@ -722,32 +750,32 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
   if (d < 4) {
     for (int j = 0; j < NJ - 1; ++j) {
       fft_pass<true, 0>(work, twl); S2CNN_FENCE();
-      S2CNN_CON(0, j + 1, 4) S2CNN_CON(1, j + 1, 5)
+      S2CNN_CON(0, j + 1) S2CNN_CON(1, j + 1)
       __syncthreads();
       fft_pass<true, 1>(work, twl); S2CNN_FENCE();
-      S2CNN_CON(2, j + 1, 6) S2CNN_CON(3, j + 2, 3)
+      S2CNN_CON(2, j + 1) S2CNN_CON(3, j + 1)
       __syncthreads();
       fft_pass<true, 2>(work, twl); S2CNN_FENCE();
-      S2CNN_CON(4, j + 2, 0) S2CNN_CON(5, j + 2, 1)
+      S2CNN_CON(4, j + 1) S2CNN_CON(5, j + 1)
       __syncthreads();
       stage_c2_store(j); S2CNN_FENCE();
-      S2CNN_CON(6, j + 2, 2)
+      S2CNN_CON(6, j + 1)
       __syncthreads();
       reduce();
       __syncthreads();
     }
   } else {
     for (int j = 0; j < NJ - 1; ++j) {
-      S2CNN_CON(0, j + 1, 4) S2CNN_CON(1, j + 1, 5)
+      S2CNN_CON(0, j + 1) S2CNN_CON(1, j + 1)
       fft_pass<true, 0>(work, twl);
       __syncthreads();
-      S2CNN_CON(2, j + 1, 6) S2CNN_CON(3, j + 2, 3)
+      S2CNN_CON(2, j + 1) S2CNN_CON(3, j + 1)
       fft_pass<true, 1>(work, twl);
       __syncthreads();
-      S2CNN_CON(4, j + 2, 0) S2CNN_CON(5, j + 2, 1)
+      S2CNN_CON(4, j + 1) S2CNN_CON(5, j + 1)
       fft_pass<true, 2>(work, twl);
       __syncthreads();
-      S2CNN_CON(6, j + 2, 2)
+      S2CNN_CON(6, j + 1)
       stage_c2_store(j);
       __syncthreads();
       reduce();
@@ -760,6 +788,22 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
   fft_pass<true, 1>(work, twl); __syncthreads();
   fft_pass<true, 2>(work, twl); __syncthreads();
   stage_c2_store(NJ - 1);
+}
+
+// Launchers: the instantiation whose item rounds cover the nl degrees present.
+inline void launch_analysis(int nl, hipStream_t st, const float* x, const float* Tf, float4* rec, long nbatch) {
+  const dim3 grid(grid_size(nbatch)), block(THREADS);
+  if (nl <= 24) hipLaunchKernelGGL(analysis_kernel<3>, grid, block, 0, st, x, Tf, rec, nbatch);
+  else if (nl <= 28) hipLaunchKernelGGL(analysis_kernel<5>, grid, block, 0, st, x, Tf, rec, nbatch);
+  else hipLaunchKernelGGL(analysis_kernel<7>, grid, block, 0, st, x, Tf, rec, nbatch);
+}
+
+inline void launch_synthesis(int nl, hipStream_t st, const float4* rec, const float* Tf, float* y, long nbatch, const float* bias,
+                             int nfeature) {
+  const dim3 grid(grid_size(nbatch)), block(THREADS);
+  if (nl <= 24) hipLaunchKernelGGL((synthesis_kernel<3, 6>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature);
+  else if (nl <= 28) hipLaunchKernelGGL((synthesis_kernel<5, 7>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature);
+  else hipLaunchKernelGGL((synthesis_kernel<7, 8>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature);
 }
 
 }  // namespace fused64
