@@ -137,6 +137,21 @@ def test_so3_one_kernel_path_is_reproducible(hip):
     for _ in range(4):
         assert torch.equal(PSO3.so3_rfft(x), a0)
         assert torch.equal(PSO3.so3_rifft(s), y0)
+    # the instantiations for truncated spectra (22 and 26 degrees), at a batch that fills the chip, with the bias
+    from s2cnn_amd.soft.so3_fft import so3_rifft_real_basis, so3_rfft_real_basis
+    xb = rnd((300, 64, 64, 64), 92).cuda()
+    bias = rnd((4,), 93).cuda()
+    for b in (22, 26):
+        r = rnd((O.nspec_so3(b), 75, 4), 94).cuda()
+        a1, y1 = so3_rfft_real_basis(xb, b_out=b), so3_rifft_real_basis(r, b_out=32, bias=bias)
+        for _ in range(3):
+            assert torch.equal(so3_rfft_real_basis(xb, b_out=b), a1)
+            assert torch.equal(so3_rifft_real_basis(r, b_out=32, bias=bias), y1)
+        # against the untruncated kernels: zero-extended spectrum in, leading rows out
+        rz = torch.zeros(O.nspec_so3(32), 75, 4, device="cuda")
+        rz[:r.size(0)] = r
+        close(y1, so3_rifft_real_basis(rz, b_out=32, bias=bias).cpu().double(), f"synthesis from {b} degrees")
+        close(a1, so3_rfft_real_basis(xb, b_out=32)[:a1.size(0)].cpu().double(), f"analysis to {b} degrees")
 
 
 def test_so3_transforms_without_prepacked_table(hip):
