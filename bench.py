@@ -151,13 +151,16 @@ def measure_rows(torch, dev, with_cpu):
     t = cpu_s(lambda: O.so3_ifft(sc[:, :1].cpu()))
     add("so3_ifft complex b=32 N=16", gpu_ms(lambda: PSO3.so3_ifft(sc)), byc, "B", t, 1 / 16, "1 volume of 16")
     del xc, sc
-    # --- kernel -> spectrum (library GEMM) at config-4 size: [64, 64, 192] -> [43680, 64, 64, 2]
+    # --- kernel -> spectrum at config-4 size: [64, 64, 192] -> [43680, 64, 64, 2]
     grid = s2cnn_amd.so3_near_identity_grid()
     kk = torch.randn(64, 64, len(grid), device=dev)
     s2cnn_amd.so3_rft(kk, 32, grid)
     t = cpu_s(lambda: O.so3_rft(kk[:8].cpu(), 32, grid))
-    add("so3_rft [64,64,192]->b32", gpu_ms(lambda: s2cnn_amd.so3_rft(kk, 32, grid)), 2.0 * 64 * 64 * 192 * nspec(32) * 2, "F", t, 8 / 64,
+    # factorised over the 3 distinct betas of the grid: bound by writing the spectrum (8 B per complex entry), not by flops
+    add("so3_rft [64,64,192]->b32", gpu_ms(lambda: s2cnn_amd.so3_rft(kk, 32, grid)), 8.0 * 64 * 64 * nspec(32) + 4.0 * kk.numel(), "B", t, 8 / 64,
         "8 of 64 input features")
+    from s2cnn_amd.so3_real import so3_rft_real
+    add("so3_rft_real (inside the layer)", gpu_ms(lambda: so3_rft_real(kk, 32, grid)), 4.0 * 64 * 64 * nspec(32) + 4.0 * kk.numel(), "B", None, 1, "")
     torch.cuda.empty_cache()
     return rows
 

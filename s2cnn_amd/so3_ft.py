@@ -1,6 +1,6 @@
-"""Spectrum of a kernel sampled on an arbitrary SO(3) grid: mirrors s2cnn/so3_ft.py of the
-reference.  The transform is one dense real GEMM with a precomputed matrix of conjugated
-Wigner-D samples; it stays a library GEMM (torch.matmul -> hipBLASLt)."""
+"""Spectrum of a kernel sampled on an arbitrary SO(3) grid (s2cnn/so3_ft.py).  In general one dense real GEMM with a
+precomputed matrix of conjugated Wigner-D samples (torch.matmul -> hipBLASLt); grids with few distinct beta values go
+through the factorised real-basis transform of s2cnn_amd.so3_real."""
 from functools import lru_cache
 
 import numpy as np
@@ -25,10 +25,20 @@ def so3_rft(x, b, grid):
     :param grid: tuple of (beta, alpha, gamma) tuples
     :return: [l * m * n, ..., complex]
     """
+    sz = x.size()
+    if x.is_cuda and so3_rft.factorised:
+        # The kernel is real, so its spectrum is that of a real signal: the real-basis transform (factorised over the
+        # few distinct beta values of the grid, s2cnn_amd.so3_real) followed by the change of basis is the same function
+        from . import so3_real
+        grid = tuple(grid)
+        if (x.numel() // sz[-1]) % 4 == 0 and so3_real._setup_so3_rft_plan(b, grid, x.device) is not None:
+            return so3_real.so3_spectrum_to_complex(so3_real.so3_rft_real(x, b, grid))
     F = _setup_so3_ft(b, grid, x.device)  # [beta_alpha_gamma, l * m * n * complex]
     assert x.size(-1) == F.size(0)
-    sz = x.size()
     # [spec*2, n_grid] @ [n_grid, rows] -> [spec, 2, rows] -> [spec, rows, 2]
     out = torch.matmul(F.t(), x.reshape(-1, sz[-1]).t())
     out = out.view(-1, 2, out.size(-1)).transpose(1, 2).contiguous()
     return out.view(-1, *sz[:-1], 2)
+
+
+so3_rft.factorised = True   # False: always the dense product with the [len(grid), nspec * 2] matrix

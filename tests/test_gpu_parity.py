@@ -520,3 +520,22 @@ def test_so3_projector_on_a_large_grid(hip):
     rel = ((up - PSO3.so3_rifft(sz)).norm() / up.norm()).item()
     print(f"zero-extended synthesis: rel L2 {rel:.2e}", flush=True)
     assert rel < TOL
+
+
+@pytest.mark.parametrize("factorised", [True, False])
+def test_so3_rft_kernel_spectrum(hip, factorised, monkeypatch):
+    """so3_rft (so3_ft.py:4-25) through the factorised real-basis transform and through the dense product:
+    values and the gradient with respect to the kernel, against the oracle."""
+    monkeypatch.setattr(s2cnn_amd.so3_rft, "factorised", factorised)
+    b = 7
+    grid = s2cnn_amd.so3_near_identity_grid(n_alpha=6, n_beta=2, n_gamma=4)
+    k = rnd((4, 3, len(grid)), 95)
+    w = rnd((O.nspec_so3(b), 4, 3, 2), 96)
+    kg = k.cuda().requires_grad_()
+    y = s2cnn_amd.so3_rft(kg, b, grid)
+    (y * w.cuda()).sum().backward()
+    ko = k.double().requires_grad_()
+    yo = O.so3_rft(ko, b, grid)
+    (yo * w.double()).sum().backward()
+    close(y, yo, "so3_rft")
+    close(kg.grad, ko.grad, "so3_rft grad")
