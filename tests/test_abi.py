@@ -51,6 +51,16 @@ def test_argument_rejection_without_gpu():
     assert lib.s2cnn_so3_packed_table_bytes(40, 40, 0) == 0 and lib.s2cnn_so3_packed_table_bytes(32, 40, 1) == 0
     assert lib.s2cnn_so3_pack_table(fake, fake, 40, 40, 0, null) == -1
     assert b"workspace" in lib.s2cnn_strerror(-2)
+    # entry points of the real-basis path and the biased synthesis
+    assert lib.s2cnn_s2_mm_real_fwd(null, null, null, 4, 2, 3, 5, null) == -1
+    assert lib.s2cnn_s2_mm_real_gradx(fake, fake, fake, 4, 0, 3, 5, null) == -1                # empty batch
+    assert lib.s2cnn_s2_mm_real_grady(ctypes.c_void_p(0x1002), fake, fake, 4, 2, 3, 5, null) == -3
+    assert lib.s2cnn_so3_mm_real_fwd(null, null, null, 4, 2, 3, 5, null) == -1
+    assert lib.s2cnn_so3_synthesis_real_bias(null, null, null, null, null, 0, 4, 4, 1, null, 1, null) == -1
+    assert lib.s2cnn_so3_synthesis_real_bias(fake, fake, null, fake, fake, 1 << 30, 4, 4, 6, fake, 4, null) == -1   # 6 volumes, 4 features
+    assert lib.s2cnn_so3_synthesis_real_basis(fake, fake, null, fake, fake, 1 << 30, 4, 4, 1, null, 1, null) == -1  # no direct kernel for this grid
+    assert lib.s2cnn_so3_real_basis_transform_available(32, 22, 0) == 1 and lib.s2cnn_so3_real_basis_transform_available(22, 22, 0) == 0
+    assert lib.s2cnn_so3_rft_expand_real(null, null, null, 4, 3, 8, null) == -1
 
 
 def test_product_has_no_cpu_path():
