@@ -389,3 +389,34 @@ def test_s2_real_product_equals_oracle_complex_product(hip):
     _close(yr, s2cnn_amd.s2_spectrum_to_real(y.float().cuda()).cpu().double().numpy())
     got = s2cnn_amd.so3_spectrum_to_complex(s2cnn_amd.s2_mm_real(xr, yr))
     _close(got, want)
+
+
+@pytest.mark.gpu
+def test_so3_mm_real_at_the_benchmark_size(hip):
+    """nl = 32, batch 16, 64 -> 64 features (the loaders with scalar stage offsets, 3 048 to 11 440 tiles per launch):
+    forward and both gradients against float64 einsums per degree on the same device."""
+    import s2cnn_amd
+    nl, B, Fi, Fo = 32, 16, 64, 64
+    ns = O.nspec_so3(nl)
+    g = torch.Generator(device="cuda").manual_seed(21)
+    x = torch.randn(ns, B, Fi, device="cuda", generator=g).requires_grad_()
+    y = (torch.randn(ns, Fi, Fo, device="cuda", generator=g) * Fi ** -0.5).requires_grad_()
+    gz = torch.randn(ns, B, Fo, device="cuda", generator=g)
+    z = s2cnn_amd.so3_mm_real(x, y)
+    gx, gy = torch.autograd.grad(z, (x, y), gz)
+    worst = 0.0
+    pos = 0
+    for l in range(nl):
+        L = 2 * l + 1
+        sl = slice(pos, pos + L * L)
+        xa = x.detach()[sl].double().reshape(L, L, B, Fi)
+        ya = y.detach()[sl].double().reshape(L, L, Fi, Fo)
+        ga = gz[sl].double().reshape(L, L, B, Fo)
+        for got, want in ((z.detach()[sl], torch.einsum("mpik,npkj->mnij", xa, ya)),
+                          (gx[sl], torch.einsum("mnij,npkj->mpik", ga, ya)),
+                          (gy[sl], torch.einsum("mnij,mpik->npkj", ga, xa))):
+            want = want.reshape(L * L, *got.shape[1:])
+            worst = max(worst, ((got.double() - want).abs().max() / want.std()).item())
+        pos += L * L
+    print(f"worst max|d|/std over degrees and the three products: {worst:.2e}", flush=True)
+    assert worst < 1e-4
