@@ -420,3 +420,32 @@ def test_so3_mm_real_at_the_benchmark_size(hip):
         pos += L * L
     print(f"worst max|d|/std over degrees and the three products: {worst:.2e}", flush=True)
     assert worst < 1e-4
+
+
+@pytest.mark.gpu
+def test_convolution_paths_agree_at_the_benchmark_size(hip, monkeypatch):
+    """The layer of the headline benchmark (batch 16, 64 -> 64 features, b = 32), forward and all gradients, through
+    two disjoint sets of kernels: real-basis spectra (per-volume transforms writing real rows, real product, factorised
+    kernel spectrum) against complex spectra (complex rows, complex product, dense kernel transform)."""
+    import s2cnn_amd
+    B, F, b = 16, 64, 32
+    torch.manual_seed(1)
+    conv = s2cnn_amd.SO3Convolution(F, F, b, b, s2cnn_amd.so3_near_identity_grid()).cuda()
+    with torch.no_grad():
+        conv.bias.normal_(0, 0.1)
+    x = torch.randn(B, F, 64, 64, 64, device="cuda", requires_grad=True)
+    res = {}
+    for flag in (True, False):
+        conv.real_basis = flag
+        monkeypatch.setattr(s2cnn_amd.so3_rft, "factorised", flag)
+        conv.zero_grad()
+        x.grad = None
+        z = conv(x)
+        loss = z.square().sum()
+        loss.backward()
+        res[flag] = (z.detach()[::5, ::7].clone(), x.grad[::5, ::7].clone(), conv.kernel.grad.clone(), conv.bias.grad.clone())
+        del z, loss
+    for name, a, c in zip(("out", "grad_x", "grad_kernel", "grad_bias"), res[True], res[False]):
+        q = ((a.double() - c.double()).abs().max() / c.double().std()).item()
+        print(name, f"{q:.2e}", flush=True)
+        assert q < 1e-4, (name, q)
