@@ -539,3 +539,19 @@ def test_so3_rft_kernel_spectrum(hip, factorised, monkeypatch):
     (yo * w.double()).sum().backward()
     close(y, yo, "so3_rft")
     close(kg.grad, ko.grad, "so3_rft grad")
+
+
+def test_so3_round_trip_at_the_benchmark_size(hip):
+    """[256, 64, 64, 64] (the transform benchmark): every volume of the batch gets the bits it gets alone (the result
+    of a volume does not depend on the workgroup that takes it), and analysis o synthesis is the identity on spectra."""
+    g = torch.Generator(device="cuda").manual_seed(33)
+    x = torch.randn(256, 64, 64, 64, device="cuda", generator=g)
+    s = PSO3.so3_rfft(x)
+    y = PSO3.so3_rifft(s)
+    for i in (0, 7, 100, 255):
+        assert torch.equal(PSO3.so3_rfft(x[i:i + 1].contiguous())[:, 0], s[:, i]), i
+        assert torch.equal(PSO3.so3_rifft(s[:, i:i + 1].contiguous())[0], y[i]), i
+    s2 = PSO3.so3_rfft(y)
+    rel = ((s2 - s).norm() / s.norm()).item()
+    print(f"analysis(synthesis(s)) - s: rel L2 {rel:.2e}", flush=True)
+    assert rel < TOL
