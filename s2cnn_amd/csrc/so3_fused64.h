@@ -172,6 +172,8 @@ inline size_t scratch_bytes(long nbatch) { return (size_t)nbatch * REC_BYTES; }
 // contracted out of the other quad buffer, two items per stage.
 // ---------------------------------------------------------------------------------------------
 constexpr int QPITCH = 32 * 4 + 6;              // complex numbers per a-row of the quad layout; the pad takes the unused n = 32
+constexpr int QHALF = 66;                       // a row holds the pairs {Z[+a,n], Z[-a,-n]} for n = 0..32, then the pairs {Z[-a,n], Z[+a,-n]}:
+                                                // consecutive items (consecutive n) read consecutive 16-byte words of either half
 constexpr int QUAD_ELEMS = 33 * QPITCH;         // row 32 takes the unused m = 32
 // table registers: four slots, item it in slot it % 4; a slot is refilled right after its item has been used:
 //   after item 0, 1, 2: items 4, 5, 6 of the same plane pair;  after 3, 4, 5, 6: items 3, 0, 1, 2 of the next pair
@@ -199,16 +201,16 @@ __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restri
   for (int it = 0; it < NIT; ++it) {
     int c, a, n;
     decode_item(it * THREADS + t, c, a, n);
-    adr[it] = (unsigned)(a * QPITCH + 4 * n) | ((unsigned)(n & 1) << 31);
+    adr[it] = (unsigned)(a * QPITCH + 2 * n) | ((unsigned)(n & 1) << 31);
   }
   // where this thread's outputs of the last gamma stage go: row slot lo holds m = sigma(lo)
   const int m = sigma(lo);
-  // quad[a][n] = { Z[+a,n], Z[-a,-n], Z[-a,n], Z[+a,-n] }; +0 and -0 are the same frequency, so
+  // row a of a quad buffer: { Z[+a,n], Z[-a,-n] } for n = 0..32, then { Z[-a,n], Z[+a,-n] }; +0 and -0 are the same frequency, so
   //   m = 0 counts as -0 when n < 0 (the item (0, n) then finds Z[0,n], Z[0,-n] in its first two places) and
   //   n = 0 is written to the place of -0 as well (the one extra store below, by the wave d = 0).
   const int qa = (m <= 32 ? m : 64 - m) * QPITCH;     // m = 32: the dump row
-  const int pos_lo = m > 32 ? 2 : 0;                  // place of an output with n >= 0
-  const int pos_hi = (m > 32 || m == 0) ? 1 : 3;      // place of an output with n < 0
+  const int pos_lo = m > 32 ? QHALF : 0;                      // place of an output with n >= 0: first of its pair
+  const int pos_hi = (m > 32 || m == 0) ? 1 : QHALF + 1;      // place of an output with n < 0: second of its pair
   const int extra = d == 0 ? qa + pos_hi : 32 * QPITCH + 130;   // n = 0 again as -0; other waves: the dump row
 
   float2 accp[NIT][4], accm[NIT][4];
@@ -261,14 +263,14 @@ __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restri
     for (int j2 = 0; j2 < 8; ++j2) v[j2] = line[j2];
     fft8<false>(v);
 #pragma unroll
-    for (int k2 = 0; k2 < 4; ++k2) q[qa + 4 * (d + 8 * k2) + pos_lo] = v[k2];
+    for (int k2 = 0; k2 < 4; ++k2) q[qa + 2 * (d + 8 * k2) + pos_lo] = v[k2];
 #pragma unroll
-    for (int k2 = 4; k2 < 8; ++k2) q[qa + 4 * (64 - d - 8 * k2) + pos_hi] = v[k2];   // n = 32 (d = 0, k2 = 4) lands in the pad of the row
+    for (int k2 = 4; k2 < 8; ++k2) q[qa + 2 * (64 - d - 8 * k2) + pos_hi] = v[k2];   // n = 32 (d = 0, k2 = 4) lands in the pad of its half
     q[extra] = v[0];
   };
   auto accumulate = [&](const float2* q, int it) {
     const float4* src = reinterpret_cast<const float4*>(q + (adr[it] & 0x7fffffffu));
-    const float4 za = src[0], zb = src[1];              // Z[+a,n], Z[-a,-n] | Z[-a,n], Z[+a,-n]
+    const float4 za = src[0], zb = src[QHALF / 2];      // Z[+a,n], Z[-a,-n] | Z[-a,n], Z[+a,-n]
     const unsigned sb = adr[it] & 0x80000000u;
     // twice the separated planes (the table carries the factor 1/2):
     // P = Z[m,n] + conj Z[-m,-n],  P' = (Z[m,n] - conj Z[-m,-n]) / i, the latter times (-1)^n
@@ -595,8 +597,9 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
                                                             float* __restrict__ y, long nbatch, const float* __restrict__ bias, int nfeature) {
   using namespace fft64;
   __shared__ __attribute__((aligned(16))) float2 work[LDS_ELEMS];
-  __shared__ __attribute__((aligned(16))) float4 stg_p[NIT * THREADS];       // item i: its share of the bins [+a,n], [-a,-n]
-  __shared__ __attribute__((aligned(16))) float4 stg_m[NIT * THREADS];       //                              [-a,n], [+a,-n]
+  constexpr int STG_PADS = 144;                                              // one pad per row: sum of (4c+4) over the 8 degree groups
+  __shared__ __attribute__((aligned(16))) float4 stg_p[NIT * THREADS + STG_PADS];   // item (c, a, n): its share of the bins [+a,n], [-a,-n]
+  __shared__ __attribute__((aligned(16))) float4 stg_m[NIT * THREADS + STG_PADS];   //                                      [-a,n], [+a,-n]
   __shared__ float2 twl[64];
   const long z = volume_of_block(nbatch);
   if (z < 0) return;
@@ -608,6 +611,12 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
 
   float2 xp[NIT][4], xm[NIT][4];
   unsigned sgn = 0;                 // bit it = n odd for item it
+  // Where an item's share goes in the staging area: the rows of degree group c are (4c+5) entries apart (one pad per
+  // row), so that the threads of reduce() that walk down a column hit different banks.  Kept as the number of pads in
+  // front of the item (at most 144), four of them per word.
+  unsigned spad[(NIT + 3) / 4];
+#pragma unroll
+  for (int w = 0; w < (NIT + 3) / 4; ++w) spad[w] = 0;
   const __amdgpu_buffer_rsrc_t rr = make_rsrc(rec + (size_t)z * REC_F4, (unsigned)REC_BYTES);
   const __amdgpu_buffer_rsrc_t rt = make_rsrc(Tf, (unsigned)(PACKED_FLOATS * 4));
   const __amdgpu_buffer_rsrc_t ry = make_rsrc(y + (size_t)z * (N * N * N), N * N * N * 4);
@@ -616,8 +625,13 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
 #pragma unroll
   for (int it = 0; it < NA; ++it) {
     int c, a, n;
-    decode_item(it * THREADS + t, c, a, n);
+    const bool item = decode_item(it * THREADS + t, c, a, n);
     sgn |= (unsigned)(n & 1) << it;
+    {
+      constexpr int PADC[8] = {0, 4, 12, 24, 40, 60, 84, 112};      // pads in front of degree group c
+      const unsigned pad = item ? (unsigned)(a + PADC[c]) : (unsigned)STG_PADS;   // padding slots land behind the last item
+      spad[it >> 2] |= pad << (8 * (it & 3));
+    }
     const float4 v0 = buf_load_f32x4(rr, toff, (it * 4 + 0) * (THREADS * 16)), v1 = buf_load_f32x4(rr, toff, (it * 4 + 1) * (THREADS * 16));
     const float4 v2 = buf_load_f32x4(rr, toff, (it * 4 + 2) * (THREADS * 16)), v3 = buf_load_f32x4(rr, toff, (it * 4 + 3) * (THREADS * 16));
     xp[it][0] = make_float2(v0.x, v0.y); xp[it][1] = make_float2(v0.z, v0.w);
@@ -661,12 +675,13 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
     }
     const unsigned sb = ((sgn >> it) & 1u) << 31;
     Qp.x = flip(Qp.x, sb); Qp.y = flip(Qp.y, sb); Qm.x = flip(Qm.x, sb); Qm.y = flip(Qm.y, sb);
-    stg_p[it * THREADS + t] = make_float4(Sp.x - Qp.y, Sp.y + Qp.x, Sp.x + Qp.y, Qp.x - Sp.y);
-    stg_m[it * THREADS + t] = make_float4(Sm.x - Qm.y, Sm.y + Qm.x, Sm.x + Qm.y, Qm.x - Sm.y);
+    const unsigned pos = it * THREADS + t + ((spad[it >> 2] >> (8 * (it & 3))) & 0xffu);
+    stg_p[pos] = make_float4(Sp.x - Qp.y, Sp.y + Qp.x, Sp.x + Qp.y, Qp.x - Sp.y);
+    stg_m[pos] = make_float4(Sm.x - Qm.y, Sm.y + Qm.x, Sm.x + Qm.y, Qm.x - Sm.y);
   };
   // staging -> work (natural order): sum over the items c = max(a,n)/4 .. 7 of each column, in that order
   auto reduce = [&]() {
-    constexpr int OFF[8] = {0, 16, 80, 224, 480, 880, 1456, 2240};
+    constexpr int OFF[8] = {0, 20, 92, 248, 520, 940, 1540, 2352};    // sum of (4c'+4)(4c'+5) over c' < c
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const int a = ca[h], n = cn[h];
@@ -675,7 +690,7 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
 #pragma unroll
       for (int c = 0; c < 8; ++c) {
         if (c >= cmin && c < CMAX) {
-          const int i = OFF[c] + a * (4 * c + 4) + n;
+          const int i = OFF[c] + a * (4 * c + 5) + n;
           const float4 u0 = stg_p[i], u1 = stg_m[i];
           s0.x += u0.x; s0.y += u0.y; s0.z += u0.z; s0.w += u0.w;
           s1.x += u1.x; s1.y += u1.y; s1.z += u1.z; s1.w += u1.w;
