@@ -172,8 +172,6 @@ inline size_t scratch_bytes(long nbatch) { return (size_t)nbatch * REC_BYTES; }
 // contracted out of the other quad buffer, two items per stage.
 // ---------------------------------------------------------------------------------------------
 constexpr int QPITCH = 32 * 4 + 6;              // complex numbers per a-row of the quad layout; the pad takes the unused n = 32
-constexpr int QHALF = 66;                       // a row holds the pairs {Z[+a,n], Z[-a,-n]} for n = 0..32, then the pairs {Z[-a,n], Z[+a,-n]}:
-                                                // consecutive items (consecutive n) read consecutive 16-byte words of either half
 constexpr int QUAD_ELEMS = 33 * QPITCH;         // row 32 takes the unused m = 32
 // table registers: four slots, item it in slot it % 4; a slot is refilled right after its item has been used:
 //   after item 0, 1, 2: items 4, 5, 6 of the same plane pair;  after 3, 4, 5, 6: items 3, 0, 1, 2 of the next pair
@@ -201,16 +199,16 @@ __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restri
   for (int it = 0; it < NIT; ++it) {
     int c, a, n;
     decode_item(it * THREADS + t, c, a, n);
-    adr[it] = (unsigned)(a * QPITCH + 2 * n) | ((unsigned)(n & 1) << 31);
+    adr[it] = (unsigned)(a * QPITCH + 4 * n) | ((unsigned)(n & 1) << 31);
   }
   // where this thread's outputs of the last gamma stage go: row slot lo holds m = sigma(lo)
   const int m = sigma(lo);
-  // row a of a quad buffer: { Z[+a,n], Z[-a,-n] } for n = 0..32, then { Z[-a,n], Z[+a,-n] }; +0 and -0 are the same frequency, so
+  // quad[a][n] = { Z[+a,n], Z[-a,-n], Z[-a,n], Z[+a,-n] }; +0 and -0 are the same frequency, so
   //   m = 0 counts as -0 when n < 0 (the item (0, n) then finds Z[0,n], Z[0,-n] in its first two places) and
   //   n = 0 is written to the place of -0 as well (the one extra store below, by the wave d = 0).
   const int qa = (m <= 32 ? m : 64 - m) * QPITCH;     // m = 32: the dump row
-  const int pos_lo = m > 32 ? QHALF : 0;                      // place of an output with n >= 0: first of its pair
-  const int pos_hi = (m > 32 || m == 0) ? 1 : QHALF + 1;      // place of an output with n < 0: second of its pair
+  const int pos_lo = m > 32 ? 2 : 0;                  // place of an output with n >= 0
+  const int pos_hi = (m > 32 || m == 0) ? 1 : 3;      // place of an output with n < 0
   const int extra = d == 0 ? qa + pos_hi : 32 * QPITCH + 130;   // n = 0 again as -0; other waves: the dump row
 
   float2 accp[NIT][4], accm[NIT][4];
@@ -263,14 +261,14 @@ __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restri
     for (int j2 = 0; j2 < 8; ++j2) v[j2] = line[j2];
     fft8<false>(v);
 #pragma unroll
-    for (int k2 = 0; k2 < 4; ++k2) q[qa + 2 * (d + 8 * k2) + pos_lo] = v[k2];
+    for (int k2 = 0; k2 < 4; ++k2) q[qa + 4 * (d + 8 * k2) + pos_lo] = v[k2];
 #pragma unroll
-    for (int k2 = 4; k2 < 8; ++k2) q[qa + 2 * (64 - d - 8 * k2) + pos_hi] = v[k2];   // n = 32 (d = 0, k2 = 4) lands in the pad of its half
+    for (int k2 = 4; k2 < 8; ++k2) q[qa + 4 * (64 - d - 8 * k2) + pos_hi] = v[k2];   // n = 32 (d = 0, k2 = 4) lands in the pad of the row
     q[extra] = v[0];
   };
   auto accumulate = [&](const float2* q, int it) {
     const float4* src = reinterpret_cast<const float4*>(q + (adr[it] & 0x7fffffffu));
-    const float4 za = src[0], zb = src[QHALF / 2];      // Z[+a,n], Z[-a,-n] | Z[-a,n], Z[+a,-n]
+    const float4 za = src[0], zb = src[1];              // Z[+a,n], Z[-a,-n] | Z[-a,n], Z[+a,-n]
     const unsigned sb = adr[it] & 0x80000000u;
     // twice the separated planes (the table carries the factor 1/2):
     // P = Z[m,n] + conj Z[-m,-n],  P' = (Z[m,n] - conj Z[-m,-n]) / i, the latter times (-1)^n
