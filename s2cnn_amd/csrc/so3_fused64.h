@@ -171,8 +171,11 @@ inline size_t scratch_bytes(long nbatch) { return (size_t)nbatch * REC_BYTES; }
 // Z[+a,n], Z[-a,-n], Z[-a,n], Z[+a,-n], side by side at quad[a][n][0..3].  Meanwhile pair j is
 // contracted out of the other quad buffer, two items per stage.
 // ---------------------------------------------------------------------------------------------
-constexpr int QPITCH = 32 * 4 + 6;              // complex numbers per a-row of the quad layout; the pad takes the unused n = 32
+constexpr int QPITCH = 32 * 4 + 14;             // complex numbers per a-row of the quad layout: 33 quads (the unused n = 32 included) + room for the skew
 constexpr int QUAD_ELEMS = 33 * QPITCH;         // row 32 takes the unused m = 32
+// Row a starts 2 (a / 8) complex numbers late.  The last gamma stage writes the rows 8r + s (r = lane % 8) at once; a pitch
+// that keeps rows 16-byte aligned puts rows 8 apart into the same banks, the skew moves them 4 banks apart instead.
+__host__ __device__ constexpr int quad_row(int a) { return a * QPITCH + 2 * (a >> 3); }
 // table registers: four slots, item it in slot it % 4; a slot is refilled right after its item has been used:
 //   after item 0, 1, 2: items 4, 5, 6 of the same plane pair;  after 3, 4, 5, 6: items 3, 0, 1, 2 of the next pair
 __device__ constexpr int table_slot(int it) { return it & 3; }
@@ -199,14 +202,14 @@ __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restri
   for (int it = 0; it < NIT; ++it) {
     int c, a, n;
     decode_item(it * THREADS + t, c, a, n);
-    adr[it] = (unsigned)(a * QPITCH + 4 * n) | ((unsigned)(n & 1) << 31);
+    adr[it] = (unsigned)(quad_row(a) + 4 * n) | ((unsigned)(n & 1) << 31);
   }
   // where this thread's outputs of the last gamma stage go: row slot lo holds m = sigma(lo)
   const int m = sigma(lo);
   // quad[a][n] = { Z[+a,n], Z[-a,-n], Z[-a,n], Z[+a,-n] }; +0 and -0 are the same frequency, so
   //   m = 0 counts as -0 when n < 0 (the item (0, n) then finds Z[0,n], Z[0,-n] in its first two places) and
   //   n = 0 is written to the place of -0 as well (the one extra store below, by the wave d = 0).
-  const int qa = (m <= 32 ? m : 64 - m) * QPITCH;     // m = 32: the dump row
+  const int qa = quad_row(m <= 32 ? m : 64 - m);      // m = 32: the dump row
   const int pos_lo = m > 32 ? 2 : 0;                  // place of an output with n >= 0
   const int pos_hi = (m > 32 || m == 0) ? 1 : 3;      // place of an output with n < 0
   const int extra = d == 0 ? qa + pos_hi : 32 * QPITCH + 130;   // n = 0 again as -0; other waves: the dump row
