@@ -137,6 +137,31 @@ __device__ __forceinline__ void fft_pass(float2* buf, const float2* twl) {
   for (int j = 0; j < 8; ++j) line[j * stride] = v[j];
 }
 
+// The same pass in two halves, so that independent work can be placed between the LDS reads and their use.
+template <int P>
+__device__ __forceinline__ void fft_pass_load(const float2* buf, float2 (&v)[8]) {
+  using namespace fft64;
+  const int lo = threadIdx.x & 63, d = threadIdx.x >> 6;
+  const float2* line = P == 0 ? buf + lo * PITCH + d : P == 1 ? buf + lo * PITCH + 8 * d : P == 2 ? buf + lo + d * PITCH : buf + lo + 8 * d * PITCH;
+  constexpr int stride = P == 0 ? 8 : P == 1 ? 1 : P == 2 ? 8 * PITCH : PITCH;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) v[j] = line[j * stride];
+}
+template <bool INV, int P>
+__device__ __forceinline__ void fft_pass_finish(float2* buf, const float2* twl, float2 (&v)[8]) {
+  using namespace fft64;
+  const int lo = threadIdx.x & 63, d = threadIdx.x >> 6;
+  float2* line = P == 0 ? buf + lo * PITCH + d : P == 1 ? buf + lo * PITCH + 8 * d : P == 2 ? buf + lo + d * PITCH : buf + lo + 8 * d * PITCH;
+  constexpr int stride = P == 0 ? 8 : P == 1 ? 1 : P == 2 ? 8 * PITCH : PITCH;
+  fft8<INV>(v);
+  if (P == 0 || P == 2) {
+#pragma unroll
+    for (int j = 1; j < 8; ++j) v[j] = cmul(v[j], twl[8 * d + j]);
+  }
+#pragma unroll
+  for (int j = 0; j < 8; ++j) line[j * stride] = v[j];
+}
+
 template <bool INV>
 __device__ __forceinline__ void fill_twiddles(float2* twl) {
   if (threadIdx.x < 64) {
@@ -348,11 +373,19 @@ __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restri
       stage_c1(); S2CNN_FENCE();
       S2CNN_PLANES(0) S2CNN_PLANES(1)
       __syncthreads();
-      S2CNN_ACC(2, j, 6) S2CNN_PLANES(2) S2CNN_ACC(3, j + 1, 3) S2CNN_PLANES(3)
-      fft_pass<false, 3>(work, twl);
+      {
+        float2 fv[8];
+        fft_pass_load<3>(work, fv); S2CNN_FENCE();          // in flight during the two items
+        S2CNN_ACC(2, j, 6) S2CNN_PLANES(2) S2CNN_ACC(3, j + 1, 3) S2CNN_PLANES(3)
+        fft_pass_finish<false, 3>(work, twl, fv);
+      }
       __syncthreads();
-      S2CNN_ACC(4, j + 1, 0) S2CNN_ACC(5, j + 1, 1)
-      fft_pass<false, 0>(work, twl);
+      {
+        float2 fv[8];
+        fft_pass_load<0>(work, fv); S2CNN_FENCE();
+        S2CNN_ACC(4, j + 1, 0) S2CNN_ACC(5, j + 1, 1)
+        fft_pass_finish<false, 0>(work, twl, fv);
+      }
       __syncthreads();
       S2CNN_ACC(6, j + 1, 2)
       stage_r2(nxt);
