@@ -333,10 +333,10 @@ int fused_analysis(const float* x, const float* table, const float* packed_table
   }
   fused64::launch_analysis(b_out, st, x, Tf, rec, nbatch);
   if (real_basis)
-    hipLaunchKernelGGL(fused64::spectrum_scatter_real, dim3((unsigned)((nbatch + fused64::ZR - 1) / fused64::ZR), fused64::NIT * 32), dim3(256), 0, st,
+    hipLaunchKernelGGL(fused64::spectrum_scatter_real, dim3((unsigned)((nbatch + fused64::ZR - 1) / fused64::ZR), fused64::active_rounds(b_out) * 32), dim3(256), 0, st,
                        rec, out, b_out, nbatch);
   else
-    hipLaunchKernelGGL(fused64::spectrum_scatter, dim3((unsigned)((nbatch + fused64::ZT - 1) / fused64::ZT), fused64::NIT * 16), dim3(256), 0, st,
+    hipLaunchKernelGGL(fused64::spectrum_scatter, dim3((unsigned)((nbatch + fused64::ZT - 1) / fused64::ZT), fused64::active_rounds(b_out) * 16), dim3(256), 0, st,
                        rec, reinterpret_cast<float2*>(out), b_out, nbatch);
   return s2cnn::launch_status();
 }
@@ -355,10 +355,10 @@ int fused_synthesis(const float* xhat, const float* table, const float* packed_t
     Tf = dst;
   }
   if (real_basis)
-    hipLaunchKernelGGL(fused64::spectrum_gather_real, dim3((unsigned)((nbatch + fused64::ZR - 1) / fused64::ZR), fused64::NIT * 32), dim3(256), 0, st,
+    hipLaunchKernelGGL(fused64::spectrum_gather_real, dim3((unsigned)((nbatch + fused64::ZR - 1) / fused64::ZR), fused64::active_rounds(nl) * 32), dim3(256), 0, st,
                        xhat, rec, nl, nbatch);
   else
-    hipLaunchKernelGGL(fused64::spectrum_gather, dim3((unsigned)((nbatch + fused64::ZT - 1) / fused64::ZT), fused64::NIT * 16), dim3(256), 0, st,
+    hipLaunchKernelGGL(fused64::spectrum_gather, dim3((unsigned)((nbatch + fused64::ZT - 1) / fused64::ZT), fused64::active_rounds(nl) * 16), dim3(256), 0, st,
                        reinterpret_cast<const float2*>(xhat), rec, nl, nbatch);
   fused64::launch_synthesis(nl, st, rec, Tf, out, nbatch, bias, nfeature);
   return s2cnn::launch_status();

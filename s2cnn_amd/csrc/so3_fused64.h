@@ -408,7 +408,7 @@ __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restri
 
   const __amdgpu_buffer_rsrc_t rr = make_rsrc(rec + (size_t)z * REC_F4, (unsigned)REC_BYTES);
 #pragma unroll
-  for (int it = 0; it < NIT; ++it) {
+  for (int it = 0; it < NA; ++it) {            // the pass that follows reads these rounds only
     buf_store_f32x4(make_float4(accp[it][0].x, accp[it][0].y, accp[it][1].x, accp[it][1].y), rr, toff, (it * 4 + 0) * (THREADS * 16));
     buf_store_f32x4(make_float4(accp[it][2].x, accp[it][2].y, accp[it][3].x, accp[it][3].y), rr, toff, (it * 4 + 1) * (THREADS * 16));
     buf_store_f32x4(make_float4(accm[it][0].x, accm[it][0].y, accm[it][1].x, accm[it][1].y), rr, toff, (it * 4 + 2) * (THREADS * 16));
@@ -838,6 +838,9 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
   fft_pass<true, 2>(work, twl); __syncthreads();
   stage_c2_store(NJ - 1);
 }
+
+// item rounds that carry degrees below nl (the template argument NA of the kernels below)
+inline int active_rounds(int nl) { return nl <= 24 ? 3 : nl <= 28 ? 5 : NIT; }
 
 // Launchers: the instantiation whose item rounds cover the nl degrees present.
 inline void launch_analysis(int nl, hipStream_t st, const float* x, const float* Tf, float4* rec, long nbatch) {
