@@ -165,6 +165,48 @@ def measure_rows(torch, dev, with_cpu):
     return rows
 
 
+def measure_network(torch, dev, steps, warmup):
+    """The SHREC17-shaped network of BASELINE config 5 (S2Conv 6->100 b 128->32, ReLU, SO3Conv 100->100 b 32->22, ReLU,
+    SO3Conv 100->55 b 22->7, so3_integrate; batch 32, near-identity grids scaled by the bandwidth ratio), forward and
+    backward with respect to the weights, timed like the headline step; time inside library calls listed beside it."""
+    import math
+
+    import s2cnn_amd
+    from s2cnn_amd import _hip
+    g1 = s2cnn_amd.s2_near_identity_grid(max_beta=math.pi / 8 * 30 / 128, n_alpha=8, n_beta=3)
+    g2 = s2cnn_amd.so3_near_identity_grid(max_beta=math.pi / 8 * 30 / 32, max_gamma=2 * math.pi, n_alpha=8, n_beta=3, n_gamma=8)
+    g3 = s2cnn_amd.so3_near_identity_grid(max_beta=math.pi / 8 * 30 / 22, max_gamma=2 * math.pi, n_alpha=8, n_beta=3, n_gamma=8)
+    torch.manual_seed(8)
+    c1 = s2cnn_amd.S2Convolution(6, 100, 128, 32, g1).to(dev)
+    c2 = s2cnn_amd.SO3Convolution(100, 100, 32, 22, g2).to(dev)
+    c3 = s2cnn_amd.SO3Convolution(100, 55, 22, 7, g3).to(dev)
+    params = [q for c in (c1, c2, c3) for q in c.parameters()]
+    x = torch.rand(32, 6, 256, 256, device=dev)
+
+    def step():
+        for q in params:
+            q.grad = None
+        out = s2cnn_amd.so3_integrate(c3(torch.relu(c2(torch.relu(c1(x))))))
+        sum_of_squares(out).backward()
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / steps * 1e3
+    with _hip.KernelTimer() as kt:
+        step()
+        torch.cuda.synchronize()
+    calls = {k: round(sum(v), 3) for k, v in sorted(kt.summary().items(), key=lambda kv: -sum(kv[1]))}
+    torch.cuda.empty_cache()
+    return {"workload": "S2Conv 6->100 (b 128->32), SO3Conv 100->100 (32->22), SO3Conv 100->55 (22->7), integrate; batch 32, fwd+bwd (BASELINE config 5)",
+            "ms_per_step": round(ms, 3), "samples_per_s": round(32 / (ms * 1e-3), 1),
+            "library_ms": round(sum(calls.values()), 3), "library_calls_ms": calls}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -175,6 +217,7 @@ def main():
     ap.add_argument("--complex-product", action="store_true",
                     help="multiply complex spectra as the reference does instead of real-basis ones")
     ap.add_argument("--rows", action="store_true", help="also time every other op of the path (adds a `rows` object)")
+    ap.add_argument("--network", action="store_true", help="also time the SHREC17-shaped network (adds a `network` object)")
     ap.add_argument("--batch", type=int, default=16)
     ap.add_argument("--b", type=int, default=32)
     ap.add_argument("--features", type=int, default=64)
@@ -279,6 +322,8 @@ def main():
 
     if args.rows:
         result["rows"] = measure_rows(torch, dev, not args.no_cpu)
+    if args.network:
+        result["network"] = measure_network(torch, dev, args.steps, args.warmup)
 
     # ---- CPU baseline: the oracle (a restatement of the reference's CPU branches) on a bounded sample
     if not args.no_cpu:
