@@ -1,13 +1,13 @@
 """Headline benchmark: one SO3Convolution layer, forward + backward, fp32, b_in = b_out = 32,
 64 -> 64 features, batch 16, default near-identity grid (192 points), Kaiming-normal kernel,
-loss = sum(out^2) - BASELINE config "Single SO3Convolution layer".  One step = one forward +
+loss = sum(out^2) - benchmark config "Single SO3Convolution layer".  One step = one forward +
 backward over one synthetic batch that is already resident in HBM.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-fft]
 
 Prints ONE JSON line.  `roofline` is for the dominant kernel (the block-diagonal spectral
 product so3_mm, bound by the fp32 matrix cores), timed with events on the launch stream inside
-the timed steps; `so3_fft` reports the standalone SO(3) FFT round trip of BASELINE config 2
+the timed steps; `so3_fft` reports the standalone SO(3) FFT round trip of benchmark config 2
 against HBM bandwidth; `cpu_baseline` is the CPU oracle timed on this host on a bounded sample.
 """
 import argparse
@@ -31,7 +31,7 @@ MM_TRAFFIC_BYTES = {"s2cnn_so3_mm_real_fwd": 6.49e9 + 0.179e9, "s2cnn_so3_mm_rea
 
 
 def sum_of_squares(t):
-    """The loss of BASELINE config 4, sum(out^2), with its gradient 2 out written out by hand: one reduction pass
+    """The loss of benchmark config 4, sum(out^2), with its gradient 2 out written out by hand: one reduction pass
     forward and one elementwise pass backward over the 1 GiB output.  (Autograd through out * out or
     vector_norm(out)**2 is the same function with three to five passes, none of them the layer's.)"""
     import torch
@@ -66,7 +66,7 @@ def so3_fft_bytes(b_in, b_out, n):
 
 
 def measure_rows(torch, dev, with_cpu):
-    """Every other op of the path at its BASELINE-config size: GPU time (events on the launch stream), the
+    """Every other op of the path at its benchmark-config size: GPU time (events on the launch stream), the
     algorithmic bytes or flops, the roofline fraction, and the CPU oracle on a bounded sample beside it."""
     import s2cnn_amd
     from s2cnn_amd import _hip
@@ -166,7 +166,7 @@ def measure_rows(torch, dev, with_cpu):
 
 
 def measure_network(torch, dev, steps, warmup):
-    """The SHREC17-shaped network of BASELINE config 5 (S2Conv 6->100 b 128->32, ReLU, SO3Conv 100->100 b 32->22, ReLU,
+    """The SHREC17-shaped network of benchmark config 5 (S2Conv 6->100 b 128->32, ReLU, SO3Conv 100->100 b 32->22, ReLU,
     SO3Conv 100->55 b 22->7, so3_integrate; batch 32, near-identity grids scaled by the bandwidth ratio), forward and
     backward with respect to the weights, timed like the headline step; time inside library calls listed beside it."""
     import math
@@ -202,7 +202,7 @@ def measure_network(torch, dev, steps, warmup):
         torch.cuda.synchronize()
     calls = {k: round(sum(v), 3) for k, v in sorted(kt.summary().items(), key=lambda kv: -sum(kv[1]))}
     torch.cuda.empty_cache()
-    return {"workload": "S2Conv 6->100 (b 128->32), SO3Conv 100->100 (32->22), SO3Conv 100->55 (22->7), integrate; batch 32, fwd+bwd (BASELINE config 5)",
+    return {"workload": "S2Conv 6->100 (b 128->32), SO3Conv 100->100 (32->22), SO3Conv 100->55 (22->7), integrate; batch 32, fwd+bwd (benchmark config 5)",
             "ms_per_step": round(ms, 3), "samples_per_s": round(32 / (ms * 1e-3), 1),
             "library_ms": round(sum(calls.values()), 3), "library_calls_ms": calls}
 
@@ -291,11 +291,11 @@ def main():
         "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "SO3Convolution fwd+bwd, batch %d, %d->%d features, b_in=b_out=%d, 192-point "
-                               "near-identity grid, loss=sum(out^2) (BASELINE config 4)" % (B, F, F, b)},
+                               "near-identity grid, loss=sum(out^2) (benchmark config 4)" % (B, F, F, b)},
         "roofline": roofline, "kernels": kernels,
     }
 
-    # ---- standalone SO(3) FFT round trip (BASELINE config 2: [256, 64, 64, 64] -> [43680, 256, 2] -> back)
+    # ---- standalone SO(3) FFT round trip (benchmark config 2: [256, 64, 64, 64] -> [43680, 256, 2] -> back)
     if not args.no_fft:
         del x, layer
         torch.cuda.empty_cache()
@@ -313,7 +313,7 @@ def main():
         bytes_dir = so3_fft_bytes(b, b, n_fft)
         rt_ms = pc["s2cnn_so3_analysis"] + pc["s2cnn_so3_synthesis"]
         gbs = 2 * bytes_dir / (rt_ms * 1e-3) / 1e9
-        result["so3_fft"] = {"workload": "SO3_fft_real -> SO3_ifft_real, [256,64,64,64] fp32 (BASELINE config 2)",
+        result["so3_fft"] = {"workload": "SO3_fft_real -> SO3_ifft_real, [256,64,64,64] fp32 (benchmark config 2)",
                              "bound": "hbm", "bytes_round_trip": 2 * bytes_dir, "ms_round_trip": round(rt_ms, 4),
                              "analysis_ms": round(pc["s2cnn_so3_analysis"], 4), "synthesis_ms": round(pc["s2cnn_so3_synthesis"], 4),
                              "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4)}

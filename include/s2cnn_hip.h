@@ -185,6 +185,25 @@ int s2cnn_so3_synthesis_real_bias(const float *xhat, const float *table, const f
                                   void *workspace, size_t workspace_bytes,
                                   int b_in, int b_out, long nbatch,
                                   const float *bias, int nfeature, void *stream);
+/* Bias (may be NULL) and max(., 0) in the epilogue: out = relu(synthesis(xhat) + bias).  real_basis = 0: xhat as
+ * above; 1: the spectrum in the real basis, one float per entry (only where
+ * s2cnn_so3_real_basis_transform_available(b_in, b_out, 1)).  Replaces F.relu applied to the output of a
+ * convolution layer (examples/mnist/run.py:88-92, examples/shrec17/model.py:28-35) without its pass over the
+ * activations.
+ */
+int s2cnn_so3_synthesis_real_relu(const float *xhat, const float *table, const float *packed_table, float *out,
+                                  void *workspace, size_t workspace_bytes,
+                                  int b_in, int b_out, long nbatch,
+                                  const float *bias, int nfeature, int real_basis, void *stream);
+/* The adjoint side of it: analysis of the real signal that equals x where mask > 0 and 0 elsewhere (mask: a
+ * tensor of the shape of x, here the OUTPUT of the relu above, so that x * [mask > 0] is the gradient that
+ * autograd would pass through it).  Workspace and tables as for s2cnn_so3_analysis with complex_in = 0;
+ * real_basis = 1 writes the real-basis spectrum [nspec(b_out), nbatch] (only where
+ * s2cnn_so3_real_basis_transform_available(b_in, b_out, 0)).
+ */
+int s2cnn_so3_analysis_real_masked(const float *x, const float *mask, const float *table, const float *packed_table,
+                                   float *out, void *workspace, size_t workspace_bytes,
+                                   int b_in, int b_out, long nbatch, int real_basis, void *stream);
 
 /* ---- table repacking for the real-signal fast path of the two transforms above ------
  * The reference uploads its Wigner table once per (b, nl, weighted, device) and reuses it

@@ -18,4 +18,8 @@ inline long so3_nspec(long b) { return b * (4 * b * b - 1) / 3; }
 
 __host__ __device__ inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
+// max(v, 0) that keeps a NaN, and the factor by which the gradient of that function passes where its OUTPUT is m
+__device__ __forceinline__ float relu_f(float v) { return v < 0.f ? 0.f : v; }
+__device__ __forceinline__ float relu_pass(float g, float m) { return m <= 0.f ? 0.f : g; }
+
 }  // namespace s2cnn

@@ -45,7 +45,7 @@ __device__ inline void fill_twiddles(float2* w, int n2) {
 // ---------------------------------------------------------------------------------------
 template <bool CPLX>
 __global__ __launch_bounds__(256) void so3_plane_dft_fwd(const float* __restrict__ x, float2* __restrict__ X,
-                                                         int n2, int nb, int ztile) {
+                                                         int n2, int nb, int ztile, const float* __restrict__ mask) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
   const int MW = 2 * nb - 1;
   const int NW = CPLX ? MW : nb;
@@ -57,7 +57,12 @@ __global__ __launch_bounds__(256) void so3_plane_dft_fwd(const float* __restrict
   fill_twiddles(w, n2);
   const int nin = (CPLX ? 2 : 1) * n2 * n2;
   const float* src = x + pl * nin;
-  for (int i = threadIdx.x; i < nin; i += blockDim.x) plane[i] = src[i];
+  if (mask) {     // samples where the mask is not positive count as zero
+    const float* msk = mask + pl * nin;
+    for (int i = threadIdx.x; i < nin; i += blockDim.x) plane[i] = s2cnn::relu_pass(src[i], msk[i]);
+  } else {
+    for (int i = threadIdx.x; i < nin; i += blockDim.x) plane[i] = src[i];
+  }
   __syncthreads();
 
   // Y[alpha][ni] = sum_gamma x[alpha][gamma] w^(n gamma)
@@ -280,10 +285,13 @@ __global__ __launch_bounds__(256) void so3_plane_dft_inv(const float2* __restric
   }
 }
 
-// y[z, :] += bias[z % nfeature] for volumes of `vol` samples (only behind the plane kernel above, which has no epilogue)
-__global__ void add_bias_kernel(float* __restrict__ y, const float* __restrict__ bias, size_t vol, int nfeature, size_t total) {
-  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x)
-    y[i] += bias[(i / vol) % nfeature];
+// y[z, :] += bias[z % nfeature] for volumes of `vol` samples (bias may be NULL), then max(y, 0) if relu; only behind
+// the plane kernels that have no epilogue of their own
+__global__ void add_bias_kernel(float* __restrict__ y, const float* __restrict__ bias, size_t vol, int nfeature, size_t total, int relu) {
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+    const float v = y[i] + (bias ? bias[(i / vol) % nfeature] : 0.f);
+    y[i] = relu ? s2cnn::relu_f(v) : v;
+  }
 }
 
 // Real signals on the 64^3 grid go through the per-volume kernels of so3_fused64.h (the planes never leave the CU).
@@ -319,9 +327,9 @@ size_t round256(size_t n) { return (n + 255) & ~(size_t)255; }
 
 // Real signals on the 64^3 grid: per-volume kernel + the pass between its records and the spectral rows.
 // real_basis: the spectrum is stored in the real basis (one float per entry) instead of complex pairs.
-int fused_analysis(const float* x, const float* table, const float* packed_table, float* out, void* workspace,
+int fused_analysis(const float* x, const float* mask, const float* table, const float* packed_table, float* out, void* workspace,
                    size_t workspace_bytes, int b_out, long nbatch, bool real_basis, hipStream_t st) {
-  if (!s2cnn::aligned16(x)) return S2CNN_EALIGN;
+  if (!s2cnn::aligned16(x) || !s2cnn::aligned16(mask)) return S2CNN_EALIGN;
   const size_t need = round256(fused64::scratch_bytes(nbatch)) + fused64::PACKED_FLOATS * sizeof(float);
   if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
   float4* rec = static_cast<float4*>(workspace);
@@ -331,7 +339,7 @@ int fused_analysis(const float* x, const float* table, const float* packed_table
     hipLaunchKernelGGL(fused64::pack_table, dim3(1024), dim3(256), 0, st, table, dst, s2cnn::so3_nspec(b_out), b_out);
     Tf = dst;
   }
-  fused64::launch_analysis(b_out, st, x, Tf, rec, nbatch);
+  fused64::launch_analysis(b_out, st, x, mask, Tf, rec, nbatch);
   if (real_basis)
     hipLaunchKernelGGL(fused64::spectrum_scatter_real, dim3((unsigned)((nbatch + fused64::ZR - 1) / fused64::ZR), fused64::active_rounds(b_out) * 32), dim3(256), 0, st,
                        rec, out, b_out, nbatch);
@@ -342,7 +350,8 @@ int fused_analysis(const float* x, const float* table, const float* packed_table
 }
 
 int fused_synthesis(const float* xhat, const float* table, const float* packed_table, float* out, void* workspace,
-                    size_t workspace_bytes, int b_in, long nbatch, bool real_basis, const float* bias, int nfeature, hipStream_t st) {
+                    size_t workspace_bytes, int b_in, long nbatch, bool real_basis, const float* bias, int nfeature, int relu,
+                    hipStream_t st) {
   if (!s2cnn::aligned16(out)) return S2CNN_EALIGN;
   const int nl = b_in < 32 ? b_in : 32;
   const size_t need = round256(fused64::scratch_bytes(nbatch)) + fused64::PACKED_FLOATS * sizeof(float);
@@ -360,7 +369,7 @@ int fused_synthesis(const float* xhat, const float* table, const float* packed_t
   else
     hipLaunchKernelGGL(fused64::spectrum_gather, dim3((unsigned)((nbatch + fused64::ZT - 1) / fused64::ZT), fused64::active_rounds(nl) * 16), dim3(256), 0, st,
                        reinterpret_cast<const float2*>(xhat), rec, nl, nbatch);
-  fused64::launch_synthesis(nl, st, rec, Tf, out, nbatch, bias, nfeature);
+  fused64::launch_synthesis(nl, st, rec, Tf, out, nbatch, bias, nfeature, relu);
   return s2cnn::launch_status();
 }
 
@@ -376,7 +385,7 @@ extern "C" int s2cnn_so3_analysis_real_basis(const float* x, const float* table,
   if (!x || !table || !out || !sizes_ok(b_in, b_out, nbatch)) return S2CNN_EINVAL;
   if (!fused_path(b_in, b_out, 0, false)) return S2CNN_EINVAL;
   if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
-  return fused_analysis(x, table, packed_table, out, workspace, workspace_bytes, b_out, nbatch, true, static_cast<hipStream_t>(stream));
+  return fused_analysis(x, nullptr, table, packed_table, out, workspace, workspace_bytes, b_out, nbatch, true, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int s2cnn_so3_synthesis_real_basis(const float* r, const float* table, const float* packed_table, float* out,
@@ -386,7 +395,7 @@ extern "C" int s2cnn_so3_synthesis_real_basis(const float* r, const float* table
   if (bias && (nfeature < 1 || nbatch % nfeature != 0)) return S2CNN_EINVAL;
   if (!fused_path(b_out, b_in, 0, true)) return S2CNN_EINVAL;
   if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
-  return fused_synthesis(r, table, packed_table, out, workspace, workspace_bytes, b_in, nbatch, true, bias, bias ? nfeature : 1,
+  return fused_synthesis(r, table, packed_table, out, workspace, workspace_bytes, b_in, nbatch, true, bias, bias ? nfeature : 1, 0,
                          static_cast<hipStream_t>(stream));
 }
 
@@ -422,15 +431,16 @@ extern "C" size_t s2cnn_so3_synthesis_workspace(int b_in, int b_out, long nbatch
   return round256(ws_bytes(b_out, b_in, nbatch, complex_out, true)) + packed_bytes(b_out, b_in, complex_out, true);
 }
 
-extern "C" int s2cnn_so3_analysis(const float* x, const float* table, const float* packed_table, float* out,
-                                  void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
-                                  int complex_in, void* stream) {
-  if (!x || !table || !out || !sizes_ok(b_in, b_out, nbatch)) return S2CNN_EINVAL;
+namespace {
+// mask: NULL, or (real signals only) a tensor of the shape of x whose positive entries select the samples that count
+int analysis_impl(const float* x, const float* mask, const float* table, const float* packed_table, float* out,
+                  void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch, int complex_in, void* stream) {
+  if (!x || !table || !out || !sizes_ok(b_in, b_out, nbatch) || (mask && complex_in)) return S2CNN_EINVAL;
   if (!s2cnn::aligned8(out) || (complex_in && !s2cnn::aligned8(x))) return S2CNN_EALIGN;
   if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (fused_path(b_in, b_out, complex_in, false))
-    return fused_analysis(x, table, packed_table, out, workspace, workspace_bytes, b_out, nbatch, false, st);
+    return fused_analysis(x, mask, table, packed_table, out, workspace, workspace_bytes, b_out, nbatch, false, st);
   const size_t need = s2cnn_so3_analysis_workspace(b_in, b_out, nbatch, complex_in);
   if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
   const int n2 = 2 * b_in, nb = b_in < b_out ? b_in : b_out;
@@ -439,23 +449,23 @@ extern "C" int s2cnn_so3_analysis(const float* x, const float* table, const floa
   const size_t lds = sizeof(float) * (2 * n2 + (complex_in ? 2 : 1) * n2 * n2 + 2 * n2 * NW);
   const unsigned planes = (unsigned)(nbatch * n2);
   const bool tiled = packed_bytes(b_in, b_out, complex_in, false) != 0;
-  const bool x16 = s2cnn::aligned16(x);
+  const bool x16 = s2cnn::aligned16(x) && s2cnn::aligned16(mask);
   const plane_real::Plan plan = complex_in ? plane_real::Plan{0, 0, 0, 0} : plane_real::plan_fwd(n2, nb, planes);
   if (lds > 160 * 1024 && plan.pl == 0) return S2CNN_EINVAL;
   if (complex_in) {
     if (lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)so3_plane_dft_fwd<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    hipLaunchKernelGGL(so3_plane_dft_fwd<true>, dim3(planes), dim3(256), lds, st, x, X, n2, nb, 0);
+    hipLaunchKernelGGL(so3_plane_dft_fwd<true>, dim3(planes), dim3(256), lds, st, x, X, n2, nb, 0, nullptr);
   } else if (n2 == 64 && x16) {
     const long npairs = nbatch * 32;
     hipLaunchKernelGGL(fft64::plane_fft64_fwd, dim3((unsigned)(npairs < 2048 ? npairs : 2048)), dim3(fft64::THREADS), 0, st, x, X, npairs, nb,
-                       tiled ? wigner_tiled::ZT : 0);
+                       tiled ? wigner_tiled::ZT : 0, mask);
   } else if (plan.pl > 0) {
     if (plan.lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)plane_real::plane_dft_fwd, hipFuncAttributeMaxDynamicSharedMemorySize, (int)plan.lds);
     hipLaunchKernelGGL(plane_real::plane_dft_fwd, dim3((planes + plan.pl - 1) / plan.pl), dim3(plan.nt), plan.lds, st, x, X, n2, nb,
-                       tiled ? wigner_tiled::ZT : 0, (long)planes, plan.pl, plan.alias);
+                       tiled ? wigner_tiled::ZT : 0, (long)planes, plan.pl, plan.alias, mask);
   } else {
     if (lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)so3_plane_dft_fwd<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    hipLaunchKernelGGL(so3_plane_dft_fwd<false>, dim3(planes), dim3(256), lds, st, x, X, n2, nb, tiled ? wigner_tiled::ZT : 0);
+    hipLaunchKernelGGL(so3_plane_dft_fwd<false>, dim3(planes), dim3(256), lds, st, x, X, n2, nb, tiled ? wigner_tiled::ZT : 0, mask);
   }
   int rc = s2cnn::launch_status();
   if (rc) return rc;
@@ -482,17 +492,17 @@ extern "C" int s2cnn_so3_analysis(const float* x, const float* table, const floa
   return s2cnn::launch_status();
 }
 
-namespace {
 int synthesis_impl(const float* xhat, const float* table, const float* packed_table, float* out, void* workspace,
                    size_t workspace_bytes, int b_in, int b_out, long nbatch, int complex_out, const float* bias, int nfeature,
-                   void* stream) {
+                   int relu, void* stream) {
   if (!xhat || !table || !out || !sizes_ok(b_out, b_in, nbatch)) return S2CNN_EINVAL;
   if (bias && (complex_out || nfeature < 1 || nbatch % nfeature != 0)) return S2CNN_EINVAL;
+  if (relu && complex_out) return S2CNN_EINVAL;
   if (!s2cnn::aligned8(xhat) || (complex_out && !s2cnn::aligned8(out))) return S2CNN_EALIGN;
   if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (fused_path(b_out, b_in, complex_out, true))
-    return fused_synthesis(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, nbatch, false, bias, bias ? nfeature : 1, st);
+    return fused_synthesis(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, nbatch, false, bias, bias ? nfeature : 1, relu, st);
   const size_t need = s2cnn_so3_synthesis_workspace(b_in, b_out, nbatch, complex_out);
   if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
   const int n2 = 2 * b_out, nb = b_in < b_out ? b_in : b_out;
@@ -530,28 +540,59 @@ int synthesis_impl(const float* xhat, const float* table, const float* packed_ta
   } else if (plan.pl > 0) {
     if (plan.lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)plane_real::plane_dft_inv, hipFuncAttributeMaxDynamicSharedMemorySize, (int)plan.lds);
     hipLaunchKernelGGL(plane_real::plane_dft_inv, dim3((planes + plan.pl - 1) / plan.pl), dim3(plan.nt), plan.lds, st, S, out, n2, nb,
-                       (long)planes, plan.pl, plan.alias, bias, bias ? nfeature : 1);
+                       (long)planes, plan.pl, plan.alias, relu, bias, bias ? nfeature : 1);
     return s2cnn::launch_status();
   } else {
     if (lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)so3_plane_dft_inv<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     hipLaunchKernelGGL(so3_plane_dft_inv<false>, dim3(planes), dim3(256), lds, st, S, out, n2, nb);
   }
-  if (bias) {
+  if (bias || relu) {
     const size_t vol = (size_t)n2 * n2 * n2;
-    hipLaunchKernelGGL(add_bias_kernel, dim3(2048), dim3(256), 0, st, out, bias, vol, nfeature, vol * nbatch);
+    hipLaunchKernelGGL(add_bias_kernel, dim3(2048), dim3(256), 0, st, out, bias, vol, bias ? nfeature : 1, vol * nbatch, relu);
   }
   return s2cnn::launch_status();
 }
 }  // namespace
 
+extern "C" int s2cnn_so3_analysis(const float* x, const float* table, const float* packed_table, float* out,
+                                  void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
+                                  int complex_in, void* stream) {
+  return analysis_impl(x, nullptr, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, complex_in, stream);
+}
+
 extern "C" int s2cnn_so3_synthesis(const float* xhat, const float* table, const float* packed_table, float* out,
                                    void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
                                    int complex_out, void* stream) {
-  return synthesis_impl(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, complex_out, nullptr, 1, stream);
+  return synthesis_impl(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, complex_out, nullptr, 1, 0, stream);
 }
 
 extern "C" int s2cnn_so3_synthesis_real_bias(const float* xhat, const float* table, const float* packed_table, float* out,
                                              void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
                                              const float* bias, int nfeature, void* stream) {
-  return synthesis_impl(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, 0, bias, nfeature, stream);
+  return synthesis_impl(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, 0, bias, nfeature, 0, stream);
+}
+
+extern "C" int s2cnn_so3_synthesis_real_relu(const float* xhat, const float* table, const float* packed_table, float* out,
+                                             void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
+                                             const float* bias, int nfeature, int real_basis, void* stream) {
+  if (!real_basis)
+    return synthesis_impl(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, 0, bias, nfeature, 1, stream);
+  if (!xhat || !table || !out || !sizes_ok(b_out, b_in, nbatch)) return S2CNN_EINVAL;
+  if (bias && (nfeature < 1 || nbatch % nfeature != 0)) return S2CNN_EINVAL;
+  if (!fused_path(b_out, b_in, 0, true)) return S2CNN_EINVAL;
+  if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
+  return fused_synthesis(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, nbatch, true, bias, bias ? nfeature : 1, 1,
+                         static_cast<hipStream_t>(stream));
+}
+
+extern "C" int s2cnn_so3_analysis_real_masked(const float* x, const float* mask, const float* table, const float* packed_table,
+                                              float* out, void* workspace, size_t workspace_bytes, int b_in, int b_out,
+                                              long nbatch, int real_basis, void* stream) {
+  if (!mask) return S2CNN_EINVAL;
+  if (!real_basis)
+    return analysis_impl(x, mask, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, 0, stream);
+  if (!x || !table || !out || !sizes_ok(b_in, b_out, nbatch)) return S2CNN_EINVAL;
+  if (!fused_path(b_in, b_out, 0, false)) return S2CNN_EINVAL;
+  if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
+  return fused_analysis(x, mask, table, packed_table, out, workspace, workspace_bytes, b_out, nbatch, true, static_cast<hipStream_t>(stream));
 }

@@ -207,9 +207,10 @@ __device__ constexpr int table_slot(int it) { return it & 3; }
 
 // NA: item rounds that carry degrees below the output bandwidth (items are ordered by degree group, so a truncated
 // spectrum leaves the later rounds without work: NA = 3 covers l < 24, 5 covers l < 28, 7 everything).
-template <int NA>
-__global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restrict__ x, const float* __restrict__ Tf,
-                                                           float4* __restrict__ rec, long nbatch) {
+// MASKED: the signal is x where mask > 0 and zero elsewhere (mask: a tensor of the shape of x).
+template <int NA, bool MASKED>
+__global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restrict__ x, const float* __restrict__ mask,
+                                                           const float* __restrict__ Tf, float4* __restrict__ rec, long nbatch) {
   using namespace fft64;
   __shared__ __attribute__((aligned(16))) float2 work[LDS_ELEMS];
   __shared__ __attribute__((aligned(16))) float2 quad[2][QUAD_ELEMS];
@@ -246,10 +247,12 @@ __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restri
     for (int u = 0; u < 4; ++u) { accp[it][u] = make_float2(0.f, 0.f); accm[it][u] = make_float2(0.f, 0.f); }
 
   const __amdgpu_buffer_rsrc_t rx = make_rsrc(x + (size_t)z * (N * N * N), N * N * N * 4);
+  const __amdgpu_buffer_rsrc_t rm = make_rsrc((MASKED ? mask : x) + (size_t)z * (N * N * N), N * N * N * 4);
   const __amdgpu_buffer_rsrc_t rt = make_rsrc(Tf, (unsigned)(PACKED_FLOATS * 4));
   const unsigned xoff = (d * N + lo) * 4;        // + (beta * 4096 + j1 * 512) * 4: row alpha = 8 j1 + d, column gamma = lo
   const unsigned toff = t * 16;
   float pa[8], pb[8];
+  float ma[MASKED ? 8 : 1], mb[MASKED ? 8 : 1];
   float4 t1[4], t2[4];
 
   auto load_planes = [&](int j) {            // planes j and 63-j: one full row (256 bytes) per wave and load
@@ -257,6 +260,10 @@ __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restri
     for (int j1 = 0; j1 < 8; ++j1) {
       pa[j1] = buf_load_f32(rx, xoff, (j * 4096 + j1 * 512) * 4);
       pb[j1] = buf_load_f32(rx, xoff, ((63 - j) * 4096 + j1 * 512) * 4);
+      if constexpr (MASKED) {
+        ma[j1] = buf_load_f32(rm, xoff, (j * 4096 + j1 * 512) * 4);
+        mb[j1] = buf_load_f32(rm, xoff, ((63 - j) * 4096 + j1 * 512) * 4);
+      }
     }
   };
   auto load_planes_part = [&](int j, int g) {   // a quarter of load_planes
@@ -264,6 +271,10 @@ __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restri
     for (int j1 = 2 * g; j1 < 2 * g + 2; ++j1) {
       pa[j1] = buf_load_f32(rx, xoff, (j * 4096 + j1 * 512) * 4);
       pb[j1] = buf_load_f32(rx, xoff, ((63 - j) * 4096 + j1 * 512) * 4);
+      if constexpr (MASKED) {
+        ma[j1] = buf_load_f32(rm, xoff, (j * 4096 + j1 * 512) * 4);
+        mb[j1] = buf_load_f32(rm, xoff, ((63 - j) * 4096 + j1 * 512) * 4);
+      }
     }
   };
   auto load_table = [&](int j, int it) {
@@ -274,7 +285,10 @@ __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restri
   auto stage_c1 = [&]() {
     float2 v[8];
 #pragma unroll
-    for (int j1 = 0; j1 < 8; ++j1) v[j1] = make_float2(pa[j1], pb[j1]);
+    for (int j1 = 0; j1 < 8; ++j1) {
+      if constexpr (MASKED) v[j1] = make_float2(s2cnn::relu_pass(pa[j1], ma[j1]), s2cnn::relu_pass(pb[j1], mb[j1]));
+      else v[j1] = make_float2(pa[j1], pb[j1]);
+    }
     fft8<false>(v);
 #pragma unroll
     for (int k = 1; k < 8; ++k) v[k] = cmul(v[k], twl[8 * d + k]);
@@ -625,10 +639,12 @@ __global__ __launch_bounds__(256) void spectrum_gather_real(const float* __restr
 // Sums are formed in a fixed order: results are reproducible bit for bit.
 // ---------------------------------------------------------------------------------------------
 // bias: NULL, or one value per feature added to every sample of volume z (feature = z % nfeature)
+// relu: nonzero = negative samples (after the bias) are stored as zero
 // NA as in analysis_kernel; CMAX: degree groups c < CMAX carry degrees of the input (6 for NA = 3, 7 for 5, 8 for 7)
 template <int NA, int CMAX>
 __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __restrict__ rec, const float* __restrict__ Tf,
-                                                            float* __restrict__ y, long nbatch, const float* __restrict__ bias, int nfeature) {
+                                                            float* __restrict__ y, long nbatch, const float* __restrict__ bias, int nfeature,
+                                                            int relu) {
   using namespace fft64;
   __shared__ __attribute__((aligned(16))) float2 work[LDS_ELEMS];
   constexpr int STG_PADS = 144;                                              // one pad per row: sum of (4c+4) over the 8 degree groups
@@ -753,6 +769,10 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
     float ra[8], rb[8];
 #pragma unroll
     for (int k = 0; k < 8; ++k) { ra[k] = v[k].x + bz; rb[k] = v[k].y + bz; }
+    if (relu) {
+#pragma unroll
+      for (int k = 0; k < 8; ++k) { ra[k] = s2cnn::relu_f(ra[k]); rb[k] = s2cnn::relu_f(rb[k]); }
+    }
     quad_transpose(ra[0], ra[1], ra[2], ra[3]); quad_transpose(ra[4], ra[5], ra[6], ra[7]);
     quad_transpose(rb[0], rb[1], rb[2], rb[3]); quad_transpose(rb[4], rb[5], rb[6], rb[7]);
     // lane (q, i) = (lo / 4, lo % 4) now holds columns 4q..4q+3 of the rows d + 8 i and d + 8 (4 + i)
@@ -843,19 +863,26 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
 inline int active_rounds(int nl) { return nl <= 24 ? 3 : nl <= 28 ? 5 : NIT; }
 
 // Launchers: the instantiation whose item rounds cover the nl degrees present.
-inline void launch_analysis(int nl, hipStream_t st, const float* x, const float* Tf, float4* rec, long nbatch) {
+template <bool MASKED>
+inline void launch_analysis_m(int nl, hipStream_t st, const float* x, const float* mask, const float* Tf, float4* rec, long nbatch) {
   const dim3 grid(grid_size(nbatch)), block(THREADS);
-  if (nl <= 24) hipLaunchKernelGGL(analysis_kernel<3>, grid, block, 0, st, x, Tf, rec, nbatch);
-  else if (nl <= 28) hipLaunchKernelGGL(analysis_kernel<5>, grid, block, 0, st, x, Tf, rec, nbatch);
-  else hipLaunchKernelGGL(analysis_kernel<7>, grid, block, 0, st, x, Tf, rec, nbatch);
+  if (nl <= 24) hipLaunchKernelGGL((analysis_kernel<3, MASKED>), grid, block, 0, st, x, mask, Tf, rec, nbatch);
+  else if (nl <= 28) hipLaunchKernelGGL((analysis_kernel<5, MASKED>), grid, block, 0, st, x, mask, Tf, rec, nbatch);
+  else hipLaunchKernelGGL((analysis_kernel<7, MASKED>), grid, block, 0, st, x, mask, Tf, rec, nbatch);
+}
+
+// mask: NULL, or the tensor whose positive entries select the samples of x that count
+inline void launch_analysis(int nl, hipStream_t st, const float* x, const float* mask, const float* Tf, float4* rec, long nbatch) {
+  if (mask) launch_analysis_m<true>(nl, st, x, mask, Tf, rec, nbatch);
+  else launch_analysis_m<false>(nl, st, x, nullptr, Tf, rec, nbatch);
 }
 
 inline void launch_synthesis(int nl, hipStream_t st, const float4* rec, const float* Tf, float* y, long nbatch, const float* bias,
-                             int nfeature) {
+                             int nfeature, int relu) {
   const dim3 grid(grid_size(nbatch)), block(THREADS);
-  if (nl <= 24) hipLaunchKernelGGL((synthesis_kernel<3, 6>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature);
-  else if (nl <= 28) hipLaunchKernelGGL((synthesis_kernel<5, 7>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature);
-  else hipLaunchKernelGGL((synthesis_kernel<7, 8>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature);
+  if (nl <= 24) hipLaunchKernelGGL((synthesis_kernel<3, 6>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu);
+  else if (nl <= 28) hipLaunchKernelGGL((synthesis_kernel<5, 7>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu);
+  else hipLaunchKernelGGL((synthesis_kernel<7, 8>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu);
 }
 
 }  // namespace fused64

@@ -107,7 +107,7 @@ struct TileLoader {
     }
   }
 
-  __device__ void init(const float* base_l, int L_, int MNI_, int KI_, int tile0) {
+  __device__ __forceinline__ void init(const float* base_l, int L_, int MNI_, int KI_, int tile0) {
     base = base_l; MNI = MNI_; KI = KI_; L = L_;
     const int t = threadIdx.x;
     const int blk_elems = MNI * KI;
@@ -314,7 +314,7 @@ __host__ __device__ inline void tile_counts(int L, int RI, int CI, int& tm, int&
   slots = tm * tn;
 }
 
-template <int MODE, int VEC, bool FAST>
+template <int MODE, int VA, int VB, bool FAST>
 __global__ __launch_bounds__(NT) void so3_block_mm_real_kernel(MmParams p) {
   typedef Cfg<MODE> C_;
 
@@ -335,8 +335,8 @@ __global__ __launch_bounds__(NT) void so3_block_mm_real_kernel(MmParams p) {
   const size_t L0 = (size_t)l * (4 * l * l - 1) / 3;
   const int M = L * p.RI, N = L * p.CI;
 
-  TileLoader<C_::A_KC, C_::A_MNMAJ, TM, VEC, FAST> la;
-  TileLoader<C_::B_KC, C_::B_MNMAJ, TN, VEC, FAST> lb;
+  TileLoader<C_::A_KC, C_::A_MNMAJ, TM, VA, FAST> la;
+  TileLoader<C_::B_KC, C_::B_MNMAJ, TN, VB, FAST> lb;
   la.init(p.A + L0 * p.RI * p.KI, L, p.RI, p.KI, tile_m);
   lb.init(p.B + L0 * p.CI * p.KI, L, p.CI, p.KI, tile_n);
 
@@ -428,19 +428,19 @@ int run(const float* a, const float* b, float* c, int nl, int RI, int CI, int KI
   if (grid < 1) return S2CNN_EINVAL;
   MmParams p{a, b, c, nl, RI, CI, KI};
   typedef Cfg<MODE> C_;
-  // four floats per access need the fast index of each operand to be a multiple of 4 and 16-byte bases
-  const bool a4 = (C_::A_KC ? KI : RI) % 4 == 0;
-  const bool b4 = (C_::B_KC ? KI : CI) % 4 == 0;
-  const bool vec4 = a4 && b4 && s2cnn::aligned16(a) && s2cnn::aligned16(b);
+  // four floats per access need the fast index of the operand to be a multiple of 4 and a 16-byte base
+  const bool a4 = (C_::A_KC ? KI : RI) % 4 == 0 && s2cnn::aligned16(a);
+  const bool b4 = (C_::B_KC ? KI : CI) % 4 == 0 && s2cnn::aligned16(b);
   hipStream_t st = static_cast<hipStream_t>(stream);
   // the fast loaders address a degree with 32-bit byte offsets
-  const bool fast = vec4 && (KI % TK == 0 || TK % KI == 0) && Lmax * Lmax * RI * KI < (1L << 30) && Lmax * Lmax * CI * KI < (1L << 30);
-  if (fast)
-    hipLaunchKernelGGL((so3_block_mm_real_kernel<MODE, 4, true>), dim3(grid), dim3(NT), 0, st, p);
-  else if (vec4)
-    hipLaunchKernelGGL((so3_block_mm_real_kernel<MODE, 4, false>), dim3(grid), dim3(NT), 0, st, p);
-  else
-    hipLaunchKernelGGL((so3_block_mm_real_kernel<MODE, 1, false>), dim3(grid), dim3(NT), 0, st, p);
+  const bool fast = a4 && b4 && (KI % TK == 0 || TK % KI == 0) && Lmax * Lmax * RI * KI < (1L << 30) && Lmax * Lmax * CI * KI < (1L << 30);
+#define S2CNN_LAUNCH(VA, VB, FAST) hipLaunchKernelGGL((so3_block_mm_real_kernel<MODE, VA, VB, FAST>), dim3(grid), dim3(NT), 0, st, p)
+  if (fast) S2CNN_LAUNCH(4, 4, true);
+  else if (a4 && b4) S2CNN_LAUNCH(4, 4, false);
+  else if (a4) S2CNN_LAUNCH(4, 1, false);
+  else if (b4) S2CNN_LAUNCH(1, 4, false);
+  else S2CNN_LAUNCH(1, 1, false);
+#undef S2CNN_LAUNCH
   return s2cnn::launch_status();
 }
 

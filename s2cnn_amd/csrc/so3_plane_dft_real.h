@@ -27,6 +27,7 @@
 // synthesis leave the LDS as one contiguous run of 16-byte stores instead of four-byte scatters.
 #pragma once
 #include <hip/hip_runtime.h>
+#include "common.h"
 #include "dft_common.h"
 
 namespace plane_real {
@@ -109,8 +110,9 @@ constexpr int LOADS = 8;   // global loads a thread has in flight while it stage
 // analysis: x [nplanes][n2][n2] -> X, laid out [plane][mi][ni] (ztile = 0) or
 // [z / Z][mi][beta][z % Z][ni] (ztile = Z, plane = z n2 + beta); mi = m + nb-1, ni = n.
 // ---------------------------------------------------------------------------------------------------
+// mask: NULL, or a tensor of the shape of x; samples of x where it is not positive count as zero
 __global__ __launch_bounds__(NT_MAX) void plane_dft_fwd(const float* __restrict__ x, float2* __restrict__ X, int n2, int nb,
-                                                        int ztile, long nplanes, int PL, int alias) {
+                                                        int ztile, long nplanes, int PL, int alias, const float* __restrict__ mask) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
   const int h = n2 / 2, nbp = pad(nb, 4), ns = pad(n2, 4);
   float2* tab = reinterpret_cast<float2*>(smem);                      // [h+1][nbp]
@@ -129,6 +131,7 @@ __global__ __launch_bounds__(NT_MAX) void plane_dft_fwd(const float* __restrict_
     const int hg = h + 1, total = PL * n2 * hg;
     const long rows_valid = (nplanes - plane0) * n2;
     const float* src = x + (size_t)plane0 * n2 * n2;
+    const float* msk = mask ? mask + (size_t)plane0 * n2 * n2 : nullptr;
     const float inv_n2 = 1.0f / (float)n2;
     Walk2 wk;
     wk.init(t, NT, hg);
@@ -143,8 +146,10 @@ __global__ __launch_bounds__(NT_MAX) void plane_dft_fwd(const float* __restrict_
         const bool valid = live && R < rows_valid;
         const bool paired = g > 0 && g < h;
         const int o1 = valid ? R * n2 + g : 0;
+        const int o2 = valid && paired ? R * n2 + n2 - g : o1;
         v1[u] = src[o1];
-        v2[u] = src[valid && paired ? R * n2 + n2 - g : o1];
+        v2[u] = src[o2];
+        if (msk) { v1[u] = s2cnn::relu_pass(v1[u], msk[o1]); v2[u] = s2cnn::relu_pass(v2[u], msk[o2]); }
         if (!valid) v1[u] = v2[u] = 0.f;
         if (!paired) v2[u] = 0.f;
         else pmask |= 1u << u;
@@ -258,8 +263,9 @@ __global__ __launch_bounds__(NT_MAX) void plane_dft_fwd(const float* __restrict_
 // synthesis: S [nplanes][2nb-1][nb] -> y [nplanes][n2][n2]
 // ---------------------------------------------------------------------------------------------------
 // bias: NULL, or nfeature values; bias[z % nfeature] is added to every sample of volume z = plane / n2
+// relu: nonzero = negative samples (after the bias) are stored as zero
 __global__ __launch_bounds__(NT_MAX) void plane_dft_inv(const float2* __restrict__ S, float* __restrict__ y, int n2, int nb,
-                                                        long nplanes, int PL, int alias, const float* __restrict__ bias,
+                                                        long nplanes, int PL, int alias, int relu, const float* __restrict__ bias,
                                                         int nfeature) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
   const int h = n2 / 2, hp = pad(h + 1, 4), nb2 = pad(nb, 2), npp = pad(h + 1, 2);
@@ -387,6 +393,7 @@ __global__ __launch_bounds__(NT_MAX) void plane_dft_inv(const float2* __restrict
     }
     if (!active || pl >= nplanes) continue;
     const float bz = bias ? bias[(int)(pl / n2) % nfeature] : 0.f;
+    auto act = [relu](float v) { return relu ? s2cnn::relu_f(v) : v; };
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int a = 2 * pb + i;
@@ -399,12 +406,12 @@ __global__ __launch_bounds__(NT_MAX) void plane_dft_inv(const float2* __restrict
         const bool mirror_g = g > 0 && g < h;
         cc[i][k] += bz;
         const float yc = cc[i][k] + sc[i][k], ys = cs[i][k] + ss[i][k];
-        dst[a * n2 + g] = yc - ys;
-        if (mirror_g) dst[a * n2 + n2 - g] = yc + ys;
+        dst[a * n2 + g] = act(yc - ys);
+        if (mirror_g) dst[a * n2 + n2 - g] = act(yc + ys);
         if (mirror_a) {
           const float zc = cc[i][k] - sc[i][k], zs = cs[i][k] - ss[i][k];
-          dst[(n2 - a) * n2 + g] = zc - zs;
-          if (mirror_g) dst[(n2 - a) * n2 + n2 - g] = zc + zs;
+          dst[(n2 - a) * n2 + g] = act(zc - zs);
+          if (mirror_g) dst[(n2 - a) * n2 + n2 - g] = act(zc + zs);
         }
       }
     }

@@ -11,6 +11,7 @@
 // Output bin k therefore sits at slot sigma(k) = 8 (k % 8) + k / 8; consumers index through sigma.
 #pragma once
 #include <hip/hip_runtime.h>
+#include "common.h"
 
 namespace fft64 {
 
@@ -121,8 +122,9 @@ __device__ __forceinline__ void make_twiddles(float2 (&tw)[8]) {
 // m = -(nb-1)..nb-1, n = 0..nb-1 of each plane's 2-D DFT.  Grid-stride over plane pairs.
 // ztile = 0: X is [plane][mi][n];  ztile = Z > 0: X is [z / Z][mi][beta][z % Z][n] (plane = z * 64 + beta),
 // the order in which the tiled Wigner contraction streams it.
+// mask: NULL, or a tensor of the shape of x; samples of x where it is not positive count as zero.
 __global__ __launch_bounds__(THREADS) void plane_fft64_fwd(const float* __restrict__ x, float2* __restrict__ X,
-                                                           long npairs, int nb, int ztile) {
+                                                           long npairs, int nb, int ztile, const float* __restrict__ mask) {
   __shared__ float2 buf[LDS_ELEMS];
   float2 tw[8];
   make_twiddles<false>(tw);
@@ -133,7 +135,13 @@ __global__ __launch_bounds__(THREADS) void plane_fft64_fwd(const float* __restri
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int q = threadIdx.x + THREADS * i;       // float4 index: row q/16, cols 4*(q%16)..
-      const float4 a = pa[q], b = pb[q];
+      float4 a = pa[q], b = pb[q];
+      if (mask) {
+        const float4* ma = reinterpret_cast<const float4*>(mask + pair * 2 * (N * N));
+        const float4 u = ma[q], v = ma[q + N * N / 4];
+        a = make_float4(s2cnn::relu_pass(a.x, u.x), s2cnn::relu_pass(a.y, u.y), s2cnn::relu_pass(a.z, u.z), s2cnn::relu_pass(a.w, u.w));
+        b = make_float4(s2cnn::relu_pass(b.x, v.x), s2cnn::relu_pass(b.y, v.y), s2cnn::relu_pass(b.z, v.z), s2cnn::relu_pass(b.w, v.w));
+      }
       float2* dst = buf + (q >> 4) * PITCH + 4 * (q & 15);
       dst[0] = make_float2(a.x, b.x); dst[1] = make_float2(a.y, b.y);
       dst[2] = make_float2(a.z, b.z); dst[3] = make_float2(a.w, b.w);

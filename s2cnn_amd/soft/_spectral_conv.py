@@ -17,8 +17,13 @@ class SpectralConvolution(nn.Module):
     # the work of the complex ones.  False selects the complex operators of the reference literally.
     real_basis = True
 
-    def __init__(self, nfeature_in, nfeature_out, b_in, b_out, grid, variance_per_sample):
+    def __init__(self, nfeature_in, nfeature_out, b_in, b_out, grid, variance_per_sample, activation=None):
         super().__init__()
+        # None: the layer of the reference.  "relu": max(., 0) applied where the output is written, and its gradient
+        # where the backward transform reads the incoming gradient: the same function as F.relu(layer(x)) without
+        # the passes of the activation over the output.
+        assert activation in (None, "relu"), activation
+        self.activation = activation
         self.nfeature_in, self.nfeature_out = nfeature_in, nfeature_out
         self.b_in, self.b_out = b_in, b_out
         self.grid = grid
@@ -26,6 +31,10 @@ class SpectralConvolution(nn.Module):
         self.bias = nn.Parameter(torch.zeros(1, nfeature_out, 1, 1, 1))
         # kept outside the parameter: activations of order one for kernel entries of order one
         self.scaling = 1.0 / math.sqrt(len(grid) * nfeature_in * variance_per_sample)
+
+    @property
+    def fused_relu(self):
+        return self.activation == "relu"
 
     def scaled_kernel(self):
         return self.kernel * self.scaling

@@ -8,13 +8,14 @@ from .so3_fft import SO3_ifft_real, SO3_ifft_real_basis
 
 
 class S2Convolution(SpectralConvolution):
-    def __init__(self, nfeature_in, nfeature_out, b_in, b_out, grid):
+    def __init__(self, nfeature_in, nfeature_out, b_in, b_out, grid, *, activation=None):
         """
         nfeature_in, nfeature_out: feature counts; b_in: bandwidth of the input (a 2 b_in x 2 b_in SOFT grid);
         b_out: bandwidth of the output; grid: the points of the sphere that carry the kernel, a tuple of
         (beta, alpha) pairs (s2cnn/soft/s2_conv.py:14-30, normalisation :27).
+        activation (not in the reference): None, or "relu" for F.relu(layer(x)) computed inside the layer.
         """
-        super().__init__(nfeature_in, nfeature_out, b_in, b_out, grid, b_out ** 4.0 / b_in ** 2.0)
+        super().__init__(nfeature_in, nfeature_out, b_in, b_out, grid, b_out ** 4.0 / b_in ** 2.0, activation)
 
     def forward(self, x):  # pylint: disable=W
         """[batch, feature_in, beta, alpha] -> [batch, feature_out, beta, alpha, gamma]"""
@@ -23,7 +24,7 @@ class S2Convolution(SpectralConvolution):
         if self.real_basis:
             yh = s2_rft_real(self.scaled_kernel(), self.b_out, self.grid)      # [l m, feature_in, feature_out]
             zh = s2_mm_real(s2_spectrum_to_real(xh), yh)                       # [l m n, batch, feature_out]
-            return SO3_ifft_real_basis.apply(zh, None, self.bias)              # the bias is added inside the transform
+            return SO3_ifft_real_basis.apply(zh, None, self.bias, self.fused_relu)   # bias added inside the transform
         yh = s2_rft(self.scaled_kernel(), self.b_out, self.grid)               # [l m, feature_in, feature_out, complex]
         zh = s2_mm(xh, yh)                                                     # [l m n, batch, feature_out, complex]
-        return SO3_ifft_real.apply(zh, None, self.bias)
+        return SO3_ifft_real.apply(zh, None, self.bias, self.fused_relu)

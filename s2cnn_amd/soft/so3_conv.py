@@ -9,13 +9,14 @@ from .so3_fft import SO3_fft_real, SO3_fft_real_basis, SO3_ifft_real, SO3_ifft_r
 
 
 class SO3Convolution(SpectralConvolution):
-    def __init__(self, nfeature_in, nfeature_out, b_in, b_out, grid):
+    def __init__(self, nfeature_in, nfeature_out, b_in, b_out, grid, *, activation=None):
         """
         nfeature_in, nfeature_out: feature counts; b_in: bandwidth of the input (a (2 b_in)^3 SOFT grid);
         b_out: bandwidth of the output; grid: the rotations that carry the kernel, a tuple of
         (beta, alpha, gamma) triples (s2cnn/soft/so3_conv.py:13-34, normalisation :31).
+        activation (not in the reference): None, or "relu" for F.relu(layer(x)) computed inside the layer.
         """
-        super().__init__(nfeature_in, nfeature_out, b_in, b_out, grid, b_out ** 3.0 / b_in ** 3.0)
+        super().__init__(nfeature_in, nfeature_out, b_in, b_out, grid, b_out ** 3.0 / b_in ** 3.0, activation)
 
     def forward(self, x):  # pylint: disable=W
         """[batch, feature_in, beta, alpha, gamma] -> [batch, feature_out, beta, alpha, gamma]"""
@@ -23,10 +24,10 @@ class SO3Convolution(SpectralConvolution):
         if self.real_basis:
             xh = SO3_fft_real_basis.apply(x, self.b_out)                       # [l m n, batch, feature_in]
             yh = so3_rft_real(self.scaled_kernel(), self.b_out, self.grid)     # [l m n, feature_in, feature_out]
-            return SO3_ifft_real_basis.apply(so3_mm_real(xh, yh), None, self.bias)   # bias added inside the transform
+            return SO3_ifft_real_basis.apply(so3_mm_real(xh, yh), None, self.bias, self.fused_relu)   # bias added inside the transform
         xh = SO3_fft_real.apply(x, self.b_out)                                 # [l m n, batch, feature_in, complex]
         yh = so3_rft(self.scaled_kernel(), self.b_out, self.grid)              # [l m n, feature_in, feature_out, complex]
-        return SO3_ifft_real.apply(so3_mm(xh, yh), None, self.bias)
+        return SO3_ifft_real.apply(so3_mm(xh, yh), None, self.bias, self.fused_relu)
 
 
 class SO3Shortcut(nn.Module):

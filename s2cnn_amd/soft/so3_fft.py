@@ -43,10 +43,20 @@ def _null_or_ptr(t):
     return _hip.ptr(t) if t is not None else None
 
 
-def _analysis(x, b_in, b_out, batch_size, for_grad, complex_in):
+def _same_shape_operand(mask, x):
+    """`mask` as a contiguous, 16-byte aligned float32 GPU tensor of the shape of x."""
+    _hip.require_gpu_f32(mask)
+    assert mask.shape == x.shape, (mask.shape, x.shape)
+    mask = mask.contiguous()
+    return mask.clone() if mask.data_ptr() % 16 else mask
+
+
+def _analysis(x, b_in, b_out, batch_size, for_grad, complex_in, mask=None):
     """x: contiguous grid tensor whose leading dims are `batch_size`; the result is allocated in its
-    final shape (never a view: autograd can then take ownership of it as a gradient without a copy)."""
+    final shape (never a view: autograd can then take ownership of it as a gradient without a copy).
+    mask (real x only): the transform is that of x where mask > 0 and of zero elsewhere."""
     _hip.require_gpu_f32(x)
+    assert mask is None or not complex_in
     if complex_in and complex_via_real:
         # the transform is linear over the complex numbers: analysis(x) = analysis(Re x) + i analysis(Im x), and the
         # kernels for real signals are the tuned ones
@@ -63,13 +73,19 @@ def _analysis(x, b_in, b_out, batch_size, for_grad, complex_in):
     packed = None if complex_in else _setup_packed_wigner(b_in, b_out, not for_grad, False, x.device)
     out = x.new_empty((_nspec(b_out), *batch_size, 2))
     ws = _hip.workspace(L.s2cnn_so3_analysis_workspace(b_in, b_out, nbatch, complex_in), x.device)
+    if mask is not None:
+        mask = _same_shape_operand(mask, x)
+        _hip.call("s2cnn_so3_analysis_real_masked", _hip.ptr(x), _hip.ptr(mask), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out),
+                  _hip.ptr(ws), ws.numel(), b_in, b_out, nbatch, 0, _hip.stream_ptr())
+        return out
     _hip.call("s2cnn_so3_analysis", _hip.ptr(x), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out), _hip.ptr(ws), ws.numel(),
                   b_in, b_out, nbatch, complex_in, _hip.stream_ptr())
     return out
 
 
-def _synthesis(x, b_in, b_out, batch_size, for_grad, complex_out, bias=None):
+def _synthesis(x, b_in, b_out, batch_size, for_grad, complex_out, bias=None, relu=False):
     _hip.require_gpu_f32(x)
+    assert not (relu and complex_out)
     if complex_out and complex_via_real:
         # y = synthesis(x) is complex-linear in x and the real-output kernels return Re y for ANY spectrum:
         # Re y = real_synthesis(x), Im y = Re(-i y) = real_synthesis(-i x)
@@ -90,6 +106,11 @@ def _synthesis(x, b_in, b_out, batch_size, for_grad, complex_out, bias=None):
         _hip.require_gpu_f32(bias)
         bias = bias.reshape(-1).contiguous()
         assert len(batch_size) >= 1 and batch_size[-1] == bias.numel()
+    if relu:
+        _hip.call("s2cnn_so3_synthesis_real_relu", _hip.ptr(x), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out), _hip.ptr(ws),
+                  ws.numel(), b_in, b_out, nbatch, _null_or_ptr(bias), 1 if bias is None else bias.numel(), 0, _hip.stream_ptr())
+        return out
+    if bias is not None:
         _hip.call("s2cnn_so3_synthesis_real_bias", _hip.ptr(x), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out), _hip.ptr(ws),
                   ws.numel(), b_in, b_out, nbatch, _hip.ptr(bias), bias.numel(), _hip.stream_ptr())
         return out
@@ -114,9 +135,10 @@ def so3_fft(x, for_grad=False, b_out=None):
     return _analysis(x.contiguous(), b_in, b_out, batch_size, for_grad, 1)
 
 
-def so3_rfft(x, for_grad=False, b_out=None):
+def so3_rfft(x, for_grad=False, b_out=None, mask=None):
     '''
     :param x: [..., beta, alpha, gamma]
+    :param mask: None, or a tensor of the shape of x: samples of x where it is not positive count as zero
     :return: [l * m * n, ..., complex]
     '''
     b_in = x.size(-1) // 2
@@ -126,7 +148,7 @@ def so3_rfft(x, for_grad=False, b_out=None):
     if b_out is None:
         b_out = b_in
     batch_size = x.size()[:-3]
-    return _analysis(x.contiguous(), b_in, b_out, batch_size, for_grad, 0)
+    return _analysis(x.contiguous(), b_in, b_out, batch_size, for_grad, 0, mask)
 
 
 def _spectrum_args(x, b_out):
@@ -149,14 +171,15 @@ def so3_ifft(x, for_grad=False, b_out=None):
     return _synthesis(x, b_in, b_out, batch_size, for_grad, 1)
 
 
-def so3_rifft(x, for_grad=False, b_out=None, bias=None):
+def so3_rifft(x, for_grad=False, b_out=None, bias=None, relu=False):
     '''
     :param x: [l * m * n, ..., complex]
     :param bias: None, or one value per entry of the last batch dimension, added to every sample of its volumes
+    :param relu: negative samples (after the bias) come out as zero
     :return: [..., beta, alpha, gamma]  (the real part of so3_ifft, whatever the symmetry of x)
     '''
     x, b_in, b_out, batch_size = _spectrum_args(x, b_out)
-    return _synthesis(x, b_in, b_out, batch_size, for_grad, 0, bias)
+    return _synthesis(x, b_in, b_out, batch_size, for_grad, 0, bias, relu)
 
 
 class SO3_fft_real(torch.autograd.Function):
@@ -177,22 +200,29 @@ class SO3_ifft_real(torch.autograd.Function):
     """s2cnn/soft/so3_fft.py:224-236, with the bias of the convolution layers as an optional third argument
     (x [l * m * n, batch, feature, complex], bias with `feature` entries in any shape): it is added in the
     epilogue of the transform, and its gradient is read off the degree-0 coefficient of the unweighted analysis
-    of grad_output, which IS the sum of grad_output over the grid."""
+    of grad_output, which IS the sum of grad_output over the grid.  relu = True applies max(., 0) in the same
+    epilogue (the activation that follows the layers in the reference's models)."""
     @staticmethod
-    def forward(ctx, x, b_out=None, bias=None):  # pylint: disable=W
+    def forward(ctx, x, b_out=None, bias=None, relu=False):  # pylint: disable=W
         nspec = x.size(0)
         ctx.b_out = b_out
         ctx.b_in = round((3 / 4 * nspec) ** (1 / 3))
         ctx.bias_shape = None if bias is None else bias.shape
-        return so3_rifft(x, b_out=ctx.b_out, bias=bias)
+        out = so3_rifft(x, b_out=ctx.b_out, bias=bias, relu=relu)
+        ctx.relu = bool(relu)
+        if relu:
+            ctx.save_for_backward(out)
+        return out
 
     @staticmethod
     def backward(ctx, grad_output):  # pylint: disable=W
-        g = so3_rfft(grad_output, for_grad=True, b_out=ctx.b_in)
+        # with the relu in the epilogue, the gradient passes where the output is positive: the mask is applied as the
+        # analysis reads grad_output
+        g = so3_rfft(grad_output, for_grad=True, b_out=ctx.b_in, mask=ctx.saved_tensors[0] if ctx.relu else None)
         gb = None
         if ctx.bias_shape is not None and ctx.needs_input_grad[2]:
             gb = g[0, ..., 0].reshape(-1, g.size(-2)).sum(0).reshape(ctx.bias_shape)
-        return g, None, gb
+        return g, None, gb, None
 
 
 # ---------------------------------------------------------------------------------------------------
@@ -204,9 +234,10 @@ def _real_basis_direct(b_in, b_out, synthesis):
     return bool(_hip.lib().s2cnn_so3_real_basis_transform_available(b_in, b_out, int(synthesis)))
 
 
-def so3_rfft_real_basis(x, for_grad=False, b_out=None):
+def so3_rfft_real_basis(x, for_grad=False, b_out=None, mask=None):
     '''
     :param x: [..., beta, alpha, gamma]
+    :param mask: None, or a tensor of the shape of x: samples of x where it is not positive count as zero
     :return: [l * m * n, ...]  = so3_spectrum_to_real(so3_rfft(x))
     '''
     b_in = x.size(-1) // 2
@@ -215,7 +246,7 @@ def so3_rfft_real_basis(x, for_grad=False, b_out=None):
         b_out = b_in
     if not (x.is_cuda and _real_basis_direct(b_in, b_out, False)):
         from ..so3_real import _convert
-        y = so3_rfft(x, for_grad, b_out)
+        y = so3_rfft(x, for_grad, b_out, mask)
         return _convert("s2cnn_so3_spectrum_to_real", y, y.shape[:-1])
     _hip.require_gpu_f32(x)
     x = x.contiguous()
@@ -230,15 +261,21 @@ def so3_rfft_real_basis(x, for_grad=False, b_out=None):
     packed = _setup_packed_wigner(b_in, b_out, not for_grad, False, x.device)
     out = x.new_empty((_nspec(b_out), *batch_size))
     ws = _hip.workspace(L.s2cnn_so3_analysis_workspace(b_in, b_out, nbatch, 0), x.device)
+    if mask is not None:
+        mask = _same_shape_operand(mask, x)
+        _hip.call("s2cnn_so3_analysis_real_masked", _hip.ptr(x), _hip.ptr(mask), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out),
+                  _hip.ptr(ws), ws.numel(), b_in, b_out, nbatch, 1, _hip.stream_ptr())
+        return out
     _hip.call("s2cnn_so3_analysis_real_basis", _hip.ptr(x), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out), _hip.ptr(ws),
               ws.numel(), b_in, b_out, nbatch, _hip.stream_ptr())
     return out
 
 
-def so3_rifft_real_basis(r, for_grad=False, b_out=None, bias=None):
+def so3_rifft_real_basis(r, for_grad=False, b_out=None, bias=None, relu=False):
     '''
     :param r: [l * m * n, ...]  real-basis spectrum
     :param bias: None, or one value per entry of the last batch dimension, added to every sample of its volumes
+    :param relu: negative samples (after the bias) come out as zero
     :return: [..., beta, alpha, gamma]  = so3_rifft(so3_spectrum_to_complex(r)) (+ bias)
     '''
     nspec = r.size(0)
@@ -248,7 +285,7 @@ def so3_rifft_real_basis(r, for_grad=False, b_out=None, bias=None):
         b_out = b_in
     if not (r.is_cuda and _real_basis_direct(b_in, b_out, True)):
         from ..so3_real import _convert
-        return so3_rifft(_convert("s2cnn_so3_spectrum_to_complex", r.contiguous(), (*r.shape, 2)), for_grad, b_out, bias)
+        return so3_rifft(_convert("s2cnn_so3_spectrum_to_complex", r.contiguous(), (*r.shape, 2)), for_grad, b_out, bias, relu)
     _hip.require_gpu_f32(r)
     r = r.contiguous()
     batch_size = r.size()[1:]
@@ -266,6 +303,10 @@ def so3_rifft_real_basis(r, for_grad=False, b_out=None, bias=None):
         bias = bias.reshape(-1).contiguous()
         nfeature = bias.numel()
         assert r.dim() >= 2 and r.size(-1) == nfeature
+    if relu:
+        _hip.call("s2cnn_so3_synthesis_real_relu", _hip.ptr(r), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out), _hip.ptr(ws),
+                  ws.numel(), b_in, b_out, nbatch, _null_or_ptr(bias), nfeature, 1, _hip.stream_ptr())
+        return out
     _hip.call("s2cnn_so3_synthesis_real_basis", _hip.ptr(r), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out), _hip.ptr(ws),
               ws.numel(), b_in, b_out, nbatch, _null_or_ptr(bias), nfeature, _hip.stream_ptr())
     return out
@@ -289,16 +330,20 @@ class SO3_ifft_real_basis(torch.autograd.Function):
     layer (r [l * m * n, batch, feature], bias with `feature` entries in any shape).  The gradient of the bias
     costs nothing: the degree-0 coefficient of the unweighted analysis of grad_output IS its sum over the grid."""
     @staticmethod
-    def forward(ctx, r, b_out=None, bias=None):  # pylint: disable=W
+    def forward(ctx, r, b_out=None, bias=None, relu=False):  # pylint: disable=W
         nspec = r.size(0)
         ctx.b_in = round((3 / 4 * nspec) ** (1 / 3))
         ctx.bias_shape = None if bias is None else bias.shape
-        return so3_rifft_real_basis(r, b_out=b_out, bias=bias)
+        out = so3_rifft_real_basis(r, b_out=b_out, bias=bias, relu=relu)
+        ctx.relu = bool(relu)
+        if relu:
+            ctx.save_for_backward(out)
+        return out
 
     @staticmethod
     def backward(ctx, grad_output):  # pylint: disable=W
-        g = so3_rfft_real_basis(grad_output, for_grad=True, b_out=ctx.b_in)
+        g = so3_rfft_real_basis(grad_output, for_grad=True, b_out=ctx.b_in, mask=ctx.saved_tensors[0] if ctx.relu else None)
         gb = None
         if ctx.bias_shape is not None and ctx.needs_input_grad[2]:
             gb = g[0].reshape(-1, g.size(-1)).sum(0).reshape(ctx.bias_shape)
-        return g, None, gb
+        return g, None, gb, None

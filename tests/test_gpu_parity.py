@@ -273,8 +273,84 @@ def test_s2_convolution_parity(hip, real_basis):
     _conv_case("s2", 3, 10, 8, 6, 6, s2cnn_amd.s2_near_identity_grid(), 66, real_basis)      # two feature passes, 16-byte rows
 
 
+@pytest.mark.parametrize("b_in,b_out,nz,nf", [(32, 32, 4, 2),     # per-volume kernels (all item rounds)
+                                              (32, 22, 6, 3), (32, 26, 2, 1),   # their truncated instantiations
+                                              (10, 32, 6, 3),     # synthesis onto the 64^3 grid from a short spectrum
+                                              (32, 34, 2, 1),     # 64-point plane kernel + Wigner stage
+                                              (22, 7, 6, 2), (6, 6, 10, 5), (5, 9, 3, 1), (11, 4, 2, 1)])   # folded plane kernels
+def test_so3_transforms_with_fused_relu(hip, b_in, b_out, nz, nf):
+    """max(., 0) in the epilogue of the synthesis and its gradient mask in the loads of the analysis against the
+    separate elementwise passes they replace: the results must be the same numbers, bit for bit, for complex and
+    real-basis spectra."""
+    from s2cnn_amd.soft import so3_fft as P
+    from s2cnn_amd.so3_real import so3_spectrum_to_real
+    print(f"fused relu b_in={b_in} b_out={b_out} nz={nz} nf={nf}", flush=True)
+    g = torch.Generator().manual_seed(1000 * b_in + b_out)
+    # synthesis b_in -> b_out
+    xh = torch.randn(O.nspec_so3(b_in), nz // nf, nf, 2, generator=g).cuda()
+    bias = torch.randn(nf, generator=g).cuda()
+    for bb in (bias, None):
+        plain = P.so3_rifft(xh, b_out=b_out, bias=bb)
+        fused = P.so3_rifft(xh, b_out=b_out, bias=bb, relu=True)
+        assert torch.equal(fused, torch.relu(plain))
+        assert (fused == 0).float().mean().item() > 0.2
+        r = so3_spectrum_to_real(xh)
+        assert torch.equal(P.so3_rifft_real_basis(r, b_out=b_out, bias=bb, relu=True), torch.relu(P.so3_rifft_real_basis(r, b_out=b_out, bias=bb)))
+    # analysis b_in -> b_out, both tables
+    x = torch.randn(nz // nf, nf, 2 * b_in, 2 * b_in, 2 * b_in, generator=g).cuda()
+    y = torch.relu(torch.randn(x.shape, generator=g)).cuda()        # what a relu leaves behind: zeros and positive values
+    for for_grad in (False, True):
+        want = P.so3_rfft(x * (y > 0), for_grad=for_grad, b_out=b_out)
+        assert torch.equal(P.so3_rfft(x, for_grad=for_grad, b_out=b_out, mask=y), want)
+        want = P.so3_rfft_real_basis(x * (y > 0), for_grad=for_grad, b_out=b_out)
+        assert torch.equal(P.so3_rfft_real_basis(x, for_grad=for_grad, b_out=b_out, mask=y), want)
+    # an operand that is not 16-byte aligned takes another loader (or a copy): same numbers
+    big = torch.randn(x.numel() + 1, generator=g).cuda()
+    xo, yo = big[1:].view(x.shape), torch.relu(big.flip(0))[1:].view(x.shape)
+    assert torch.equal(P.so3_rfft(xo, b_out=b_out, mask=yo), P.so3_rfft(xo * (yo > 0), b_out=b_out))
+
+
+@pytest.mark.parametrize("kind,real_basis", [("so3", True), ("so3", False), ("s2", True), ("s2", False)])
+def test_layers_with_fused_relu(hip, kind, real_basis):
+    """activation="relu" is F.relu(layer(x)): same output, same gradients wrt input, kernel and bias; and the
+    output against the oracle's layer followed by relu."""
+    shapes = [(3, 4, 6, 5, 5), (2, 3, 5, 32, 32)] if kind == "so3" else [(3, 2, 6, 8, 5), (2, 3, 4, 40, 32)]
+    for (B, fi, fo, b_in, b_out) in shapes:
+        print(f"fused relu layer {kind} real_basis={real_basis} B={B} {fi}->{fo} b {b_in}->{b_out}", flush=True)
+        torch.manual_seed(b_in)
+        if kind == "so3":
+            grid = s2cnn_amd.so3_near_identity_grid()
+            ref = s2cnn_amd.SO3Convolution(fi, fo, b_in, b_out, grid)
+            fus = s2cnn_amd.SO3Convolution(fi, fo, b_in, b_out, grid, activation="relu")
+            x = torch.randn(B, fi, 2 * b_in, 2 * b_in, 2 * b_in)
+        else:
+            grid = s2cnn_amd.s2_near_identity_grid()
+            ref = s2cnn_amd.S2Convolution(fi, fo, b_in, b_out, grid)
+            fus = s2cnn_amd.S2Convolution(fi, fo, b_in, b_out, grid, activation="relu")
+            x = torch.randn(B, fi, 2 * b_in, 2 * b_in)
+        with torch.no_grad():
+            ref.bias.normal_()
+        fus.load_state_dict(ref.state_dict())
+        ref.real_basis = fus.real_basis = real_basis
+        if b_in <= 8:
+            conv = O.so3_conv if kind == "so3" else O.s2_conv
+            want = torch.relu(conv(x.double(), ref.kernel.detach().double(), ref.bias.detach().double(), b_in, b_out, grid))
+        ref, fus = ref.cuda(), fus.cuda()
+        xa, xb = x.cuda().requires_grad_(), x.cuda().requires_grad_()
+        ya, yb = torch.relu(ref(xa)), fus(xb)
+        assert torch.equal(ya, yb)
+        if b_in <= 8:
+            close(yb, want, "layer + relu against the oracle")
+        w = torch.randn(ya.shape, generator=torch.Generator().manual_seed(5)).cuda()
+        (ya * w).sum().backward()
+        (yb * w).sum().backward()
+        for a, b, name in ((xa.grad, xb.grad, "input"), (ref.kernel.grad, fus.kernel.grad, "kernel"), (ref.bias.grad, fus.bias.grad, "bias")):
+            err = (a - b).abs().max().item() / a.abs().max().item()
+            assert err < 1e-6, (name, err)
+
+
 def test_config1_shaped_network(hip):
-    """BASELINE config 1 shapes at reduced batch: S2Conv 1->20 (b 30->10), ReLU, SO3Conv 20->40
+    """benchmark config 1 shapes at reduced batch: S2Conv 1->20 (b 30->10), ReLU, SO3Conv 20->40
     (b 10->6), ReLU, so3_integrate; forward only."""
     g = torch.Generator().manual_seed(1)
     x = torch.rand(4, 1, 60, 60, generator=g) * (torch.rand(4, 1, 60, 60, generator=g) < 0.3)
@@ -292,7 +368,7 @@ def test_config1_shaped_network(hip):
 
 
 def _config5_layers(seed=8):
-    """BASELINE config 5 (SHREC17-shaped): S2Conv 6->100 b128->32, SO3Conv 100->100 b32->22, SO3Conv 100->55 b22->7,
+    """benchmark config 5 (SHREC17-shaped): S2Conv 6->100 b128->32, SO3Conv 100->100 b32->22, SO3Conv 100->55 b22->7,
     near-identity grids with max_beta scaled by the bandwidth ratio (examples/shrec17/model_original.py:12-40)."""
     import math
     g1 = s2cnn_amd.s2_near_identity_grid(max_beta=math.pi / 8 * 30 / 128, n_alpha=8, n_beta=3)

@@ -134,7 +134,9 @@ def test_basis_kernels_against_dense(hip, nl, cols):
                                         (12, 16, 32, 48), (9, 4, 100, 36),
                                         # block sizes that divide / are multiples of the K stage (32): scalar-stepped loaders,
                                         # several blocks per stage (8, 16), several stages per block (96, 128), ragged last stage
-                                        (5, 8, 64, 32), (4, 4, 128, 64), (7, 32, 96, 32), (6, 16, 16, 8)])
+                                        (5, 8, 64, 32), (4, 4, 128, 64), (7, 32, 96, 32), (6, 16, 16, 8),
+                                        # one operand with 16-byte accesses, the other with 4-byte ones
+                                        (5, 6, 20, 7), (4, 3, 7, 8), (7, 32, 100, 55)])
 def test_so3_mm_real_forward_backward(hip, nl, B, Fi, Fo):
     import s2cnn_amd
     print(f"so3_mm_real nl={nl} B={B} Fi={Fi} Fo={Fo}", flush=True)
