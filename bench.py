@@ -168,7 +168,9 @@ def measure_rows(torch, dev, with_cpu):
 def measure_network(torch, dev, steps, warmup):
     """The SHREC17-shaped network of benchmark config 5 (S2Conv 6->100 b 128->32, ReLU, SO3Conv 100->100 b 32->22, ReLU,
     SO3Conv 100->55 b 22->7, so3_integrate; batch 32, near-identity grids scaled by the bandwidth ratio), forward and
-    backward with respect to the weights, timed like the headline step; time inside library calls listed beside it."""
+    backward with respect to the weights, timed like the headline step; time inside library calls listed beside it.
+    Timed twice: with the activations inside the layers (activation="relu") and, as the reference's models are written,
+    as separate torch.relu calls on the layers' outputs; both are the same function."""
     import math
 
     import s2cnn_amd
@@ -176,35 +178,44 @@ def measure_network(torch, dev, steps, warmup):
     g1 = s2cnn_amd.s2_near_identity_grid(max_beta=math.pi / 8 * 30 / 128, n_alpha=8, n_beta=3)
     g2 = s2cnn_amd.so3_near_identity_grid(max_beta=math.pi / 8 * 30 / 32, max_gamma=2 * math.pi, n_alpha=8, n_beta=3, n_gamma=8)
     g3 = s2cnn_amd.so3_near_identity_grid(max_beta=math.pi / 8 * 30 / 22, max_gamma=2 * math.pi, n_alpha=8, n_beta=3, n_gamma=8)
-    torch.manual_seed(8)
-    c1 = s2cnn_amd.S2Convolution(6, 100, 128, 32, g1).to(dev)
-    c2 = s2cnn_amd.SO3Convolution(100, 100, 32, 22, g2).to(dev)
-    c3 = s2cnn_amd.SO3Convolution(100, 55, 22, 7, g3).to(dev)
-    params = [q for c in (c1, c2, c3) for q in c.parameters()]
     x = torch.rand(32, 6, 256, 256, device=dev)
 
-    def step():
-        for q in params:
-            q.grad = None
-        out = s2cnn_amd.so3_integrate(c3(torch.relu(c2(torch.relu(c1(x))))))
-        sum_of_squares(out).backward()
+    def timed(activation):
+        torch.manual_seed(8)
+        c1 = s2cnn_amd.S2Convolution(6, 100, 128, 32, g1, activation=activation).to(dev)
+        c2 = s2cnn_amd.SO3Convolution(100, 100, 32, 22, g2, activation=activation).to(dev)
+        c3 = s2cnn_amd.SO3Convolution(100, 55, 22, 7, g3).to(dev)
+        params = [q for c in (c1, c2, c3) for q in c.parameters()]
+        act = torch.relu if activation is None else (lambda t: t)
 
-    for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step()
-    torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) / steps * 1e3
-    with _hip.KernelTimer() as kt:
-        step()
+        def step():
+            for q in params:
+                q.grad = None
+            out = s2cnn_amd.so3_integrate(c3(act(c2(act(c1(x))))))
+            sum_of_squares(out).backward()
+
+        for _ in range(warmup):
+            step()
         torch.cuda.synchronize()
-    calls = {k: round(sum(v), 3) for k, v in sorted(kt.summary().items(), key=lambda kv: -sum(kv[1]))}
-    torch.cuda.empty_cache()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) / steps * 1e3
+        with _hip.KernelTimer() as kt:
+            step()
+            torch.cuda.synchronize()
+        calls = {k: round(sum(v), 3) for k, v in sorted(kt.summary().items(), key=lambda kv: -sum(kv[1]))}
+        del c1, c2, c3, params
+        torch.cuda.empty_cache()
+        return ms, calls
+
+    ms, calls = timed("relu")
+    ms_sep, calls_sep = timed(None)
     return {"workload": "S2Conv 6->100 (b 128->32), SO3Conv 100->100 (32->22), SO3Conv 100->55 (22->7), integrate; batch 32, fwd+bwd (benchmark config 5)",
             "ms_per_step": round(ms, 3), "samples_per_s": round(32 / (ms * 1e-3), 1),
-            "library_ms": round(sum(calls.values()), 3), "library_calls_ms": calls}
+            "library_ms": round(sum(calls.values()), 3), "library_calls_ms": calls,
+            "separate_relu": {"ms_per_step": round(ms_sep, 3), "library_ms": round(sum(calls_sep.values()), 3)}}
 
 
 def main():
