@@ -27,6 +27,7 @@
 // synthesis leave the LDS as one contiguous run of 16-byte stores instead of four-byte scatters.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <type_traits>
 #include "common.h"
 #include "dft_common.h"
 
@@ -133,35 +134,45 @@ __global__ __launch_bounds__(NT_MAX) void plane_dft_fwd(const float* __restrict_
     const float* src = x + (size_t)plane0 * n2 * n2;
     const float* msk = mask ? mask + (size_t)plane0 * n2 * n2 : nullptr;
     const float inv_n2 = 1.0f / (float)n2;
-    Walk2 wk;
-    wk.init(t, NT, hg);
-    for (int e = t; e < total; e += LOADS * NT) {
-      float v1[LOADS], v2[LOADS];
-      int dst[LOADS];
-      unsigned pmask = 0;
+    // one copy of the loop per case, so that the batched loads of the plain case stay one run of loads
+    auto fold_rows = [&](auto masked) {
+      Walk2 wk;
+      wk.init(t, NT, hg);
+      for (int e = t; e < total; e += LOADS * NT) {
+        float v1[LOADS], v2[LOADS], m1[LOADS], m2[LOADS];
+        int dst[LOADS];
+        unsigned pmask = 0, vmask = 0;
 #pragma unroll
-      for (int u = 0; u < LOADS; ++u) {
-        const int R = wk.row, g = wk.col;
-        const bool live = e + u * NT < total;
-        const bool valid = live && R < rows_valid;
-        const bool paired = g > 0 && g < h;
-        const int o1 = valid ? R * n2 + g : 0;
-        const int o2 = valid && paired ? R * n2 + n2 - g : o1;
-        v1[u] = src[o1];
-        v2[u] = src[o2];
-        if (msk) { v1[u] = s2cnn::relu_pass(v1[u], msk[o1]); v2[u] = s2cnn::relu_pass(v2[u], msk[o2]); }
-        if (!valid) v1[u] = v2[u] = 0.f;
-        if (!paired) v2[u] = 0.f;
-        else pmask |= 1u << u;
-        const int q = (int)(((float)R + 0.5f) * inv_n2), a = R - q * n2;
-        const int slot = a == 0 ? 0 : a == h ? 1 : a < h ? 2 * a : 2 * (n2 - a) + 1;
-        dst[u] = live ? (q * hg + g) * ns + slot : -1;
-        wk.step();
+        for (int u = 0; u < LOADS; ++u) {
+          const int R = wk.row, g = wk.col;
+          const bool live = e + u * NT < total;
+          const bool valid = live && R < rows_valid;
+          const bool paired = g > 0 && g < h;
+          const int o1 = valid ? R * n2 + g : 0;
+          const int o2 = valid && paired ? R * n2 + n2 - g : o1;
+          v1[u] = src[o1];
+          v2[u] = src[o2];
+          if constexpr (decltype(masked)::value) { m1[u] = msk[o1]; m2[u] = msk[o2]; }
+          if (valid) vmask |= 1u << u;
+          if (paired) pmask |= 1u << u;
+          const int q = (int)(((float)R + 0.5f) * inv_n2), a = R - q * n2;
+          const int slot = a == 0 ? 0 : a == h ? 1 : a < h ? 2 * a : 2 * (n2 - a) + 1;
+          dst[u] = live ? (q * hg + g) * ns + slot : -1;
+          wk.step();
+        }
+#pragma unroll
+        for (int u = 0; u < LOADS; ++u) {
+          float a = v1[u], b = v2[u];
+          if constexpr (decltype(masked)::value) { a = s2cnn::relu_pass(a, m1[u]); b = s2cnn::relu_pass(b, m2[u]); }
+          if (!((vmask >> u) & 1u)) a = b = 0.f;
+          const bool paired = (pmask >> u) & 1u;
+          if (!paired) b = 0.f;
+          if (dst[u] >= 0) EO[dst[u]] = make_float2(a + b, paired ? a - b : 0.f);
+        }
       }
-#pragma unroll
-      for (int u = 0; u < LOADS; ++u)
-        if (dst[u] >= 0) EO[dst[u]] = make_float2(v1[u] + v2[u], (pmask >> u) & 1u ? v1[u] - v2[u] : 0.f);
-    }
+    };
+    if (msk) fold_rows(std::true_type{});
+    else fold_rows(std::false_type{});
     if (ns > n2)   // n2 = 2 mod 4: two empty slots
       for (int i = t; i < PL * hg * (ns - n2); i += NT) EO[(i / (ns - n2)) * ns + n2 + i % (ns - n2)] = make_float2(0.f, 0.f);
   }

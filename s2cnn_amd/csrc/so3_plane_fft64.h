@@ -132,19 +132,27 @@ __global__ __launch_bounds__(THREADS) void plane_fft64_fwd(const float* __restri
   for (long pair = blockIdx.x; pair < npairs; pair += gridDim.x) {
     const float4* pa = reinterpret_cast<const float4*>(x + pair * 2 * (N * N));
     const float4* pb = pa + N * N / 4;
+    float4 a[4], b[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {                    // float4 index q: row q/16, cols 4*(q%16)..
+      a[i] = pa[threadIdx.x + THREADS * i];
+      b[i] = pb[threadIdx.x + THREADS * i];
+    }
+    if (mask) {
+      const float4* ma = reinterpret_cast<const float4*>(mask + pair * 2 * (N * N));
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float4 u = ma[threadIdx.x + THREADS * i], v = ma[threadIdx.x + THREADS * i + N * N / 4];
+        a[i] = make_float4(s2cnn::relu_pass(a[i].x, u.x), s2cnn::relu_pass(a[i].y, u.y), s2cnn::relu_pass(a[i].z, u.z), s2cnn::relu_pass(a[i].w, u.w));
+        b[i] = make_float4(s2cnn::relu_pass(b[i].x, v.x), s2cnn::relu_pass(b[i].y, v.y), s2cnn::relu_pass(b[i].z, v.z), s2cnn::relu_pass(b[i].w, v.w));
+      }
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int q = threadIdx.x + THREADS * i;       // float4 index: row q/16, cols 4*(q%16)..
-      float4 a = pa[q], b = pb[q];
-      if (mask) {
-        const float4* ma = reinterpret_cast<const float4*>(mask + pair * 2 * (N * N));
-        const float4 u = ma[q], v = ma[q + N * N / 4];
-        a = make_float4(s2cnn::relu_pass(a.x, u.x), s2cnn::relu_pass(a.y, u.y), s2cnn::relu_pass(a.z, u.z), s2cnn::relu_pass(a.w, u.w));
-        b = make_float4(s2cnn::relu_pass(b.x, v.x), s2cnn::relu_pass(b.y, v.y), s2cnn::relu_pass(b.z, v.z), s2cnn::relu_pass(b.w, v.w));
-      }
+      const int q = threadIdx.x + THREADS * i;
       float2* dst = buf + (q >> 4) * PITCH + 4 * (q & 15);
-      dst[0] = make_float2(a.x, b.x); dst[1] = make_float2(a.y, b.y);
-      dst[2] = make_float2(a.z, b.z); dst[3] = make_float2(a.w, b.w);
+      dst[0] = make_float2(a[i].x, b[i].x); dst[1] = make_float2(a[i].y, b[i].y);
+      dst[2] = make_float2(a[i].z, b[i].z); dst[3] = make_float2(a[i].w, b[i].w);
     }
     __syncthreads();
     transform_2d<false>(buf, tw);
