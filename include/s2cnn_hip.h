@@ -188,7 +188,7 @@ int s2cnn_so3_synthesis_real_bias(const float *xhat, const float *table, const f
 /* Bias (may be NULL) and max(., 0) in the epilogue: out = relu(synthesis(xhat) + bias).  real_basis = 0: xhat as
  * above; 1: the spectrum in the real basis, one float per entry (only where
  * s2cnn_so3_real_basis_transform_available(b_in, b_out, 1)).  Replaces F.relu applied to the output of a
- * convolution layer (examples/mnist/run.py:88-92, examples/shrec17/model.py:28-35) without its pass over the
+ * convolution layer (examples/mnist/run.py:88-92) without its pass over the
  * activations.
  */
 int s2cnn_so3_synthesis_real_relu(const float *xhat, const float *table, const float *packed_table, float *out,
