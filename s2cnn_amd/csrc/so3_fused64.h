@@ -547,13 +547,34 @@ constexpr int IT_TILE_R = 16;
 constexpr int VLD_R = 16 * ZR + 1;
 constexpr float SQRT2 = 1.41421356237309504880f, RSQRT2 = 0.70710678118654752440f;
 
+// where one output row of the tile comes from: out[row] = alpha * vals[comp] + beta * vals[comp + 8] (row < 0: no such row)
+struct RowRule { int row, comp; float alpha, beta; };
+
+// rule of row slot rs = 4 u + kind (degree 4 c + u; kind: 0 (+a,+n)  1 (+a,-n)  2 (-a,+n)  3 (-a,-n)) of an item
+__device__ __forceinline__ RowRule row_rule(int inf, int rs, int nl) {
+  const int u = rs >> 2, kind = rs & 3;
+  const int c = inf & 0xff, a = (inf >> 8) & 0xff, n = (inf >> 16) & 0xff;
+  const int l = 4 * c + u;
+  RowRule r{-1, 0, 0.f, 0.f};
+  if (!(inf >> 24) || l < a || l < n || l >= nl || ((kind & 1) && n == 0) || ((kind & 2) && a == 0)) return r;
+  r.row = lmn_index(l, (kind & 2) ? -a : a, (kind & 1) ? -n : n);
+  // A = (+a) half: components 4 (u / 2) + 2 (u % 2) + (0 re, 1 im);  C = (-a) half: the same + 8
+  r.comp = 4 * (u >> 1) + 2 * (u & 1) + ((kind == 1 || kind == 2) ? 1 : 0);
+  const float s = (a & 1) ? -1.f : 1.f;
+  r.alpha = kind == 1 ? -1.f : 1.f;
+  r.beta = (kind == 0) ? s : -s;
+  if (a == 0) { r.alpha *= SQRT2; r.beta = 0.f; if (n == 0) r.alpha = 1.f; }
+  else if (n == 0) { r.alpha *= RSQRT2; r.beta *= RSQRT2; }
+  return r;
+}
+
 __global__ __launch_bounds__(256) void spectrum_scatter_real(const float4* __restrict__ rec, float* __restrict__ out, int nl, long nbatch) {
   __shared__ float vals[IT_TILE_R * VLD_R];
-  __shared__ int info[IT_TILE_R];
+  __shared__ RowRule rules[IT_TILE_R * 16];
   const int th = threadIdx.x;
   const long z0 = (long)blockIdx.x * ZR;
   const int it = blockIdx.y >> 5, t0 = (blockIdx.y & 31) * IT_TILE_R;
-  if (th < IT_TILE_R) info[th] = pack_item_info(it * THREADS + t0 + th);
+  rules[th] = row_rule(pack_item_info(it * THREADS + t0 + (th >> 4)), th & 15, nl);   // 16 items x 16 row slots: one per thread
 #pragma unroll
   for (int r = 0; r < 8; ++r) {
     const int e = th + 256 * r;
@@ -564,55 +585,60 @@ __global__ __launch_bounds__(256) void spectrum_scatter_real(const float4* __res
     d[0] = v.x; d[ZR] = v.y; d[2 * ZR] = v.z; d[3 * ZR] = v.w;
   }
   __syncthreads();
-  const int zz = th & 31, sub = th >> 5;       // sub = 0..7: row slots 2 p + (0, 1) -> (u, kind) = ((sub & 1) * 2 + p / 2 ... see below)
+  const int zz = th & 31, sub = th >> 5;       // 8 row slots at a time, 32 volumes (128 bytes of a row) each
   if (z0 + zz >= nbatch) return;
-  for (int p = 0; p < 2 * IT_TILE_R; ++p) {    // 16 rows per item (4 degrees x 4 kinds), 8 at a time
+  float* dst = out + z0 + zz;
+  for (int p = 0; p < 2 * IT_TILE_R; ++p) {
     const int item = p >> 1;
-    const int rs = (p & 1) * 8 + sub;          // 0..15
-    const int u = rs >> 2, kind = rs & 3;      // kind: 0 (+a,+n)  1 (+a,-n)  2 (-a,+n)  3 (-a,-n)
-    const int inf = info[item];
-    const int c = inf & 0xff, a = (inf >> 8) & 0xff, n = (inf >> 16) & 0xff;
-    const int l = 4 * c + u;
-    if (!(inf >> 24) || l < a || l < n || l >= nl || ((kind & 1) && n == 0) || ((kind & 2) && a == 0)) continue;
-    const int row = lmn_index(l, (kind & 2) ? -a : a, (kind & 1) ? -n : n);
-    // A = (+a) half: components 4 (u / 2) + 2 (u % 2) + (0 re, 1 im);  C = (-a) half: the same + 8
-    const int comp = 4 * (u >> 1) + 2 * (u & 1) + ((kind == 1 || kind == 2) ? 1 : 0);
-    const float av = vals[item * VLD_R + comp * ZR + zz], cv = vals[item * VLD_R + (comp + 8) * ZR + zz];
-    const float s = (a & 1) ? -1.f : 1.f;
-    float alpha = kind == 1 ? -1.f : 1.f;
-    float beta = (kind == 0) ? s : -s;
-    if (a == 0) { alpha *= SQRT2; beta = 0.f; if (n == 0) alpha = 1.f; }
-    else if (n == 0) { alpha *= RSQRT2; beta *= RSQRT2; }
-    out[(size_t)row * nbatch + z0 + zz] = alpha * av + beta * cv;
+    const RowRule r = rules[item * 16 + (p & 1) * 8 + sub];
+    if (r.row < 0) continue;
+    const float* v = vals + item * VLD_R + r.comp * ZR + zz;
+    dst[(size_t)r.row * nbatch] = r.alpha * v[0] + r.beta * v[8 * ZR];
   }
+}
+
+// the four rows R[+a,+n], R[+a,-n], R[-a,+n], R[-a,-n] of degree 4 c + u of an item (-1: none; rows[0] < 0: no such degree)
+struct QuadRows { int rows[4]; float s; };
+
+__device__ __forceinline__ QuadRows quad_rows(int inf, int u, int nl) {
+  const int c = inf & 0xff, a = (inf >> 8) & 0xff, n = (inf >> 16) & 0xff;
+  const int l = 4 * c + u;
+  QuadRows q{{-1, -1, -1, -1}, (a & 1) ? -1.f : 1.f};
+  if ((inf >> 24) && l >= a && l >= n && l < nl) {
+    q.rows[0] = lmn_index(l, a, n);
+    if (n > 0) q.rows[1] = lmn_index(l, a, -n);
+    if (a > 0) q.rows[2] = lmn_index(l, -a, n);
+    if (a > 0 && n > 0) q.rows[3] = lmn_index(l, -a, -n);
+  }
+  return q;
 }
 
 __global__ __launch_bounds__(256) void spectrum_gather_real(const float* __restrict__ rr, float4* __restrict__ rec, int nl, long nbatch) {
   __shared__ float vals[IT_TILE_R * VLD_R];
-  __shared__ int info[IT_TILE_R];
+  __shared__ QuadRows quads[IT_TILE_R * 4];
   const int th = threadIdx.x;
   const long z0 = (long)blockIdx.x * ZR;
   const int it = blockIdx.y >> 5, t0 = (blockIdx.y & 31) * IT_TILE_R;
-  if (th < IT_TILE_R) info[th] = pack_item_info(it * THREADS + t0 + th);
+  if (th < IT_TILE_R * 4) quads[th] = quad_rows(pack_item_info(it * THREADS + t0 + (th >> 2)), th & 3, nl);
   __syncthreads();
   {
     const int zz = th & 31, u = (th >> 5) & 3, sub = th >> 7;
     const long zc = z0 + zz < nbatch ? z0 + zz : nbatch - 1;
+    const float* src = rr + zc;
     for (int item = sub; item < IT_TILE_R; item += 2) {
-      const int inf = info[item];
-      const int c = inf & 0xff, a = (inf >> 8) & 0xff, n = (inf >> 16) & 0xff;
-      const int l = 4 * c + u;
+      const QuadRows q = quads[item * 4 + u];
       float2 A = make_float2(0.f, 0.f), C = A;
-      if ((inf >> 24) && l >= a && l >= n && l < nl) {
-        const float cc = rr[(size_t)lmn_index(l, a, n) * nbatch + zc];
-        const float cs = n > 0 ? rr[(size_t)lmn_index(l, a, -n) * nbatch + zc] : 0.f;
-        const float sc = a > 0 ? rr[(size_t)lmn_index(l, -a, n) * nbatch + zc] : 0.f;
-        const float ss = (a > 0 && n > 0) ? rr[(size_t)lmn_index(l, -a, -n) * nbatch + zc] : 0.f;
-        const float s = (a & 1) ? -1.f : 1.f;
-        if (a > 0 && n > 0) { A = make_float2(cc + ss, sc - cs); C = make_float2(s * (cc - ss), -s * (cs + sc)); }
-        else if (a > 0)     { A = make_float2(SQRT2 * cc, SQRT2 * sc); C = make_float2(s * SQRT2 * cc, -s * SQRT2 * sc); }
-        else if (n > 0)     { A = make_float2(SQRT2 * cc, -SQRT2 * cs); }
-        else                { A = make_float2(2.f * cc, 0.f); }
+      if (q.rows[0] >= 0) {
+        const bool hn = q.rows[1] >= 0, ha = q.rows[2] >= 0;
+        const float cc = src[(size_t)q.rows[0] * nbatch];
+        const float cs = hn ? src[(size_t)q.rows[1] * nbatch] : 0.f;
+        const float sc = ha ? src[(size_t)q.rows[2] * nbatch] : 0.f;
+        const float ss = q.rows[3] >= 0 ? src[(size_t)q.rows[3] * nbatch] : 0.f;
+        const float s = q.s;
+        if (ha && hn) { A = make_float2(cc + ss, sc - cs); C = make_float2(s * (cc - ss), -s * (cs + sc)); }
+        else if (ha)  { A = make_float2(SQRT2 * cc, SQRT2 * sc); C = make_float2(s * SQRT2 * cc, -s * SQRT2 * sc); }
+        else if (hn)  { A = make_float2(SQRT2 * cc, -SQRT2 * cs); }
+        else          { A = make_float2(2.f * cc, 0.f); }
       }
       const int comp = 4 * (u >> 1) + 2 * (u & 1);
       float* d = vals + item * VLD_R + comp * ZR + zz;
