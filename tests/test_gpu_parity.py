@@ -617,6 +617,55 @@ def test_so3_rft_kernel_spectrum(hip, factorised, monkeypatch):
     close(kg.grad, ko.grad, "so3_rft grad")
 
 
+@pytest.mark.parametrize("b,nz", [(32, 8200), (22, 25300)])
+def test_so3_transforms_beyond_32_bit_offsets(hip, b, nz):
+    """Batches whose tensors pass 2^31 elements (and 2^33 bytes): the last volumes must get the bits they get alone,
+    for the complex-pair and the real-basis spectra (64^3 grid: per-volume kernels; 44^3: plane + Wigner stages)."""
+    if torch.cuda.mem_get_info()[0] < 60 * 2 ** 30:
+        pytest.skip("needs 60 GiB of free device memory")
+    n = 2 * b
+    assert nz * n ** 3 > 2 ** 31
+    print(f"large batch b={b} nz={nz}", flush=True)
+    g = torch.Generator(device="cuda").manual_seed(b)
+    x = torch.randn(nz, n, n, n, device="cuda", generator=g)
+    last = x[-3:].clone()
+    s = PSO3.so3_rfft(x)
+    assert torch.equal(s[:, -3:], PSO3.so3_rfft(last))
+    assert torch.equal(s[:, 5:8], PSO3.so3_rfft(x[5:8].clone()))
+    r = PSO3.so3_rfft_real_basis(x)
+    assert torch.equal(r[:, -3:], PSO3.so3_rfft_real_basis(last))
+    del x
+    y = PSO3.so3_rifft(s)
+    assert torch.equal(y[-3:], PSO3.so3_rifft(s[:, -3:].contiguous()))
+    assert torch.equal(y[5:8], PSO3.so3_rifft(s[:, 5:8].contiguous()))
+    del y, s
+    y = PSO3.so3_rifft_real_basis(r)
+    assert torch.equal(y[-3:], PSO3.so3_rifft_real_basis(r[:, -3:].contiguous()))
+    del y, r
+    torch.cuda.empty_cache()
+
+
+def test_s2_transforms_and_integral_beyond_32_bit_offsets(hip):
+    """The same property for the S^2 transforms ([33 000, 256, 256] -> b 32 and back) and for so3_integrate."""
+    if torch.cuda.mem_get_info()[0] < 60 * 2 ** 30:
+        pytest.skip("needs 60 GiB of free device memory")
+    g = torch.Generator(device="cuda").manual_seed(128)
+    x = torch.randn(33000, 256, 256, device="cuda", generator=g)
+    assert x.numel() > 2 ** 31
+    s = PS2.s2_rfft(x, b_out=32)
+    assert torch.equal(s[:, -3:], PS2.s2_rfft(x[-3:].clone(), b_out=32))
+    del x
+    y = PS2.s2_rifft(s, for_grad=True, b_out=128)
+    assert y.numel() > 2 ** 31
+    assert torch.equal(y[-3:], PS2.s2_rifft(s[:, -3:].contiguous(), for_grad=True, b_out=128))
+    del y, s
+    x = torch.randn(8200, 64, 64, 64, device="cuda", generator=g)
+    v = s2cnn_amd.so3_integrate(x)
+    assert torch.equal(v[-3:], s2cnn_amd.so3_integrate(x[-3:].clone()))
+    del x
+    torch.cuda.empty_cache()
+
+
 def test_so3_round_trip_at_the_benchmark_size(hip):
     """[256, 64, 64, 64] (the transform benchmark): every volume of the batch gets the bits it gets alone (the result
     of a volume does not depend on the workgroup that takes it), and analysis o synthesis is the identity on spectra."""
