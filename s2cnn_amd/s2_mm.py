@@ -9,7 +9,6 @@ class _S2_mm(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, y):
-        _hip.require_gpu_f32(x, y)
         assert y.size(3) == 2
         assert x.size(3) == 2
         nbatch, f_in, f_out = x.size(1), x.size(2), y.size(2)
@@ -17,6 +16,7 @@ class _S2_mm(torch.autograd.Function):
         assert y.size(0) == x.size(0)
         nl = round(x.size(0) ** 0.5)
         assert x.size(0) == nl ** 2
+        _hip.require_gpu_f32(x, y)
         nspec = (4 * nl ** 2 - 1) * nl // 3
         x = x.contiguous()
         y = y.contiguous()

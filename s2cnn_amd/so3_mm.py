@@ -15,7 +15,6 @@ class _SO3_mm(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, y):
-        _hip.require_gpu_f32(x, y)
         assert y.size(3) == 2
         assert x.size(3) == 2
         nspec, nbatch, f_in = x.size(0), x.size(1), x.size(2)
@@ -23,6 +22,7 @@ class _SO3_mm(torch.autograd.Function):
         assert y.size(1) == f_in
         assert y.size(0) == nspec
         nl = _nl_from_nspec(nspec)
+        _hip.require_gpu_f32(x, y)
         x = x.contiguous()
         y = y.contiguous()
         ctx.save_for_backward(x, y)

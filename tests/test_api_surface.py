@@ -95,3 +95,30 @@ def test_layer_state_matches_the_reference():
     assert list(s.state_dict()) == []                                       # identity: no parameters
     s = so3_conv.SO3Shortcut(4, 6, 6, 4)
     assert {k: tuple(v.shape) for k, v in s.state_dict().items()} == {"conv.kernel": (4, 6, 1), "conv.bias": (1, 6, 1, 1, 1)}
+
+
+def test_shape_errors_are_assertion_errors():
+    """As in the reference (asserts at s2cnn/so3_mm.py:17-26, s2_mm.py:17-27, soft/so3_fft.py:17-21, soft/s2_fft.py:24,71,
+    soft/so3_conv.py:41-42): a call with inconsistent shapes fails with AssertionError before anything touches a device."""
+    import torch
+    z = torch.zeros
+    with pytest.raises(AssertionError):
+        s2cnn_amd.so3_mm(z(10, 2, 3, 2), z(10, 4, 5, 2))            # feature counts differ
+    with pytest.raises(AssertionError):
+        s2cnn_amd.so3_mm(z(11, 2, 3, 2), z(11, 3, 5, 2))            # 11 is no nspec(b)
+    with pytest.raises(AssertionError):
+        s2cnn_amd.s2_mm(z(9, 2, 3, 2), z(4, 3, 5, 2))               # spectra of different bandwidth
+    with pytest.raises(AssertionError):
+        s2cnn_amd.s2_mm(z(8, 2, 3, 2), z(8, 3, 5, 2))               # 8 is no b^2
+    with pytest.raises(AssertionError):
+        s2_fft.s2_fft(z(2, 8, 8, 2), b_out=5)                       # b_out > b_in
+    with pytest.raises(AssertionError):
+        s2_fft.s2_ifft(z(16, 2, 2), b_out=3)                        # b_out < b_in
+    with pytest.raises(AssertionError):
+        so3_fft.so3_rfft(z(2, 8, 8, 6))                             # not a cube
+    with pytest.raises(AssertionError):
+        so3_fft.so3_rifft(z(11, 2, 2))                              # 11 is no nspec(b)
+    with pytest.raises(AssertionError):
+        s2cnn_amd.SO3Convolution(2, 3, 4, 4, s2cnn_amd.so3_near_identity_grid())(z(1, 2, 8, 8, 6))
+    with pytest.raises(AssertionError):
+        s2cnn_amd.S2Convolution(2, 3, 4, 4, s2cnn_amd.s2_near_identity_grid())(z(1, 3, 8, 8))
