@@ -56,7 +56,9 @@ def nspec(b):
 
 def mm_flops(nl, B, Fi, Fo, real=True):
     """Algorithmic flops of one block product: B Fi Fo sum_l (2l+1)^3 = B Fi Fo nl^2 (2 nl^2 - 1) multiply-adds,
-    real (2 flops each) in the real basis the layer uses, complex (8 flops each) in so3_mm proper."""
+    real (2 flops each) in the real basis the layer uses, complex (8 flops each) in so3_mm proper.  The complex kernels
+    form a complex product from three real ones, so the matrix cores execute 6 flops per complex multiply-add: their
+    rows also give `mfma_executed_frac` = 3/4 of the algorithmic fraction."""
     return (2.0 if real else 8.0) * B * Fi * Fo * nl * nl * (2 * nl * nl - 1)
 
 
@@ -137,6 +139,19 @@ def measure_rows(torch, dev, with_cpu):
     add("s2_mm_real grad (x and y)", gpu_ms(lambda: torch.autograd.grad(zr, (xr, yr), gzr, retain_graph=True)),
         4.0 * 2 * (zr.numel() + xr.numel() + yr.numel()), "B", None, 1, "")
     del zk, gzk, xkg, ykg, s2spec, gspec, xs2g, xr, yr, zr, gzr
+    # --- the complex block product alone (config 3): x [43680, 16, 64, 2], y [43680, 64, 64, 2], forward and both gradients
+    xm = (torch.randn(nspec(32), 16, 64, 2, generator=g) * 0.125)
+    xmg = xm.to(dev).requires_grad_()
+    ymg = (torch.randn(nspec(32), 64, 64, 2, device=dev) * 0.125).requires_grad_()
+    zm = s2cnn_amd.so3_mm(xmg, ymg)
+    gzm = torch.randn_like(zm)
+    fl = mm_flops(32, 16, 64, 64, real=False)
+    t = cpu_s(lambda: O.so3_mm(xm[:, :1], ymg.detach().cpu()))
+    add("so3_mm fwd nl=32 B=16 64->64", gpu_ms(lambda: s2cnn_amd.so3_mm(xmg, ymg)), fl, "F", t, 1 / 16, "batch 1 of 16")
+    add("so3_mm grad (x and y)", gpu_ms(lambda: torch.autograd.grad(zm, (xmg, ymg), gzm, retain_graph=True)), 2 * fl, "F", None, 1, "")
+    for k in ("so3_mm fwd nl=32 B=16 64->64", "so3_mm grad (x and y)"):
+        rows[k]["mfma_executed_frac"] = round(0.75 * rows[k]["frac"], 4)
+    del xm, xmg, ymg, zm, gzm
     # --- Haar integral at config-4 output size [16, 64, 64, 64, 64]
     xi = torch.randn(16, 64, 64, 64, 64, device=dev)
     t = cpu_s(lambda: O.so3_integrate(xi[:2].cpu()))
@@ -288,6 +303,8 @@ def main():
                 "unit": "TFLOP/s", "frac": round(ach / PEAK_FP32_MFMA_TFLOPS, 4),
                 "traffic": MM_TRAFFIC_BYTES.get(dominant) if (B, F, b) == (16, 64, 32) else None,
                 "flop_per_launch": flops, "ms_per_launch": round(per_call[dominant], 3)}
+    if "_real_" not in dominant:   # three real products per complex one: the matrix cores execute 3/4 of the algorithmic flops
+        roofline["mfma_executed_frac"] = round(0.75 * roofline["frac"], 4)
     kernels = {n: {"ms": round(ms, 3)} for n, ms in per_call.items()}
     for n in mm_names:
         kernels[n]["tflops"] = round(flops_of[n] / (per_call[n] * 1e-3) / 1e12, 2)

@@ -14,15 +14,18 @@
 // The kernel keeps each operand tile in LDS in the orientation it has in memory, so loads
 // from HBM are coalesced and nothing is transposed on the way.
 //
-// Complex arithmetic on a real matrix core: one MFMA 32x32x2 takes two contraction steps,
-// one per half-wave.  The lower half is fed the real parts and the upper half the
-// imaginary parts of the same complex column, so that with b' = (br, bi) the instruction
-// accumulates ar*br + ai*bi (the real part of a*conj(b)), and with b'' = (-bi, br) the
-// imaginary part; without conjugation b' = (br, -bi), b'' = (bi, br).  Four real MACs per
-// complex MAC - the algorithmic minimum - and the A operand register is shared by both.
+// Complex arithmetic on a real matrix core, three real products per complex one (Gauss): with
+// b = br + i bi' (bi' = -bi where the operand is conjugated)
+//     P1 = sum ar br,   P2 = sum ai bi',   P3 = sum (ar + ai)(br + bi')
+//     re = P1 - P2,     im = P3 - P1 - P2.
+// One MFMA 32x32x2 takes two contraction steps, one per half-wave; a lane holds two consecutive complex
+// steps of its row / column (four floats), forms the two sums in registers and feeds six MFMAs: 1.5 per
+// complex multiply-add instead of the 2 of the direct form, at the price of a third accumulator per block.
+// The sums are formed in fp32 before the product, so the imaginary part carries a rounding error of the
+// size of |a||b| eps rather than of its own size: the same bound as any fp32 complex product.
 //
-// Tiling.  A workgroup (4 waves) owns 128 rows x 128 columns = 4 x 4 blocks of 32.  Wave (wm, wn)
-// takes row blocks wm, wm+2 and column blocks wn, wn+2, so a ragged tile (fewer live blocks) still
+// Tiling.  A workgroup (4 waves) owns 128 rows x 64 columns = 4 x 2 blocks of 32.  Wave (wm, wn)
+// takes row blocks wm, wm+2 and column block wn, so a ragged tile (fewer live blocks) still
 // splits evenly over the waves; blocks that lie wholly outside the matrix are skipped per wave.
 // The grid lists exactly the tiles of all degrees, heaviest degree first (no idle workgroups:
 // a workgroup that exits at once still waits for a full slot and stalls the in-order dispatch).
@@ -34,7 +37,7 @@ namespace {
 typedef float v16f __attribute__((ext_vector_type(16)));
 
 constexpr int NRB = 2;            // 32-row blocks per wave
-constexpr int NCB = 2;            // 32-column blocks per wave
+constexpr int NCB = 1;            // 32-column blocks per wave (three accumulators per block: 96 registers per wave)
 constexpr int TM = 64 * NRB;      // tile rows   (flattened (spectral, feature) index): 2 waves x NRB blocks
 constexpr int TN = 64 * NCB;      // tile cols
 constexpr int BSTR = 64, WSTR = 32;   // a wave's blocks are 64 apart, the two waves of a dimension offset by 32
@@ -151,8 +154,8 @@ struct TileLoader {
   }
 };
 
-// The four reals (re k0, im k0, re k0+1, im k0+1) one lane feeds to four consecutive MFMAs,
-// for tile row/col `idx` and the lane's pair of contraction steps k0 = 4s + 2h.
+// The four reals (re k0, im k0, re k0+1, im k0+1) of tile row/col `idx` and the lane's pair of
+// contraction steps k0 = 4s + 2h.
 template <bool KC, int LD>
 __device__ __forceinline__ float4 fetch_operand(const float2* tile, int idx, int k0) {
   if (KC) {
@@ -164,12 +167,14 @@ __device__ __forceinline__ float4 fetch_operand(const float2* tile, int idx, int
   }
 }
 
+// the three accumulators of a 32x32 block of complex outputs
+struct Acc3 { v16f p1, p2, p3; };
+
 // All matrix-core work of one LDS stage for a wave with NI live row blocks (rows arow + 64 i) and NJ
 // live column blocks (columns bcol + 64 j).  Operand registers are double buffered: the LDS reads of
 // step s+1 are issued before the MFMAs of step s.
 template <typename C_, int NI, int NJ>
-__device__ __forceinline__ void stage_mma(const float2* As, const float2* Bs, v16f (&acc_re)[NRB][NCB], v16f (&acc_im)[NRB][NCB],
-                                          int arow, int bcol, int h) {
+__device__ __forceinline__ void stage_mma(const float2* As, const float2* Bs, Acc3 (&acc)[NRB][NCB], int arow, int bcol, int h) {
   constexpr int ALD = TileShape<C_::A_KC, TM>::LD, BLD = TileShape<C_::B_KC, TN>::LD;
   float4 a[2][NI], b[2][NJ];
 #pragma unroll
@@ -186,29 +191,27 @@ __device__ __forceinline__ void stage_mma(const float2* As, const float2* Bs, v1
       for (int j = 0; j < NJ; ++j) b[nxt][j] = fetch_operand<C_::B_KC, BLD>(Bs, bcol + BSTR * j, 4 * (s + 1) + 2 * h);
     }
     __builtin_amdgcn_sched_barrier(0);   // keep the LDS reads of the next step ahead of this step's MFMAs
-    float4 bre[NJ], bim[NJ];
+    float2 asum[NI], bim[NJ], bsum[NJ];  // per contraction step of the lane's pair: ar + ai | bi' | br + bi'
+#pragma unroll
+    for (int i = 0; i < NI; ++i) asum[i] = make_float2(a[cur][i].x + a[cur][i].y, a[cur][i].z + a[cur][i].w);
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
       const float4 v = b[cur][j];
-      if (C_::CONJ) {
-        bre[j] = v;
-        bim[j] = make_float4(-v.y, v.x, -v.w, v.z);
-      } else {
-        bre[j] = make_float4(v.x, -v.y, v.z, -v.w);
-        bim[j] = make_float4(v.y, v.x, v.w, v.z);
-      }
+      bim[j] = C_::CONJ ? make_float2(-v.y, -v.w) : make_float2(v.y, v.w);
+      bsum[j] = make_float2(v.x + bim[j].x, v.z + bim[j].y);
     }
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
+    for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int i = 0; i < NI; ++i)
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
-          const float av = t == 0 ? a[cur][i].x : t == 1 ? a[cur][i].y : t == 2 ? a[cur][i].z : a[cur][i].w;
-          const float br = t == 0 ? bre[j].x : t == 1 ? bre[j].y : t == 2 ? bre[j].z : bre[j].w;
-          const float bi = t == 0 ? bim[j].x : t == 1 ? bim[j].y : t == 2 ? bim[j].z : bim[j].w;
-          acc_re[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, br, acc_re[i][j], 0, 0, 0);
-          acc_im[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bi, acc_im[i][j], 0, 0, 0);
+          const float ar = t == 0 ? a[cur][i].x : a[cur][i].z, ai = t == 0 ? a[cur][i].y : a[cur][i].w;
+          const float br = t == 0 ? b[cur][j].x : b[cur][j].z;
+          acc[i][j].p1 = __builtin_amdgcn_mfma_f32_32x32x2f32(ar, br, acc[i][j].p1, 0, 0, 0);
+          acc[i][j].p2 = __builtin_amdgcn_mfma_f32_32x32x2f32(ai, t == 0 ? bim[j].x : bim[j].y, acc[i][j].p2, 0, 0, 0);
+          acc[i][j].p3 = __builtin_amdgcn_mfma_f32_32x32x2f32(t == 0 ? asum[i].x : asum[i].y, t == 0 ? bsum[j].x : bsum[j].y,
+                                                              acc[i][j].p3, 0, 0, 0);
         }
   }
 }
@@ -217,7 +220,7 @@ __device__ __forceinline__ void stage_mma(const float2* As, const float2* Bs, v1
 // buffer, the operands of stage s+1 (fetched during stage s-1) are written to the other and the global loads
 // of stage s+2 are issued; one barrier per stage.
 template <typename C_, int NI, int NJ, typename LA, typename LB>
-__device__ __forceinline__ void contract(LA& la, LB& lb, float2* As, float2* Bs, v16f (&acc_re)[NRB][NCB], v16f (&acc_im)[NRB][NCB],
+__device__ __forceinline__ void contract(LA& la, LB& lb, float2* As, float2* Bs, Acc3 (&acc)[NRB][NCB],
                                          int nstage, int nkc, int arow, int bcol, int h) {
   constexpr int AEL = TileShape<C_::A_KC, TM>::ELEMS, BEL = TileShape<C_::B_KC, TN>::ELEMS;
   int kb = 0, kc = 0;
@@ -244,7 +247,7 @@ __device__ __forceinline__ void contract(LA& la, LB& lb, float2* As, float2* Bs,
       }
     }
     if (NI > 0 && NJ > 0)
-      stage_mma<C_, (NI > 0 ? NI : 1), (NJ > 0 ? NJ : 1)>(As + cur * AEL, Bs + cur * BEL, acc_re, acc_im, arow, bcol, h);
+      stage_mma<C_, (NI > 0 ? NI : 1), (NJ > 0 ? NJ : 1)>(As + cur * AEL, Bs + cur * BEL, acc, arow, bcol, h);
     __syncthreads();
   }
 }
@@ -287,13 +290,13 @@ __global__ __launch_bounds__(NT) void so3_block_mm_kernel(MmParams p) {
   const int r32 = lane & 31, h = lane >> 5;
   const int wrow = (wave >> 1) * WSTR, wcol = (wave & 1) * WSTR;
 
-  v16f acc_re[NRB][NCB], acc_im[NRB][NCB];
+  Acc3 acc[NRB][NCB];
 #pragma unroll
   for (int i = 0; i < NRB; ++i)
 #pragma unroll
     for (int j = 0; j < NCB; ++j)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) { acc_re[i][j][v] = 0.f; acc_im[i][j][v] = 0.f; }
+      for (int v = 0; v < 16; ++v) { acc[i][j].p1[v] = 0.f; acc[i][j].p2[v] = 0.f; acc[i][j].p3[v] = 0.f; }
 
   // live blocks of this wave: rows tile_m + wrow + 64 i < M, columns tile_n + wcol + 64 j < N (prefixes of i, j)
   const int remr = M - tile_m - wrow, remc = N - tile_n - wcol;
@@ -305,7 +308,7 @@ __global__ __launch_bounds__(NT) void so3_block_mm_kernel(MmParams p) {
   const int nkc = s2cnn::ceil_div(p.KI, TK);
   const int nstage = L * nkc;
   // one specialised copy of the whole contraction loop per count of live blocks (wave-uniform choice)
-#define S2CNN_CONTRACT(I, J) contract<C_, I, J>(la, lb, As, Bs, acc_re, acc_im, nstage, nkc, wrow + r32, wcol + r32, h)
+#define S2CNN_CONTRACT(I, J) contract<C_, I, J>(la, lb, As, Bs, acc, nstage, nkc, wrow + r32, wcol + r32, h)
   if (nj == NCB) {
     switch (ni) {
       case 4: if (NRB >= 4) { S2CNN_CONTRACT((NRB >= 4 ? 4 : 1), NCB); } break;
@@ -316,7 +319,7 @@ __global__ __launch_bounds__(NT) void so3_block_mm_kernel(MmParams p) {
     }
   } else if (nj == 0) {
     S2CNN_CONTRACT(0, 0);
-  } else {  // NCB == 2 and one live column block
+  } else if constexpr (NCB > 1) {  // one live column block of two
     switch (ni) {
       case 4: if (NRB >= 4) { S2CNN_CONTRACT((NRB >= 4 ? 4 : 1), 1); } break;
       case 3: if (NRB >= 3) { S2CNN_CONTRACT((NRB >= 3 ? 3 : 1), 1); } break;
@@ -344,7 +347,8 @@ __global__ __launch_bounds__(NT) void so3_block_mm_kernel(MmParams p) {
         if (row < M) {
           const int rb = row / p.RI, ri = row - rb * p.RI;
           const int blk = C_::C_RMAJ ? rb * L + cb : cb * L + rb;
-          Cl[(size_t)blk * blk_elems + ri * p.CI + ci] = make_float2(acc_re[i][j][v], acc_im[i][j][v]);
+          const float p1 = acc[i][j].p1[v], p2 = acc[i][j].p2[v];
+          Cl[(size_t)blk * blk_elems + ri * p.CI + ci] = make_float2(p1 - p2, acc[i][j].p3[v] - p1 - p2);
         }
       }
     }
