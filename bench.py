@@ -26,8 +26,8 @@ PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
 # HBM-side bytes per launch of the three product kernels at this workload, from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE scaled by a 1 GiB elementwise kernel of the same run (profiles/so3_mm_real_b32_B16_F64_hbm_traffic.md);
 # not re-measured at run time.
-MM_TRAFFIC_BYTES = {"s2cnn_so3_mm_real_fwd": 6.49e9 + 0.179e9, "s2cnn_so3_mm_real_gradx": 6.63e9 + 0.179e9,
-                    "s2cnn_so3_mm_real_grady": 5.01e9 + 0.716e9}
+MM_TRAFFIC_BYTES = {"s2cnn_so3_mm_real_fwd": 6.67e9 + 0.179e9, "s2cnn_so3_mm_real_gradx": 6.61e9 + 0.179e9,
+                    "s2cnn_so3_mm_real_grady": 5.04e9 + 0.716e9}
 
 
 def sum_of_squares(t):
