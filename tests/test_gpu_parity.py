@@ -568,6 +568,65 @@ def test_network_forward_replays_from_a_hip_graph(hip):
             assert torch.equal(static_y, want), f"replay {i} differs from the eager pass"
 
 
+def test_training_step_replays_from_a_hip_graph(hip):
+    """Forward, backward and an SGD update of the MNIST-shaped network (layers with the activation inside) captured
+    into one HIP graph: after the same inputs, every replayed step must leave the weights of an eager twin, bit for bit,
+    with eager work and synchronisations between the replays."""
+    pi = 3.141592653589793
+    g1 = s2cnn_amd.s2_near_identity_grid(max_beta=pi / 8, n_alpha=8, n_beta=3)
+    g2 = s2cnn_amd.so3_near_identity_grid(max_beta=pi / 8, max_gamma=2 * pi, n_alpha=8, n_beta=3, n_gamma=8)
+
+    def build():
+        torch.manual_seed(5)
+        c1 = s2cnn_amd.S2Convolution(1, 20, 30, 10, g1, activation="relu").cuda()
+        c2 = s2cnn_amd.SO3Convolution(20, 40, 10, 6, g2, activation="relu").cuda()
+        head = torch.nn.Linear(40, 10).cuda()
+        params = [*c1.parameters(), *c2.parameters(), *head.parameters()]
+        return (lambda x: head(s2cnn_amd.so3_integrate(c2(c1(x))))), params, torch.optim.SGD(params, lr=0.05)
+
+    net_g, params_g, opt_g = build()
+    net_e, params_e, opt_e = build()
+    gen = torch.Generator().manual_seed(6)
+    batches = [(torch.rand(8, 1, 60, 60, generator=gen).cuda(), torch.randint(0, 10, (8,), generator=gen).cuda()) for _ in range(3)]
+    static_x, static_t = batches[0][0].clone(), batches[0][1].clone()
+    start = [q.detach().clone() for q in params_g]
+
+    def step(net, opt, x, t):
+        opt.zero_grad(set_to_none=True)
+        loss = torch.nn.functional.cross_entropy(net(x), t)
+        loss.backward()
+        opt.step()
+        return loss
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            step(net_g, opt_g, static_x, static_t)      # tables, workspaces and allocator pools exist before the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    with torch.no_grad():
+        for q, q0 in zip(params_g, start):
+            q.copy_(q0)                                 # back to the weights the eager twin starts from
+    graph = torch.cuda.CUDAGraph()
+    opt_g.zero_grad(set_to_none=True)
+    with torch.cuda.graph(graph):
+        static_loss = step(net_g, opt_g, static_x, static_t)
+    with torch.no_grad():
+        for q, q0 in zip(params_g, start):
+            q.copy_(q0)                                 # the capture itself ran nothing, but keep the state explicit
+    for i, (x, t) in enumerate(batches):
+        static_x.copy_(x)
+        static_t.copy_(t)
+        graph.replay()
+        torch.cuda.synchronize()
+        loss_e = step(net_e, opt_e, x, t)               # eager work between the replays
+        torch.cuda.synchronize()
+        assert torch.equal(static_loss, loss_e), f"replay {i}: loss differs"
+        for k, (a, b) in enumerate(zip(params_g, params_e)):
+            assert torch.equal(a, b), f"replay {i}: parameter {k} differs from the eager step"
+
+
 def test_so3_projector_on_a_large_grid(hip):
     """b = 48 (96^3 grid, 147 440 coefficients): planes with more register blocks than 256 threads hold and degrees
     beyond the tiled Wigner kernels.  No oracle at this size: synthesis followed by analysis is the identity on
