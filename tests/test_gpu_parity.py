@@ -230,14 +230,14 @@ def test_so3_integrate(hip):
 
 
 # ------------------------------------------------------------------ layers, forward and gradients
-def _conv_case(kind, B, Fi, Fo, b_in, b_out, grid, seed, real_basis=None):
+def _conv_case(kind, B, Fi, Fo, b_in, b_out, grid, seed, real_basis=None, activation=None):
     if kind == "so3":
         x = rnd((B, Fi, 2 * b_in, 2 * b_in, 2 * b_in), seed)
-        layer = s2cnn_amd.SO3Convolution(Fi, Fo, b_in, b_out, grid)
+        layer = s2cnn_amd.SO3Convolution(Fi, Fo, b_in, b_out, grid, activation=activation)
         ofun = O.so3_conv
     else:
         x = rnd((B, Fi, 2 * b_in, 2 * b_in), seed)
-        layer = s2cnn_amd.S2Convolution(Fi, Fo, b_in, b_out, grid)
+        layer = s2cnn_amd.S2Convolution(Fi, Fo, b_in, b_out, grid, activation=activation)
         ofun = O.s2_conv
     k = torch.rand(Fi, Fo, len(grid), generator=torch.Generator().manual_seed(seed + 1)) * 2 - 1
     bias = rnd((1, Fo, 1, 1, 1), seed + 2, 0.1)
@@ -252,11 +252,48 @@ def _conv_case(kind, B, Fi, Fo, b_in, b_out, grid, seed, real_basis=None):
     (out ** 2).sum().backward()
     xo, ko, bo = x.double().requires_grad_(), k.double().requires_grad_(), bias.double().requires_grad_()
     outo = ofun(xo, ko, bo, b_in, b_out, grid)
+    if activation == "relu":
+        outo = torch.relu(outo)
     (outo ** 2).sum().backward()
     close(out, outo, kind + " conv out")
     close(xg.grad, xo.grad, kind + " conv grad x")
     close(layer.kernel.grad, ko.grad, kind + " conv grad kernel")
     close(layer.bias.grad, bo.grad, kind + " conv grad bias")
+
+
+def _random_grid(kind, rng):
+    import math
+    if kind == "so3":
+        pick = rng.randrange(3)
+        if pick == 0:
+            return s2cnn_amd.so3_near_identity_grid(max_beta=math.pi / rng.choice((4, 8, 16)), n_alpha=rng.choice((3, 4, 6, 8)),
+                                                    n_beta=rng.choice((1, 2, 3)), n_gamma=rng.choice((None, 1, 3, 5)))
+        if pick == 1:
+            return s2cnn_amd.so3_equatorial_grid(max_beta=rng.choice((0, 0.2)), max_gamma=rng.choice((0, 0.4)), n_alpha=rng.choice((4, 7, 12)),
+                                                 n_beta=rng.choice((1, 2)), n_gamma=rng.choice((1, 2, 3)))
+        return ((0.3, 1.0, 2.0), (1.1, 0.2, 5.0), (2.9, 4.0, 0.1), (0.3, 2.0, 2.5), (1.7, 3.3, 3.3))   # no two points share beta rings evenly
+    pick = rng.randrange(2)
+    if pick == 0:
+        return s2cnn_amd.s2_near_identity_grid(max_beta=math.pi / rng.choice((4, 8)), n_alpha=rng.choice((3, 5, 8)), n_beta=rng.choice((1, 2, 3)))
+    return s2cnn_amd.s2_equatorial_grid(max_beta=rng.choice((0, 0.3)), n_alpha=rng.choice((4, 9, 16)), n_beta=rng.choice((1, 3)))
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_layers_on_random_shapes(hip, seed):
+    """Seeded random draws of batch, feature counts, bandwidths (b_out <= b_in as the layers are used, both parities,
+    grids the fast paths do not cover) and kernel grids: forward and all gradients of both layers against the oracle,
+    in the real-basis and the complex formulation, with and without the activation inside."""
+    import random
+    rng = random.Random(1234 + seed)
+    for kind in ("so3", "s2"):
+        b_in = rng.randint(2, 7) if kind == "so3" else rng.randint(2, 12)
+        b_out = rng.randint(2, min(b_in, 6))       # b_out = 1 gives constant outputs: the std of the error metric vanishes
+        B, Fi, Fo = rng.randint(1, 5), rng.randint(1, 9), rng.randint(1, 9)
+        grid = _random_grid(kind, rng)
+        real_basis = rng.random() < 0.6
+        activation = rng.choice((None, "relu"))
+        print(f"random case {seed} {kind}: B={B} {Fi}->{Fo} b {b_in}->{b_out} grid {len(grid)} real_basis={real_basis} activation={activation}", flush=True)
+        _conv_case(kind, B, Fi, Fo, b_in, b_out, grid, 7000 + 10 * seed, real_basis, activation)
 
 
 def test_so3_convolution_parity(hip):
