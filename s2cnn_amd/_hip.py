@@ -120,11 +120,16 @@ def check(code):
 
 
 def require_gpu_f32(*tensors):
+    """Operands must be float32 tensors on the current GPU: kernels are launched on the current device's current
+    stream (as the reference's are, s2cnn/soft/so3_fft.py:341), so an operand elsewhere would be read across devices."""
     for t in tensors:
         if not (t.is_cuda and t.dtype == torch.float32):
             raise RuntimeError(
                 "s2cnn_amd runs float32 tensors on the GPU only (got %s on %s); there is no CPU path"
                 % (t.dtype, t.device))
+        if t.device.index != torch.cuda.current_device():
+            raise RuntimeError("operand on %s but the current device is cuda:%d: call inside torch.cuda.device(%d)"
+                               % (t.device, torch.cuda.current_device(), t.device.index))
 
 
 def stream_ptr():
