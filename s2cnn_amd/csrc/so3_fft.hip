@@ -318,9 +318,9 @@ bool sizes_ok(int b_grid, int b_spec, long nbatch) {
 size_t packed_bytes(int b_grid, int b_spec, int cplx, bool synthesis) {
   if (fused_path(b_grid, b_spec, cplx, synthesis)) return fused64::PACKED_FLOATS * sizeof(float);
   const int nb = b_grid < b_spec ? b_grid : b_spec;
-  if (cplx || nb > 32) return 0;
-  if (synthesis) return 2 * b_grid <= 64 ? wigner_tiled::packed_floats_synthesis(nb) * sizeof(float) : 0;
-  return b_spec <= 32 ? wigner_tiled::packed_floats_analysis(2 * b_grid, nb) * sizeof(float) : 0;
+  if (cplx || nb > 64) return 0;
+  if (synthesis) return 2 * b_grid <= 128 ? wigner_tiled::packed_floats_synthesis(2 * b_grid, nb) * sizeof(float) : 0;
+  return b_spec <= 64 ? wigner_tiled::packed_floats_analysis(2 * b_grid, nb, b_spec) * sizeof(float) : 0;
 }
 
 size_t round256(size_t n) { return (n + 255) & ~(size_t)255; }
@@ -480,8 +480,13 @@ int analysis_impl(const float* x, const float* mask, const float* table, const f
       hipLaunchKernelGGL(wigner_tiled::pack_table_analysis, dim3(2048), dim3(256), 0, st, table, dst, n2, nb, b_out);
       Tp = dst;
     }
-    hipLaunchKernelGGL(wigner_tiled::wigner_fwd_tiled, dim3(wigner_tiled::grid_size(MW, nbatch)), dim3(256), 0, st, X, Tp,
-                       reinterpret_cast<float2*>(out), n2, nb, b_out, nbatch);
+    const int parts = wigner_tiled::parts_analysis(nb, b_out);
+    if (parts == 1)
+      hipLaunchKernelGGL(wigner_tiled::wigner_fwd_tiled<false>, dim3(wigner_tiled::grid_size(MW, nbatch)), dim3(256), 0, st, X, Tp,
+                         reinterpret_cast<float2*>(out), n2, nb, b_out, nbatch);
+    else
+      hipLaunchKernelGGL(wigner_tiled::wigner_fwd_tiled<true>, dim3(wigner_tiled::grid_size(MW, nbatch), parts), dim3(256), 0, st, X, Tp,
+                         reinterpret_cast<float2*>(out), n2, nb, b_out, nbatch);
     return s2cnn::launch_status();
   }
   dim3 grid(s2cnn::ceil_div(NW, 16), MW, (unsigned)((nbatch + 15) / 16));
@@ -521,8 +526,8 @@ int synthesis_impl(const float* xhat, const float* table, const float* packed_ta
       hipLaunchKernelGGL(wigner_tiled::pack_table_synthesis, dim3(2048), dim3(256), 0, st, table, dst, n2, nb, b_in);
       Tq = dst;
     }
-    hipLaunchKernelGGL(wigner_tiled::wigner_inv_tiled, dim3(wigner_tiled::grid_size(MW, nbatch)), dim3(512), 0, st, xh, Tq, S,
-                       n2, nb, b_in, nbatch);
+    hipLaunchKernelGGL(wigner_tiled::wigner_inv_tiled, dim3(wigner_tiled::grid_size(MW, nbatch), wigner_tiled::parts_synthesis(n2, nb)),
+                       dim3(512), 0, st, xh, Tq, S, n2, nb, b_in, nbatch);
   } else if (complex_out) {
     hipLaunchKernelGGL(so3_wigner_inv<true>, grid, dim3(16, 16), 0, st, xh, table, S, n2, nb, b_in, nbatch);
   } else {

@@ -7,10 +7,13 @@
 //              xs = (xhat[l,m,n] + (-1)^(m-n) conj xhat[l,-m,-n]) / 2
 //
 // The table is consumed in a packed, zero-padded order that makes every chunk one contiguous block:
-//   analysis : Tp[mi][beta][n (32)][l (32)]        (pack_table_analysis)
-//   synthesis: Tq[mi][l (nb)][n (32)][beta (64)]   (pack_table_synthesis)
+//   analysis : Tp[part][mi][beta][n (32)][l (32)]        (pack_table_analysis)
+//   synthesis: Tq[part][mi][l (nb)][n (32)][beta (64)]   (pack_table_synthesis)
 // with zeros outside max(|m|, n) <= l < number of degrees, n < nb, beta < 2 b_grid.
-// Requirements: nb = min(b_grid, b_spec) <= 32, degrees <= 32 (analysis), 2 b_grid <= 64 (synthesis).
+// A workgroup covers 32 values of n and 32 degrees (analysis) or 64 betas (synthesis); larger problems are cut
+// into parts, one more grid dimension: analysis (l0, n0) = (0,0), (32,0), (32,32) (n <= l), synthesis
+// (n0, beta0) in {0, 32} x {0, 64}.
+// Requirements: nb = min(b_grid, b_spec) <= 64, degrees <= 64 (analysis), 2 b_grid <= 128 (synthesis).
 #pragma once
 #include <hip/hip_runtime.h>
 
@@ -44,16 +47,31 @@ inline int grid_size(int MW, long nbatch) {
   return (int)(8L * ((MW + 7) / 8) * nzt);
 }
 
-__host__ __device__ inline size_t packed_floats_analysis(int n2, int nb) { return (size_t)(2 * nb - 1) * n2 * 1024; }
-__host__ __device__ inline size_t packed_floats_synthesis(int nb) { return (size_t)(2 * nb - 1) * nb * 32 * 64; }
+// parts of the analysis: degrees [l0, l0 + 32) x frequencies n in [n0, n0 + 32)
+__host__ __device__ inline int parts_analysis(int nb, int nl) { return nl <= 32 ? 1 : nb <= 32 ? 2 : 3; }
+__host__ __device__ inline void part_analysis(int part, int& l0, int& n0) { l0 = part >= 1 ? 32 : 0; n0 = part == 2 ? 32 : 0; }
+// parts of the synthesis: n in [n0, n0 + 32) x betas [beta0, beta0 + 64)
+__host__ __device__ inline int parts_synthesis(int n2, int nb) { return (nb > 32 ? 2 : 1) * (n2 > 64 ? 2 : 1); }
+__host__ __device__ inline void part_synthesis(int part, int nb, int& n0, int& beta0) {
+  const int pn = nb > 32 ? 2 : 1;
+  n0 = 32 * (part % pn); beta0 = 64 * (part / pn);
+}
+
+__host__ __device__ inline size_t packed_floats_analysis_part(int n2, int nb) { return (size_t)(2 * nb - 1) * n2 * 1024; }
+__host__ __device__ inline size_t packed_floats_synthesis_part(int nb) { return (size_t)(2 * nb - 1) * nb * 32 * 64; }
+__host__ __device__ inline size_t packed_floats_analysis(int n2, int nb, int nl) { return parts_analysis(nb, nl) * packed_floats_analysis_part(n2, nb); }
+__host__ __device__ inline size_t packed_floats_synthesis(int n2, int nb) { return parts_synthesis(n2, nb) * packed_floats_synthesis_part(nb); }
 
 // one thread per packed element
 __global__ void pack_table_analysis(const float* __restrict__ T, float* __restrict__ Tp, int n2, int nb, int nl) {
-  const size_t total = packed_floats_analysis(n2, nb);
+  const size_t per_part = packed_floats_analysis_part(n2, nb), total = packed_floats_analysis(n2, nb, nl);
   const long nspec = (long)nl * (4L * nl * nl - 1) / 3;
   for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
-    const int l = i & 31, n = (i >> 5) & 31;
-    const size_t r = i >> 10;
+    int l0, n0;
+    part_analysis((int)(i / per_part), l0, n0);
+    const size_t ip = i % per_part;
+    const int l = l0 + (int)(ip & 31), n = n0 + (int)((ip >> 5) & 31);
+    const size_t r = ip >> 10;
     const int bt = (int)(r % n2), m = (int)(r / n2) - (nb - 1);
     const int am = m < 0 ? -m : m;
     float v = 0.f;
@@ -63,11 +81,14 @@ __global__ void pack_table_analysis(const float* __restrict__ T, float* __restri
 }
 
 __global__ void pack_table_synthesis(const float* __restrict__ T, float* __restrict__ Tq, int n2, int nb, int b_spec) {
-  const size_t total = packed_floats_synthesis(nb);
+  const size_t per_part = packed_floats_synthesis_part(nb), total = packed_floats_synthesis(n2, nb);
   const long nspec = (long)b_spec * (4L * b_spec * b_spec - 1) / 3;
   for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
-    const int bt = i & 63, n = (i >> 6) & 31;
-    const size_t r = i >> 11;
+    int n0, beta0;
+    part_synthesis((int)(i / per_part), nb, n0, beta0);
+    const size_t ip = i % per_part;
+    const int bt = beta0 + (int)(ip & 63), n = n0 + (int)((ip >> 6) & 31);
+    const size_t r = ip >> 11;
     const int l = (int)(r % nb), m = (int)(r / nb) - (nb - 1);
     const int am = m < 0 ? -m : m;
     float v = 0.f;
@@ -86,6 +107,9 @@ __global__ void pack_table_synthesis(const float* __restrict__ T, float* __restr
 typedef float v16f __attribute__((ext_vector_type(16)));
 constexpr int XLD_M = 33;     // z stride (complex) of the X chunk: (z, c) lanes hit 32 distinct banks
 
+// PARTS = false: one part (nb, nl <= 32), the chunk of X is one contiguous run; true: the parts above, the chunk is
+// KB*16 row pieces.
+template <bool PARTS>
 __global__ __launch_bounds__(256, 2) void wigner_fwd_tiled(const float2* __restrict__ X, const float* __restrict__ Tp,
                                                            float2* __restrict__ out, int n2, int nb, int nl, long nbatch) {
   __shared__ __attribute__((aligned(16))) float2 Xs[KB * ZT * XLD_M];
@@ -97,6 +121,10 @@ __global__ __launch_bounds__(256, 2) void wigner_fwd_tiled(const float2* __restr
   const int mi = m + nb - 1;
   const long z0 = (long)zt * ZT;
   const int am = abs(m);
+  int l0 = 0, n0 = 0;                           // this workgroup's part: degrees l0 .. l0+31, frequencies n0 .. n0+31
+  if constexpr (PARTS) part_analysis(blockIdx.y, l0, n0);
+  if (am >= l0 + 32) return;                    // no degree of the part reaches |m|
+  const int CW = NW - n0 < 32 ? NW - n0 : 32;   // columns of the part
 
   const int t = threadIdx.x;
   const int lane = t & 63, wave = t >> 6;
@@ -113,24 +141,34 @@ __global__ __launch_bounds__(256, 2) void wigner_fwd_tiled(const float2* __restr
   float4 tr_[KB];
   // packed table: the chunk of KB betas is KB*1024 contiguous floats; slot i covers floats 4 (t + 256 i)..+3,
   // i.e. beta_local = i, n = t / 8, l = 4 (t % 8)
-  const float4* tbase = reinterpret_cast<const float4*>(Tp + (size_t)mi * n2 * 1024);
+  const float4* tbase = reinterpret_cast<const float4*>(Tp + (PARTS ? blockIdx.y * packed_floats_analysis_part(n2, nb) : 0) + (size_t)mi * n2 * 1024);
   const int tlds = (t >> 3) * TLD + 4 * (t & 7);
-  // X is laid out [z tile][mi][beta][z % 16][n]: one chunk (KB betas) is KB*16*NW contiguous complex
-  // numbers; thread slot i covers element e = t + 256 i of the chunk.
-  const int chunk_elems = KB * ZT * NW;
-  const float2* xbase = X + ((size_t)zt * MW + mi) * n2 * ZT * NW;
-  const int n2elems = n2 * ZT * NW;
+  // X is laid out [z tile][mi][beta][z % 16][n]: a chunk (KB betas) is KB*16 rows of NW complex numbers.
+  // One part: the chunk is KB*16*NW contiguous numbers; thread slot i covers element e = t + 256 i of it.
+  // Several parts: the part takes the CW columns from n0 of every row; a thread keeps one column (lc) and takes rows
+  // lr, lr + 8, ...: offsets that advance by constants, nothing per slot to keep in registers.
+  const int lc = t & 31, lr = t >> 5;
+  const bool colok = lc < CW;
+  const float2* xbase = X + ((size_t)zt * MW + mi) * n2 * ZT * NW + (PARTS ? n0 + (colok ? lc : 0) : 0);
+  const int nrows = n2 * ZT;
+  const int chunk_elems = KB * ZT * NW, n2elems = n2 * ZT * NW;
   const float inv_nw = 1.0f / (float)NW;         // e / NW for e < 4096, NW <= 32: (e + 0.5) * inv_nw truncates exactly
-  // columns n >= NW of the X chunk are never loaded: clear them once (T is zero there, but 0 * NaN is not)
+  // columns n >= CW of the X chunk are never loaded: clear them once (T is zero there, but 0 * NaN is not)
   for (int i = t; i < KB * ZT * XLD_M; i += 256) Xs[i] = make_float2(0.f, 0.f);
 
   auto load_chunk = [&](int b0) {
-    const int e0 = b0 * ZT * NW;
 #pragma unroll
     for (int i = 0; i < KB * 2; ++i) {
-      const int e = e0 + t + 256 * i;
-      const float2 v = xbase[e < n2elems ? e : 0];
-      xr[i] = e < n2elems ? v : make_float2(0.f, 0.f);
+      if constexpr (PARTS) {
+        const int row = b0 * ZT + lr + 8 * i;                  // beta * 16 + z
+        const bool ok = colok && row < nrows;
+        const float2 v = xbase[ok ? row * NW : 0];
+        xr[i] = ok ? v : make_float2(0.f, 0.f);
+      } else {
+        const int e = b0 * ZT * NW + t + 256 * i;
+        const float2 v = xbase[e < n2elems ? e : 0];
+        xr[i] = e < n2elems ? v : make_float2(0.f, 0.f);
+      }
     }
 #pragma unroll
     for (int bt = 0; bt < KB; ++bt) {
@@ -148,11 +186,18 @@ __global__ __launch_bounds__(256, 2) void wigner_fwd_tiled(const float2* __restr
   load_chunk(0);
   for (int b0 = 0; b0 < n2; b0 += KB) {
     __syncthreads();
+    if constexpr (PARTS) {
+      if (colok) {
 #pragma unroll
-    for (int i = 0; i < KB * 2; ++i) {
-      const int e = t + 256 * i;
-      const int row = (int)(((float)e + 0.5f) * inv_nw);     // beta_local * 16 + z
-      if (e < chunk_elems) Xs[row * XLD_M + (e - row * NW)] = xr[i];
+        for (int i = 0; i < KB * 2; ++i) Xs[(lr + 8 * i) * XLD_M + lc] = xr[i];
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < KB * 2; ++i) {
+        const int e = t + 256 * i;
+        const int row = (int)(((float)e + 0.5f) * inv_nw);     // beta_local * 16 + z
+        if (e < chunk_elems) Xs[row * XLD_M + (e - row * NW)] = xr[i];
+      }
     }
 #pragma unroll
     for (int bt = 0; bt < KB; ++bt) *reinterpret_cast<float4*>(Ts + bt * 32 * TLD + tlds) = tr_[bt];
@@ -170,35 +215,27 @@ __global__ __launch_bounds__(256, 2) void wigner_fwd_tiled(const float2* __restr
   }
 
   // ---- write out[lmn][z].c and its mirror (-m,-n); (m < 0, n = 0) is written by the workgroup of -m.
-  // Accumulator register v of lane (l32 = 2 z + c, h) holds degree l = 8 (v / 4) + 4 h + v % 4.
+  // Accumulator register v of lane (l32 = 2 z + c, h) holds degree l = l0 + 8 (v / 4) + 4 h + v % 4.
   const long z = z0 + (l32 >> 1);
   if (z >= nbatch) return;
   const int c = l32 & 1;
   float* outf = reinterpret_cast<float*>(out) + z * 2 + c;
   const size_t rowf = (size_t)nbatch * 2;        // floats per spectral row
-  // lmn(l, m, n) = lbase[l] + m (2l+1) + n with lbase[l] = l(4l^2-1)/3 + l(2l+1) + l; the mirror is lbase[l] - m(2l+1) - n
-  int lbase[16], lcoef[16];
+  // lmn(l, m, n) = lbase + m (2l+1) + n with lbase = l(4l^2-1)/3 + l(2l+1) + l; the mirror is lbase - m(2l+1) - n
 #pragma unroll
   for (int v = 0; v < 16; ++v) {
-    const int l = 8 * (v / 4) + 4 * h + (v % 4);
-    lcoef[v] = 2 * l + 1;
-    lbase[v] = l * (4 * l * l - 1) / 3 + l * (2 * l + 1) + l;
-  }
+    const int l = l0 + 8 * (v / 4) + 4 * h + (v % 4);
+    if (l >= nl || l < am) continue;
+    const int lcoef = 2 * l + 1;
+    const int lbase = l * (4 * l * l - 1) / 3 + l * lcoef + l;
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const int n = 8 * wave + j;
-    if (n >= NW || (n == 0 && m < 0)) continue;
-    const bool mirror = (n > 0 || m > 0);
-    const float sg = (((m - n) & 1) ? -1.f : 1.f) * (c ? -1.f : 1.f);
-    const int lmin = am > n ? am : n;
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int l = 8 * (v / 4) + 4 * h + (v % 4);
-      if (l >= lmin && l < nl) {
-        const int d = m * lcoef[v] + n;
-        outf[(size_t)(lbase[v] + d) * rowf] = acc[j][v];
-        if (mirror) outf[(size_t)(lbase[v] - d) * rowf] = sg * acc[j][v];
-      }
+    for (int j = 0; j < 8; ++j) {
+      const int n = n0 + 8 * wave + j;
+      if (n >= NW || n > l || (n == 0 && m < 0)) continue;
+      const float sg = (((m - n) & 1) ? -1.f : 1.f) * (c ? -1.f : 1.f);
+      const int d = m * lcoef + n;
+      outf[(size_t)(lbase + d) * rowf] = acc[j][v];
+      if (n > 0 || m > 0) outf[(size_t)(lbase - d) * rowf] = sg * acc[j][v];
     }
   }
 }
@@ -216,8 +253,9 @@ __global__ __launch_bounds__(512) void wigner_inv_tiled(const float2* __restrict
   if (!decode_block(MW, nb, nzt, m, zt)) return;
   const int mi = m + nb - 1;
   const long z0 = (long)zt * ZT;
-  const long nspec = (long)b_spec * (4L * b_spec * b_spec - 1) / 3;
   const int am = abs(m);
+  int n0, beta0;                                // this workgroup's part: frequencies n0 .. n0+31, betas beta0 .. beta0+63
+  part_synthesis(blockIdx.y, nb, n0, beta0);
 
   const int t = threadIdx.x;
   const int n = t & 31, zq = (t >> 5) & 7, bh = t >> 8;
@@ -225,7 +263,7 @@ __global__ __launch_bounds__(512) void wigner_inv_tiled(const float2* __restrict
 #pragma unroll
   for (int j = 0; j < 32; ++j) { acc[j][0] = make_float2(0.f, 0.f); acc[j][1] = make_float2(0.f, 0.f); }
 
-  const int xz = t & 15, xn = t >> 4;           // spectrum loader: z fastest (contiguous in memory), n = 0..31
+  const int xz = t & 15, xn = n0 + (t >> 4);    // spectrum loader: z fastest (contiguous in memory), 32 values of n
   const float hs = ((m & 1) ? -0.5f : 0.5f);    // (-1)^(m-n)/2 = hs * (-1)^n
 
   // Unconditional (clamped) loads, next chunk fetched while the current one is consumed.
@@ -233,7 +271,7 @@ __global__ __launch_bounds__(512) void wigner_inv_tiled(const float2* __restrict
   float4 tq[LC];
   // packed table: degree l of this m is 32*64 contiguous floats; slot i covers floats 4 t..+3 of degree l0 + i,
   // i.e. n = t / 16, beta = 4 (t % 16)
-  const float4* tbase = reinterpret_cast<const float4*>(Tq_g + (size_t)mi * nb * 2048);
+  const float4* tbase = reinterpret_cast<const float4*>(Tq_g + blockIdx.y * packed_floats_synthesis_part(nb) + (size_t)mi * nb * 2048);
   const int tlds = (t >> 4) * QLD + 4 * (t & 15);
   const long zc = z0 + xz < nbatch ? z0 + xz : nbatch - 1;
 
@@ -250,7 +288,7 @@ __global__ __launch_bounds__(512) void wigner_inv_tiled(const float2* __restrict
     }
   };
 
-  const int lstart = (am / LC) * LC;
+  const int lstart = ((am > n0 ? am : n0) / LC) * LC;   // no degree below max(|m|, n0) contributes
   load_chunk(lstart);
   for (int l0 = lstart; l0 < nb; l0 += LC) {
     __syncthreads();
@@ -260,7 +298,7 @@ __global__ __launch_bounds__(512) void wigner_inv_tiled(const float2* __restrict
       const bool okx = (l < nb && l >= am && l >= xn && xn < NW && z0 + xz < nbatch);
       const float sg = (xn & 1) ? -hs : hs;
       const float2 a = xa[i], b = xb[i];
-      xs[(i * ZT + xz) * SLD + xn] = okx ? make_float2(0.5f * a.x + sg * b.x, 0.5f * a.y - sg * b.y) : make_float2(0.f, 0.f);
+      xs[(i * ZT + xz) * SLD + (t >> 4)] = okx ? make_float2(0.5f * a.x + sg * b.x, 0.5f * a.y - sg * b.y) : make_float2(0.f, 0.f);
       *reinterpret_cast<float4*>(Tq + i * 32 * QLD + tlds) = tq[i];
     }
     __syncthreads();
@@ -284,16 +322,16 @@ __global__ __launch_bounds__(512) void wigner_inv_tiled(const float2* __restrict
     }
   }
 
-  if (n >= NW) return;
+  if (n0 + n >= NW) return;
   const size_t plane = (size_t)MW * NW;
 #pragma unroll
   for (int zz = 0; zz < 2; ++zz) {
     const long z = z0 + 2 * zq + zz;
     if (z >= nbatch) continue;
-    float2* p = S + ((size_t)z * n2 * MW + mi) * NW + n;
+    float2* p = S + ((size_t)z * n2 * MW + mi) * NW + n0 + n;
 #pragma unroll
     for (int j = 0; j < 32; ++j) {
-      const int bt = 32 * bh + j;
+      const int bt = beta0 + 32 * bh + j;
       if (bt < n2) p[(size_t)bt * plane] = acc[j][zz];
     }
   }

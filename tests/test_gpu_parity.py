@@ -537,7 +537,9 @@ def test_so3_mm_at_config3_features_linearity(hip):
     assert z2.abs().max().item() < 1e-4 * z.std().item()
 
 
-@pytest.mark.parametrize("b_grid,b_spec,nz", [(22, 22, 2), (22, 7, 5), (40, 8, 1), (5, 5, 60), (1, 1, 300)])
+@pytest.mark.parametrize("b_grid,b_spec,nz", [(22, 22, 2), (22, 7, 5), (40, 8, 1), (5, 5, 60), (1, 1, 300),
+                                              # more than 32 frequencies or degrees: the Wigner stage runs in parts
+                                              (36, 36, 3), (34, 40, 2), (40, 34, 17), (32, 37, 2), (50, 33, 1)])
 def test_so3_real_transforms_on_other_grids(hip, b_grid, b_spec, nz):
     """Real signals on grids other than 64^3: the folded plane transform takes several planes per workgroup
     (ragged last workgroup included) or one large plane; analysis truncates, synthesis zero-extends."""
@@ -666,7 +668,7 @@ def test_training_step_replays_from_a_hip_graph(hip):
 
 def test_so3_projector_on_a_large_grid(hip):
     """b = 48 (96^3 grid, 147 440 coefficients): planes with more register blocks than 256 threads hold and degrees
-    beyond the tiled Wigner kernels.  No oracle at this size: synthesis followed by analysis is the identity on
+    beyond one part of the tiled Wigner kernels.  No oracle at this size: synthesis followed by analysis is the identity on
     spectra of real signals, analysis followed by synthesis a projector, and truncation commutes with both."""
     b = 48
     g = torch.Generator().manual_seed(90)
