@@ -17,7 +17,8 @@
 // One MFMA 32x32x2 takes two contraction steps, one per half-wave; a lane reads four consecutive steps
 // at once (k = 8s + 4h .. +3) and feeds them to four consecutive MFMAs.
 //
-// Tiling.  A workgroup (4 waves) owns TM x TN = (64 NRB) x (64 NCB) outputs; wave (wm, wn) takes row
+// Tiling.  A workgroup (4 waves) owns TM x TN = (64 NRB) x (64 NCB) outputs (NCB = 2, or 1 when the 128 x 128 tiles
+// of a small problem would leave CUs without work); wave (wm, wn) takes row
 // blocks wm + 2i and column blocks wn + 2j (interleaved, so ragged tiles still split evenly).  The grid
 // lists exactly the tiles of all degrees, heaviest degree first.
 #include <type_traits>
@@ -28,13 +29,12 @@ namespace {
 typedef float v16f __attribute__((ext_vector_type(16)));
 
 constexpr int NRB = 2;            // 32-row blocks per wave
-constexpr int NCB = 2;            // 32-column blocks per wave
 constexpr int TM = 64 * NRB;
-constexpr int TN = 64 * NCB;
 constexpr int BSTR = 64, WSTR = 32;
 constexpr int TK = 32;            // contraction steps per LDS stage
 constexpr int NT = 256;
 constexpr int KC_LD = TK + 4;     // leading dim of a K-contiguous LDS tile: 144 B rows
+constexpr int SMALL_GRID = 512;   // workgroups that fill the chip (2 per CU)
 
 enum Mode { FWD = 0, GRADX = 1, GRADY = 2 };
 
@@ -244,8 +244,9 @@ __device__ __forceinline__ float4 fetch_operand(const float* tile, int idx, int 
   }
 }
 
-template <typename C_, int NI, int NJ>
+template <typename C_, int NCB, int NI, int NJ>
 __device__ __forceinline__ void stage_mma(const float* As, const float* Bs, v16f (&acc)[NRB][NCB], int arow, int bcol, int h) {
+  constexpr int TN = 64 * NCB;
   constexpr int ALD = TileShape<C_::A_KC, TM>::LD, BLD = TileShape<C_::B_KC, TN>::LD;
   constexpr int NS = TK / 8;
   float4 a[2][NI], b[2][NJ];
@@ -279,9 +280,10 @@ __device__ __forceinline__ void stage_mma(const float* As, const float* Bs, v16f
 // Double-buffered LDS: while the matrix cores consume stage s from one buffer, the operands of stage s+1
 // (fetched during stage s-1) are written to the other and the global loads of stage s+2 are issued; one
 // barrier per stage.
-template <typename C_, int NI, int NJ, typename LA, typename LB>
+template <typename C_, int NCB, int NI, int NJ, typename LA, typename LB>
 __device__ __forceinline__ void contract(LA& la, LB& lb, float* As, float* Bs, v16f (&acc)[NRB][NCB],
                                          int nstage, int arow, int bcol, int h) {
+  constexpr int TN = 64 * NCB;
   constexpr int AEL = TileShape<C_::A_KC, TM>::ELEMS, BEL = TileShape<C_::B_KC, TN>::ELEMS;
   la.load();
   lb.load();
@@ -303,20 +305,21 @@ __device__ __forceinline__ void contract(LA& la, LB& lb, float* As, float* Bs, v
       }
     }
     if (NI > 0 && NJ > 0)
-      stage_mma<C_, (NI > 0 ? NI : 1), (NJ > 0 ? NJ : 1)>(As + cur * AEL, Bs + cur * BEL, acc, arow, bcol, h);
+      stage_mma<C_, NCB, (NI > 0 ? NI : 1), (NJ > 0 ? NJ : 1)>(As + cur * AEL, Bs + cur * BEL, acc, arow, bcol, h);
     __syncthreads();
   }
 }
 
-__host__ __device__ inline void tile_counts(int L, int RI, int CI, int& tm, int& tn, int& slots) {
+__host__ __device__ inline void tile_counts(int L, int RI, int CI, int TN, int& tm, int& tn, int& slots) {
   tm = s2cnn::ceil_div(L * RI, TM);
   tn = s2cnn::ceil_div(L * CI, TN);
   slots = tm * tn;
 }
 
-template <int MODE, int VA, int VB, bool FAST>
+template <int MODE, int VA, int VB, bool FAST, int NCB>
 __global__ __launch_bounds__(NT) void so3_block_mm_real_kernel(MmParams p) {
   typedef Cfg<MODE> C_;
+  constexpr int TN = 64 * NCB;
 
   __shared__ __attribute__((aligned(16))) float As[2 * TileShape<C_::A_KC, TM>::ELEMS];
   __shared__ __attribute__((aligned(16))) float Bs[2 * TileShape<C_::B_KC, TN>::ELEMS];
@@ -324,7 +327,7 @@ __global__ __launch_bounds__(NT) void so3_block_mm_real_kernel(MmParams p) {
   int t = blockIdx.x;
   int l = p.nl - 1, tm = 0, tn = 0, slots = 0;
   for (;; --l) {
-    tile_counts(2 * l + 1, p.RI, p.CI, tm, tn, slots);
+    tile_counts(2 * l + 1, p.RI, p.CI, TN, tm, tn, slots);
     if (t < slots || l == 0) break;
     t -= slots;
   }
@@ -360,7 +363,7 @@ __global__ __launch_bounds__(NT) void so3_block_mm_real_kernel(MmParams p) {
   if (ni == 0 || nj == 0) ni = nj = 0;
 
   const int nstage = s2cnn::ceil_div(L * p.KI, TK);
-#define S2CNN_CONTRACT(I, J) contract<C_, I, J>(la, lb, As, Bs, acc, nstage, wrow + r32, wcol + r32, h)
+#define S2CNN_CONTRACT(I, J) contract<C_, NCB, I, J>(la, lb, As, Bs, acc, nstage, wrow + r32, wcol + r32, h)
   if (nj == NCB) {
     switch (ni) {
       case 4: if (NRB >= 4) { S2CNN_CONTRACT((NRB >= 4 ? 4 : 1), NCB); } break;
@@ -371,7 +374,7 @@ __global__ __launch_bounds__(NT) void so3_block_mm_real_kernel(MmParams p) {
     }
   } else if (nj == 0) {
     S2CNN_CONTRACT(0, 0);
-  } else {
+  } else if constexpr (NCB > 1) {
     switch (ni) {
       case 4: if (NRB >= 4) { S2CNN_CONTRACT((NRB >= 4 ? 4 : 1), 1); } break;
       case 3: if (NRB >= 3) { S2CNN_CONTRACT((NRB >= 3 ? 3 : 1), 1); } break;
@@ -405,11 +408,11 @@ __global__ __launch_bounds__(NT) void so3_block_mm_real_kernel(MmParams p) {
   }
 }
 
-int total_slots(int nl, int RI, int CI) {
+int total_slots(int nl, int RI, int CI, int TN) {
   long n = 0;
   for (int l = 0; l < nl; ++l) {
     int tm, tn, slots;
-    tile_counts(2 * l + 1, RI, CI, tm, tn, slots);
+    tile_counts(2 * l + 1, RI, CI, TN, tm, tn, slots);
     n += slots;
   }
   return n > 0x7fffffffL ? -1 : (int)n;
@@ -424,7 +427,9 @@ int run(const float* a, const float* b, float* c, int nl, int RI, int CI, int KI
   const long Lmax = 2L * nl - 1;
   if (Lmax * Lmax * RI * KI >= (1L << 31) || Lmax * Lmax * CI * KI >= (1L << 31)) return S2CNN_EINVAL;
   if (!aligned4(a) || !aligned4(b) || !aligned4(c)) return S2CNN_EALIGN;
-  const int grid = total_slots(nl, RI, CI);
+  // 128 x 128 tiles unless they are too few to give every CU its two workgroups: then 128 x 64
+  const bool narrow = total_slots(nl, RI, CI, 128) < SMALL_GRID;
+  const int grid = total_slots(nl, RI, CI, narrow ? 64 : 128);
   if (grid < 1) return S2CNN_EINVAL;
   MmParams p{a, b, c, nl, RI, CI, KI};
   typedef Cfg<MODE> C_;
@@ -434,7 +439,11 @@ int run(const float* a, const float* b, float* c, int nl, int RI, int CI, int KI
   hipStream_t st = static_cast<hipStream_t>(stream);
   // the fast loaders address a degree with 32-bit byte offsets
   const bool fast = a4 && b4 && (KI % TK == 0 || TK % KI == 0) && Lmax * Lmax * RI * KI < (1L << 30) && Lmax * Lmax * CI * KI < (1L << 30);
-#define S2CNN_LAUNCH(VA, VB, FAST) hipLaunchKernelGGL((so3_block_mm_real_kernel<MODE, VA, VB, FAST>), dim3(grid), dim3(NT), 0, st, p)
+#define S2CNN_LAUNCH(VA, VB, FAST)                                                                                    \
+  do {                                                                                                                \
+    if (narrow) hipLaunchKernelGGL((so3_block_mm_real_kernel<MODE, VA, VB, FAST, 1>), dim3(grid), dim3(NT), 0, st, p); \
+    else hipLaunchKernelGGL((so3_block_mm_real_kernel<MODE, VA, VB, FAST, 2>), dim3(grid), dim3(NT), 0, st, p);        \
+  } while (0)
   if (fast) S2CNN_LAUNCH(4, 4, true);
   else if (a4 && b4) S2CNN_LAUNCH(4, 4, false);
   else if (a4) S2CNN_LAUNCH(4, 1, false);
