@@ -83,7 +83,8 @@ class _S2_mm_real(torch.autograd.Function):
         y = y.contiguous()
         ctx.save_for_backward(x, y)
         z = x.new_empty((nspec, nbatch, f_out))
-        _hip.call("s2cnn_s2_mm_real_fwd", _hip.ptr(x), _hip.ptr(y), _hip.ptr(z), nl, nbatch, f_in, f_out, _hip.stream_ptr())
+        if nbatch > 0:
+            _hip.call("s2cnn_s2_mm_real_fwd", _hip.ptr(x), _hip.ptr(y), _hip.ptr(z), nl, nbatch, f_in, f_out, _hip.stream_ptr())
         return z
 
     @staticmethod
@@ -95,10 +96,14 @@ class _S2_mm_real(torch.autograd.Function):
         gx = gy = None
         if ctx.needs_input_grad[0]:
             gx = gz.new_empty((nl ** 2, nbatch, f_in))
-            _hip.call("s2cnn_s2_mm_real_gradx", _hip.ptr(gz), _hip.ptr(y), _hip.ptr(gx), nl, nbatch, f_in, f_out, _hip.stream_ptr())
+            if nbatch > 0:
+                _hip.call("s2cnn_s2_mm_real_gradx", _hip.ptr(gz), _hip.ptr(y), _hip.ptr(gx), nl, nbatch, f_in, f_out, _hip.stream_ptr())
         if ctx.needs_input_grad[1]:
             gy = gz.new_empty((nl ** 2, f_in, f_out))
-            _hip.call("s2cnn_s2_mm_real_grady", _hip.ptr(gz), _hip.ptr(x), _hip.ptr(gy), nl, nbatch, f_in, f_out, _hip.stream_ptr())
+            if nbatch > 0:
+                _hip.call("s2cnn_s2_mm_real_grady", _hip.ptr(gz), _hip.ptr(x), _hip.ptr(gy), nl, nbatch, f_in, f_out, _hip.stream_ptr())
+            else:
+                gy.zero_()
         return gx, gy
 
 

@@ -21,6 +21,8 @@ def _convert(name, x, out_shape):
     nl = _nl_from_nspec(nspec)
     out = x.new_empty(out_shape)
     ncols = out.numel() // out.size(0) // (2 if name.endswith("to_complex") else 1)
+    if ncols == 0:
+        return out
     _hip.call(name, _hip.ptr(x), _hip.ptr(out), nl, ncols, _hip.stream_ptr())
     return out
 
@@ -72,8 +74,9 @@ class _SO3_mm_real(torch.autograd.Function):
         y = y.contiguous()
         ctx.save_for_backward(x, y)
         z = x.new_empty((nspec, nbatch, f_out))
-        _hip.call("s2cnn_so3_mm_real_fwd", _hip.ptr(x), _hip.ptr(y), _hip.ptr(z), nl, nbatch, f_in, f_out,
-                  _hip.stream_ptr())
+        if nbatch > 0:
+            _hip.call("s2cnn_so3_mm_real_fwd", _hip.ptr(x), _hip.ptr(y), _hip.ptr(z), nl, nbatch, f_in, f_out,
+                      _hip.stream_ptr())
         return z
 
     @staticmethod
@@ -86,12 +89,16 @@ class _SO3_mm_real(torch.autograd.Function):
         gx = gy = None
         if ctx.needs_input_grad[0]:
             gx = gz.new_empty((nspec, nbatch, f_in))
-            _hip.call("s2cnn_so3_mm_real_gradx", _hip.ptr(gz), _hip.ptr(y), _hip.ptr(gx), nl, nbatch, f_in, f_out,
-                      _hip.stream_ptr())
+            if nbatch > 0:
+                _hip.call("s2cnn_so3_mm_real_gradx", _hip.ptr(gz), _hip.ptr(y), _hip.ptr(gx), nl, nbatch, f_in, f_out,
+                          _hip.stream_ptr())
         if ctx.needs_input_grad[1]:
             gy = gz.new_empty((nspec, f_in, f_out))
-            _hip.call("s2cnn_so3_mm_real_grady", _hip.ptr(gz), _hip.ptr(x), _hip.ptr(gy), nl, nbatch, f_in, f_out,
-                      _hip.stream_ptr())
+            if nbatch > 0:
+                _hip.call("s2cnn_so3_mm_real_grady", _hip.ptr(gz), _hip.ptr(x), _hip.ptr(gy), nl, nbatch, f_in, f_out,
+                          _hip.stream_ptr())
+            else:
+                gy.zero_()
         return gx, gy
 
 

@@ -19,6 +19,8 @@ def _analysis(x, b_in, b_out, for_grad, complex_in):
     nbatch = x.size(0)
     table = _setup_wigner(b_in, nl=b_out, weighted=not for_grad, device=x.device)
     out = x.new_empty((b_out ** 2, nbatch, 2))
+    if nbatch == 0:
+        return out
     ws = _hip.workspace(L.s2cnn_s2_analysis_workspace(b_in, b_out, nbatch, complex_in), x.device)
     _hip.call("s2cnn_s2_analysis", _hip.ptr(x), _hip.ptr(table), _hip.ptr(out), _hip.ptr(ws), ws.numel(),
                   b_in, b_out, nbatch, complex_in, _hip.stream_ptr())
@@ -31,10 +33,20 @@ def _synthesis(x, b_in, b_out, for_grad, complex_out):
     nbatch = x.size(1)
     table = _setup_wigner(b_out, nl=b_in, weighted=for_grad, device=x.device)
     out = x.new_empty((nbatch, 2 * b_out, 2 * b_out) + ((2,) if complex_out else ()))
+    if nbatch == 0:
+        return out
     ws = _hip.workspace(L.s2cnn_s2_synthesis_workspace(b_in, b_out, nbatch, complex_out), x.device)
     _hip.call("s2cnn_s2_synthesis", _hip.ptr(x), _hip.ptr(table), _hip.ptr(out), _hip.ptr(ws), ws.numel(),
                   b_in, b_out, nbatch, complex_out, _hip.stream_ptr())
     return out
+
+
+def _count(sizes):
+    """Product of the batch dimensions (explicit, so that views of empty batches are not ambiguous)."""
+    n = 1
+    for d in sizes:
+        n *= d
+    return n
 
 
 def _grid_args(x, b_out, complex_in):
@@ -56,8 +68,8 @@ def s2_fft(x, for_grad=False, b_out=None):
     '''
     assert x.size(-1) == 2
     b_in, b_out, batch_size = _grid_args(x, b_out, True)
-    x = x.contiguous().view(-1, 2 * b_in, 2 * b_in, 2)
-    return _analysis(x, b_in, b_out, for_grad, 1).view(-1, *batch_size, 2)
+    x = x.contiguous().view(_count(batch_size), 2 * b_in, 2 * b_in, 2)
+    return _analysis(x, b_in, b_out, for_grad, 1).view(b_out ** 2, *batch_size, 2)
 
 
 def s2_rfft(x, for_grad=False, b_out=None):
@@ -68,8 +80,8 @@ def s2_rfft(x, for_grad=False, b_out=None):
     :return:  [l * m, ..., complex]
     '''
     b_in, b_out, batch_size = _grid_args(x, b_out, False)
-    x = x.contiguous().view(-1, 2 * b_in, 2 * b_in)
-    return _analysis(x, b_in, b_out, for_grad, 0).view(-1, *batch_size, 2)
+    x = x.contiguous().view(_count(batch_size), 2 * b_in, 2 * b_in)
+    return _analysis(x, b_in, b_out, for_grad, 0).view(b_out ** 2, *batch_size, 2)
 
 
 def _spectrum_args(x, b_out):
@@ -81,7 +93,7 @@ def _spectrum_args(x, b_out):
         b_out = b_in
     assert b_out >= b_in
     batch_size = x.size()[1:-1]
-    return x.contiguous().view(nspec, -1, 2), b_in, b_out, batch_size
+    return x.contiguous().view(nspec, _count(batch_size), 2), b_in, b_out, batch_size
 
 
 def s2_ifft(x, for_grad=False, b_out=None):

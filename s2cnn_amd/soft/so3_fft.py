@@ -72,6 +72,8 @@ def _analysis(x, b_in, b_out, batch_size, for_grad, complex_in, mask=None):
     table = _setup_wigner(b_in, nl=b_out, weighted=not for_grad, device=x.device)
     packed = None if complex_in else _setup_packed_wigner(b_in, b_out, not for_grad, False, x.device)
     out = x.new_empty((_nspec(b_out), *batch_size, 2))
+    if nbatch == 0:
+        return out
     ws = _hip.workspace(L.s2cnn_so3_analysis_workspace(b_in, b_out, nbatch, complex_in), x.device)
     if mask is not None:
         mask = _same_shape_operand(mask, x)
@@ -100,6 +102,8 @@ def _synthesis(x, b_in, b_out, batch_size, for_grad, complex_out, bias=None, rel
     packed = None if complex_out else _setup_packed_wigner(b_in, b_out, for_grad, True, x.device)
     shape = (*batch_size, 2 * b_out, 2 * b_out, 2 * b_out) + ((2,) if complex_out else ())
     out = x.new_empty(shape)
+    if nbatch == 0:
+        return out
     ws = _hip.workspace(L.s2cnn_so3_synthesis_workspace(b_in, b_out, nbatch, complex_out), x.device)
     if bias is not None:
         assert not complex_out
@@ -221,7 +225,7 @@ class SO3_ifft_real(torch.autograd.Function):
         g = so3_rfft(grad_output, for_grad=True, b_out=ctx.b_in, mask=ctx.saved_tensors[0] if ctx.relu else None)
         gb = None
         if ctx.bias_shape is not None and ctx.needs_input_grad[2]:
-            gb = g[0, ..., 0].reshape(-1, g.size(-2)).sum(0).reshape(ctx.bias_shape)
+            gb = g[0, ..., 0].reshape(g[0, ..., 0].numel() // g.size(-2), g.size(-2)).sum(0).reshape(ctx.bias_shape)
         return g, None, gb, None
 
 
@@ -260,6 +264,8 @@ def so3_rfft_real_basis(x, for_grad=False, b_out=None, mask=None):
     table = _setup_wigner(b_in, nl=b_out, weighted=not for_grad, device=x.device)
     packed = _setup_packed_wigner(b_in, b_out, not for_grad, False, x.device)
     out = x.new_empty((_nspec(b_out), *batch_size))
+    if nbatch == 0:
+        return out
     ws = _hip.workspace(L.s2cnn_so3_analysis_workspace(b_in, b_out, nbatch, 0), x.device)
     if mask is not None:
         mask = _same_shape_operand(mask, x)
@@ -296,6 +302,8 @@ def so3_rifft_real_basis(r, for_grad=False, b_out=None, bias=None, relu=False):
     table = _setup_wigner(b_out, nl=b_in, weighted=for_grad, device=r.device)
     packed = _setup_packed_wigner(b_in, b_out, for_grad, True, r.device)
     out = r.new_empty((*batch_size, 2 * b_out, 2 * b_out, 2 * b_out))
+    if nbatch == 0:
+        return out
     ws = _hip.workspace(L.s2cnn_so3_synthesis_workspace(b_in, b_out, nbatch, 0), r.device)
     nfeature = 1
     if bias is not None:
@@ -345,5 +353,5 @@ class SO3_ifft_real_basis(torch.autograd.Function):
         g = so3_rfft_real_basis(grad_output, for_grad=True, b_out=ctx.b_in, mask=ctx.saved_tensors[0] if ctx.relu else None)
         gb = None
         if ctx.bias_shape is not None and ctx.needs_input_grad[2]:
-            gb = g[0].reshape(-1, g.size(-1)).sum(0).reshape(ctx.bias_shape)
+            gb = g[0].reshape(g[0].numel() // g.size(-1), g.size(-1)).sum(0).reshape(ctx.bias_shape)
         return g, None, gb, None

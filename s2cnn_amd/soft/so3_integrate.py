@@ -19,9 +19,14 @@ class _SO3_integrate(torch.autograd.Function):
         ctx.b = b
         ctx.shape = x.size()
         lead = x.size()[:-3]
-        x = x.contiguous().view(-1, 2 * b, 2 * b, 2 * b)
+        n = 1
+        for d in lead:
+            n *= d
+        x = x.contiguous().view(n, 2 * b, 2 * b, 2 * b)
         w = _setup_so3_integrate(b, x.device)
         out = x.new_empty((x.size(0),))
+        if x.size(0) == 0:
+            return out.view(*lead)
         _hip.call("s2cnn_so3_integrate", _hip.ptr(x), _hip.ptr(w), _hip.ptr(out), b, x.size(0),
                   _hip.stream_ptr())
         return out.view(*lead)
@@ -29,9 +34,11 @@ class _SO3_integrate(torch.autograd.Function):
     @staticmethod
     def backward(ctx, g):
         b = ctx.b
-        g = g.contiguous().view(-1)
+        g = g.contiguous().view(g.numel())
         w = _setup_so3_integrate(b, g.device)
         gx = g.new_empty((g.numel(), 2 * b, 2 * b, 2 * b))
+        if g.numel() == 0:
+            return gx.view(ctx.shape)
         _hip.call("s2cnn_so3_integrate_grad", _hip.ptr(g), _hip.ptr(w), _hip.ptr(gx), b, g.numel(),
                   _hip.stream_ptr())
         return gx.view(ctx.shape)

@@ -48,8 +48,11 @@ def test_argument_rejection_without_gpu():
     assert lib.s2cnn_so3_analysis_workspace(16, 16, 256, 0) == 256 * 32 * 31 * 16 * 8 + packed16
     assert lib.s2cnn_so3_analysis(ctypes.c_void_p(0x1008), fake, fake, fake, null, 0, 32, 32, 1, 0, null) == -3   # 64^3 real input: 16-byte alignment
     assert lib.s2cnn_so3_synthesis_workspace(4, 6, 3, 1) == 16 * 12 * 7 * 7 * 8      # batch padded to the z tile, no fast path
-    assert lib.s2cnn_so3_packed_table_bytes(40, 40, 0) == 0 and lib.s2cnn_so3_packed_table_bytes(32, 40, 1) == 0
-    assert lib.s2cnn_so3_pack_table(fake, fake, 40, 40, 0, null) == -1
+    # more than 32 frequencies / degrees or 64 betas: one packed table per part of the Wigner stage; none beyond 64 / 128
+    assert lib.s2cnn_so3_packed_table_bytes(40, 40, 0) == 3 * 79 * 80 * 1024 * 4
+    assert lib.s2cnn_so3_packed_table_bytes(32, 40, 1) == 2 * 63 * 32 * 2048 * 4
+    assert lib.s2cnn_so3_packed_table_bytes(70, 70, 0) == 0 and lib.s2cnn_so3_packed_table_bytes(70, 70, 1) == 0
+    assert lib.s2cnn_so3_pack_table(fake, fake, 70, 70, 0, null) == -1
     assert b"workspace" in lib.s2cnn_strerror(-2)
     # entry points of the real-basis path and the biased synthesis
     assert lib.s2cnn_s2_mm_real_fwd(null, null, null, 4, 2, 3, 5, null) == -1

@@ -296,6 +296,34 @@ def test_layers_on_random_shapes(hip, seed):
         _conv_case(kind, B, Fi, Fo, b_in, b_out, grid, 7000 + 10 * seed, real_basis, activation)
 
 
+def test_empty_batch(hip):
+    """A batch of zero samples runs through operators and layers like any other: empty outputs of the right shape,
+    zero gradients for the weights (the reference's CPU branches behave so, being plain tensor algebra)."""
+    c1 = s2cnn_amd.S2Convolution(2, 3, 6, 4, s2cnn_amd.s2_near_identity_grid()).cuda()
+    c2 = s2cnn_amd.SO3Convolution(3, 5, 4, 3, s2cnn_amd.so3_near_identity_grid(), activation="relu").cuda()
+    for real_basis in (True, False):
+        c1.real_basis = c2.real_basis = real_basis
+        x = torch.zeros(0, 2, 12, 12, device="cuda", requires_grad=True)
+        y = c2(c1(x))
+        assert y.shape == (0, 5, 6, 6, 6)
+        v = s2cnn_amd.so3_integrate(y)
+        assert v.shape == (0, 5)
+        v.sum().backward()
+        assert x.grad.shape == x.shape
+        for c in (c1, c2):
+            assert c.kernel.grad.shape == c.kernel.shape and float(c.kernel.grad.abs().max()) == 0.0
+            assert float(c.bias.grad.abs().max()) == 0.0
+            c.zero_grad()
+    s = PSO3.so3_rfft(torch.zeros(0, 8, 8, 8, device="cuda"))
+    assert s.shape == (O.nspec_so3(4), 0, 2) and PSO3.so3_rifft(s).shape == (0, 8, 8, 8)
+    s = PS2.s2_rfft(torch.zeros(3, 0, 8, 8, device="cuda"))
+    assert s.shape == (16, 3, 0, 2) and PS2.s2_rifft(s).shape == (3, 0, 8, 8)
+    z = s2cnn_amd.so3_mm(torch.zeros(10, 0, 3, 2, device="cuda"), torch.zeros(10, 3, 4, 2, device="cuda"))
+    assert z.shape == (10, 0, 4, 2)
+    z = s2cnn_amd.s2_mm(torch.zeros(4, 0, 3, 2, device="cuda"), torch.zeros(4, 3, 4, 2, device="cuda"))
+    assert z.shape == (10, 0, 4, 2)
+
+
 def test_so3_convolution_parity(hip):
     _conv_case("so3", 2, 3, 4, 5, 4, s2cnn_amd.so3_near_identity_grid(n_alpha=4, n_beta=2, n_gamma=3), 50)
     _conv_case("so3", 3, 8, 8, 6, 6, s2cnn_amd.so3_near_identity_grid(), 53)
