@@ -259,7 +259,7 @@ __host__ __device__ inline void tile_counts(int L, int RI, int CI, int& tm, int&
 }
 
 template <int MODE, int VEC>
-__global__ __launch_bounds__(NT, 3) void so3_block_mm_kernel(MmParams p) {
+__global__ __launch_bounds__(NT, MODE == GRADX ? 2 : 3) void so3_block_mm_kernel(MmParams p) {   // grad x: two K-contiguous tiles leave LDS for two workgroups
   typedef Cfg<MODE> C_;
   __shared__ __attribute__((aligned(16))) float2 As[2 * TileShape<C_::A_KC, TM>::ELEMS];
   __shared__ __attribute__((aligned(16))) float2 Bs[2 * TileShape<C_::B_KC, TN>::ELEMS];
