@@ -694,13 +694,14 @@ def test_training_step_replays_from_a_hip_graph(hip):
             assert torch.equal(a, b), f"replay {i}: parameter {k} differs from the eager step"
 
 
-def test_so3_projector_on_a_large_grid(hip):
-    """b = 48 (96^3 grid, 147 440 coefficients): planes with more register blocks than 256 threads hold and degrees
-    beyond one part of the tiled Wigner kernels.  No oracle at this size: synthesis followed by analysis is the identity on
-    spectra of real signals, analysis followed by synthesis a projector, and truncation commutes with both."""
-    b = 48
+@pytest.mark.parametrize("b,nz", [(48, 2), (64, 3), (33, 17)])
+def test_so3_projector_on_a_large_grid(hip, b, nz):
+    """b = 48 (96^3 grid, 147 440 coefficients), 64 (every part of the Wigner stage full: 64 frequencies, 64 degrees,
+    128 betas) and 33 (parts of one column / one degree): planes with more register blocks than 256 threads hold and
+    degrees beyond one part of the tiled Wigner kernels.  No oracle at these sizes: synthesis followed by analysis is
+    the identity on spectra of real signals, analysis followed by synthesis a projector, and truncation commutes with both."""
     g = torch.Generator().manual_seed(90)
-    x = torch.randn(2, 2 * b, 2 * b, 2 * b, generator=g).cuda()
+    x = torch.randn(nz, 2 * b, 2 * b, 2 * b, generator=g).cuda()
     s = PSO3.so3_rfft(x)                                   # spectrum of a real signal
     y = PSO3.so3_rifft(s)                                  # its band-limited projection
     s2 = PSO3.so3_rfft(y)
