@@ -342,7 +342,8 @@ def test_s2_convolution_parity(hip, real_basis):
                                               (32, 22, 6, 3), (32, 26, 2, 1),   # their truncated instantiations
                                               (10, 32, 6, 3),     # synthesis onto the 64^3 grid from a short spectrum
                                               (32, 34, 2, 1),     # 64-point plane kernel + Wigner stage
-                                              (22, 7, 6, 2), (6, 6, 10, 5), (5, 9, 3, 1), (11, 4, 2, 1)])   # folded plane kernels
+                                              (22, 7, 6, 2), (6, 6, 10, 5), (5, 9, 3, 1), (11, 4, 2, 1),   # folded plane kernels
+                                              (36, 36, 2, 1), (40, 33, 2, 2)])   # ... with the Wigner stage in parts
 def test_so3_transforms_with_fused_relu(hip, b_in, b_out, nz, nf):
     """max(., 0) in the epilogue of the synthesis and its gradient mask in the loads of the analysis against the
     separate elementwise passes they replace: the results must be the same numbers, bit for bit, for complex and
