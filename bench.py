@@ -180,6 +180,46 @@ def measure_rows(torch, dev, with_cpu):
     return rows
 
 
+def measure_so3_mm(torch, dev, reps=5):
+    """Benchmark config 3: the complex block product alone, x [43680, 16, 64, 2], y [43680, 64, 64, 2] with entries
+    N(0, 1/64), forward and the gradients with respect to x and y, each timed with events on the launch stream.  `frac` is
+    algorithmic flops (8 per complex multiply-add) over the fp32 matrix peak; the kernels form a complex product from three
+    real ones, so the matrix cores execute 3/4 of that: `mfma_executed_frac`."""
+    import s2cnn_amd
+    from s2cnn_amd import _hip
+    nl, B, Fi, Fo = 32, 16, 64, 64
+    g = torch.Generator(device=dev).manual_seed(3)
+    x = (torch.randn(nspec(nl), B, Fi, 2, device=dev, generator=g) * 0.125).requires_grad_()
+    y = (torch.randn(nspec(nl), Fi, Fo, 2, device=dev, generator=g) * 0.125).requires_grad_()
+    gz = torch.randn(nspec(nl), B, Fo, 2, device=dev, generator=g)
+
+    def step():
+        z = s2cnn_amd.so3_mm(x, y)
+        torch.autograd.grad(z, (x, y), gz)
+
+    for _ in range(2):
+        step()
+    torch.cuda.synchronize()
+    with _hip.KernelTimer() as kt:
+        for _ in range(reps):
+            step()
+        torch.cuda.synchronize()
+    pc = {k: sum(v) / len(v) for k, v in kt.summary().items()}
+    fl = mm_flops(nl, B, Fi, Fo, real=False)
+    out = {"workload": "so3_mm fwd + grad x + grad y, x [43680,16,64,2], y [43680,64,64,2] (benchmark config 3)", "bound": "mfma",
+           "flop_per_launch": fl, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s"}
+    total = 0.0
+    for name in ("s2cnn_so3_mm_fwd", "s2cnn_so3_mm_gradx", "s2cnn_so3_mm_grady"):
+        ach = fl / (pc[name] * 1e-3) / 1e12
+        total += pc[name]
+        out[name] = {"ms": round(pc[name], 3), "achieved": round(ach, 2), "frac": round(ach / PEAK_FP32_MFMA_TFLOPS, 4),
+                     "mfma_executed_frac": round(0.75 * ach / PEAK_FP32_MFMA_TFLOPS, 4)}
+    out["ms_fwd_bwd"] = round(total, 3)
+    del x, y, gz
+    torch.cuda.empty_cache()
+    return out
+
+
 def measure_network(torch, dev, steps, warmup):
     """The SHREC17-shaped network of benchmark config 5 (S2Conv 6->100 b 128->32, ReLU, SO3Conv 100->100 b 32->22, ReLU,
     SO3Conv 100->55 b 22->7, so3_integrate; batch 32, near-identity grids scaled by the bandwidth ratio), forward and
@@ -240,6 +280,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-fft", action="store_true", help="skip the standalone FFT round trip")
+    ap.add_argument("--no-mm", action="store_true", help="skip the standalone complex so3_mm (benchmark config 3)")
     ap.add_argument("--complex-product", action="store_true",
                     help="multiply complex spectra as the reference does instead of real-basis ones")
     ap.add_argument("--rows", action="store_true", help="also time every other op of the path (adds a `rows` object)")
@@ -302,6 +343,8 @@ def main():
     roofline = {"bound": "mfma", "kernel": dominant, "achieved": round(ach, 2), "peak": PEAK_FP32_MFMA_TFLOPS,
                 "unit": "TFLOP/s", "frac": round(ach / PEAK_FP32_MFMA_TFLOPS, 4),
                 "traffic": MM_TRAFFIC_BYTES.get(dominant) if (B, F, b) == (16, 64, 32) else None,
+                "traffic_source": "profiles/so3_mm_real_b32_B16_F64_hbm_traffic.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of "
+                                  "this workload; not re-measured in this run)",
                 "flop_per_launch": flops, "ms_per_launch": round(per_call[dominant], 3)}
     if "_real_" not in dominant:   # three real products per complex one: the matrix cores execute 3/4 of the algorithmic flops
         roofline["mfma_executed_frac"] = round(0.75 * roofline["frac"], 4)
@@ -348,6 +391,8 @@ def main():
         del xf
         torch.cuda.empty_cache()
 
+    if not args.no_mm:
+        result["so3_mm"] = measure_so3_mm(torch, dev)
     if args.rows:
         result["rows"] = measure_rows(torch, dev, not args.no_cpu)
     if args.network:
@@ -372,12 +417,17 @@ def main():
             out = O.so3_conv(xc, kc, bc, b, b, grid)
             sum_of_squares(out).backward()
 
-        c0 = time.perf_counter()
-        cpu_step()
-        c1 = time.perf_counter()
-        result["cpu_baseline"] = {"value": round(Bc / (c1 - c0), 4), "unit": "samples/s", "cores": cores, "kind": "port",
-                                  "sample": "same layer and sizes at batch %d of %d, one fwd+bwd (%.1f s), fp32, "
-                                            "torch threads = %d" % (Bc, B, c1 - c0, cores)}
+        cpu_step()                                       # warm-up: autograd graph, allocator, thread pool
+        reps = []
+        for _ in range(3):
+            c0 = time.perf_counter()
+            cpu_step()
+            reps.append(time.perf_counter() - c0)
+        med = sorted(reps)[1]
+        result["cpu_baseline"] = {"value": round(Bc / med, 4), "unit": "samples/s", "cores": cores, "kind": "port",
+                                  "sample": "same layer and sizes at batch %d of %d, fwd+bwd, fp32, torch threads = %d: one warm-up, "
+                                            "then 3 repetitions of %s s, median taken"
+                                            % (Bc, B, cores, " / ".join("%.1f" % r for r in reps))}
 
     print(json.dumps(result), flush=True)
 

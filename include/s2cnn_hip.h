@@ -31,7 +31,8 @@ extern "C" {
 #define S2CNN_OK 0
 #define S2CNN_EINVAL (-1)      /* a size is out of range or inconsistent              */
 #define S2CNN_EWORKSPACE (-2)  /* workspace pointer NULL or smaller than required     */
-#define S2CNN_EALIGN (-3)      /* a pointer is not aligned to 8 bytes                  */
+#define S2CNN_EALIGN (-3)      /* a pointer misses the alignment its entry documents   */
+                               /* (4, 8 or 16 bytes)                                   */
 
 /* ABI version of this header; bumped when a signature changes. */
 int s2cnn_abi_version(void);

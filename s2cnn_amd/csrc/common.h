@@ -6,10 +6,14 @@
 
 namespace s2cnn {
 
+// Status of the launches an entry point has just made.  hipGetLastError returns (and clears) the last error of
+// this host thread, whoever caused it: entry points call clear_stale_error() before their first launch so that an
+// error left behind by other code on the thread is not reported as theirs.
 inline int launch_status() {
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? S2CNN_OK : static_cast<int>(e);
 }
+inline void clear_stale_error() { (void)hipGetLastError(); }
 
 inline bool aligned8(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 7u) == 0; }
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

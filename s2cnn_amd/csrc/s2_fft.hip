@@ -135,6 +135,7 @@ extern "C" size_t s2cnn_s2_synthesis_workspace(int b_in, int b_out, long nbatch,
 
 extern "C" int s2cnn_s2_analysis(const float* x, const float* table, float* out, void* workspace, size_t workspace_bytes,
                                  int b_in, int b_out, long nbatch, int complex_in, void* stream) {
+  s2cnn::clear_stale_error();
   if (!x || !table || !out || !sizes_ok(b_in, b_out, nbatch)) return S2CNN_EINVAL;
   if (!s2cnn::aligned8(out) || (complex_in && !s2cnn::aligned8(x))) return S2CNN_EALIGN;
   if (!workspace || workspace_bytes < ws_bytes(b_in, b_out, nbatch) || !s2cnn::aligned8(workspace)) return S2CNN_EWORKSPACE;
@@ -163,6 +164,7 @@ extern "C" int s2cnn_s2_analysis(const float* x, const float* table, float* out,
 
 extern "C" int s2cnn_s2_synthesis(const float* xhat, const float* table, float* out, void* workspace, size_t workspace_bytes,
                                   int b_in, int b_out, long nbatch, int complex_out, void* stream) {
+  s2cnn::clear_stale_error();
   if (!xhat || !table || !out || !sizes_ok(b_out, b_in, nbatch)) return S2CNN_EINVAL;
   if (!s2cnn::aligned8(xhat) || (complex_out && !s2cnn::aligned8(out))) return S2CNN_EALIGN;
   if (!workspace || workspace_bytes < ws_bytes(b_out, b_in, nbatch) || !s2cnn::aligned8(workspace)) return S2CNN_EWORKSPACE;

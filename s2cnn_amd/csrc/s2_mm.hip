@@ -156,6 +156,7 @@ int check(const void* a, const void* b, const void* c, int nl, int nbatch, int f
 }  // namespace
 
 extern "C" int s2cnn_s2_mm_fwd(const float* x, const float* y, float* z, int nl, int nbatch, int f_in, int f_out, void* stream) {
+  s2cnn::clear_stale_error();
   if (int rc = check(x, y, z, nl, nbatch, f_in, f_out)) return rc;
   hipLaunchKernelGGL(s2_mm_fwd_kernel, dim3(nl * nl, NSPLIT, (unsigned)(((long)nbatch * f_out + 255) / 256)), dim3(256), 0,
                      static_cast<hipStream_t>(stream),
@@ -165,6 +166,7 @@ extern "C" int s2cnn_s2_mm_fwd(const float* x, const float* y, float* z, int nl,
 }
 
 extern "C" int s2cnn_s2_mm_gradx(const float* gz, const float* y, float* gx, int nl, int nbatch, int f_in, int f_out, void* stream) {
+  s2cnn::clear_stale_error();
   if (int rc = check(gz, y, gx, nl, nbatch, f_in, f_out)) return rc;
   hipLaunchKernelGGL(s2_mm_gradx_kernel, dim3(nl * nl, nbatch, (f_in + KC - 1) / KC), dim3(256), 0, static_cast<hipStream_t>(stream),
                      reinterpret_cast<const float2*>(gz), reinterpret_cast<const float2*>(y), reinterpret_cast<float2*>(gx),
@@ -173,6 +175,7 @@ extern "C" int s2cnn_s2_mm_gradx(const float* gz, const float* y, float* gx, int
 }
 
 extern "C" int s2cnn_s2_mm_grady(const float* gz, const float* x, float* gy, int nl, int nbatch, int f_in, int f_out, void* stream) {
+  s2cnn::clear_stale_error();
   if (int rc = check(gz, x, gy, nl, nbatch, f_in, f_out)) return rc;
   hipLaunchKernelGGL(s2_mm_grady_kernel, dim3(nl * nl, (f_out + 63) / 64, (f_in + KC - 1) / KC), dim3(256), 0,
                      static_cast<hipStream_t>(stream), reinterpret_cast<const float2*>(gz), reinterpret_cast<const float2*>(x),

@@ -207,6 +207,7 @@ bool vec4(const void* a, const void* b, const void* c, int fo) {
 }  // namespace
 
 extern "C" int s2cnn_s2_mm_real_fwd(const float* x, const float* y, float* z, int nl, int nbatch, int f_in, int f_out, void* stream) {
+  s2cnn::clear_stale_error();
   if (int rc = check(x, y, z, nl, nbatch, f_in, f_out)) return rc;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int npair = (nbatch + 1) / 2;
@@ -221,6 +222,7 @@ extern "C" int s2cnn_s2_mm_real_fwd(const float* x, const float* y, float* z, in
 }
 
 extern "C" int s2cnn_s2_mm_real_gradx(const float* gz, const float* y, float* gx, int nl, int nbatch, int f_in, int f_out, void* stream) {
+  s2cnn::clear_stale_error();
   if (int rc = check(gz, y, gx, nl, nbatch, f_in, f_out)) return rc;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const dim3 grid(nl * nl, (nbatch + IB - 1) / IB, (f_in + KC - 1) / KC);
@@ -232,6 +234,7 @@ extern "C" int s2cnn_s2_mm_real_gradx(const float* gz, const float* y, float* gx
 }
 
 extern "C" int s2cnn_s2_mm_real_grady(const float* gz, const float* x, float* gy, int nl, int nbatch, int f_in, int f_out, void* stream) {
+  s2cnn::clear_stale_error();
   if (int rc = check(gz, x, gy, nl, nbatch, f_in, f_out)) return rc;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (vec4(gz, gz, gy, f_out)) {

@@ -382,6 +382,7 @@ extern "C" int s2cnn_so3_real_basis_transform_available(int b_in, int b_out, int
 
 extern "C" int s2cnn_so3_analysis_real_basis(const float* x, const float* table, const float* packed_table, float* out,
                                              void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch, void* stream) {
+  s2cnn::clear_stale_error();
   if (!x || !table || !out || !sizes_ok(b_in, b_out, nbatch)) return S2CNN_EINVAL;
   if (!fused_path(b_in, b_out, 0, false)) return S2CNN_EINVAL;
   if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
@@ -391,6 +392,7 @@ extern "C" int s2cnn_so3_analysis_real_basis(const float* x, const float* table,
 extern "C" int s2cnn_so3_synthesis_real_basis(const float* r, const float* table, const float* packed_table, float* out,
                                               void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
                                               const float* bias, int nfeature, void* stream) {
+  s2cnn::clear_stale_error();
   if (!r || !table || !out || !sizes_ok(b_out, b_in, nbatch)) return S2CNN_EINVAL;
   if (bias && (nfeature < 1 || nbatch % nfeature != 0)) return S2CNN_EINVAL;
   if (!fused_path(b_out, b_in, 0, true)) return S2CNN_EINVAL;
@@ -405,6 +407,7 @@ extern "C" size_t s2cnn_so3_packed_table_bytes(int b_in, int b_out, int synthesi
 }
 
 extern "C" int s2cnn_so3_pack_table(const float* table, float* packed, int b_in, int b_out, int synthesis, void* stream) {
+  s2cnn::clear_stale_error();
   if (!table || !packed || b_in < 1 || b_out < 1 || b_in > 512 || b_out > 512) return S2CNN_EINVAL;
   if (s2cnn_so3_packed_table_bytes(b_in, b_out, synthesis) == 0) return S2CNN_EINVAL;
   if (!s2cnn::aligned16(packed)) return S2CNN_EALIGN;
@@ -562,24 +565,28 @@ int synthesis_impl(const float* xhat, const float* table, const float* packed_ta
 extern "C" int s2cnn_so3_analysis(const float* x, const float* table, const float* packed_table, float* out,
                                   void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
                                   int complex_in, void* stream) {
+  s2cnn::clear_stale_error();
   return analysis_impl(x, nullptr, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, complex_in, stream);
 }
 
 extern "C" int s2cnn_so3_synthesis(const float* xhat, const float* table, const float* packed_table, float* out,
                                    void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
                                    int complex_out, void* stream) {
+  s2cnn::clear_stale_error();
   return synthesis_impl(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, complex_out, nullptr, 1, 0, stream);
 }
 
 extern "C" int s2cnn_so3_synthesis_real_bias(const float* xhat, const float* table, const float* packed_table, float* out,
                                              void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
                                              const float* bias, int nfeature, void* stream) {
+  s2cnn::clear_stale_error();
   return synthesis_impl(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, 0, bias, nfeature, 0, stream);
 }
 
 extern "C" int s2cnn_so3_synthesis_real_relu(const float* xhat, const float* table, const float* packed_table, float* out,
                                              void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
                                              const float* bias, int nfeature, int real_basis, void* stream) {
+  s2cnn::clear_stale_error();
   if (!real_basis)
     return synthesis_impl(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, 0, bias, nfeature, 1, stream);
   if (!xhat || !table || !out || !sizes_ok(b_out, b_in, nbatch)) return S2CNN_EINVAL;
@@ -593,6 +600,7 @@ extern "C" int s2cnn_so3_synthesis_real_relu(const float* xhat, const float* tab
 extern "C" int s2cnn_so3_analysis_real_masked(const float* x, const float* mask, const float* table, const float* packed_table,
                                               float* out, void* workspace, size_t workspace_bytes, int b_in, int b_out,
                                               long nbatch, int real_basis, void* stream) {
+  s2cnn::clear_stale_error();
   if (!mask) return S2CNN_EINVAL;
   if (!real_basis)
     return analysis_impl(x, mask, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, 0, stream);

@@ -58,12 +58,14 @@ __global__ __launch_bounds__(256) void so3_integrate_grad_kernel(const float* __
 }  // namespace
 
 extern "C" int s2cnn_so3_integrate(const float* x, const float* w, float* out, int b, long n, void* stream) {
+  s2cnn::clear_stale_error();
   if (!x || !w || !out || b < 1 || b > 1024 || n < 1 || n >= (1L << 31)) return S2CNN_EINVAL;
   hipLaunchKernelGGL(so3_integrate_kernel, dim3((unsigned)n), dim3(256), 0, static_cast<hipStream_t>(stream), x, w, out, 2 * b);
   return s2cnn::launch_status();
 }
 
 extern "C" int s2cnn_so3_integrate_grad(const float* g, const float* w, float* gx, int b, long n, void* stream) {
+  s2cnn::clear_stale_error();
   if (!g || !w || !gx || b < 1 || b > 1024 || n < 1 || n >= (1L << 31)) return S2CNN_EINVAL;
   hipLaunchKernelGGL(so3_integrate_grad_kernel, dim3((unsigned)n), dim3(256), 0, static_cast<hipStream_t>(stream), g, w, gx, 2 * b);
   return s2cnn::launch_status();
@@ -76,7 +78,7 @@ extern "C" const char* s2cnn_strerror(int code) {
     case S2CNN_OK: return "ok";
     case S2CNN_EINVAL: return "a size is out of range or inconsistent, or a pointer is NULL";
     case S2CNN_EWORKSPACE: return "workspace is NULL, misaligned or smaller than the *_workspace() size";
-    case S2CNN_EALIGN: return "a complex tensor is not aligned to 8 bytes";
+    case S2CNN_EALIGN: return "a pointer does not meet the alignment documented for this entry (4, 8 or 16 bytes)";
     default: return code > 0 ? hipGetErrorString(static_cast<hipError_t>(code)) : "unknown s2cnn error";
   }
 }

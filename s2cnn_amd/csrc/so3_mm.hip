@@ -394,15 +394,18 @@ int run(const float* a, const float* b, float* c, int nl, int RI, int CI, int KI
 
 extern "C" int s2cnn_so3_mm_fwd(const float* x, const float* y, float* z, int nl, int nbatch, int f_in,
                                 int f_out, void* stream) {
+  s2cnn::clear_stale_error();
   return run<FWD>(x, y, z, nl, nbatch, f_out, f_in, stream);
 }
 
 extern "C" int s2cnn_so3_mm_gradx(const float* gz, const float* y, float* gx, int nl, int nbatch, int f_in,
                                   int f_out, void* stream) {
+  s2cnn::clear_stale_error();
   return run<GRADX>(gz, y, gx, nl, nbatch, f_in, f_out, stream);
 }
 
 extern "C" int s2cnn_so3_mm_grady(const float* gz, const float* x, float* gy, int nl, int nbatch, int f_in,
                                   int f_out, void* stream) {
+  s2cnn::clear_stale_error();
   return run<GRADY>(x, gz, gy, nl, f_in, f_out, nbatch, stream);
 }

@@ -111,6 +111,7 @@ dim3 grid_for(int nl, long ncols) {
 }  // namespace
 
 extern "C" int s2cnn_so3_spectrum_to_real(const float* x, float* r, int nl, long ncols, void* stream) {
+  s2cnn::clear_stale_error();
   if (int rc = check(x, r, nl, ncols)) return rc;
   if (!s2cnn::aligned8(x)) return S2CNN_EALIGN;
   hipLaunchKernelGGL(to_real_kernel, grid_for(nl, ncols), dim3(256), 0, static_cast<hipStream_t>(stream),
@@ -119,6 +120,7 @@ extern "C" int s2cnn_so3_spectrum_to_real(const float* x, float* r, int nl, long
 }
 
 extern "C" int s2cnn_so3_spectrum_to_complex(const float* r, float* x, int nl, long ncols, void* stream) {
+  s2cnn::clear_stale_error();
   if (int rc = check(r, x, nl, ncols)) return rc;
   if (!s2cnn::aligned8(x)) return S2CNN_EALIGN;
   hipLaunchKernelGGL(to_complex_kernel, grid_for(nl, ncols), dim3(256), 0, static_cast<hipStream_t>(stream),

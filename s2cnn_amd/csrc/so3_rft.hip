@@ -140,6 +140,7 @@ int check(const void* p, const void* q, const void* r, int b, int nbeta, long nc
 }  // namespace
 
 extern "C" int s2cnn_so3_rft_expand_real(const float* G, const float* dtab, float* y, int b, int nbeta, long ncols, void* stream) {
+  s2cnn::clear_stale_error();
   if (int rc = check(G, dtab, y, b, nbeta, ncols)) return rc;
   const dim3 grid((unsigned)(b * b), (unsigned)((ncols / 4 + 255) / 256));
   hipStream_t st = static_cast<hipStream_t>(stream);
@@ -153,6 +154,7 @@ extern "C" int s2cnn_so3_rft_expand_real(const float* G, const float* dtab, floa
 }
 
 extern "C" int s2cnn_so3_rft_expand_real_grad(const float* gy, const float* dtab, float* gG, int b, int nbeta, long ncols, void* stream) {
+  s2cnn::clear_stale_error();
   if (int rc = check(gy, dtab, gG, b, nbeta, ncols)) return rc;
   const dim3 grid((unsigned)(b * b), (unsigned)((ncols / 4 + 255) / 256));
   hipStream_t st = static_cast<hipStream_t>(stream);

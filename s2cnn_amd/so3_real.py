@@ -140,9 +140,12 @@ class _SO3RftRealFactorised(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x2, b, plan):
         idx, valid, E, dtab = plan[:4]
+        _hip.require_gpu_f32(x2)
         ncols = x2.size(0)
-        xg = x2.t()[idx] * valid.unsqueeze(-1)                    # [nbeta, P, ncols]
-        G = torch.bmm(E.transpose(1, 2), xg).contiguous()        # [nbeta, R, ncols]
+        with torch.autocast(device_type="cuda", enabled=False):  # the expansion kernel reads G as float32
+            xg = x2.t()[idx] * valid.unsqueeze(-1)                # [nbeta, P, ncols]
+            G = torch.bmm(E.transpose(1, 2), xg).contiguous()    # [nbeta, R, ncols]
+        _hip.require_gpu_f32(G)
         y = x2.new_empty((b * (4 * b * b - 1) // 3, ncols))
         _hip.call("s2cnn_so3_rft_expand_real", _hip.ptr(G), _hip.ptr(dtab), _hip.ptr(y), b, idx.size(0), ncols, _hip.stream_ptr())
         ctx.plan, ctx.b, ctx.n_grid = plan, b, x2.size(1)
@@ -152,10 +155,12 @@ class _SO3RftRealFactorised(torch.autograd.Function):
     def backward(ctx, gy):
         idx, valid, E, dtab, sel, idx_sel = ctx.plan
         gy = gy.contiguous()
+        _hip.require_gpu_f32(gy)
         ncols = gy.size(1)
         gG = gy.new_empty((idx.size(0), E.size(2), ncols))
         _hip.call("s2cnn_so3_rft_expand_real_grad", _hip.ptr(gy), _hip.ptr(dtab), _hip.ptr(gG), ctx.b, idx.size(0), ncols, _hip.stream_ptr())
-        gxg = torch.bmm(E, gG)                                    # [nbeta, P, ncols]
+        with torch.autocast(device_type="cuda", enabled=False):
+            gxg = torch.bmm(E, gG)                                # [nbeta, P, ncols]
         gx = gy.new_zeros((ctx.n_grid, ncols))
         gx.index_add_(0, idx_sel, gxg.reshape(-1, ncols).index_select(0, sel))   # no boolean masks: they would sync with the host
         return gx.t(), None, None
@@ -169,7 +174,8 @@ def so3_rft_real(x, b, grid):
     """
     sz = x.size()
     ncols = x.numel() // sz[-1]
-    plan = _setup_so3_rft_plan(b, tuple(grid), x.device) if (x.is_cuda and ncols % 4 == 0 and so3_rft_real.factorised) else None
+    fast = x.is_cuda and x.dtype == torch.float32 and ncols % 4 == 0 and so3_rft_real.factorised
+    plan = _setup_so3_rft_plan(b, tuple(grid), x.device) if fast else None
     if plan is not None:
         assert sz[-1] == len(grid)
         out = _SO3RftRealFactorised.apply(x.reshape(-1, sz[-1]), b, plan)

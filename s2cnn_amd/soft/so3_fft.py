@@ -13,15 +13,21 @@ def _nspec(b):
 
 
 @lru_cache(maxsize=32)
-def _setup_wigner(b, nl, weighted, device):
-    """[2b, nspec(nl)] float32 on `device`, computed in float64 (s2cnn/soft/so3_fft.py:205-243)."""
-    dss = wigner.so3_wigner_table(b, nl, bool(weighted))
+def _wigner_table(b, nl, weighted, device):
+    dss = wigner.so3_wigner_table(b, nl, weighted)
     return torch.tensor(dss, dtype=torch.float32, device=device).contiguous()
+
+
+def _setup_wigner(b, nl, weighted, device):
+    """[2b, nspec(nl)] float32 on `device`, computed in float64 (s2cnn/soft/so3_fft.py:205-243).  One cache entry per
+    table, whichever way the arguments are passed (lru_cache keys positional and keyword calls differently)."""
+    return _wigner_table(int(b), int(nl), bool(weighted), torch.device(device))
 
 
 @lru_cache(maxsize=32)
 def _setup_packed_wigner(b_in, b_out, weighted, synthesis, device):
-    """The table of `_setup_wigner` repacked once for the tiled kernels (None where they do not apply)."""
+    """The table of `_setup_wigner` repacked once for the tiled kernels (None where they do not apply).  The first
+    call for a table synchronizes: make it (one transform of each size) before capturing a HIP graph."""
     L = _hip.lib()
     nbytes = L.s2cnn_so3_packed_table_bytes(b_in, b_out, int(synthesis))
     if nbytes == 0:

@@ -98,6 +98,19 @@ def test_rfft_equals_rft_on_soft_grid():
         assert (y1 - y2).abs().max().item() < 1e-10 * y1.abs().mean().item()
 
 
+@pytest.mark.parametrize("b_in,b_out", [(7, 5), (6, 6), (9, 2)])
+def test_s2_fft_equals_s2_rft_on_soft_grid(b_in, b_out):
+    """The S^2 twin of tests/so3_fft.py:8-24 of the reference: s2_fft's table carries 2 b_in w_beta
+    (s2cnn/soft/s2_fft.py:124) and s2_rft's matrix 2 b_out (s2cnn/s2_ft.py:38-45), hence
+    s2_fft(x, b_out) = (b_in / b_out) s2_rft(w * x, b_out, s2_soft_grid(b_in)).  s2_fft is pinned by brute force above,
+    so a dropped factor, a wrong column of D or a swapped (beta, alpha) in s2_rft fails here."""
+    x = torch.randn(2, 2 * b_in, 2 * b_in, dtype=D)
+    y1 = O.s2_fft(O.as_complex(x), b_out=b_out)
+    xw = torch.einsum("zba,b->zba", x, O.quadrature_weights(b_in, D))
+    y2 = O.s2_rft(xw.reshape(2, -1), b_out, O.s2_soft_grid(b_in)) * (b_in / b_out)
+    assert (y1 - y2).abs().max().item() < 1e-12 * y1.abs().mean().item()
+
+
 def _idem(f, g, x, b_in, b_out):
     x = g(f(x, b_out=b_out), b_out=b_in)
     y = g(f(x, b_out=b_out), b_out=b_in)
