@@ -33,6 +33,7 @@ extern "C" {
 #define S2CNN_EWORKSPACE (-2)  /* workspace pointer NULL or smaller than required     */
 #define S2CNN_EALIGN (-3)      /* a pointer misses the alignment its entry documents   */
                                /* (4, 8 or 16 bytes)                                   */
+#define S2CNN_ETOOBIG (-4)     /* needs more scratch than the library's own buffer     */
 
 /* ABI version of this header; bumped when a signature changes. */
 int s2cnn_abi_version(void);
@@ -160,6 +161,22 @@ size_t s2cnn_so3_analysis_workspace(int b_in, int b_out, long nbatch, int comple
 int s2cnn_so3_analysis(const float *x, const float *table, const float *packed_table, float *out,
                        void *workspace, size_t workspace_bytes,
                        int b_in, int b_out, long nbatch, int complex_in, void *stream);
+
+/* ---- the analysis above without a workspace argument ---------------------------------
+ * No counterpart in the reference.  For callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): the same transform as s2cnn_so3_analysis
+ * with its scratch in a buffer that the library itself holds, S2CNN_STATIC_SCRATCH_BYTES per GPU from the
+ * moment the library is loaded until the process ends.  Calls nothing that allocates.
+ *   - sizes whose s2cnn_so3_analysis_workspace(...) exceeds S2CNN_STATIC_SCRATCH_BYTES are rejected with
+ *     S2CNN_ETOOBIG (real signals on the 64^3 grid: up to 130 volumes per call);
+ *   - all calls on one GPU share that GPU's buffer: calls that overlap in time on one GPU (different
+ *     streams or threads) race; calls on one stream are ordered and safe;
+ *   - the first call on a GPU resolves the buffer's address for it (no allocation; make it outside a graph capture);
+ *   - results are those of s2cnn_so3_analysis bit for bit.
+ */
+#define S2CNN_STATIC_SCRATCH_BYTES (32u << 20)
+int s2cnn_so3_analysis_static(const float *x, const float *table, const float *packed_table, float *out,
+                              int b_in, int b_out, long nbatch, int complex_in, void *stream);
 
 /* ---- SO(3) Fourier synthesis: spectrum -> grid -------------------------------------
  * xhat  [nspec(b_in), nbatch, 2]

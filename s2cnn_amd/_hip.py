@@ -43,6 +43,7 @@ SIGNATURES = {
     "s2cnn_s2_mm_real_grady": (_int, _MM_SIG),
     "s2cnn_so3_analysis_workspace": (_size_t, _WS_SIG),
     "s2cnn_so3_analysis": (_int, _FT3_SIG),
+    "s2cnn_so3_analysis_static": (_int, [_c_float_p, _c_float_p, _c_float_p, _c_float_p, _int, _int, _long, _int, _vp]),
     "s2cnn_so3_synthesis_workspace": (_size_t, _WS_SIG),
     "s2cnn_so3_synthesis": (_int, _FT3_SIG),
     "s2cnn_so3_synthesis_real_bias": (_int, _FT3R_SIG[:-1] + [_c_float_p, _int, _vp]),

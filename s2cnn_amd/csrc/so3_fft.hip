@@ -21,6 +21,7 @@
 #include "so3_wigner_tiled.h"
 #include "so3_fused64.h"
 #include "so3_plane_dft_real.h"
+#include <mutex>
 
 namespace {
 
@@ -608,4 +609,47 @@ extern "C" int s2cnn_so3_analysis_real_masked(const float* x, const float* mask,
   if (!fused_path(b_in, b_out, 0, false)) return S2CNN_EINVAL;
   if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
   return fused_analysis(x, mask, table, packed_table, out, workspace, workspace_bytes, b_out, nbatch, true, static_cast<hipStream_t>(stream));
+}
+
+// ---------------------------------------------------------------------------------------------
+// s2cnn_so3_analysis for callers that cannot allocate: the scratch is a buffer of the library's own.
+// `scratch` below is the host-side stand-in of the device array, not a device address: host code uses the
+// address that hipGetSymbolAddress returns for the current device (every GPU holds its own copy).
+// ---------------------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[S2CNN_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int MAX_DEVICES = 64;
+void* scratch_ptr[MAX_DEVICES];     // device address of `scratch` per GPU, resolved on the first call with that GPU current
+std::mutex scratch_mutex;
+
+int static_scratch(void** p) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return static_cast<int>(e);
+  if (dev < 0 || dev >= MAX_DEVICES) return S2CNN_EINVAL;
+  std::lock_guard<std::mutex> lock(scratch_mutex);
+  if (!scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return static_cast<int>(e);
+    if (!ptr) return S2CNN_EINVAL;
+    scratch_ptr[dev] = ptr;
+  }
+  *p = scratch_ptr[dev];
+  return S2CNN_OK;
+}
+}  // namespace
+
+extern "C" int s2cnn_so3_analysis_static(const float* x, const float* table, const float* packed_table, float* out,
+                                         int b_in, int b_out, long nbatch, int complex_in, void* stream) {
+  s2cnn::clear_stale_error();
+  if (!x || !table || !out || !sizes_ok(b_in, b_out, nbatch)) return S2CNN_EINVAL;
+  const size_t need = s2cnn_so3_analysis_workspace(b_in, b_out, nbatch, complex_in);
+  if (need == 0) return S2CNN_EINVAL;
+  if (need > (size_t)S2CNN_STATIC_SCRATCH_BYTES) return S2CNN_ETOOBIG;
+  void* ws = nullptr;
+  const int rc = static_scratch(&ws);
+  if (rc) return rc;
+  return analysis_impl(x, nullptr, table, packed_table, out, ws, (size_t)S2CNN_STATIC_SCRATCH_BYTES, b_in, b_out, nbatch, complex_in, stream);
 }

@@ -79,6 +79,7 @@ extern "C" const char* s2cnn_strerror(int code) {
     case S2CNN_EINVAL: return "a size is out of range or inconsistent, or a pointer is NULL";
     case S2CNN_EWORKSPACE: return "workspace is NULL, misaligned or smaller than the *_workspace() size";
     case S2CNN_EALIGN: return "a pointer does not meet the alignment documented for this entry (4, 8 or 16 bytes)";
+    case S2CNN_ETOOBIG: return "the sizes need more scratch than the library's static buffer holds (S2CNN_STATIC_SCRATCH_BYTES)";
     default: return code > 0 ? hipGetErrorString(static_cast<hipError_t>(code)) : "unknown s2cnn error";
   }
 }
