@@ -61,18 +61,6 @@ __device__ __forceinline__ void buf_store_f32x4(float4 x, __amdgpu_buffer_rsrc_t
   __builtin_amdgcn_raw_buffer_store_b128(v, r, (int)voff, (int)soff, 0);
 }
 
-// 4 x 4 transpose across the four lanes of a quad: afterwards r_k of lane i is what r_i of lane k was.
-__device__ __forceinline__ float dpp_quad_xor1(float x) { return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0xB1, 0xf, 0xf, false)); }
-__device__ __forceinline__ float dpp_quad_xor2(float x) { return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x4E, 0xf, 0xf, false)); }
-__device__ __forceinline__ void quad_transpose(float& r0, float& r1, float& r2, float& r3) {
-  const bool b0 = threadIdx.x & 1, b1 = threadIdx.x & 2;
-  float u;
-  u = dpp_quad_xor1(b0 ? r0 : r1); if (b0) r0 = u; else r1 = u;
-  u = dpp_quad_xor1(b0 ? r2 : r3); if (b0) r2 = u; else r3 = u;
-  u = dpp_quad_xor2(b1 ? r0 : r2); if (b1) r0 = u; else r2 = u;
-  u = dpp_quad_xor2(b1 ? r1 : r3); if (b1) r1 = u; else r3 = u;
-}
-
 // x with its sign flipped where `signbit` (0 or 0x80000000) is set
 __device__ __forceinline__ float flip(float x, unsigned signbit) { return __uint_as_float(__float_as_uint(x) ^ signbit); }
 
@@ -115,11 +103,30 @@ __global__ void pack_table(const float* __restrict__ T, float* __restrict__ Tf, 
   }
 }
 
+// w64^(d k), k = 0..7, for this wave's d = threadIdx.x / 64 (conjugated for the inverse) as wave-uniform values: they
+// live in scalar registers, so the twiddled passes read nothing but their data from LDS.
+struct Twiddles { float c[8], s[8]; };
+__device__ __forceinline__ float uniform(float x) { return __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(x))); }
+template <bool INV>
+__device__ __forceinline__ void make_twiddles(Twiddles& tw) {
+  const int d = threadIdx.x >> 6;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    float s, c;
+    sincospif((float)(d * k) / 32.0f, &s, &c);   // angle 2 pi d k / 64
+    tw.c[k] = uniform(c);
+    tw.s[k] = uniform(INV ? s : -s);
+  }
+}
+__device__ __forceinline__ float2 twmul(float2 v, const Twiddles& tw, int k) {
+  return make_float2(v.x * tw.c[k] - v.y * tw.s[k], v.x * tw.s[k] + v.y * tw.c[k]);
+}
+
 // One radix-8 pass of the in-place 2-D transform of a 64x64 complex plane in LDS by 512 threads
 // (natural order in, sigma order out on both axes): P = 0, 1 rows, P = 2, 3 columns.
-// twl[8*d + k] = w64^(d k) (conjugated for the inverse).  A barrier must follow each pass.
+// A barrier must follow each pass.
 template <bool INV, int P>
-__device__ __forceinline__ void fft_pass(float2* buf, const float2* twl) {
+__device__ __forceinline__ void fft_pass(float2* buf, const Twiddles& tw) {
   using namespace fft64;
   const int lo = threadIdx.x & 63;   // line
   const int d = threadIdx.x >> 6;    // j2 in the first pass of an axis, k1 in the second
@@ -131,7 +138,7 @@ __device__ __forceinline__ void fft_pass(float2* buf, const float2* twl) {
   fft8<INV>(v);
   if (P == 0 || P == 2) {
 #pragma unroll
-    for (int j = 1; j < 8; ++j) v[j] = cmul(v[j], twl[8 * d + j]);
+    for (int j = 1; j < 8; ++j) v[j] = twmul(v[j], tw, j);
   }
 #pragma unroll
   for (int j = 0; j < 8; ++j) line[j * stride] = v[j];
@@ -148,7 +155,7 @@ __device__ __forceinline__ void fft_pass_load(const float2* buf, float2 (&v)[8])
   for (int j = 0; j < 8; ++j) v[j] = line[j * stride];
 }
 template <bool INV, int P>
-__device__ __forceinline__ void fft_pass_finish(float2* buf, const float2* twl, float2 (&v)[8]) {
+__device__ __forceinline__ void fft_pass_finish(float2* buf, const Twiddles& tw, float2 (&v)[8]) {
   using namespace fft64;
   const int lo = threadIdx.x & 63, d = threadIdx.x >> 6;
   float2* line = P == 0 ? buf + lo * PITCH + d : P == 1 ? buf + lo * PITCH + 8 * d : P == 2 ? buf + lo + d * PITCH : buf + lo + 8 * d * PITCH;
@@ -156,20 +163,10 @@ __device__ __forceinline__ void fft_pass_finish(float2* buf, const float2* twl, 
   fft8<INV>(v);
   if (P == 0 || P == 2) {
 #pragma unroll
-    for (int j = 1; j < 8; ++j) v[j] = cmul(v[j], twl[8 * d + j]);
+    for (int j = 1; j < 8; ++j) v[j] = twmul(v[j], tw, j);
   }
 #pragma unroll
   for (int j = 0; j < 8; ++j) line[j * stride] = v[j];
-}
-
-template <bool INV>
-__device__ __forceinline__ void fill_twiddles(float2* twl) {
-  if (threadIdx.x < 64) {
-    const int d = threadIdx.x >> 3, k = threadIdx.x & 7;
-    float s, c;
-    sincospif((float)(d * k) / 32.0f, &s, &c);   // angle 2 pi d k / 64
-    twl[threadIdx.x] = make_float2(c, INV ? s : -s);
-  }
 }
 
 // Workgroup -> volume.  Consecutive workgroups go round-robin over the 8 XCDs; the workgroups of one
@@ -214,12 +211,12 @@ __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restri
   using namespace fft64;
   __shared__ __attribute__((aligned(16))) float2 work[LDS_ELEMS];
   __shared__ __attribute__((aligned(16))) float2 quad[2][QUAD_ELEMS];
-  __shared__ float2 twl[64];
   const long z = volume_of_block(nbatch);
   if (z < 0) return;
   const int t = threadIdx.x;
   const int lo = t & 63, d = t >> 6;
-  fill_twiddles<false>(twl);
+  Twiddles twl;
+  make_twiddles<false>(twl);
   for (int i = t; i < 2 * QUAD_ELEMS; i += THREADS) (&quad[0][0])[i] = make_float2(0.f, 0.f);   // places nobody writes (the -a half of a = 0) read as zero
 
   // quad address of the item (complex index), bit 31 = sign bit of (-1)^n
@@ -291,7 +288,7 @@ __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restri
     }
     fft8<false>(v);
 #pragma unroll
-    for (int k = 1; k < 8; ++k) v[k] = cmul(v[k], twl[8 * d + k]);
+    for (int k = 1; k < 8; ++k) v[k] = twmul(v[k], twl, k);
 #pragma unroll
     for (int k = 0; k < 8; ++k) work[(8 * k + d) * PITCH + lo] = v[k];
   };
@@ -338,7 +335,7 @@ __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restri
   if constexpr (NA > 1) load_table(0, 1);
   if constexpr (NA > 2) load_table(0, 2);
   if constexpr (NA > 3) load_table(0, 3);
-  __syncthreads();                              // twiddles, cleared quads
+  __syncthreads();                              // cleared quads
   stage_c1();
   load_planes(1);
   __syncthreads();
@@ -676,13 +673,13 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
   constexpr int STG_PADS = 144;                                              // one pad per row: sum of (4c+4) over the 8 degree groups
   __shared__ __attribute__((aligned(16))) float4 stg_p[NIT * THREADS + STG_PADS];   // item (c, a, n): its share of the bins [+a,n], [-a,-n]
   __shared__ __attribute__((aligned(16))) float4 stg_m[NIT * THREADS + STG_PADS];   //                                      [-a,n], [+a,-n]
-  __shared__ float2 twl[64];
   const long z = volume_of_block(nbatch);
   if (z < 0) return;
   const int t = threadIdx.x;
   const int lo = t & 63, d = t >> 6;
   const float bz = bias ? bias[z % nfeature] : 0.f;
-  fill_twiddles<true>(twl);
+  Twiddles twl;
+  make_twiddles<true>(twl);
   for (int i = t; i < LDS_ELEMS; i += THREADS) work[i] = make_float2(0.f, 0.f);   // bins of m = 32 and n = 32 stay zero ... until a transform overwrites them: cleared again in reduce()
 
   float2 xp[NIT][4], xm[NIT][4];
@@ -697,7 +694,7 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
   const __amdgpu_buffer_rsrc_t rt = make_rsrc(Tf, (unsigned)(PACKED_FLOATS * 4));
   const __amdgpu_buffer_rsrc_t ry = make_rsrc(y + (size_t)z * (N * N * N), N * N * N * 4);
   const unsigned toff = t * 16;
-  const unsigned yoff = ((d + 8 * (lo & 3)) * N + 4 * (lo >> 2)) * 4;   // + (beta * 4096 + 2048 h) * 4: row d + 8 (lo % 4) + 32 h, columns 4 (lo / 4)..+3
+  const unsigned yoff = (d * N + lo) * 4;          // + (beta * 4096 + k * 512) * 4: row alpha = d + 8 k, column gamma = lo
 #pragma unroll
   for (int it = 0; it < NA; ++it) {
     int c, a, n;
@@ -783,40 +780,21 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
     if (t < 64) { work[32 * PITCH + t] = make_float2(0.f, 0.f); work[t * PITCH + 32] = make_float2(0.f, 0.f); }
   };
   // second alpha stage: lane lo takes the column slot sigma(lo), i.e. column gamma = lo; inputs at row slots
-  // 8 d + j, outputs rows alpha = d + 8 k2.  The four lanes of a quad then exchange their values (4 x 4
-  // transposes) so that a lane holds four adjacent columns of one row: 16-byte stores, whole rows per wave.
-  // Real part -> plane j, imaginary part -> plane 63-j.
+  // 8 d + j, outputs rows alpha = d + 8 k.  Real part -> plane j, imaginary part -> plane 63-j, one whole 256-byte row
+  // per wave and store.
   auto stage_c2_store = [&](int j) {
     float2 v[8];
     const float2* line = work + sigma(lo) + 8 * d * PITCH;
 #pragma unroll
     for (int k = 0; k < 8; ++k) v[k] = line[k * PITCH];
     fft8<true>(v);
-    float ra[8], rb[8];
 #pragma unroll
-    for (int k = 0; k < 8; ++k) { ra[k] = v[k].x + bz; rb[k] = v[k].y + bz; }
-    if (relu) {
-#pragma unroll
-      for (int k = 0; k < 8; ++k) { ra[k] = s2cnn::relu_f(ra[k]); rb[k] = s2cnn::relu_f(rb[k]); }
+    for (int k = 0; k < 8; ++k) {
+      float ra = v[k].x + bz, rb = v[k].y + bz;
+      if (relu) { ra = s2cnn::relu_f(ra); rb = s2cnn::relu_f(rb); }
+      buf_store_f32(ra, ry, yoff, (j * 4096 + k * 512) * 4);
+      buf_store_f32(rb, ry, yoff, ((63 - j) * 4096 + k * 512) * 4);
     }
-    quad_transpose(ra[0], ra[1], ra[2], ra[3]); quad_transpose(ra[4], ra[5], ra[6], ra[7]);
-    quad_transpose(rb[0], rb[1], rb[2], rb[3]); quad_transpose(rb[4], rb[5], rb[6], rb[7]);
-    // lane (q, i) = (lo / 4, lo % 4) now holds columns 4q..4q+3 of the rows d + 8 i and d + 8 (4 + i)
-    // Four 16-byte stores.  Observed on gfx950: when such stores follow each other within a few cycles (or their
-    // data registers are refilled for the next store), the first component of the earlier store can come out
-    // holding the later store's value in lanes 12-15 of each 16-lane row - run-to-run varying, and only when loads
-    // had just been queued.  Hence: 16 distinct data registers, idle cycles between and after the stores, and the
-    // plane offset in the lane offset (an integer add between the stores) instead of the scalar offset.
-    __builtin_amdgcn_sched_barrier(0);
-    buf_store_f32x4(make_float4(ra[0], ra[1], ra[2], ra[3]), ry, yoff + (j * 4096) * 4, 0);
-    asm volatile("s_nop 7" ::: "memory");
-    buf_store_f32x4(make_float4(ra[4], ra[5], ra[6], ra[7]), ry, yoff + (j * 4096 + 2048) * 4, 0);
-    asm volatile("s_nop 7" ::: "memory");
-    buf_store_f32x4(make_float4(rb[0], rb[1], rb[2], rb[3]), ry, yoff + ((63 - j) * 4096) * 4, 0);
-    asm volatile("s_nop 7" ::: "memory");
-    buf_store_f32x4(make_float4(rb[4], rb[5], rb[6], rb[7]), ry, yoff + ((63 - j) * 4096 + 2048) * 4, 0);
-    asm volatile("s_nop 7\n\ts_nop 7" ::: "memory");
-    __builtin_amdgcn_sched_barrier(0);
   };
 
 #define S2CNN_FENCE() __builtin_amdgcn_sched_barrier(0)
