@@ -273,6 +273,23 @@ def measure_network(torch, dev, steps, warmup):
             "separate_relu": {"ms_per_step": round(ms_sep, 3), "library_ms": round(sum(calls_sep.values()), 3)}}
 
 
+def measure_example_network(torch, name, steps, warmup, batch=32):
+    """One of the reference's example networks (examples/mnist/run.py:55-98, examples/shrec17/model.py, model_original.py) in
+    its training step (forward, loss, backward, SGD with momentum) on a fixed synthetic batch; time inside library calls
+    listed beside the step time."""
+    from s2cnn_amd import _hip, harness
+    if name == "shrec17_original":
+        batch = 16
+    model, losses, ms = harness.train_steps(name, batch=batch, steps=steps, warmup=warmup, lr=0.01)
+    with _hip.KernelTimer() as kt:
+        harness.train_steps(name, batch=batch, steps=1, warmup=0, lr=0.01, model=model)
+        torch.cuda.synchronize()
+    calls = {k: round(sum(v), 3) for k, v in sorted(kt.summary().items(), key=lambda kv: -sum(kv[1]))}
+    return {"workload": "%s training step (s2cnn_amd/harness.py), batch %d, synthetic data" % (name, batch),
+            "ms_per_step": round(ms, 3), "samples_per_s": round(batch / (ms * 1e-3), 1), "first_loss": round(losses[0], 4),
+            "last_loss": round(losses[-1], 4), "library_ms": round(sum(calls.values()), 3), "library_calls_ms": calls}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -284,7 +301,10 @@ def main():
     ap.add_argument("--complex-product", action="store_true",
                     help="multiply complex spectra as the reference does instead of real-basis ones")
     ap.add_argument("--rows", action="store_true", help="also time every other op of the path (adds a `rows` object)")
-    ap.add_argument("--network", action="store_true", help="also time the SHREC17-shaped network (adds a `network` object)")
+    ap.add_argument("--network", nargs="?", const="config5", default=None, choices=["config5", "mnist", "shrec17", "shrec17_original"],
+                    help="also time a whole network, forward + backward (adds a `network` object): config5 = the SHREC17-shaped "
+                         "network of benchmark config 5 (default); mnist, shrec17, shrec17_original = the reference's example "
+                         "networks (s2cnn_amd/harness.py) in a training step with SGD on a synthetic batch of 32")
     ap.add_argument("--batch", type=int, default=16)
     ap.add_argument("--b", type=int, default=32)
     ap.add_argument("--features", type=int, default=64)
@@ -395,8 +415,10 @@ def main():
         result["so3_mm"] = measure_so3_mm(torch, dev)
     if args.rows:
         result["rows"] = measure_rows(torch, dev, not args.no_cpu)
-    if args.network:
+    if args.network == "config5":
         result["network"] = measure_network(torch, dev, args.steps, args.warmup)
+    elif args.network:
+        result["network"] = measure_example_network(torch, args.network, args.steps, args.warmup)
 
     # ---- CPU baseline: the oracle (a restatement of the reference's CPU branches) on a bounded sample
     if not args.no_cpu:

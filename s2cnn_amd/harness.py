@@ -1,0 +1,148 @@
+"""The reference's example networks on this package's layers, and a training step on synthetic data.
+
+The module and parameter names are those of the reference's scripts, so a state dict saved by either loads into the
+other (examples/shrec17/train.py:123 saves `model.state_dict()`, examples/shrec17/test.py:49 loads it):
+
+  S2ConvNet_original   examples/mnist/run.py:55-98          S2Conv 1->20 (b 30->10), ReLU, SO3Conv 20->40 (b 10->6), ReLU,
+                                                            so3_integrate, Linear 40->10; near-identity grids
+  Shrec17Model         examples/shrec17/model.py:7-48       S2Conv 6->100 (b 64->16), [BatchNorm3d, ReLU, SO3Conv 100->100
+                                                            (b 16->10)], BatchNorm3d, ReLU, so3_integrate, Linear, log_softmax;
+                                                            equatorial grids with 2 b_in points on one ring
+  Shrec17ModelOriginal examples/shrec17/model_original.py   features 6, 50, 70, 350, bandwidths 128, 32, 22, 7, maximum over the
+                                                            grid instead of the integral, BatchNorm1d in the output layer
+
+Data sets, loaders and logging of the reference's scripts are not reproduced: `train_steps` feeds a fixed synthetic batch.
+"""
+import time
+
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+from . import (S2Convolution, SO3Convolution, s2_equatorial_grid, s2_near_identity_grid, so3_equatorial_grid, so3_integrate,
+               so3_near_identity_grid)
+
+
+class S2ConvNet_original(nn.Module):
+    """examples/mnist/run.py:55-98.  fused_activation: the two ReLUs inside the layers' last transforms (same function)."""
+
+    def __init__(self, fused_activation=False):
+        super().__init__()
+        f1, f2, f_output = 20, 40, 10
+        b_in, b_l1, b_l2 = 30, 10, 6
+        act = "relu" if fused_activation else None
+        self.fused_activation = fused_activation
+        self.conv1 = S2Convolution(nfeature_in=1, nfeature_out=f1, b_in=b_in, b_out=b_l1, grid=s2_near_identity_grid(), activation=act)
+        self.conv2 = SO3Convolution(nfeature_in=f1, nfeature_out=f2, b_in=b_l1, b_out=b_l2, grid=so3_near_identity_grid(), activation=act)
+        self.out_layer = nn.Linear(f2, f_output)
+
+    def forward(self, x):  # pylint: disable=W0221
+        x = self.conv1(x)
+        if not self.fused_activation:
+            x = F.relu(x)
+        x = self.conv2(x)
+        if not self.fused_activation:
+            x = F.relu(x)
+        x = so3_integrate(x)
+        return self.out_layer(x)
+
+
+def _shrec17_sequence(features, bandwidths):
+    """S2 layer, then (BatchNorm3d, ReLU, SO3 layer) per further bandwidth, then BatchNorm3d, ReLU
+    (examples/shrec17/model.py:17-38, model_original.py:17-38)."""
+    assert len(bandwidths) == len(features) - 1
+    sequence = []
+    grid = s2_equatorial_grid(max_beta=0, n_alpha=2 * bandwidths[0], n_beta=1)
+    sequence.append(S2Convolution(features[0], features[1], bandwidths[0], bandwidths[1], grid))
+    for l in range(1, len(features) - 2):
+        b_in, b_out = bandwidths[l], bandwidths[l + 1]
+        sequence.append(nn.BatchNorm3d(features[l], affine=True))
+        sequence.append(nn.ReLU())
+        grid = so3_equatorial_grid(max_beta=0, max_gamma=0, n_alpha=2 * b_in, n_beta=1, n_gamma=1)
+        sequence.append(SO3Convolution(features[l], features[l + 1], b_in, b_out, grid))
+    sequence.append(nn.BatchNorm3d(features[-2], affine=True))
+    sequence.append(nn.ReLU())
+    return nn.Sequential(*sequence)
+
+
+class Shrec17Model(nn.Module):
+    """examples/shrec17/model.py:7-48."""
+
+    def __init__(self, nclasses):
+        super().__init__()
+        self.features = [6, 100, 100, nclasses]
+        self.bandwidths = [64, 16, 10]
+        self.sequential = _shrec17_sequence(self.features, self.bandwidths)
+        self.out_layer = nn.Linear(self.features[-2], self.features[-1])
+
+    def forward(self, x):  # pylint: disable=W0221
+        x = self.sequential(x)      # [batch, feature, beta, alpha, gamma]
+        x = so3_integrate(x)        # [batch, feature]
+        return F.log_softmax(self.out_layer(x), dim=1)
+
+
+class Shrec17ModelOriginal(nn.Module):
+    """examples/shrec17/model_original.py:7-50."""
+
+    def __init__(self, nclasses):
+        super().__init__()
+        self.features = [6, 50, 70, 350, nclasses]
+        self.bandwidths = [128, 32, 22, 7]
+        self.sequential = _shrec17_sequence(self.features, self.bandwidths)
+        self.out_layer = nn.Sequential(nn.BatchNorm1d(self.features[-2], affine=False), nn.Linear(self.features[-2], self.features[-1]))
+
+    def forward(self, x):  # pylint: disable=W0221
+        x = self.sequential(x)
+        x = x.view(x.size(0), x.size(1), -1).max(-1)[0]
+        return F.log_softmax(self.out_layer(x), dim=1)
+
+
+NETWORKS = {
+    # name: (constructor, input shape without the batch, number of classes, loss on the network's output)
+    "mnist": (S2ConvNet_original, (1, 60, 60), 10, F.cross_entropy),                       # examples/mnist/run.py:211-223
+    "shrec17": (lambda: Shrec17Model(55), (6, 128, 128), 55, F.nll_loss),                  # examples/shrec17/train.py:70-82
+    "shrec17_original": (lambda: Shrec17ModelOriginal(55), (6, 256, 256), 55, F.nll_loss),
+}
+
+
+def synthetic_batch(name, batch, device, seed=0):
+    """A fixed batch of the network's input shape: uniform values with 70 % of the samples zero for the digit network
+    (projected digits are sparse), uniform values for the six ray-cast channels of the shape networks; random labels."""
+    _, shape, nclasses, _ = NETWORKS[name]
+    g = torch.Generator().manual_seed(seed)
+    x = torch.rand(batch, *shape, generator=g)
+    if name == "mnist":
+        x = x * (torch.rand(batch, *shape, generator=g) < 0.3)
+    y = torch.randint(0, nclasses, (batch,), generator=g)
+    return x.to(device), y.to(device)
+
+
+def train_steps(name, batch=32, steps=10, warmup=2, lr=0.05, device="cuda:0", seed=0, model=None):
+    """`warmup + steps` SGD steps (momentum 0.9, as examples/shrec17/train.py:66) on one synthetic batch.
+    Returns (model, losses of all steps, milliseconds per timed step)."""
+    ctor, _, _, loss_fn = NETWORKS[name]
+    torch.manual_seed(seed)
+    if model is None:
+        model = ctor()
+    model = model.to(device)
+    model.train()
+    x, y = synthetic_batch(name, batch, device, seed)
+    opt = torch.optim.SGD(model.parameters(), lr=lr, momentum=0.9)
+    losses = []
+
+    def step():
+        opt.zero_grad(set_to_none=True)
+        loss = loss_fn(model(x), y)
+        loss.backward()
+        opt.step()
+        losses.append(loss.detach())
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / max(steps, 1) * 1e3
+    return model, [float(l) for l in losses], ms
