@@ -223,6 +223,22 @@ int s2cnn_so3_analysis_real_masked(const float *x, const float *mask, const floa
                                    float *out, void *workspace, size_t workspace_bytes,
                                    int b_in, int b_out, long nbatch, int real_basis, void *stream);
 
+/* The same pair with the mask as ONE BIT per sample (real signals on the 64^3 grid only: where
+ * s2cnn_so3_relu_bits_bytes(b_grid, nbatch) is not 0).  The synthesis writes, beside `out`, bit = "out is not <= 0" for
+ * every sample ([nbatch][beta][alpha % 8][alpha / 8] 64-bit words, bit = gamma; 32 KiB per volume, 16-byte aligned); the
+ * masked analysis reads those bits instead of a tensor of the shape of x: a thirty-second of the mask traffic of the
+ * backward pass, and the saved state of the activation shrinks by the same factor.  Results are those of the pair above
+ * bit for bit.  No counterpart in the reference (its models call F.relu on the layer's output, examples/mnist/run.py:88-92).
+ */
+size_t s2cnn_so3_relu_bits_bytes(int b_grid, long nbatch);
+int s2cnn_so3_synthesis_real_relu_bits(const float *xhat, const float *table, const float *packed_table, float *out,
+                                       void *bits, void *workspace, size_t workspace_bytes,
+                                       int b_in, int b_out, long nbatch,
+                                       const float *bias, int nfeature, int real_basis, void *stream);
+int s2cnn_so3_analysis_real_masked_bits(const float *x, const void *bits, const float *table, const float *packed_table,
+                                        float *out, void *workspace, size_t workspace_bytes,
+                                        int b_in, int b_out, long nbatch, int real_basis, void *stream);
+
 /* ---- table repacking for the real-signal fast path of the two transforms above ------
  * The reference uploads its Wigner table once per (b, nl, weighted, device) and reuses it
  * (soft/so3_fft.py:205-209); a caller of this library does the same with the packed copy:

@@ -328,8 +328,8 @@ size_t round256(size_t n) { return (n + 255) & ~(size_t)255; }
 
 // Real signals on the 64^3 grid: per-volume kernel + the pass between its records and the spectral rows.
 // real_basis: the spectrum is stored in the real basis (one float per entry) instead of complex pairs.
-int fused_analysis(const float* x, const float* mask, const float* table, const float* packed_table, float* out, void* workspace,
-                   size_t workspace_bytes, int b_out, long nbatch, bool real_basis, hipStream_t st) {
+int fused_analysis(const float* x, const float* mask, bool mask_bits, const float* table, const float* packed_table, float* out,
+                   void* workspace, size_t workspace_bytes, int b_out, long nbatch, bool real_basis, hipStream_t st) {
   if (!s2cnn::aligned16(x) || !s2cnn::aligned16(mask)) return S2CNN_EALIGN;
   const size_t need = round256(fused64::scratch_bytes(nbatch)) + fused64::PACKED_FLOATS * sizeof(float);
   if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
@@ -340,7 +340,7 @@ int fused_analysis(const float* x, const float* mask, const float* table, const 
     hipLaunchKernelGGL(fused64::pack_table, dim3(1024), dim3(256), 0, st, table, dst, s2cnn::so3_nspec(b_out), b_out);
     Tf = dst;
   }
-  fused64::launch_analysis(b_out, st, x, mask, Tf, rec, nbatch);
+  fused64::launch_analysis(b_out, st, x, mask, mask_bits, Tf, rec, nbatch);
   if (real_basis)
     hipLaunchKernelGGL(fused64::spectrum_scatter_real, dim3((unsigned)((nbatch + fused64::ZR - 1) / fused64::ZR), fused64::active_rounds(b_out) * 32), dim3(256), 0, st,
                        rec, out, b_out, nbatch);
@@ -352,8 +352,8 @@ int fused_analysis(const float* x, const float* mask, const float* table, const 
 
 int fused_synthesis(const float* xhat, const float* table, const float* packed_table, float* out, void* workspace,
                     size_t workspace_bytes, int b_in, long nbatch, bool real_basis, const float* bias, int nfeature, int relu,
-                    hipStream_t st) {
-  if (!s2cnn::aligned16(out)) return S2CNN_EALIGN;
+                    unsigned long long* bits, hipStream_t st) {
+  if (!s2cnn::aligned16(out) || !s2cnn::aligned16(bits)) return S2CNN_EALIGN;
   const int nl = b_in < 32 ? b_in : 32;
   const size_t need = round256(fused64::scratch_bytes(nbatch)) + fused64::PACKED_FLOATS * sizeof(float);
   if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
@@ -370,7 +370,7 @@ int fused_synthesis(const float* xhat, const float* table, const float* packed_t
   else
     hipLaunchKernelGGL(fused64::spectrum_gather, dim3((unsigned)((nbatch + fused64::ZT - 1) / fused64::ZT), fused64::active_rounds(nl) * 16), dim3(256), 0, st,
                        reinterpret_cast<const float2*>(xhat), rec, nl, nbatch);
-  fused64::launch_synthesis(nl, st, rec, Tf, out, nbatch, bias, nfeature, relu);
+  fused64::launch_synthesis(nl, st, rec, Tf, out, nbatch, bias, nfeature, relu, bits);
   return s2cnn::launch_status();
 }
 
@@ -387,7 +387,7 @@ extern "C" int s2cnn_so3_analysis_real_basis(const float* x, const float* table,
   if (!x || !table || !out || !sizes_ok(b_in, b_out, nbatch)) return S2CNN_EINVAL;
   if (!fused_path(b_in, b_out, 0, false)) return S2CNN_EINVAL;
   if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
-  return fused_analysis(x, nullptr, table, packed_table, out, workspace, workspace_bytes, b_out, nbatch, true, static_cast<hipStream_t>(stream));
+  return fused_analysis(x, nullptr, false, table, packed_table, out, workspace, workspace_bytes, b_out, nbatch, true, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int s2cnn_so3_synthesis_real_basis(const float* r, const float* table, const float* packed_table, float* out,
@@ -399,7 +399,7 @@ extern "C" int s2cnn_so3_synthesis_real_basis(const float* r, const float* table
   if (!fused_path(b_out, b_in, 0, true)) return S2CNN_EINVAL;
   if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
   return fused_synthesis(r, table, packed_table, out, workspace, workspace_bytes, b_in, nbatch, true, bias, bias ? nfeature : 1, 0,
-                         static_cast<hipStream_t>(stream));
+                         nullptr, static_cast<hipStream_t>(stream));
 }
 
 extern "C" size_t s2cnn_so3_packed_table_bytes(int b_in, int b_out, int synthesis) {
@@ -437,14 +437,15 @@ extern "C" size_t s2cnn_so3_synthesis_workspace(int b_in, int b_out, long nbatch
 
 namespace {
 // mask: NULL, or (real signals only) a tensor of the shape of x whose positive entries select the samples that count
-int analysis_impl(const float* x, const float* mask, const float* table, const float* packed_table, float* out,
+int analysis_impl(const float* x, const float* mask, bool mask_bits, const float* table, const float* packed_table, float* out,
                   void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch, int complex_in, void* stream) {
   if (!x || !table || !out || !sizes_ok(b_in, b_out, nbatch) || (mask && complex_in)) return S2CNN_EINVAL;
+  if (mask_bits && !(mask && fused_path(b_in, b_out, complex_in, false))) return S2CNN_EINVAL;
   if (!s2cnn::aligned8(out) || (complex_in && !s2cnn::aligned8(x))) return S2CNN_EALIGN;
   if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (fused_path(b_in, b_out, complex_in, false))
-    return fused_analysis(x, mask, table, packed_table, out, workspace, workspace_bytes, b_out, nbatch, false, st);
+    return fused_analysis(x, mask, mask_bits, table, packed_table, out, workspace, workspace_bytes, b_out, nbatch, false, st);
   const size_t need = s2cnn_so3_analysis_workspace(b_in, b_out, nbatch, complex_in);
   if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
   const int n2 = 2 * b_in, nb = b_in < b_out ? b_in : b_out;
@@ -503,15 +504,16 @@ int analysis_impl(const float* x, const float* mask, const float* table, const f
 
 int synthesis_impl(const float* xhat, const float* table, const float* packed_table, float* out, void* workspace,
                    size_t workspace_bytes, int b_in, int b_out, long nbatch, int complex_out, const float* bias, int nfeature,
-                   int relu, void* stream) {
+                   int relu, unsigned long long* bits, void* stream) {
   if (!xhat || !table || !out || !sizes_ok(b_out, b_in, nbatch)) return S2CNN_EINVAL;
+  if (bits && !fused_path(b_out, b_in, complex_out, true)) return S2CNN_EINVAL;
   if (bias && (complex_out || nfeature < 1 || nbatch % nfeature != 0)) return S2CNN_EINVAL;
   if (relu && complex_out) return S2CNN_EINVAL;
   if (!s2cnn::aligned8(xhat) || (complex_out && !s2cnn::aligned8(out))) return S2CNN_EALIGN;
   if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (fused_path(b_out, b_in, complex_out, true))
-    return fused_synthesis(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, nbatch, false, bias, bias ? nfeature : 1, relu, st);
+    return fused_synthesis(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, nbatch, false, bias, bias ? nfeature : 1, relu, bits, st);
   const size_t need = s2cnn_so3_synthesis_workspace(b_in, b_out, nbatch, complex_out);
   if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
   const int n2 = 2 * b_out, nb = b_in < b_out ? b_in : b_out;
@@ -567,48 +569,84 @@ extern "C" int s2cnn_so3_analysis(const float* x, const float* table, const floa
                                   void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
                                   int complex_in, void* stream) {
   s2cnn::clear_stale_error();
-  return analysis_impl(x, nullptr, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, complex_in, stream);
+  return analysis_impl(x, nullptr, false, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, complex_in, stream);
 }
 
 extern "C" int s2cnn_so3_synthesis(const float* xhat, const float* table, const float* packed_table, float* out,
                                    void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
                                    int complex_out, void* stream) {
   s2cnn::clear_stale_error();
-  return synthesis_impl(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, complex_out, nullptr, 1, 0, stream);
+  return synthesis_impl(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, complex_out, nullptr, 1, 0, nullptr, stream);
 }
 
 extern "C" int s2cnn_so3_synthesis_real_bias(const float* xhat, const float* table, const float* packed_table, float* out,
                                              void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
                                              const float* bias, int nfeature, void* stream) {
   s2cnn::clear_stale_error();
-  return synthesis_impl(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, 0, bias, nfeature, 0, stream);
+  return synthesis_impl(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, 0, bias, nfeature, 0, nullptr, stream);
 }
 
-extern "C" int s2cnn_so3_synthesis_real_relu(const float* xhat, const float* table, const float* packed_table, float* out,
-                                             void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
-                                             const float* bias, int nfeature, int real_basis, void* stream) {
-  s2cnn::clear_stale_error();
+namespace {
+int synthesis_relu_impl(const float* xhat, const float* table, const float* packed_table, float* out, unsigned long long* bits,
+                        void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch, const float* bias, int nfeature,
+                        int real_basis, void* stream) {
   if (!real_basis)
-    return synthesis_impl(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, 0, bias, nfeature, 1, stream);
+    return synthesis_impl(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, 0, bias, nfeature, 1, bits, stream);
   if (!xhat || !table || !out || !sizes_ok(b_out, b_in, nbatch)) return S2CNN_EINVAL;
   if (bias && (nfeature < 1 || nbatch % nfeature != 0)) return S2CNN_EINVAL;
   if (!fused_path(b_out, b_in, 0, true)) return S2CNN_EINVAL;
   if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
   return fused_synthesis(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, nbatch, true, bias, bias ? nfeature : 1, 1,
-                         static_cast<hipStream_t>(stream));
+                         bits, static_cast<hipStream_t>(stream));
+}
+
+int analysis_masked_impl(const float* x, const float* mask, bool mask_bits, const float* table, const float* packed_table, float* out,
+                         void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch, int real_basis, void* stream) {
+  if (!mask) return S2CNN_EINVAL;
+  if (!real_basis)
+    return analysis_impl(x, mask, mask_bits, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, 0, stream);
+  if (!x || !table || !out || !sizes_ok(b_in, b_out, nbatch)) return S2CNN_EINVAL;
+  if (!fused_path(b_in, b_out, 0, false)) return S2CNN_EINVAL;
+  if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
+  return fused_analysis(x, mask, mask_bits, table, packed_table, out, workspace, workspace_bytes, b_out, nbatch, true, static_cast<hipStream_t>(stream));
+}
+}  // namespace
+
+extern "C" int s2cnn_so3_synthesis_real_relu(const float* xhat, const float* table, const float* packed_table, float* out,
+                                             void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
+                                             const float* bias, int nfeature, int real_basis, void* stream) {
+  s2cnn::clear_stale_error();
+  return synthesis_relu_impl(xhat, table, packed_table, out, nullptr, workspace, workspace_bytes, b_in, b_out, nbatch, bias, nfeature, real_basis, stream);
+}
+
+extern "C" size_t s2cnn_so3_relu_bits_bytes(int b_grid, long nbatch) {
+  if (nbatch < 1 || !fused_path(b_grid, b_grid, 0, true)) return 0;
+  return (size_t)nbatch * fused64::BITS_WORDS * sizeof(unsigned long long);
+}
+
+extern "C" int s2cnn_so3_synthesis_real_relu_bits(const float* xhat, const float* table, const float* packed_table, float* out,
+                                                  void* bits, void* workspace, size_t workspace_bytes, int b_in, int b_out,
+                                                  long nbatch, const float* bias, int nfeature, int real_basis, void* stream) {
+  s2cnn::clear_stale_error();
+  if (!bits || s2cnn_so3_relu_bits_bytes(b_out, nbatch) == 0) return S2CNN_EINVAL;
+  return synthesis_relu_impl(xhat, table, packed_table, out, static_cast<unsigned long long*>(bits), workspace, workspace_bytes, b_in, b_out,
+                             nbatch, bias, nfeature, real_basis, stream);
 }
 
 extern "C" int s2cnn_so3_analysis_real_masked(const float* x, const float* mask, const float* table, const float* packed_table,
                                               float* out, void* workspace, size_t workspace_bytes, int b_in, int b_out,
                                               long nbatch, int real_basis, void* stream) {
   s2cnn::clear_stale_error();
-  if (!mask) return S2CNN_EINVAL;
-  if (!real_basis)
-    return analysis_impl(x, mask, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, 0, stream);
-  if (!x || !table || !out || !sizes_ok(b_in, b_out, nbatch)) return S2CNN_EINVAL;
-  if (!fused_path(b_in, b_out, 0, false)) return S2CNN_EINVAL;
-  if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
-  return fused_analysis(x, mask, table, packed_table, out, workspace, workspace_bytes, b_out, nbatch, true, static_cast<hipStream_t>(stream));
+  return analysis_masked_impl(x, mask, false, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, real_basis, stream);
+}
+
+extern "C" int s2cnn_so3_analysis_real_masked_bits(const float* x, const void* bits, const float* table, const float* packed_table,
+                                                   float* out, void* workspace, size_t workspace_bytes, int b_in, int b_out,
+                                                   long nbatch, int real_basis, void* stream) {
+  s2cnn::clear_stale_error();
+  if (s2cnn_so3_relu_bits_bytes(b_in, nbatch) == 0) return S2CNN_EINVAL;
+  return analysis_masked_impl(x, static_cast<const float*>(bits), true, table, packed_table, out, workspace, workspace_bytes, b_in, b_out,
+                              nbatch, real_basis, stream);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -651,5 +689,5 @@ extern "C" int s2cnn_so3_analysis_static(const float* x, const float* table, con
   void* ws = nullptr;
   const int rc = static_scratch(&ws);
   if (rc) return rc;
-  return analysis_impl(x, nullptr, table, packed_table, out, ws, (size_t)S2CNN_STATIC_SCRATCH_BYTES, b_in, b_out, nbatch, complex_in, stream);
+  return analysis_impl(x, nullptr, false, table, packed_table, out, ws, (size_t)S2CNN_STATIC_SCRATCH_BYTES, b_in, b_out, nbatch, complex_in, stream);
 }

@@ -204,10 +204,14 @@ __device__ constexpr int table_slot(int it) { return it & 3; }
 
 // NA: item rounds that carry degrees below the output bandwidth (items are ordered by degree group, so a truncated
 // spectrum leaves the later rounds without work: NA = 3 covers l < 24, 5 covers l < 28, 7 everything).
-// MASKED: the signal is x where mask > 0 and zero elsewhere (mask: a tensor of the shape of x).
-template <int NA, bool MASKED>
+// MASK: 0: the signal is x; 1: x where mask > 0 and zero elsewhere (mask: a tensor of the shape of x); 2: the same with
+// `mask` holding one BIT per sample instead (bits_index below), as the synthesis writes them.
+constexpr int BITS_WORDS = N * N;      // 64-bit words per volume: [beta][alpha % 8][alpha / 8], bit = gamma
+__host__ __device__ inline size_t bits_index(long z, int beta, int d) { return ((size_t)z * N + beta) * N + 8 * d; }   // + alpha / 8
+template <int NA, int MASK>
 __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restrict__ x, const float* __restrict__ mask,
                                                            const float* __restrict__ Tf, float4* __restrict__ rec, long nbatch) {
+  constexpr bool MASKED = MASK == 1;
   using namespace fft64;
   __shared__ __attribute__((aligned(16))) float2 work[LDS_ELEMS];
   __shared__ __attribute__((aligned(16))) float2 quad[2][QUAD_ELEMS];
@@ -250,29 +254,31 @@ __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restri
   const unsigned toff = t * 16;
   float pa[8], pb[8];
   float ma[MASKED ? 8 : 1], mb[MASKED ? 8 : 1];
+  // bit masks of the wave's eight rows of either plane: uniform over the wave (scalar loads), one lane mask per row
+  unsigned long long ba[MASK == 2 ? 8 : 1], bb[MASK == 2 ? 8 : 1];
+  const unsigned long long* const bits = reinterpret_cast<const unsigned long long*>(mask);
+  const int du = __builtin_amdgcn_readfirstlane(d);
   float4 t1[4], t2[4];
 
-  auto load_planes = [&](int j) {            // planes j and 63-j: one full row (256 bytes) per wave and load
-#pragma unroll
-    for (int j1 = 0; j1 < 8; ++j1) {
-      pa[j1] = buf_load_f32(rx, xoff, (j * 4096 + j1 * 512) * 4);
-      pb[j1] = buf_load_f32(rx, xoff, ((63 - j) * 4096 + j1 * 512) * 4);
-      if constexpr (MASKED) {
-        ma[j1] = buf_load_f32(rm, xoff, (j * 4096 + j1 * 512) * 4);
-        mb[j1] = buf_load_f32(rm, xoff, ((63 - j) * 4096 + j1 * 512) * 4);
-      }
+  auto load_rows = [&](int j, int j1) {      // row 8 j1 + d of the planes j and 63-j: one full row (256 bytes) per wave and load
+    pa[j1] = buf_load_f32(rx, xoff, (j * 4096 + j1 * 512) * 4);
+    pb[j1] = buf_load_f32(rx, xoff, ((63 - j) * 4096 + j1 * 512) * 4);
+    if constexpr (MASKED) {
+      ma[j1] = buf_load_f32(rm, xoff, (j * 4096 + j1 * 512) * 4);
+      mb[j1] = buf_load_f32(rm, xoff, ((63 - j) * 4096 + j1 * 512) * 4);
     }
+    if constexpr (MASK == 2) {
+      ba[j1] = bits[bits_index(z, j, du) + j1];
+      bb[j1] = bits[bits_index(z, 63 - j, du) + j1];
+    }
+  };
+  auto load_planes = [&](int j) {
+#pragma unroll
+    for (int j1 = 0; j1 < 8; ++j1) load_rows(j, j1);
   };
   auto load_planes_part = [&](int j, int g) {   // a quarter of load_planes
 #pragma unroll
-    for (int j1 = 2 * g; j1 < 2 * g + 2; ++j1) {
-      pa[j1] = buf_load_f32(rx, xoff, (j * 4096 + j1 * 512) * 4);
-      pb[j1] = buf_load_f32(rx, xoff, ((63 - j) * 4096 + j1 * 512) * 4);
-      if constexpr (MASKED) {
-        ma[j1] = buf_load_f32(rm, xoff, (j * 4096 + j1 * 512) * 4);
-        mb[j1] = buf_load_f32(rm, xoff, ((63 - j) * 4096 + j1 * 512) * 4);
-      }
-    }
+    for (int j1 = 2 * g; j1 < 2 * g + 2; ++j1) load_rows(j, j1);
   };
   auto load_table = [&](int j, int it) {
     t1[table_slot(it)] = buf_load_f32x4(rt, toff, ((j * NIT + it) * 2 + 0) * (THREADS * 16));
@@ -284,6 +290,8 @@ __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restri
 #pragma unroll
     for (int j1 = 0; j1 < 8; ++j1) {
       if constexpr (MASKED) v[j1] = make_float2(s2cnn::relu_pass(pa[j1], ma[j1]), s2cnn::relu_pass(pb[j1], mb[j1]));
+      else if constexpr (MASK == 2) v[j1] = make_float2(__builtin_amdgcn_inverse_ballot_w64(ba[j1]) ? pa[j1] : 0.f,
+                                                        __builtin_amdgcn_inverse_ballot_w64(bb[j1]) ? pb[j1] : 0.f);
       else v[j1] = make_float2(pa[j1], pb[j1]);
     }
     fft8<false>(v);
@@ -667,7 +675,7 @@ __global__ __launch_bounds__(256) void spectrum_gather_real(const float* __restr
 template <int NA, int CMAX>
 __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __restrict__ rec, const float* __restrict__ Tf,
                                                             float* __restrict__ y, long nbatch, const float* __restrict__ bias, int nfeature,
-                                                            int relu) {
+                                                            int relu, unsigned long long* __restrict__ bits) {
   using namespace fft64;
   __shared__ __attribute__((aligned(16))) float2 work[LDS_ELEMS];
   constexpr int STG_PADS = 144;                                              // one pad per row: sum of (4c+4) over the 8 degree groups
@@ -788,12 +796,21 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
 #pragma unroll
     for (int k = 0; k < 8; ++k) v[k] = line[k * PITCH];
     fft8<true>(v);
+    unsigned long long wa = 0, wb = 0;               // lane k: which samples of row d + 8 k are positive (one bit per column)
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
       float ra = v[k].x + bz, rb = v[k].y + bz;
       if (relu) { ra = s2cnn::relu_f(ra); rb = s2cnn::relu_f(rb); }
       buf_store_f32(ra, ry, yoff, (j * 4096 + k * 512) * 4);
       buf_store_f32(rb, ry, yoff, ((63 - j) * 4096 + k * 512) * 4);
+      if (bits) {                                   // the gradient of max(., 0) passes where the output is not <= 0 (a NaN passes)
+        const unsigned long long qa = __ballot(!(ra <= 0.f)), qb = __ballot(!(rb <= 0.f));
+        if (lo == k) { wa = qa; wb = qb; }
+      }
+    }
+    if (bits && lo < 8) {                           // 64 contiguous bytes per plane and wave
+      bits[bits_index(z, j, d) + lo] = wa;
+      bits[bits_index(z, 63 - j, d) + lo] = wb;
     }
   };
 
@@ -867,7 +884,7 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
 inline int active_rounds(int nl) { return nl <= 24 ? 3 : nl <= 28 ? 5 : NIT; }
 
 // Launchers: the instantiation whose item rounds cover the nl degrees present.
-template <bool MASKED>
+template <int MASKED>
 inline void launch_analysis_m(int nl, hipStream_t st, const float* x, const float* mask, const float* Tf, float4* rec, long nbatch) {
   const dim3 grid(grid_size(nbatch)), block(THREADS);
   if (nl <= 24) hipLaunchKernelGGL((analysis_kernel<3, MASKED>), grid, block, 0, st, x, mask, Tf, rec, nbatch);
@@ -875,18 +892,21 @@ inline void launch_analysis_m(int nl, hipStream_t st, const float* x, const floa
   else hipLaunchKernelGGL((analysis_kernel<7, MASKED>), grid, block, 0, st, x, mask, Tf, rec, nbatch);
 }
 
-// mask: NULL, or the tensor whose positive entries select the samples of x that count
-inline void launch_analysis(int nl, hipStream_t st, const float* x, const float* mask, const float* Tf, float4* rec, long nbatch) {
-  if (mask) launch_analysis_m<true>(nl, st, x, mask, Tf, rec, nbatch);
-  else launch_analysis_m<false>(nl, st, x, nullptr, Tf, rec, nbatch);
+// mask: NULL, or the tensor whose positive entries select the samples of x that count; mask_bits: `mask` holds one bit
+// per sample (BITS_WORDS 64-bit words per volume, written by the synthesis) instead of one float
+inline void launch_analysis(int nl, hipStream_t st, const float* x, const float* mask, bool mask_bits, const float* Tf, float4* rec, long nbatch) {
+  if (mask && mask_bits) launch_analysis_m<2>(nl, st, x, mask, Tf, rec, nbatch);
+  else if (mask) launch_analysis_m<1>(nl, st, x, mask, Tf, rec, nbatch);
+  else launch_analysis_m<0>(nl, st, x, nullptr, Tf, rec, nbatch);
 }
 
+// bits: NULL, or BITS_WORDS 64-bit words per volume that receive one bit per sample: the output is not <= 0
 inline void launch_synthesis(int nl, hipStream_t st, const float4* rec, const float* Tf, float* y, long nbatch, const float* bias,
-                             int nfeature, int relu) {
+                             int nfeature, int relu, unsigned long long* bits) {
   const dim3 grid(grid_size(nbatch)), block(THREADS);
-  if (nl <= 24) hipLaunchKernelGGL((synthesis_kernel<3, 6>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu);
-  else if (nl <= 28) hipLaunchKernelGGL((synthesis_kernel<5, 7>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu);
-  else hipLaunchKernelGGL((synthesis_kernel<7, 8>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu);
+  if (nl <= 24) hipLaunchKernelGGL((synthesis_kernel<3, 6>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits);
+  else if (nl <= 28) hipLaunchKernelGGL((synthesis_kernel<5, 7>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits);
+  else hipLaunchKernelGGL((synthesis_kernel<7, 8>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits);
 }
 
 }  // namespace fused64

@@ -57,6 +57,18 @@ def _same_shape_operand(mask, x):
     return mask.clone() if mask.data_ptr() % 16 else mask
 
 
+def _is_bit_mask(mask):
+    """A mask of one bit per sample, as `_relu_bits` allocates it and the transforms with relu=True fill it."""
+    return mask is not None and mask.dtype == torch.int64
+
+
+def _relu_bits(b_grid, nbatch, device):
+    """Where the synthesis onto the (2 b_grid)^3 grid can record the sign of its output as one bit per sample: an int64
+    tensor for them (s2cnn_so3_relu_bits_bytes), else None (the float output then serves as the mask)."""
+    nbytes = _hip.lib().s2cnn_so3_relu_bits_bytes(b_grid, nbatch) if nbatch > 0 else 0
+    return torch.empty(nbytes // 8, dtype=torch.int64, device=device) if nbytes else None
+
+
 def _analysis(x, b_in, b_out, batch_size, for_grad, complex_in, mask=None):
     """x: contiguous grid tensor whose leading dims are `batch_size`; the result is allocated in its
     final shape (never a view: autograd can then take ownership of it as a gradient without a copy).
@@ -81,6 +93,10 @@ def _analysis(x, b_in, b_out, batch_size, for_grad, complex_in, mask=None):
     if nbatch == 0:
         return out
     ws = _hip.workspace(L.s2cnn_so3_analysis_workspace(b_in, b_out, nbatch, complex_in), x.device)
+    if _is_bit_mask(mask):
+        _hip.call("s2cnn_so3_analysis_real_masked_bits", _hip.ptr(x), _hip.ptr(mask), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out),
+                  _hip.ptr(ws), ws.numel(), b_in, b_out, nbatch, 0, _hip.stream_ptr())
+        return out
     if mask is not None:
         mask = _same_shape_operand(mask, x)
         _hip.call("s2cnn_so3_analysis_real_masked", _hip.ptr(x), _hip.ptr(mask), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out),
@@ -91,7 +107,8 @@ def _analysis(x, b_in, b_out, batch_size, for_grad, complex_in, mask=None):
     return out
 
 
-def _synthesis(x, b_in, b_out, batch_size, for_grad, complex_out, bias=None, relu=False):
+def _synthesis(x, b_in, b_out, batch_size, for_grad, complex_out, bias=None, relu=False, bits=None):
+    """bits (with relu): an int64 tensor from `_relu_bits` that receives one bit per sample (the output is not <= 0)."""
     _hip.require_gpu_f32(x)
     assert not (relu and complex_out)
     if complex_out and complex_via_real:
@@ -116,6 +133,10 @@ def _synthesis(x, b_in, b_out, batch_size, for_grad, complex_out, bias=None, rel
         _hip.require_gpu_f32(bias)
         bias = bias.reshape(-1).contiguous()
         assert len(batch_size) >= 1 and batch_size[-1] == bias.numel()
+    if relu and bits is not None:
+        _hip.call("s2cnn_so3_synthesis_real_relu_bits", _hip.ptr(x), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out), _hip.ptr(bits),
+                  _hip.ptr(ws), ws.numel(), b_in, b_out, nbatch, _null_or_ptr(bias), 1 if bias is None else bias.numel(), 0, _hip.stream_ptr())
+        return out
     if relu:
         _hip.call("s2cnn_so3_synthesis_real_relu", _hip.ptr(x), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out), _hip.ptr(ws),
                   ws.numel(), b_in, b_out, nbatch, _null_or_ptr(bias), 1 if bias is None else bias.numel(), 0, _hip.stream_ptr())
@@ -149,6 +170,7 @@ def so3_rfft(x, for_grad=False, b_out=None, mask=None):
     '''
     :param x: [..., beta, alpha, gamma]
     :param mask: None, or a tensor of the shape of x: samples of x where it is not positive count as zero
+                 (or the bit mask that so3_rifft(..., relu=True, bits=...) filled)
     :return: [l * m * n, ..., complex]
     '''
     b_in = x.size(-1) // 2
@@ -181,15 +203,16 @@ def so3_ifft(x, for_grad=False, b_out=None):
     return _synthesis(x, b_in, b_out, batch_size, for_grad, 1)
 
 
-def so3_rifft(x, for_grad=False, b_out=None, bias=None, relu=False):
+def so3_rifft(x, for_grad=False, b_out=None, bias=None, relu=False, bits=None):
     '''
     :param x: [l * m * n, ..., complex]
     :param bias: None, or one value per entry of the last batch dimension, added to every sample of its volumes
     :param relu: negative samples (after the bias) come out as zero
+    :param bits: None, or (with relu) the int64 tensor of `_relu_bits` that receives one bit per sample: the output is not <= 0
     :return: [..., beta, alpha, gamma]  (the real part of so3_ifft, whatever the symmetry of x)
     '''
     x, b_in, b_out, batch_size = _spectrum_args(x, b_out)
-    return _synthesis(x, b_in, b_out, batch_size, for_grad, 0, bias, relu)
+    return _synthesis(x, b_in, b_out, batch_size, for_grad, 0, bias, relu, bits)
 
 
 class SO3_fft_real(torch.autograd.Function):
@@ -218,10 +241,14 @@ class SO3_ifft_real(torch.autograd.Function):
         ctx.b_out = b_out
         ctx.b_in = round((3 / 4 * nspec) ** (1 / 3))
         ctx.bias_shape = None if bias is None else bias.shape
-        out = so3_rifft(x, b_out=ctx.b_out, bias=bias, relu=relu)
+        bits = None
+        b_grid = ctx.b_in if b_out is None else b_out
+        if relu and x.is_cuda and ctx.b_in <= b_grid:      # one bit per sample where the library can record it and its
+            bits = _relu_bits(b_grid, x[..., 0].numel() // nspec, x.device)     # analysis can read it; else the output is the mask
+        out = so3_rifft(x, b_out=ctx.b_out, bias=bias, relu=relu, bits=bits)
         ctx.relu = bool(relu)
         if relu:
-            ctx.save_for_backward(out)
+            ctx.save_for_backward(out if bits is None else bits)
         return out
 
     @staticmethod
@@ -273,6 +300,10 @@ def so3_rfft_real_basis(x, for_grad=False, b_out=None, mask=None):
     if nbatch == 0:
         return out
     ws = _hip.workspace(L.s2cnn_so3_analysis_workspace(b_in, b_out, nbatch, 0), x.device)
+    if _is_bit_mask(mask):
+        _hip.call("s2cnn_so3_analysis_real_masked_bits", _hip.ptr(x), _hip.ptr(mask), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out),
+                  _hip.ptr(ws), ws.numel(), b_in, b_out, nbatch, 1, _hip.stream_ptr())
+        return out
     if mask is not None:
         mask = _same_shape_operand(mask, x)
         _hip.call("s2cnn_so3_analysis_real_masked", _hip.ptr(x), _hip.ptr(mask), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out),
@@ -283,7 +314,7 @@ def so3_rfft_real_basis(x, for_grad=False, b_out=None, mask=None):
     return out
 
 
-def so3_rifft_real_basis(r, for_grad=False, b_out=None, bias=None, relu=False):
+def so3_rifft_real_basis(r, for_grad=False, b_out=None, bias=None, relu=False, bits=None):
     '''
     :param r: [l * m * n, ...]  real-basis spectrum
     :param bias: None, or one value per entry of the last batch dimension, added to every sample of its volumes
@@ -297,7 +328,7 @@ def so3_rifft_real_basis(r, for_grad=False, b_out=None, bias=None, relu=False):
         b_out = b_in
     if not (r.is_cuda and _real_basis_direct(b_in, b_out, True)):
         from ..so3_real import _convert
-        return so3_rifft(_convert("s2cnn_so3_spectrum_to_complex", r.contiguous(), (*r.shape, 2)), for_grad, b_out, bias, relu)
+        return so3_rifft(_convert("s2cnn_so3_spectrum_to_complex", r.contiguous(), (*r.shape, 2)), for_grad, b_out, bias, relu, bits)
     _hip.require_gpu_f32(r)
     r = r.contiguous()
     batch_size = r.size()[1:]
@@ -317,6 +348,10 @@ def so3_rifft_real_basis(r, for_grad=False, b_out=None, bias=None, relu=False):
         bias = bias.reshape(-1).contiguous()
         nfeature = bias.numel()
         assert r.dim() >= 2 and r.size(-1) == nfeature
+    if relu and bits is not None:
+        _hip.call("s2cnn_so3_synthesis_real_relu_bits", _hip.ptr(r), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out), _hip.ptr(bits),
+                  _hip.ptr(ws), ws.numel(), b_in, b_out, nbatch, _null_or_ptr(bias), nfeature, 1, _hip.stream_ptr())
+        return out
     if relu:
         _hip.call("s2cnn_so3_synthesis_real_relu", _hip.ptr(r), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out), _hip.ptr(ws),
                   ws.numel(), b_in, b_out, nbatch, _null_or_ptr(bias), nfeature, 1, _hip.stream_ptr())
@@ -348,10 +383,14 @@ class SO3_ifft_real_basis(torch.autograd.Function):
         nspec = r.size(0)
         ctx.b_in = round((3 / 4 * nspec) ** (1 / 3))
         ctx.bias_shape = None if bias is None else bias.shape
-        out = so3_rifft_real_basis(r, b_out=b_out, bias=bias, relu=relu)
+        bits = None
+        b_grid = ctx.b_in if b_out is None else b_out
+        if relu and r.is_cuda and ctx.b_in <= b_grid:
+            bits = _relu_bits(b_grid, r.numel() // nspec, r.device)
+        out = so3_rifft_real_basis(r, b_out=b_out, bias=bias, relu=relu, bits=bits)
         ctx.relu = bool(relu)
         if relu:
-            ctx.save_for_backward(out)
+            ctx.save_for_backward(out if bits is None else bits)
         return out
 
     @staticmethod

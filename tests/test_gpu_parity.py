@@ -376,6 +376,46 @@ def test_so3_transforms_with_fused_relu(hip, b_in, b_out, nz, nf):
     assert torch.equal(P.so3_rfft(xo, b_out=b_out, mask=yo), P.so3_rfft(xo * (yo > 0), b_out=b_out))
 
 
+@pytest.mark.parametrize("b_in", [32, 10, 22])
+def test_one_bit_relu_mask_on_the_64_grid(hip, b_in):
+    """The synthesis onto the 64^3 grid can record "the output is not <= 0" as one bit per sample (word
+    [volume][beta][alpha % 8][alpha / 8], bit gamma), and the analysis from that grid can take those bits for the mask:
+    the bits must say exactly what the float output says, and the masked analysis must give the numbers of the analysis
+    with the float mask up to rounding (the two instantiations of the kernel need not contract their multiply-adds alike:
+    2e-6 of the largest coefficient), for both kinds of spectra and both tables.  Other grids report that they keep no bits."""
+    from s2cnn_amd.soft import so3_fft as P
+    from s2cnn_amd.so3_real import so3_spectrum_to_real
+    assert P._relu_bits(22, 3, "cuda") is None and P._relu_bits(32, 0, "cuda") is None
+    nz, nf = 6, 3
+    g = torch.Generator().manual_seed(77 + b_in)
+    xh = torch.randn(O.nspec_so3(b_in), nz // nf, nf, 2, generator=g).cuda()
+    bias = torch.randn(nf, generator=g).cuda()
+    gy = torch.randn(nz // nf, nf, 64, 64, 64, generator=g).cuda()
+    for real_basis in (False, True):
+        spec = so3_spectrum_to_real(xh) if real_basis else xh
+        synth = P.so3_rifft_real_basis if real_basis else P.so3_rifft
+        ana = P.so3_rfft_real_basis if real_basis else P.so3_rfft
+        bits = P._relu_bits(32, nz, "cuda")
+        assert bits.numel() == nz * 64 * 64 and bits.dtype == torch.int64
+        bits.fill_(0x5555555555555555)                                        # every word must be overwritten
+        out = synth(spec, b_out=32, bias=bias, relu=True, bits=bits)
+        assert torch.equal(out, synth(spec, b_out=32, bias=bias, relu=True))
+        # unpack: [z, beta, alpha % 8, alpha / 8] words, bit gamma
+        shifts = torch.arange(64, device="cuda")
+        got = ((bits.view(nz, 64, 8, 8, 1) >> shifts) & 1).bool()             # [z, beta, a_lo, a_hi, gamma]
+        got = got.permute(0, 1, 3, 2, 4).reshape(nz, 64, 64, 64)              # alpha = 8 a_hi + a_lo
+        assert torch.equal(got, out.view(nz, 64, 64, 64) > 0)
+        for for_grad in (False, True):
+            for b_out in (32, 22, b_in):
+                want = ana(gy, for_grad=for_grad, b_out=b_out, mask=out)
+                got = ana(gy, for_grad=for_grad, b_out=b_out, mask=bits)
+                err = (got - want).abs().max().item() / want.abs().max().item()
+                assert err < 2e-6, (real_basis, for_grad, b_out, err)
+        # a mask of all ones is no mask, a mask of zeros leaves nothing
+        close(ana(gy, b_out=b_in, mask=torch.full_like(bits, -1)), ana(gy, b_out=b_in).double().cpu(), "all-ones bit mask")
+        assert not ana(gy, b_out=b_in, mask=torch.zeros_like(bits)).any()
+
+
 @pytest.mark.parametrize("kind,real_basis", [("so3", True), ("so3", False), ("s2", True), ("s2", False)])
 def test_layers_with_fused_relu(hip, kind, real_basis):
     """activation="relu" is F.relu(layer(x)): same output, same gradients wrt input, kernel and bias; and the
