@@ -233,7 +233,8 @@ def measure_network(torch, dev, steps, warmup):
     g1 = s2cnn_amd.s2_near_identity_grid(max_beta=math.pi / 8 * 30 / 128, n_alpha=8, n_beta=3)
     g2 = s2cnn_amd.so3_near_identity_grid(max_beta=math.pi / 8 * 30 / 32, max_gamma=2 * math.pi, n_alpha=8, n_beta=3, n_gamma=8)
     g3 = s2cnn_amd.so3_near_identity_grid(max_beta=math.pi / 8 * 30 / 22, max_gamma=2 * math.pi, n_alpha=8, n_beta=3, n_gamma=8)
-    x = torch.rand(32, 6, 256, 256, device=dev)
+    from s2cnn_amd.harness import smooth_spherical_batch
+    x = smooth_spherical_batch(32, 6, 128, dev, seed=5)     # uniform-range values with smooth structure of degrees l < 16 plus noise
 
     def timed(activation):
         torch.manual_seed(8)

@@ -28,6 +28,21 @@ __global__ __launch_bounds__(256) void so3_integrate_kernel(const float* __restr
       }
       acc += w[bt] * (((s0.x + s0.y) + (s0.z + s0.w)) + ((s1.x + s1.y) + (s1.z + s1.w)) + ((s2.x + s2.y) + (s2.z + s2.w)) + ((s3.x + s3.y) + (s3.z + s3.w)));
     }
+  } else if ((reinterpret_cast<uintptr_t>(x) & 15u) == 0) {
+    // any other grid: n2 is even, so planes and volumes are whole numbers of 16-byte words
+    const float4* x4 = reinterpret_cast<const float4*>(xs);
+    const int p4 = (int)(plane / 4);
+    for (int bt = 0; bt < n2; ++bt) {
+      float4 s0 = make_float4(0.f, 0.f, 0.f, 0.f), s1 = s0;
+      const float4* pl = x4 + (size_t)bt * p4;
+      for (int i = threadIdx.x; i < p4; i += 512) {
+        const float4 v0 = pl[i];
+        const float4 v1 = i + 256 < p4 ? pl[i + 256] : make_float4(0.f, 0.f, 0.f, 0.f);
+        s0.x += v0.x; s0.y += v0.y; s0.z += v0.z; s0.w += v0.w;
+        s1.x += v1.x; s1.y += v1.y; s1.z += v1.z; s1.w += v1.w;
+      }
+      acc += w[bt] * (((s0.x + s0.y) + (s0.z + s0.w)) + ((s1.x + s1.y) + (s1.z + s1.w)));
+    }
   } else {
     for (int bt = 0; bt < n2; ++bt) {
       float s = 0.f;
@@ -49,6 +64,16 @@ __global__ __launch_bounds__(256) void so3_integrate_grad_kernel(const float* __
   const size_t plane = (size_t)n2 * n2;
   float* dst = gx + blockIdx.x * plane * n2;
   const float gv = g[blockIdx.x];
+  if ((reinterpret_cast<uintptr_t>(gx) & 15u) == 0) {      // n2 is even: every plane is a whole number of 16-byte words
+    float4* dst4 = reinterpret_cast<float4*>(dst);
+    const int p4 = (int)(plane / 4);
+    for (int bt = 0; bt < n2; ++bt) {
+      const float v = gv * w[bt];
+      const float4 v4 = make_float4(v, v, v, v);
+      for (int i = threadIdx.x; i < p4; i += blockDim.x) dst4[(size_t)bt * p4 + i] = v4;
+    }
+    return;
+  }
   for (int bt = 0; bt < n2; ++bt) {
     const float v = gv * w[bt];
     for (size_t i = threadIdx.x; i < plane; i += blockDim.x) dst[bt * plane + i] = v;

@@ -117,6 +117,22 @@ def synthetic_batch(name, batch, device, seed=0):
     return x.to(device), y.to(device)
 
 
+def smooth_spherical_batch(batch, channels, b, device, seed=0, lmax=16, noise=0.1):
+    """Signals on the 2b x 2b grid of the sphere with smooth low-bandwidth structure: the synthesis of a random spectrum of
+    degrees l < lmax (amplitudes falling like 1 / (l + 1)), rescaled per signal to [0, 1 - noise], plus uniform noise in
+    [0, noise): the ray-cast depth / normal look of the inputs of the shape networks, values in [0, 1)."""
+    from .soft.s2_fft import S2_ifft_real
+    g = torch.Generator().manual_seed(seed)
+    spec = torch.randn(lmax * lmax, batch * channels, 2, generator=g)
+    falloff = torch.cat([torch.full((2 * l + 1,), 1.0 / (l + 1)) for l in range(lmax)])
+    y = S2_ifft_real.apply((spec * falloff.view(-1, 1, 1)).to(device), b)          # [batch * channels, 2b, 2b]
+    flat = y.reshape(y.size(0), -1)
+    lo, hi = flat.min(1, keepdim=True)[0], flat.max(1, keepdim=True)[0]
+    flat = (flat - lo) / (hi - lo).clamp_min(1e-12) * (1.0 - noise)
+    flat = flat + noise * torch.rand(flat.shape, generator=g).to(device)
+    return flat.clamp_(0.0, 1.0 - 1e-7).view(batch, channels, 2 * b, 2 * b)
+
+
 def train_steps(name, batch=32, steps=10, warmup=2, lr=0.05, device="cuda:0", seed=0, model=None):
     """`warmup + steps` SGD steps (momentum 0.9, as examples/shrec17/train.py:66) on one synthetic batch.
     Returns (model, losses of all steps, milliseconds per timed step)."""

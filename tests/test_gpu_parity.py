@@ -227,6 +227,10 @@ def test_so3_integrate(hip):
         close(gx, gxo, f"integrate grad b={b}")
     ones = torch.ones(3, 8, 8, 8, device="cuda")
     assert (s2cnn_amd.so3_integrate(ones) - 1).abs().max().item() < 1e-5
+    # an input that is not 16-byte aligned takes the 4-byte loads: same numbers up to the order of the sums
+    big = rnd((3 * 14 ** 3 + 1,), 43).cuda()
+    xo = big[1:].view(3, 14, 14, 14)
+    close(s2cnn_amd.so3_integrate(xo), O.so3_integrate(xo.cpu().double()), "integrate, unaligned input")
 
 
 # ------------------------------------------------------------------ layers, forward and gradients
@@ -489,7 +493,9 @@ def test_config5_shaped_network(hip):
     """Forward parity against the oracle at batch 1; forward + backward at batch 4 on the GPU must reproduce the
     batch-1 result for its first sample (batch independence) and give finite gradients."""
     (c1, c2, c3), (g1, g2, g3) = _config5_layers()
-    x = torch.rand(4, 6, 256, 256, generator=torch.Generator().manual_seed(9))
+    from s2cnn_amd.harness import smooth_spherical_batch
+    x = smooth_spherical_batch(4, 6, 128, "cuda", seed=9).cpu()       # the input the configuration names: smooth, l < 16, plus noise
+    assert 0.0 <= x.min().item() and x.max().item() < 1.0 and x.std().item() > 0.05
     x1 = x[:1].double()
 
     def kb(c):
