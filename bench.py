@@ -286,9 +286,25 @@ def measure_example_network(torch, name, steps, warmup, batch=32):
         harness.train_steps(name, batch=batch, steps=1, warmup=0, lr=0.01, model=model)
         torch.cuda.synchronize()
     calls = {k: round(sum(v), 3) for k, v in sorted(kt.summary().items(), key=lambda kv: -sum(kv[1]))}
-    return {"workload": "%s training step (s2cnn_amd/harness.py), batch %d, synthetic data" % (name, batch),
-            "ms_per_step": round(ms, 3), "samples_per_s": round(batch / (ms * 1e-3), 1), "first_loss": round(losses[0], 4),
-            "last_loss": round(losses[-1], 4), "library_ms": round(sum(calls.values()), 3), "library_calls_ms": calls}
+    out = {"workload": "%s training step (s2cnn_amd/harness.py), batch %d, synthetic data" % (name, batch),
+           "ms_per_step": round(ms, 3), "samples_per_s": round(batch / (ms * 1e-3), 1), "first_loss": round(losses[0], 4),
+           "last_loss": round(losses[-1], 4), "library_ms": round(sum(calls.values()), 3), "library_calls_ms": calls}
+    if name.startswith("shrec17"):
+        # the same network with its BatchNorm3d + ReLU pairs evaluated inside the neighbouring transforms (same function)
+        del model
+        torch.cuda.empty_cache()
+        torch.manual_seed(0)
+        fused = harness.NETWORKS[name][0]()
+        fused.fused_norm = True
+        model, flosses, fms = harness.train_steps(name, batch=batch, steps=steps, warmup=warmup, lr=0.01, model=fused)
+        with _hip.KernelTimer() as kt:
+            harness.train_steps(name, batch=batch, steps=1, warmup=0, lr=0.01, model=model)
+            torch.cuda.synchronize()
+        fcalls = {k: round(sum(v), 3) for k, v in sorted(kt.summary().items(), key=lambda kv: -sum(kv[1]))}
+        out["fused_norm"] = {"ms_per_step": round(fms, 3), "samples_per_s": round(batch / (fms * 1e-3), 1),
+                             "first_loss": round(flosses[0], 4), "last_loss": round(flosses[-1], 4),
+                             "library_ms": round(sum(fcalls.values()), 3), "library_calls_ms": fcalls}
+    return out
 
 
 def main():

@@ -239,6 +239,38 @@ int s2cnn_so3_analysis_real_masked_bits(const float *x, const void *bits, const 
                                         float *out, void *workspace, size_t workspace_bytes,
                                         int b_in, int b_out, long nbatch, int real_basis, void *stream);
 
+/* ---- batch normalisation and max(., 0) between two layers, inside the transforms --------
+ * The reference's shape networks put nn.BatchNorm3d and nn.ReLU between their layers (examples/shrec17/model.py:28-35,
+ * model_original.py:28-35): three passes over the activations forward and five backward.  Here the next layer's analysis
+ * applies the normalisation and the activation as it loads the previous layer's output y, and the backward analysis of
+ * the previous layer forms the gradient with respect to y as it loads the incoming gradient:
+ *   s2cnn_volume_moments            out[z] = (sum y, sum y^2) of each of the nvol volumes of n samples: the batch
+ *                                   statistics of a feature are sums of these over the batch
+ *   s2cnn_so3_analysis_real_affine_relu     the analysis of max(a y + b, 0), a = params[z % nfeature],
+ *                                   b = params[nfeature + z % nfeature]  (a = weight / sqrt(var + eps), b = bias - mean a)
+ *   s2cnn_bn_relu_grad_moments      out[z] = (sum g m, sum g m y), m = (a y + b > 0): the two reductions of the backward
+ *                                   pass of the normalisation (g: gradient with respect to the activation)
+ *   s2cnn_so3_analysis_real_bn_relu_grad    the analysis of a (m ? g : 0) + p + q y, params [4][nfeature] = a, b, p, q:
+ *                                   the gradient with respect to y (p, q from the reductions; p = q = 0 with fixed statistics)
+ * x / g / y: [nbatch, 2b_in, 2b_in, 2b_in], 16-byte aligned on the 64^3 grid; other arguments as s2cnn_so3_analysis
+ * (real_basis = 1 only where s2cnn_so3_real_basis_transform_available says so).  Available where
+ * s2cnn_so3_analysis_prologue_available(b_in, b_out) returns 1: the 64^3 grid with b_out <= 32 and every other grid whose
+ * planes fit the LDS; elsewhere S2CNN_EINVAL (apply the function with a pass of its own, then s2cnn_so3_analysis).
+ * nbatch must be a multiple of nfeature.  No counterpart in the reference.
+ */
+int s2cnn_so3_analysis_prologue_available(int b_in, int b_out);
+int s2cnn_volume_moments(const float *x, float *out, long nvol, long n, void *stream);
+int s2cnn_bn_relu_grad_moments(const float *g, const float *y, const float *params, int nfeature, float *out,
+                               long nvol, long n, void *stream);
+int s2cnn_so3_analysis_real_affine_relu(const float *x, const float *params, int nfeature,
+                                        const float *table, const float *packed_table, float *out,
+                                        void *workspace, size_t workspace_bytes,
+                                        int b_in, int b_out, long nbatch, int real_basis, void *stream);
+int s2cnn_so3_analysis_real_bn_relu_grad(const float *g, const float *y, const float *params, int nfeature,
+                                         const float *table, const float *packed_table, float *out,
+                                         void *workspace, size_t workspace_bytes,
+                                         int b_in, int b_out, long nbatch, int real_basis, void *stream);
+
 /* ---- table repacking for the real-signal fast path of the two transforms above ------
  * The reference uploads its Wigner table once per (b, nl, weighted, device) and reuses it
  * (soft/so3_fft.py:205-209); a caller of this library does the same with the packed copy:

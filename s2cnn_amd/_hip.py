@@ -52,6 +52,11 @@ SIGNATURES = {
     "s2cnn_so3_relu_bits_bytes": (_size_t, [_int, _long]),
     "s2cnn_so3_synthesis_real_relu_bits": (_int, _FT3R_SIG[:4] + [_vp] + _FT3R_SIG[4:-1] + [_c_float_p, _int, _int, _vp]),
     "s2cnn_so3_analysis_real_masked_bits": (_int, [_c_float_p, _vp] + _FT3R_SIG[1:-1] + [_int, _vp]),
+    "s2cnn_so3_analysis_prologue_available": (_int, [_int, _int]),
+    "s2cnn_volume_moments": (_int, [_c_float_p, _c_float_p, _long, _long, _vp]),
+    "s2cnn_bn_relu_grad_moments": (_int, [_c_float_p, _c_float_p, _c_float_p, _int, _c_float_p, _long, _long, _vp]),
+    "s2cnn_so3_analysis_real_affine_relu": (_int, [_c_float_p, _c_float_p, _int] + _FT3R_SIG[1:-1] + [_int, _vp]),
+    "s2cnn_so3_analysis_real_bn_relu_grad": (_int, [_c_float_p, _c_float_p, _c_float_p, _int] + _FT3R_SIG[1:-1] + [_int, _vp]),
     "s2cnn_so3_real_basis_transform_available": (_int, [_int, _int, _int]),
     "s2cnn_so3_analysis_real_basis": (_int, _FT3R_SIG),
     "s2cnn_so3_synthesis_real_basis": (_int, _FT3R_SIG[:-1] + [_c_float_p, _int, _vp]),

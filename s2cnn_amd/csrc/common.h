@@ -26,4 +26,27 @@ __host__ __device__ inline int ceil_div(int a, int b) { return (a + b - 1) / b; 
 __device__ __forceinline__ float relu_f(float v) { return v < 0.f ? 0.f : v; }
 __device__ __forceinline__ float relu_pass(float g, float m) { return m <= 0.f ? 0.f : g; }
 
+// What an analysis does to its input as it loads it (the signal v that is transformed):
+//   NONE            v = x
+//   MASK            v = x where w > 0, else 0                       (w: a tensor of the shape of x)
+//   BITS            the same with one bit per sample in w           (per-volume kernels of the 64^3 grid only)
+//   AFFINE_RELU     v = max(a x + b, 0)                             (a, b: per feature, params [2][nfeature])
+//   BN_RELU_GRAD    v = a (a w + b > 0 ? x : 0) + p + q w           (x: incoming gradient, w: the tensor the forward
+//                   pass normalised; a, b, p, q per feature, params [4][nfeature]: the gradient of a batch normalisation
+//                   followed by max(., 0) with respect to its input)
+// The feature of volume z is z % nfeature.
+enum Prologue { PRO_NONE = 0, PRO_MASK = 1, PRO_BITS = 2, PRO_AFFINE_RELU = 3, PRO_BN_RELU_GRAD = 4 };
+struct Input {
+  const float* x;
+  const float* w = nullptr;
+  int kind = PRO_NONE;
+  const float* params = nullptr;
+  int nfeature = 1;
+  bool second_tensor() const { return kind == PRO_MASK || kind == PRO_BN_RELU_GRAD; }
+};
+__device__ __forceinline__ float affine_relu(float x, float a, float b) { return relu_f(fmaf(a, x, b)); }
+__device__ __forceinline__ float bn_relu_grad(float g, float w, float a, float b, float p, float q) {
+  return fmaf(q, w, p) + relu_pass(a * g, fmaf(a, w, b));
+}
+
 }  // namespace s2cnn

@@ -328,9 +328,9 @@ size_t round256(size_t n) { return (n + 255) & ~(size_t)255; }
 
 // Real signals on the 64^3 grid: per-volume kernel + the pass between its records and the spectral rows.
 // real_basis: the spectrum is stored in the real basis (one float per entry) instead of complex pairs.
-int fused_analysis(const float* x, const float* mask, bool mask_bits, const float* table, const float* packed_table, float* out,
+int fused_analysis(const s2cnn::Input& in, const float* table, const float* packed_table, float* out,
                    void* workspace, size_t workspace_bytes, int b_out, long nbatch, bool real_basis, hipStream_t st) {
-  if (!s2cnn::aligned16(x) || !s2cnn::aligned16(mask)) return S2CNN_EALIGN;
+  if (!s2cnn::aligned16(in.x) || !s2cnn::aligned16(in.w)) return S2CNN_EALIGN;
   const size_t need = round256(fused64::scratch_bytes(nbatch)) + fused64::PACKED_FLOATS * sizeof(float);
   if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
   float4* rec = static_cast<float4*>(workspace);
@@ -340,7 +340,7 @@ int fused_analysis(const float* x, const float* mask, bool mask_bits, const floa
     hipLaunchKernelGGL(fused64::pack_table, dim3(1024), dim3(256), 0, st, table, dst, s2cnn::so3_nspec(b_out), b_out);
     Tf = dst;
   }
-  fused64::launch_analysis(b_out, st, x, mask, mask_bits, Tf, rec, nbatch);
+  fused64::launch_analysis(b_out, st, in, Tf, rec, nbatch);
   if (real_basis)
     hipLaunchKernelGGL(fused64::spectrum_scatter_real, dim3((unsigned)((nbatch + fused64::ZR - 1) / fused64::ZR), fused64::active_rounds(b_out) * 32), dim3(256), 0, st,
                        rec, out, b_out, nbatch);
@@ -387,7 +387,7 @@ extern "C" int s2cnn_so3_analysis_real_basis(const float* x, const float* table,
   if (!x || !table || !out || !sizes_ok(b_in, b_out, nbatch)) return S2CNN_EINVAL;
   if (!fused_path(b_in, b_out, 0, false)) return S2CNN_EINVAL;
   if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
-  return fused_analysis(x, nullptr, false, table, packed_table, out, workspace, workspace_bytes, b_out, nbatch, true, static_cast<hipStream_t>(stream));
+  return fused_analysis(s2cnn::Input{x}, table, packed_table, out, workspace, workspace_bytes, b_out, nbatch, true, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int s2cnn_so3_synthesis_real_basis(const float* r, const float* table, const float* packed_table, float* out,
@@ -436,16 +436,29 @@ extern "C" size_t s2cnn_so3_synthesis_workspace(int b_in, int b_out, long nbatch
 }
 
 namespace {
-// mask: NULL, or (real signals only) a tensor of the shape of x whose positive entries select the samples that count
-int analysis_impl(const float* x, const float* mask, bool mask_bits, const float* table, const float* packed_table, float* out,
+// Where the loads of an analysis can do more than select samples (s2cnn::PRO_AFFINE_RELU, PRO_BN_RELU_GRAD): the per-volume
+// kernels of the 64^3 grid and the folded plane kernel of the other grids that fit the LDS.
+bool prologue_path(int b_in, int b_out) {
+  if (!sizes_ok(b_in, b_out, 1)) return false;
+  if (fused_path(b_in, b_out, 0, false)) return true;
+  return 2 * b_in != 64 && plane_real::plan_fwd(2 * b_in, b_in < b_out ? b_in : b_out, 2 * b_in).pl > 0;
+}
+
+// in: the signal and what its loads do to it (real signals only for anything but PRO_NONE)
+int analysis_impl(const s2cnn::Input& in, const float* table, const float* packed_table, float* out,
                   void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch, int complex_in, void* stream) {
-  if (!x || !table || !out || !sizes_ok(b_in, b_out, nbatch) || (mask && complex_in)) return S2CNN_EINVAL;
-  if (mask_bits && !(mask && fused_path(b_in, b_out, complex_in, false))) return S2CNN_EINVAL;
+  const float* x = in.x;
+  const float* mask = in.second_tensor() ? in.w : nullptr;
+  if (!x || !table || !out || !sizes_ok(b_in, b_out, nbatch) || (in.kind != s2cnn::PRO_NONE && complex_in)) return S2CNN_EINVAL;
+  if (in.kind != s2cnn::PRO_NONE && in.kind != s2cnn::PRO_AFFINE_RELU && !in.w) return S2CNN_EINVAL;
+  if (in.kind == s2cnn::PRO_BITS && !fused_path(b_in, b_out, complex_in, false)) return S2CNN_EINVAL;
+  if (in.kind >= s2cnn::PRO_AFFINE_RELU && (!in.params || in.nfeature < 1 || nbatch % in.nfeature != 0 || !prologue_path(b_in, b_out)))
+    return S2CNN_EINVAL;
   if (!s2cnn::aligned8(out) || (complex_in && !s2cnn::aligned8(x))) return S2CNN_EALIGN;
   if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (fused_path(b_in, b_out, complex_in, false))
-    return fused_analysis(x, mask, mask_bits, table, packed_table, out, workspace, workspace_bytes, b_out, nbatch, false, st);
+    return fused_analysis(in, table, packed_table, out, workspace, workspace_bytes, b_out, nbatch, false, st);
   const size_t need = s2cnn_so3_analysis_workspace(b_in, b_out, nbatch, complex_in);
   if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
   const int n2 = 2 * b_in, nb = b_in < b_out ? b_in : b_out;
@@ -467,7 +480,7 @@ int analysis_impl(const float* x, const float* mask, bool mask_bits, const float
   } else if (plan.pl > 0) {
     if (plan.lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)plane_real::plane_dft_fwd, hipFuncAttributeMaxDynamicSharedMemorySize, (int)plan.lds);
     hipLaunchKernelGGL(plane_real::plane_dft_fwd, dim3((planes + plan.pl - 1) / plan.pl), dim3(plan.nt), plan.lds, st, x, X, n2, nb,
-                       tiled ? wigner_tiled::ZT : 0, (long)planes, plan.pl, plan.alias, mask);
+                       tiled ? wigner_tiled::ZT : 0, (long)planes, plan.pl, plan.alias, mask, in.kind, in.params, in.nfeature);
   } else {
     if (lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)so3_plane_dft_fwd<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     hipLaunchKernelGGL(so3_plane_dft_fwd<false>, dim3(planes), dim3(256), lds, st, x, X, n2, nb, tiled ? wigner_tiled::ZT : 0, mask);
@@ -569,7 +582,7 @@ extern "C" int s2cnn_so3_analysis(const float* x, const float* table, const floa
                                   void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
                                   int complex_in, void* stream) {
   s2cnn::clear_stale_error();
-  return analysis_impl(x, nullptr, false, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, complex_in, stream);
+  return analysis_impl(s2cnn::Input{x}, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, complex_in, stream);
 }
 
 extern "C" int s2cnn_so3_synthesis(const float* xhat, const float* table, const float* packed_table, float* out,
@@ -600,15 +613,17 @@ int synthesis_relu_impl(const float* xhat, const float* table, const float* pack
                          bits, static_cast<hipStream_t>(stream));
 }
 
-int analysis_masked_impl(const float* x, const float* mask, bool mask_bits, const float* table, const float* packed_table, float* out,
-                         void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch, int real_basis, void* stream) {
-  if (!mask) return S2CNN_EINVAL;
+int analysis_prologue_impl(const s2cnn::Input& in, const float* table, const float* packed_table, float* out,
+                           void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch, int real_basis, void* stream) {
+  if (in.kind == s2cnn::PRO_NONE) return S2CNN_EINVAL;
   if (!real_basis)
-    return analysis_impl(x, mask, mask_bits, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, 0, stream);
-  if (!x || !table || !out || !sizes_ok(b_in, b_out, nbatch)) return S2CNN_EINVAL;
+    return analysis_impl(in, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, 0, stream);
+  if (!in.x || !table || !out || !sizes_ok(b_in, b_out, nbatch)) return S2CNN_EINVAL;
+  if (in.kind != s2cnn::PRO_AFFINE_RELU && !in.w) return S2CNN_EINVAL;
+  if (in.kind >= s2cnn::PRO_AFFINE_RELU && (!in.params || in.nfeature < 1 || nbatch % in.nfeature != 0)) return S2CNN_EINVAL;
   if (!fused_path(b_in, b_out, 0, false)) return S2CNN_EINVAL;
   if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
-  return fused_analysis(x, mask, mask_bits, table, packed_table, out, workspace, workspace_bytes, b_out, nbatch, true, static_cast<hipStream_t>(stream));
+  return fused_analysis(in, table, packed_table, out, workspace, workspace_bytes, b_out, nbatch, true, static_cast<hipStream_t>(stream));
 }
 }  // namespace
 
@@ -637,7 +652,8 @@ extern "C" int s2cnn_so3_analysis_real_masked(const float* x, const float* mask,
                                               float* out, void* workspace, size_t workspace_bytes, int b_in, int b_out,
                                               long nbatch, int real_basis, void* stream) {
   s2cnn::clear_stale_error();
-  return analysis_masked_impl(x, mask, false, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, real_basis, stream);
+  return analysis_prologue_impl(s2cnn::Input{x, mask, s2cnn::PRO_MASK}, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch,
+                                real_basis, stream);
 }
 
 extern "C" int s2cnn_so3_analysis_real_masked_bits(const float* x, const void* bits, const float* table, const float* packed_table,
@@ -645,8 +661,26 @@ extern "C" int s2cnn_so3_analysis_real_masked_bits(const float* x, const void* b
                                                    long nbatch, int real_basis, void* stream) {
   s2cnn::clear_stale_error();
   if (s2cnn_so3_relu_bits_bytes(b_in, nbatch) == 0) return S2CNN_EINVAL;
-  return analysis_masked_impl(x, static_cast<const float*>(bits), true, table, packed_table, out, workspace, workspace_bytes, b_in, b_out,
-                              nbatch, real_basis, stream);
+  return analysis_prologue_impl(s2cnn::Input{x, static_cast<const float*>(bits), s2cnn::PRO_BITS}, table, packed_table, out, workspace,
+                                workspace_bytes, b_in, b_out, nbatch, real_basis, stream);
+}
+
+extern "C" int s2cnn_so3_analysis_prologue_available(int b_in, int b_out) { return prologue_path(b_in, b_out) ? 1 : 0; }
+
+extern "C" int s2cnn_so3_analysis_real_affine_relu(const float* x, const float* params, int nfeature, const float* table,
+                                                   const float* packed_table, float* out, void* workspace, size_t workspace_bytes,
+                                                   int b_in, int b_out, long nbatch, int real_basis, void* stream) {
+  s2cnn::clear_stale_error();
+  return analysis_prologue_impl(s2cnn::Input{x, nullptr, s2cnn::PRO_AFFINE_RELU, params, nfeature}, table, packed_table, out, workspace,
+                                workspace_bytes, b_in, b_out, nbatch, real_basis, stream);
+}
+
+extern "C" int s2cnn_so3_analysis_real_bn_relu_grad(const float* g, const float* y, const float* params, int nfeature, const float* table,
+                                                    const float* packed_table, float* out, void* workspace, size_t workspace_bytes,
+                                                    int b_in, int b_out, long nbatch, int real_basis, void* stream) {
+  s2cnn::clear_stale_error();
+  return analysis_prologue_impl(s2cnn::Input{g, y, s2cnn::PRO_BN_RELU_GRAD, params, nfeature}, table, packed_table, out, workspace,
+                                workspace_bytes, b_in, b_out, nbatch, real_basis, stream);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -689,5 +723,5 @@ extern "C" int s2cnn_so3_analysis_static(const float* x, const float* table, con
   void* ws = nullptr;
   const int rc = static_scratch(&ws);
   if (rc) return rc;
-  return analysis_impl(x, nullptr, false, table, packed_table, out, ws, (size_t)S2CNN_STATIC_SCRATCH_BYTES, b_in, b_out, nbatch, complex_in, stream);
+  return analysis_impl(s2cnn::Input{x}, table, packed_table, out, ws, (size_t)S2CNN_STATIC_SCRATCH_BYTES, b_in, b_out, nbatch, complex_in, stream);
 }

@@ -204,14 +204,17 @@ __device__ constexpr int table_slot(int it) { return it & 3; }
 
 // NA: item rounds that carry degrees below the output bandwidth (items are ordered by degree group, so a truncated
 // spectrum leaves the later rounds without work: NA = 3 covers l < 24, 5 covers l < 28, 7 everything).
-// MASK: 0: the signal is x; 1: x where mask > 0 and zero elsewhere (mask: a tensor of the shape of x); 2: the same with
-// `mask` holding one BIT per sample instead (bits_index below), as the synthesis writes them.
+// MASK: what is done to x as it is loaded, one of s2cnn::Prologue: 0: nothing; 1: x where mask > 0 and zero elsewhere
+// (mask: a tensor of the shape of x); 2: the same with `mask` holding one BIT per sample instead (bits_index below), as
+// the synthesis writes them; 3: max(a x + b, 0); 4: a (a mask + b > 0 ? x : 0) + p + q mask, with a, b, p, q of the
+// volume's feature z % nfeature in params [.][nfeature].
 constexpr int BITS_WORDS = N * N;      // 64-bit words per volume: [beta][alpha % 8][alpha / 8], bit = gamma
 __host__ __device__ inline size_t bits_index(long z, int beta, int d) { return ((size_t)z * N + beta) * N + 8 * d; }   // + alpha / 8
 template <int NA, int MASK>
 __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restrict__ x, const float* __restrict__ mask,
-                                                           const float* __restrict__ Tf, float4* __restrict__ rec, long nbatch) {
-  constexpr bool MASKED = MASK == 1;
+                                                           const float* __restrict__ Tf, float4* __restrict__ rec, long nbatch,
+                                                           const float* __restrict__ params, int nfeature) {
+  constexpr bool MASKED = MASK == 1 || MASK == 4;      // a second tensor is loaded beside x
   using namespace fft64;
   __shared__ __attribute__((aligned(16))) float2 work[LDS_ELEMS];
   __shared__ __attribute__((aligned(16))) float2 quad[2][QUAD_ELEMS];
@@ -222,6 +225,13 @@ __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restri
   Twiddles twl;
   make_twiddles<false>(twl);
   for (int i = t; i < 2 * QUAD_ELEMS; i += THREADS) (&quad[0][0])[i] = make_float2(0.f, 0.f);   // places nobody writes (the -a half of a = 0) read as zero
+  float pr_a = 0.f, pr_b = 0.f, pr_p = 0.f, pr_q = 0.f;      // the feature's constants: the same for the whole workgroup
+  if constexpr (MASK >= 3) {
+    const int c = (int)(z % nfeature);
+    pr_a = params[c];
+    pr_b = params[nfeature + c];
+    if constexpr (MASK == 4) { pr_p = params[2 * nfeature + c]; pr_q = params[3 * nfeature + c]; }
+  }
 
   // quad address of the item (complex index), bit 31 = sign bit of (-1)^n
   unsigned adr[NIT];
@@ -289,7 +299,10 @@ __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restri
     float2 v[8];
 #pragma unroll
     for (int j1 = 0; j1 < 8; ++j1) {
-      if constexpr (MASKED) v[j1] = make_float2(s2cnn::relu_pass(pa[j1], ma[j1]), s2cnn::relu_pass(pb[j1], mb[j1]));
+      if constexpr (MASK == 1) v[j1] = make_float2(s2cnn::relu_pass(pa[j1], ma[j1]), s2cnn::relu_pass(pb[j1], mb[j1]));
+      else if constexpr (MASK == 3) v[j1] = make_float2(s2cnn::affine_relu(pa[j1], pr_a, pr_b), s2cnn::affine_relu(pb[j1], pr_a, pr_b));
+      else if constexpr (MASK == 4) v[j1] = make_float2(s2cnn::bn_relu_grad(pa[j1], ma[j1], pr_a, pr_b, pr_p, pr_q),
+                                                        s2cnn::bn_relu_grad(pb[j1], mb[j1], pr_a, pr_b, pr_p, pr_q));
       else if constexpr (MASK == 2) v[j1] = make_float2(__builtin_amdgcn_inverse_ballot_w64(ba[j1]) ? pa[j1] : 0.f,
                                                         __builtin_amdgcn_inverse_ballot_w64(bb[j1]) ? pb[j1] : 0.f);
       else v[j1] = make_float2(pa[j1], pb[j1]);
@@ -884,20 +897,23 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
 inline int active_rounds(int nl) { return nl <= 24 ? 3 : nl <= 28 ? 5 : NIT; }
 
 // Launchers: the instantiation whose item rounds cover the nl degrees present.
-template <int MASKED>
-inline void launch_analysis_m(int nl, hipStream_t st, const float* x, const float* mask, const float* Tf, float4* rec, long nbatch) {
+template <int MASK>
+inline void launch_analysis_m(int nl, hipStream_t st, const s2cnn::Input& in, const float* Tf, float4* rec, long nbatch) {
   const dim3 grid(grid_size(nbatch)), block(THREADS);
-  if (nl <= 24) hipLaunchKernelGGL((analysis_kernel<3, MASKED>), grid, block, 0, st, x, mask, Tf, rec, nbatch);
-  else if (nl <= 28) hipLaunchKernelGGL((analysis_kernel<5, MASKED>), grid, block, 0, st, x, mask, Tf, rec, nbatch);
-  else hipLaunchKernelGGL((analysis_kernel<7, MASKED>), grid, block, 0, st, x, mask, Tf, rec, nbatch);
+  if (nl <= 24) hipLaunchKernelGGL((analysis_kernel<3, MASK>), grid, block, 0, st, in.x, in.w, Tf, rec, nbatch, in.params, in.nfeature);
+  else if (nl <= 28) hipLaunchKernelGGL((analysis_kernel<5, MASK>), grid, block, 0, st, in.x, in.w, Tf, rec, nbatch, in.params, in.nfeature);
+  else hipLaunchKernelGGL((analysis_kernel<7, MASK>), grid, block, 0, st, in.x, in.w, Tf, rec, nbatch, in.params, in.nfeature);
 }
 
-// mask: NULL, or the tensor whose positive entries select the samples of x that count; mask_bits: `mask` holds one bit
-// per sample (BITS_WORDS 64-bit words per volume, written by the synthesis) instead of one float
-inline void launch_analysis(int nl, hipStream_t st, const float* x, const float* mask, bool mask_bits, const float* Tf, float4* rec, long nbatch) {
-  if (mask && mask_bits) launch_analysis_m<2>(nl, st, x, mask, Tf, rec, nbatch);
-  else if (mask) launch_analysis_m<1>(nl, st, x, mask, Tf, rec, nbatch);
-  else launch_analysis_m<0>(nl, st, x, nullptr, Tf, rec, nbatch);
+// in: the signal and what is done to it in the loads (s2cnn::Input)
+inline void launch_analysis(int nl, hipStream_t st, const s2cnn::Input& in, const float* Tf, float4* rec, long nbatch) {
+  switch (in.kind) {
+    case s2cnn::PRO_MASK: launch_analysis_m<1>(nl, st, in, Tf, rec, nbatch); break;
+    case s2cnn::PRO_BITS: launch_analysis_m<2>(nl, st, in, Tf, rec, nbatch); break;
+    case s2cnn::PRO_AFFINE_RELU: launch_analysis_m<3>(nl, st, in, Tf, rec, nbatch); break;
+    case s2cnn::PRO_BN_RELU_GRAD: launch_analysis_m<4>(nl, st, in, Tf, rec, nbatch); break;
+    default: launch_analysis_m<0>(nl, st, in, Tf, rec, nbatch);
+  }
 }
 
 // bits: NULL, or BITS_WORDS 64-bit words per volume that receive one bit per sample: the output is not <= 0

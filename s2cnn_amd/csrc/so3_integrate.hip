@@ -80,7 +80,76 @@ __global__ __launch_bounds__(256) void so3_integrate_grad_kernel(const float* __
   }
 }
 
+// Two sums per volume in one read, in a fixed order (bit-reproducible): what a batch normalisation over the volumes
+// of a feature needs of them.
+//   GRAD = false: out[z] = (sum x, sum x^2)
+//   GRAD = true : out[z] = (sum g m, sum g m y) with m = (a y + b > 0), a = params[z % F], b = params[F + z % F]
+template <bool GRAD>
+__global__ __launch_bounds__(256) void volume_moments_kernel(const float* __restrict__ x, const float* __restrict__ y,
+                                                             const float* __restrict__ params, int nfeature,
+                                                             float2* __restrict__ out, long n) {
+  __shared__ double part[2][256];
+  const long z = blockIdx.x;
+  const float* xs = x + z * n;
+  const float* ys = GRAD ? y + z * n : nullptr;
+  float a = 0.f, b = 0.f;
+  if constexpr (GRAD) { a = params[z % nfeature]; b = params[nfeature + z % nfeature]; }
+  auto term = [&](float xv, float yv, float& s1, float& s2) {
+    if constexpr (GRAD) {
+      const float gm = s2cnn::relu_pass(xv, fmaf(a, yv, b));
+      s1 += gm; s2 = fmaf(gm, yv, s2);
+    } else {
+      s1 += xv; s2 = fmaf(xv, xv, s2);
+    }
+  };
+  float s1[4] = {0.f, 0.f, 0.f, 0.f}, s2[4] = {0.f, 0.f, 0.f, 0.f};
+  const bool wide = n % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15u) == 0 && (!GRAD || (reinterpret_cast<uintptr_t>(y) & 15u) == 0);
+  if (wide) {
+    const float4* x4 = reinterpret_cast<const float4*>(xs);
+    const float4* y4 = reinterpret_cast<const float4*>(ys);
+    const long n4 = n / 4;
+    for (long i = threadIdx.x; i < n4; i += 256) {
+      const float4 xv = x4[i];
+      const float4 yv = GRAD ? y4[i] : xv;
+      term(xv.x, yv.x, s1[0], s2[0]); term(xv.y, yv.y, s1[1], s2[1]);
+      term(xv.z, yv.z, s1[2], s2[2]); term(xv.w, yv.w, s1[3], s2[3]);
+    }
+  } else {
+    for (long i = threadIdx.x; i < n; i += 256) term(xs[i], GRAD ? ys[i] : 0.f, s1[0], s2[0]);
+  }
+  part[0][threadIdx.x] = ((double)s1[0] + (double)s1[1]) + ((double)s1[2] + (double)s1[3]);
+  part[1][threadIdx.x] = ((double)s2[0] + (double)s2[1]) + ((double)s2[2] + (double)s2[3]);
+  __syncthreads();
+  for (int s = 128; s > 0; s >>= 1) {
+    if ((int)threadIdx.x < s) {
+      part[0][threadIdx.x] += part[0][threadIdx.x + s];
+      part[1][threadIdx.x] += part[1][threadIdx.x + s];
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) out[z] = make_float2((float)part[0][0], (float)part[1][0]);
+}
+
 }  // namespace
+
+extern "C" int s2cnn_volume_moments(const float* x, float* out, long nvol, long n, void* stream) {
+  s2cnn::clear_stale_error();
+  if (!x || !out || nvol < 1 || nvol >= (1L << 31) || n < 1) return S2CNN_EINVAL;
+  if (!s2cnn::aligned8(out)) return S2CNN_EALIGN;
+  hipLaunchKernelGGL(volume_moments_kernel<false>, dim3((unsigned)nvol), dim3(256), 0, static_cast<hipStream_t>(stream), x, nullptr, nullptr, 1,
+                     reinterpret_cast<float2*>(out), n);
+  return s2cnn::launch_status();
+}
+
+extern "C" int s2cnn_bn_relu_grad_moments(const float* g, const float* y, const float* params, int nfeature, float* out, long nvol, long n,
+                                          void* stream) {
+  s2cnn::clear_stale_error();
+  if (!g || !y || !params || !out || nfeature < 1 || nvol < 1 || nvol >= (1L << 31) || nvol % nfeature != 0 || n < 1) return S2CNN_EINVAL;
+  if (!s2cnn::aligned8(out)) return S2CNN_EALIGN;
+  hipLaunchKernelGGL(volume_moments_kernel<true>, dim3((unsigned)nvol), dim3(256), 0, static_cast<hipStream_t>(stream), g, y, params, nfeature,
+                     reinterpret_cast<float2*>(out), n);
+  return s2cnn::launch_status();
+}
 
 extern "C" int s2cnn_so3_integrate(const float* x, const float* w, float* out, int b, long n, void* stream) {
   s2cnn::clear_stale_error();

@@ -111,10 +111,13 @@ constexpr int LOADS = 8;   // global loads a thread has in flight while it stage
 // analysis: x [nplanes][n2][n2] -> X, laid out [plane][mi][ni] (ztile = 0) or
 // [z / Z][mi][beta][z % Z][ni] (ztile = Z, plane = z n2 + beta); mi = m + nb-1, ni = n.
 // ---------------------------------------------------------------------------------------------------
-// mask: NULL, or a tensor of the shape of x; samples of x where it is not positive count as zero
+// kind, mask, params, nfeature: what is done to x as it is loaded (s2cnn::Prologue; mask = the second tensor, if any;
+// kind 2, bit masks, is not supported here)
 __global__ __launch_bounds__(NT_MAX) void plane_dft_fwd(const float* __restrict__ x, float2* __restrict__ X, int n2, int nb,
-                                                        int ztile, long nplanes, int PL, int alias, const float* __restrict__ mask) {
+                                                        int ztile, long nplanes, int PL, int alias, const float* __restrict__ mask,
+                                                        int kind, const float* __restrict__ params, int nfeature) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
+  __shared__ float4 par[PL_MAX];                                      // (a, b, p, q) of the feature of each plane of the workgroup
   const int h = n2 / 2, nbp = pad(nb, 4), ns = pad(n2, 4);
   float2* tab = reinterpret_cast<float2*>(smem);                      // [h+1][nbp]
   float2* EO = tab + (h + 1) * nbp;                                   // [PL][h+1][ns]
@@ -126,6 +129,11 @@ __global__ __launch_bounds__(NT_MAX) void plane_dft_fwd(const float* __restrict_
     const int j = i / nbp, k = i - j * nbp;
     tab[i] = k < nb ? cs_entry(j, k, n2) : make_float2(0.f, 0.f);
   }
+  if (kind >= 3 && t < PL) {
+    const int c = (int)(((plane0 + t) / n2) % nfeature);
+    par[t] = make_float4(params[c], params[nfeature + c], kind == 4 ? params[2 * nfeature + c] : 0.f, kind == 4 ? params[3 * nfeature + c] : 0.f);
+  }
+  if (kind >= 3) __syncthreads();
   // fold gamma; rows go to slots so that the pair (a, n2-a) is adjacent: 0 -> 0, h -> 1, a -> 2a, n2-a -> 2a+1.
   // The planes of a workgroup are one contiguous run of rows; LOADS of them are issued before the first is used.
   {
@@ -135,12 +143,14 @@ __global__ __launch_bounds__(NT_MAX) void plane_dft_fwd(const float* __restrict_
     const float* msk = mask ? mask + (size_t)plane0 * n2 * n2 : nullptr;
     const float inv_n2 = 1.0f / (float)n2;
     // one copy of the loop per case, so that the batched loads of the plain case stay one run of loads
-    auto fold_rows = [&](auto masked) {
+    auto fold_rows = [&](auto kind_c) {
+      constexpr int KIND = decltype(kind_c)::value;
+      constexpr bool SECOND = KIND == 1 || KIND == 4;
       Walk2 wk;
       wk.init(t, NT, hg);
       for (int e = t; e < total; e += LOADS * NT) {
         float v1[LOADS], v2[LOADS], m1[LOADS], m2[LOADS];
-        int dst[LOADS];
+        int dst[LOADS], pln[LOADS];
         unsigned pmask = 0, vmask = 0;
 #pragma unroll
         for (int u = 0; u < LOADS; ++u) {
@@ -152,10 +162,11 @@ __global__ __launch_bounds__(NT_MAX) void plane_dft_fwd(const float* __restrict_
           const int o2 = valid && paired ? R * n2 + n2 - g : o1;
           v1[u] = src[o1];
           v2[u] = src[o2];
-          if constexpr (decltype(masked)::value) { m1[u] = msk[o1]; m2[u] = msk[o2]; }
+          if constexpr (SECOND) { m1[u] = msk[o1]; m2[u] = msk[o2]; }
           if (valid) vmask |= 1u << u;
           if (paired) pmask |= 1u << u;
           const int q = (int)(((float)R + 0.5f) * inv_n2), a = R - q * n2;
+          pln[u] = live ? q : 0;
           const int slot = a == 0 ? 0 : a == h ? 1 : a < h ? 2 * a : 2 * (n2 - a) + 1;
           dst[u] = live ? (q * hg + g) * ns + slot : -1;
           wk.step();
@@ -163,7 +174,15 @@ __global__ __launch_bounds__(NT_MAX) void plane_dft_fwd(const float* __restrict_
 #pragma unroll
         for (int u = 0; u < LOADS; ++u) {
           float a = v1[u], b = v2[u];
-          if constexpr (decltype(masked)::value) { a = s2cnn::relu_pass(a, m1[u]); b = s2cnn::relu_pass(b, m2[u]); }
+          if constexpr (KIND == 1) { a = s2cnn::relu_pass(a, m1[u]); b = s2cnn::relu_pass(b, m2[u]); }
+          if constexpr (KIND == 3) {
+            const float4 c = par[pln[u]];
+            a = s2cnn::affine_relu(a, c.x, c.y); b = s2cnn::affine_relu(b, c.x, c.y);
+          }
+          if constexpr (KIND == 4) {
+            const float4 c = par[pln[u]];
+            a = s2cnn::bn_relu_grad(a, m1[u], c.x, c.y, c.z, c.w); b = s2cnn::bn_relu_grad(b, m2[u], c.x, c.y, c.z, c.w);
+          }
           if (!((vmask >> u) & 1u)) a = b = 0.f;
           const bool paired = (pmask >> u) & 1u;
           if (!paired) b = 0.f;
@@ -171,8 +190,10 @@ __global__ __launch_bounds__(NT_MAX) void plane_dft_fwd(const float* __restrict_
         }
       }
     };
-    if (msk) fold_rows(std::true_type{});
-    else fold_rows(std::false_type{});
+    if (kind == 1) fold_rows(std::integral_constant<int, 1>{});
+    else if (kind == 3) fold_rows(std::integral_constant<int, 3>{});
+    else if (kind == 4) fold_rows(std::integral_constant<int, 4>{});
+    else fold_rows(std::integral_constant<int, 0>{});
     if (ns > n2)   // n2 = 2 mod 4: two empty slots
       for (int i = t; i < PL * hg * (ns - n2); i += NT) EO[(i / (ns - n2)) * ns + n2 + i % (ns - n2)] = make_float2(0.f, 0.f);
   }

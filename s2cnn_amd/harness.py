@@ -19,6 +19,7 @@ import torch
 import torch.nn.functional as F
 from torch import nn
 
+from .soft.bn_relu import run_sequence
 from . import (S2Convolution, SO3Convolution, s2_equatorial_grid, s2_near_identity_grid, so3_equatorial_grid, so3_integrate,
                so3_near_identity_grid)
 
@@ -66,33 +67,36 @@ def _shrec17_sequence(features, bandwidths):
 
 
 class Shrec17Model(nn.Module):
-    """examples/shrec17/model.py:7-48."""
+    """examples/shrec17/model.py:7-48.  fused_norm: the BatchNorm3d + ReLU pairs between two layers are evaluated inside
+    the layers' transforms (s2cnn_amd/soft/bn_relu.py): same modules, parameters and buffers, same function."""
 
-    def __init__(self, nclasses):
+    def __init__(self, nclasses, fused_norm=False):
         super().__init__()
+        self.fused_norm = fused_norm
         self.features = [6, 100, 100, nclasses]
         self.bandwidths = [64, 16, 10]
         self.sequential = _shrec17_sequence(self.features, self.bandwidths)
         self.out_layer = nn.Linear(self.features[-2], self.features[-1])
 
     def forward(self, x):  # pylint: disable=W0221
-        x = self.sequential(x)      # [batch, feature, beta, alpha, gamma]
+        x = run_sequence(self.sequential, x) if self.fused_norm else self.sequential(x)      # [batch, feature, beta, alpha, gamma]
         x = so3_integrate(x)        # [batch, feature]
         return F.log_softmax(self.out_layer(x), dim=1)
 
 
 class Shrec17ModelOriginal(nn.Module):
-    """examples/shrec17/model_original.py:7-50."""
+    """examples/shrec17/model_original.py:7-50.  fused_norm: as in Shrec17Model."""
 
-    def __init__(self, nclasses):
+    def __init__(self, nclasses, fused_norm=False):
         super().__init__()
+        self.fused_norm = fused_norm
         self.features = [6, 50, 70, 350, nclasses]
         self.bandwidths = [128, 32, 22, 7]
         self.sequential = _shrec17_sequence(self.features, self.bandwidths)
         self.out_layer = nn.Sequential(nn.BatchNorm1d(self.features[-2], affine=False), nn.Linear(self.features[-2], self.features[-1]))
 
     def forward(self, x):  # pylint: disable=W0221
-        x = self.sequential(x)
+        x = run_sequence(self.sequential, x) if self.fused_norm else self.sequential(x)
         x = x.view(x.size(0), x.size(1), -1).max(-1)[0]
         return F.log_softmax(self.out_layer(x), dim=1)
 

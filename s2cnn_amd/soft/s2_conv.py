@@ -20,11 +20,21 @@ class S2Convolution(SpectralConvolution):
     def forward(self, x):  # pylint: disable=W
         """[batch, feature_in, beta, alpha] -> [batch, feature_out, beta, alpha, gamma]"""
         self.check_input(x, 2)
-        xh = S2_fft_real.apply(x, self.b_out)                                  # [l m, batch, feature_in, complex]
         if self.real_basis:
-            yh = s2_rft_real(self.scaled_kernel(), self.b_out, self.grid)      # [l m, feature_in, feature_out]
-            zh = s2_mm_real(s2_spectrum_to_real(xh), yh)                       # [l m n, batch, feature_out]
-            return SO3_ifft_real_basis.apply(zh, None, self.bias, self.fused_relu)   # bias added inside the transform
+            return self.from_spectrum(self.product_spectrum(x))
+        xh = S2_fft_real.apply(x, self.b_out)                                  # [l m, batch, feature_in, complex]
         yh = s2_rft(self.scaled_kernel(), self.b_out, self.grid)               # [l m, feature_in, feature_out, complex]
         zh = s2_mm(xh, yh)                                                     # [l m n, batch, feature_out, complex]
         return SO3_ifft_real.apply(zh, None, self.bias, self.fused_relu)
+
+    # The two halves of the real-basis forward pass (see SO3Convolution.product_spectrum).
+    def product_spectrum(self, x, xh=None):
+        """[l m n, batch, feature_out] in the real basis, from the input x (xh: its complex S^2 spectrum, if at hand)."""
+        if xh is None:
+            self.check_input(x, 2)
+            xh = S2_fft_real.apply(x, self.b_out)                              # [l m, batch, feature_in, complex]
+        yh = s2_rft_real(self.scaled_kernel(), self.b_out, self.grid)          # [l m, feature_in, feature_out]
+        return s2_mm_real(s2_spectrum_to_real(xh), yh)                         # [l m n, batch, feature_out]
+
+    def from_spectrum(self, zh):
+        return SO3_ifft_real_basis.apply(zh, None, self.bias, self.fused_relu)  # bias added inside the transform

@@ -22,12 +22,24 @@ class SO3Convolution(SpectralConvolution):
         """[batch, feature_in, beta, alpha, gamma] -> [batch, feature_out, beta, alpha, gamma]"""
         self.check_input(x, 3)
         if self.real_basis:
-            xh = SO3_fft_real_basis.apply(x, self.b_out)                       # [l m n, batch, feature_in]
-            yh = so3_rft_real(self.scaled_kernel(), self.b_out, self.grid)     # [l m n, feature_in, feature_out]
-            return SO3_ifft_real_basis.apply(so3_mm_real(xh, yh), None, self.bias, self.fused_relu)   # bias added inside the transform
+            return self.from_spectrum(self.product_spectrum(x))
         xh = SO3_fft_real.apply(x, self.b_out)                                 # [l m n, batch, feature_in, complex]
         yh = so3_rft(self.scaled_kernel(), self.b_out, self.grid)              # [l m n, feature_in, feature_out, complex]
         return SO3_ifft_real.apply(so3_mm(xh, yh), None, self.bias, self.fused_relu)
+
+
+    # The two halves of the real-basis forward pass, for callers that put something else between the layers' transforms
+    # (s2cnn_amd/soft/bn_relu.py): the spectrum of the output before the last transform, and that transform.
+    def product_spectrum(self, x, xh=None):
+        """[l m n, batch, feature_out] in the real basis, from the input x or from its spectrum xh [l m n, batch, feature_in]."""
+        if xh is None:
+            self.check_input(x, 3)
+            xh = SO3_fft_real_basis.apply(x, self.b_out)                       # [l m n, batch, feature_in]
+        yh = so3_rft_real(self.scaled_kernel(), self.b_out, self.grid)         # [l m n, feature_in, feature_out]
+        return so3_mm_real(xh, yh)
+
+    def from_spectrum(self, zh):
+        return SO3_ifft_real_basis.apply(zh, None, self.bias, self.fused_relu)  # bias added inside the transform
 
 
 class SO3Shortcut(nn.Module):

@@ -57,6 +57,50 @@ def _same_shape_operand(mask, x):
     return mask.clone() if mask.data_ptr() % 16 else mask
 
 
+class LoadAffineReLU:
+    """Passed as `mask` to the real analyses: the signal that is transformed is max(a x + b, 0), a = params[0][z % F],
+    b = params[1][z % F] for volume z (params: float32 [2, F] on the device of x)."""
+
+    def __init__(self, params):
+        _hip.require_gpu_f32(params)
+        assert params.dim() == 2 and params.size(0) == 2
+        self.params = params.contiguous()
+
+
+class LoadBNReLUGrad:
+    """Passed as `mask` to the real analyses of a gradient g: the signal that is transformed is
+    a (a y + b > 0 ? g : 0) + p + q y, with a, b, p, q = params[0..3][z % F] (float32 [4, F]) and y of the shape of g:
+    the gradient of max(batch_norm(y), 0) with respect to y."""
+
+    def __init__(self, y, params):
+        _hip.require_gpu_f32(params)
+        assert params.dim() == 2 and params.size(0) == 4
+        self.y, self.params = y, params.contiguous()
+
+
+def analysis_prologue_available(b_in, b_out):
+    """Whether the real analysis b_in -> b_out can apply LoadAffineReLU / LoadBNReLUGrad in its loads."""
+    return bool(_hip.lib().s2cnn_so3_analysis_prologue_available(b_in, b_out))
+
+
+def _analysis_with_loads(x, mask, table, packed, out, ws, b_in, b_out, nbatch, real_basis):
+    """The analysis of x with what `mask` asks for done in its loads."""
+    tail = (_hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out), _hip.ptr(ws), ws.numel(), b_in, b_out, nbatch, real_basis, _hip.stream_ptr())
+    if isinstance(mask, LoadAffineReLU):
+        assert nbatch % mask.params.size(1) == 0
+        _hip.call("s2cnn_so3_analysis_real_affine_relu", _hip.ptr(x), _hip.ptr(mask.params), mask.params.size(1), *tail)
+    elif isinstance(mask, LoadBNReLUGrad):
+        assert nbatch % mask.params.size(1) == 0
+        y = _same_shape_operand(mask.y, x)
+        _hip.call("s2cnn_so3_analysis_real_bn_relu_grad", _hip.ptr(x), _hip.ptr(y), _hip.ptr(mask.params), mask.params.size(1), *tail)
+    elif _is_bit_mask(mask):
+        _hip.call("s2cnn_so3_analysis_real_masked_bits", _hip.ptr(x), _hip.ptr(mask), *tail)
+    else:
+        mask = _same_shape_operand(mask, x)
+        _hip.call("s2cnn_so3_analysis_real_masked", _hip.ptr(x), _hip.ptr(mask), *tail)
+    return out
+
+
 def _is_bit_mask(mask):
     """A mask of one bit per sample, as `_relu_bits` allocates it and the transforms with relu=True fill it."""
     return mask is not None and mask.dtype == torch.int64
@@ -93,15 +137,8 @@ def _analysis(x, b_in, b_out, batch_size, for_grad, complex_in, mask=None):
     if nbatch == 0:
         return out
     ws = _hip.workspace(L.s2cnn_so3_analysis_workspace(b_in, b_out, nbatch, complex_in), x.device)
-    if _is_bit_mask(mask):
-        _hip.call("s2cnn_so3_analysis_real_masked_bits", _hip.ptr(x), _hip.ptr(mask), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out),
-                  _hip.ptr(ws), ws.numel(), b_in, b_out, nbatch, 0, _hip.stream_ptr())
-        return out
     if mask is not None:
-        mask = _same_shape_operand(mask, x)
-        _hip.call("s2cnn_so3_analysis_real_masked", _hip.ptr(x), _hip.ptr(mask), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out),
-                  _hip.ptr(ws), ws.numel(), b_in, b_out, nbatch, 0, _hip.stream_ptr())
-        return out
+        return _analysis_with_loads(x, mask, table, packed, out, ws, b_in, b_out, nbatch, 0)
     _hip.call("s2cnn_so3_analysis", _hip.ptr(x), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out), _hip.ptr(ws), ws.numel(),
                   b_in, b_out, nbatch, complex_in, _hip.stream_ptr())
     return out
@@ -300,15 +337,8 @@ def so3_rfft_real_basis(x, for_grad=False, b_out=None, mask=None):
     if nbatch == 0:
         return out
     ws = _hip.workspace(L.s2cnn_so3_analysis_workspace(b_in, b_out, nbatch, 0), x.device)
-    if _is_bit_mask(mask):
-        _hip.call("s2cnn_so3_analysis_real_masked_bits", _hip.ptr(x), _hip.ptr(mask), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out),
-                  _hip.ptr(ws), ws.numel(), b_in, b_out, nbatch, 1, _hip.stream_ptr())
-        return out
     if mask is not None:
-        mask = _same_shape_operand(mask, x)
-        _hip.call("s2cnn_so3_analysis_real_masked", _hip.ptr(x), _hip.ptr(mask), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out),
-                  _hip.ptr(ws), ws.numel(), b_in, b_out, nbatch, 1, _hip.stream_ptr())
-        return out
+        return _analysis_with_loads(x, mask, table, packed, out, ws, b_in, b_out, nbatch, 1)
     _hip.call("s2cnn_so3_analysis_real_basis", _hip.ptr(x), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out), _hip.ptr(ws),
               ws.numel(), b_in, b_out, nbatch, _hip.stream_ptr())
     return out

@@ -1,0 +1,171 @@
+"""Batch normalisation + ReLU between two layers evaluated inside the layers' transforms (s2cnn_amd/soft/bn_relu.py)
+against the modules they replace: nn.BatchNorm3d and nn.ReLU of torch between this package's layers, as the reference's
+shape networks are written (examples/shrec17/model.py:17-38).  The pieces through the C ABI first: the two sums per
+volume, the analysis that applies max(a y + b, 0) in its loads and the one that forms the gradient of the pair in its
+loads, each against the same arithmetic as torch tensor expressions followed by the plain analysis."""
+import pytest
+import torch
+from torch import nn
+
+import s2cnn_amd
+from s2cnn_amd import harness
+from s2cnn_amd.soft import bn_relu
+from s2cnn_amd.soft import so3_fft as P
+
+pytestmark = pytest.mark.gpu
+
+PAIRS = [(32, 32), (32, 22), (22, 22), (22, 7), (16, 10), (10, 6), (6, 6), (7, 7), (3, 3)]
+
+
+def _rel(got, want):
+    return (got - want).abs().max().item() / max(want.abs().max().item(), 1e-30)
+
+
+def test_volume_moments(hip):
+    g = torch.Generator().manual_seed(1)
+    for n2, nvol in ((64, 6), (44, 4), (14, 9), (6, 5)):
+        x = (torch.randn(nvol, n2, n2, n2, generator=g) + 0.5).cuda()
+        got = bn_relu._moments("s2cnn_volume_moments", n2 ** 3, x).double()
+        want = torch.stack([x.double().sum((1, 2, 3)), (x.double() ** 2).sum((1, 2, 3))], 1)
+        assert _rel(got, want) < 2e-6, n2
+        # the sums of the backward pass: sum g m and sum g m y with m = (a y + b > 0), feature = volume % 3
+        y = torch.randn(nvol // 3 * 3, n2, n2, n2, generator=g).cuda()
+        gr = torch.randn(y.shape, generator=g).cuda()
+        ab = torch.tensor([[0.7, -1.3, 2.0], [0.1, 0.4, -0.5]]).cuda()
+        a = ab[0].repeat(y.size(0) // 3).view(-1, 1, 1, 1)
+        b = ab[1].repeat(y.size(0) // 3).view(-1, 1, 1, 1)
+        m = (a * y + b > 0)
+        got = bn_relu._moments("s2cnn_bn_relu_grad_moments", n2 ** 3, gr, y, ab, 3).double()
+        gm = (gr * m).double()
+        want = torch.stack([gm.sum((1, 2, 3)), (gm * y.double()).sum((1, 2, 3))], 1)
+        assert (got - want).abs().max().item() < 2e-5 * want.abs().max().item(), n2    # a sample at the threshold may fall either way
+
+
+@pytest.mark.parametrize("b_in,b_out", PAIRS)
+def test_analysis_with_the_normalisation_in_its_loads(hip, b_in, b_out):
+    """max(a y + b, 0) and a (a y + b > 0 ? g : 0) + p + q y formed by the loads of the analysis against the same
+    functions as tensor expressions followed by the plain analysis; complex and real-basis spectra, both tables."""
+    assert P.analysis_prologue_available(b_in, b_out)
+    print(f"normalisation in the loads b_in={b_in} b_out={b_out}", flush=True)
+    nb, nf = 2, 3
+    g = torch.Generator().manual_seed(100 * b_in + b_out)
+    y = torch.randn(nb, nf, 2 * b_in, 2 * b_in, 2 * b_in, generator=g).cuda()
+    gr = torch.randn(y.shape, generator=g).cuda()
+    par = torch.tensor([[0.7, -1.3, 2.0], [0.1, 0.4, -0.5], [0.02, -0.01, 0.03], [-0.05, 0.04, 0.01]]).cuda()
+    a, b, p, q = (par[i].view(1, nf, 1, 1, 1) for i in range(4))
+    u = torch.relu(a * y + b)
+    v = a * gr * (a * y + b > 0) + p + q * y
+    for for_grad in (False, True):
+        for ana in (P.so3_rfft, P.so3_rfft_real_basis):
+            want = ana(u, for_grad=for_grad, b_out=b_out)
+            got = ana(y, for_grad=for_grad, b_out=b_out, mask=P.LoadAffineReLU(par[:2].contiguous()))
+            assert _rel(got, want) < 2e-5, ("affine relu", for_grad, ana.__name__, _rel(got, want))
+            want = ana(v, for_grad=for_grad, b_out=b_out)
+            got = ana(gr, for_grad=for_grad, b_out=b_out, mask=P.LoadBNReLUGrad(y, par))
+            assert _rel(got, want) < 2e-5, ("bn relu grad", for_grad, ana.__name__, _rel(got, want))
+
+
+class _Norm64(nn.Module):
+    """nn.BatchNorm3d evaluated in float64 on float32 activations: the checker's normalisation (the float32 kernels of
+    the library behind torch's module lose digits of the statistics at 10^6 samples per feature)."""
+
+    def __init__(self, n):
+        super().__init__()
+        self.bn = nn.BatchNorm3d(n, dtype=torch.float64)
+        self.weight, self.bias = self.bn.weight, self.bn.bias
+
+    def forward(self, x):  # pylint: disable=W0221
+        return self.bn(x.double()).float()
+
+
+def _as_checker(seq):
+    """The same sequence with every BatchNorm3d replaced by its float64 twin (same parameters and buffers)."""
+    mods = []
+    for m in seq:
+        if isinstance(m, nn.BatchNorm3d):
+            twin = _Norm64(m.num_features).to(m.weight.device)
+            twin.bn.load_state_dict({k: (v.double() if v.is_floating_point() else v) for k, v in m.state_dict().items()})
+            mods.append(twin)
+        else:
+            mods.append(m)
+    return nn.Sequential(*mods)
+
+
+def _sequence(sizes, feats, seed):
+    """S2Conv, then (BatchNorm3d, ReLU, SO3Conv) per further bandwidth, then BatchNorm3d, ReLU: the reference's pattern."""
+    torch.manual_seed(seed)
+    mods = [s2cnn_amd.S2Convolution(feats[0], feats[1], sizes[0], sizes[1], s2cnn_amd.s2_near_identity_grid())]
+    for i in range(1, len(sizes) - 1):
+        mods += [nn.BatchNorm3d(feats[i]), nn.ReLU(),
+                 s2cnn_amd.SO3Convolution(feats[i], feats[i + 1], sizes[i], sizes[i + 1], s2cnn_amd.so3_near_identity_grid())]
+    mods += [nn.BatchNorm3d(feats[-1]), nn.ReLU()]
+    seq = nn.Sequential(*mods)
+    with torch.no_grad():
+        for m in seq:
+            if isinstance(m, nn.BatchNorm3d):
+                m.weight.uniform_(0.5, 1.5)
+                m.bias.normal_(0, 0.3)
+            elif hasattr(m, "kernel"):
+                m.bias.normal_(0, 0.3)
+    return seq
+
+
+@pytest.mark.parametrize("sizes,feats", [((12, 8, 6, 4), (2, 4, 5, 3)),          # small grids: folded plane kernels
+                                         ((40, 32, 22, 7), (2, 3, 4, 3))])       # 64^3 and 44^3: per-volume kernels, truncated spectra
+def test_sequence_with_fused_normalisation(hip, sizes, feats):
+    import copy
+    fus = _sequence(sizes, feats, 5).cuda()
+    ref = _as_checker(copy.deepcopy(fus))
+    # One sample of 10^6 whose normalised value lies within rounding of the threshold of the ReLU may pass in one
+    # evaluation and not in the other, which moves a spectral gradient by 10^-3 of its size: the comparison is made on an
+    # input for which the checker sees no such sample (three evaluations: two training steps and one in evaluation mode).
+    closest = []
+    hooks = [m.register_forward_hook(lambda _m, _i, out: closest.append(out.abs().min().item())) for m in ref if isinstance(m, _Norm64)]
+    for seed in range(6, 36):
+        x = torch.randn(3, feats[0], 2 * sizes[0], 2 * sizes[0], generator=torch.Generator().manual_seed(seed)).cuda()
+        probe = copy.deepcopy(ref)
+        phooks = [m.register_forward_hook(lambda _m, _i, out: closest.append(out.abs().min().item())) for m in probe if isinstance(m, _Norm64)]
+        del closest[:]
+        with torch.no_grad():
+            probe.train(); probe(x); probe(x); probe.eval(); probe(x)
+        if min(closest) > 5e-7:                 # the two evaluations of a normalised value differ by 1.5e-7 at most
+            break
+    else:
+        pytest.skip("no input without a sample at the threshold among thirty seeds")
+    for h in hooks + phooks:
+        h.remove()
+    print(f"input seed {seed}: closest normalised value to the threshold {min(closest):.1e}", flush=True)
+    for mode in ("train", "train", "eval"):                 # two training steps (running averages move twice), then evaluation
+        ref.train(mode == "train")
+        fus.train(mode == "train")
+        xa, xb = x.clone().requires_grad_(), x.clone().requires_grad_()
+        ya, yb = ref(xa), bn_relu.run_sequence(fus, xb)
+        assert _rel(yb, ya) < 1e-4, (mode, _rel(yb, ya))
+        w = torch.randn(ya.shape, generator=torch.Generator().manual_seed(7)).cuda()
+        for net in (ref, fus):
+            net.zero_grad(set_to_none=True)
+        (ya * w).sum().backward()
+        (yb * w).sum().backward()
+        assert _rel(xb.grad, xa.grad) < 2e-4, (mode, "input", _rel(xb.grad, xa.grad))
+        # a bias in front of a normalisation with batch statistics has gradient zero (rounding noise on either side):
+        # differences are measured against the largest gradient of the network where a parameter's own is smaller
+        scale = max(q.grad.abs().max().item() for q in ref.parameters())
+        for (name, pa), (_, pb) in zip(ref.named_parameters(), fus.named_parameters()):
+            err = (pb.grad - pa.grad.float()).abs().max().item() / max(pa.grad.abs().max().item(), 0.1 * scale)
+            assert err < 2e-4, (mode, name, err)
+        for (name, ba), (_, bb) in zip(ref.named_buffers(), fus.named_buffers()):
+            assert _rel(bb.double(), ba.double()) < 1e-5, (mode, name)
+        print(f"{sizes} {mode}: output {_rel(yb, ya):.1e}, input gradient {_rel(xb.grad, xa.grad):.1e}", flush=True)
+
+
+def test_shape_network_with_fused_normalisation(hip):
+    """The SHREC17 network of the harness with the normalisations inside the transforms: the same losses over training
+    steps as the plain module sequence, from the same initial weights."""
+    torch.manual_seed(0)
+    plain = harness.Shrec17Model(55)
+    torch.manual_seed(0)
+    fused = harness.Shrec17Model(55, fused_norm=True)
+    _, la, _ = harness.train_steps("shrec17", batch=4, steps=4, warmup=0, lr=0.02, model=plain)
+    _, lb, _ = harness.train_steps("shrec17", batch=4, steps=4, warmup=0, lr=0.02, model=fused)
+    print("plain", ["%.5f" % l for l in la], "fused", ["%.5f" % l for l in lb], flush=True)
+    assert max(abs(a - b) for a, b in zip(la, lb)) < 2e-4 * abs(la[0])
