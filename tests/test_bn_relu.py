@@ -69,10 +69,9 @@ class _Norm64(nn.Module):
     """nn.BatchNorm3d evaluated in float64 on float32 activations: the checker's normalisation (the float32 kernels of
     the library behind torch's module lose digits of the statistics at 10^6 samples per feature)."""
 
-    def __init__(self, n):
+    def __init__(self, n, **kwargs):
         super().__init__()
-        self.bn = nn.BatchNorm3d(n, dtype=torch.float64)
-        self.weight, self.bias = self.bn.weight, self.bn.bias
+        self.bn = nn.BatchNorm3d(n, dtype=torch.float64, **kwargs)
 
     def forward(self, x):  # pylint: disable=W0221
         return self.bn(x.double()).float()
@@ -83,7 +82,7 @@ def _as_checker(seq):
     mods = []
     for m in seq:
         if isinstance(m, nn.BatchNorm3d):
-            twin = _Norm64(m.num_features).to(m.weight.device)
+            twin = _Norm64(m.num_features, affine=m.affine, momentum=m.momentum, eps=m.eps, track_running_stats=m.track_running_stats).cuda()
             twin.bn.load_state_dict({k: (v.double() if v.is_floating_point() else v) for k, v in m.state_dict().items()})
             mods.append(twin)
         else:
@@ -91,18 +90,18 @@ def _as_checker(seq):
     return nn.Sequential(*mods)
 
 
-def _sequence(sizes, feats, seed):
+def _sequence(sizes, feats, seed, **bn_kwargs):
     """S2Conv, then (BatchNorm3d, ReLU, SO3Conv) per further bandwidth, then BatchNorm3d, ReLU: the reference's pattern."""
     torch.manual_seed(seed)
     mods = [s2cnn_amd.S2Convolution(feats[0], feats[1], sizes[0], sizes[1], s2cnn_amd.s2_near_identity_grid())]
     for i in range(1, len(sizes) - 1):
-        mods += [nn.BatchNorm3d(feats[i]), nn.ReLU(),
+        mods += [nn.BatchNorm3d(feats[i], **bn_kwargs), nn.ReLU(),
                  s2cnn_amd.SO3Convolution(feats[i], feats[i + 1], sizes[i], sizes[i + 1], s2cnn_amd.so3_near_identity_grid())]
-    mods += [nn.BatchNorm3d(feats[-1]), nn.ReLU()]
+    mods += [nn.BatchNorm3d(feats[-1], **bn_kwargs), nn.ReLU()]
     seq = nn.Sequential(*mods)
     with torch.no_grad():
         for m in seq:
-            if isinstance(m, nn.BatchNorm3d):
+            if isinstance(m, nn.BatchNorm3d) and m.affine:
                 m.weight.uniform_(0.5, 1.5)
                 m.bias.normal_(0, 0.3)
             elif hasattr(m, "kernel"):
@@ -110,11 +109,14 @@ def _sequence(sizes, feats, seed):
     return seq
 
 
-@pytest.mark.parametrize("sizes,feats", [((12, 8, 6, 4), (2, 4, 5, 3)),          # small grids: folded plane kernels
-                                         ((40, 32, 22, 7), (2, 3, 4, 3))])       # 64^3 and 44^3: per-volume kernels, truncated spectra
-def test_sequence_with_fused_normalisation(hip, sizes, feats):
+@pytest.mark.parametrize("sizes,feats,bn_kwargs", [
+    ((12, 8, 6, 4), (2, 4, 5, 3), {}),                                       # small grids: folded plane kernels
+    ((40, 32, 22, 7), (2, 3, 4, 3), {}),                                     # 64^3 and 44^3: per-volume kernels, truncated spectra
+    ((12, 8, 6, 4), (2, 4, 5, 3), {"affine": False, "momentum": None}),      # no weights, cumulative running averages
+    ((10, 8, 6), (2, 4, 5), {"track_running_stats": False})])                # batch statistics in evaluation mode as well
+def test_sequence_with_fused_normalisation(hip, sizes, feats, bn_kwargs):
     import copy
-    fus = _sequence(sizes, feats, 5).cuda()
+    fus = _sequence(sizes, feats, 5, **bn_kwargs).cuda()
     ref = _as_checker(copy.deepcopy(fus))
     # One sample of 10^6 whose normalised value lies within rounding of the threshold of the ReLU may pass in one
     # evaluation and not in the other, which moves a spectral gradient by 10^-3 of its size: the comparison is made on an
