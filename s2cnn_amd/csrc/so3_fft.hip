@@ -545,8 +545,12 @@ int synthesis_impl(const float* xhat, const float* table, const float* packed_ta
       hipLaunchKernelGGL(wigner_tiled::pack_table_synthesis, dim3(2048), dim3(256), 0, st, table, dst, n2, nb, b_in);
       Tq = dst;
     }
-    hipLaunchKernelGGL(wigner_tiled::wigner_inv_tiled, dim3(wigner_tiled::grid_size(MW, nbatch), wigner_tiled::parts_synthesis(n2, nb)),
-                       dim3(512), 0, st, xh, Tq, S, n2, nb, b_in, nbatch);
+    if (wigner_tiled::small_synthesis(n2, nb))
+      hipLaunchKernelGGL((wigner_tiled::wigner_inv_tiled<16, 32>), dim3(wigner_tiled::grid_size(MW, nbatch)), dim3(512), 0, st, xh, Tq, S, n2, nb,
+                         b_in, nbatch);
+    else
+      hipLaunchKernelGGL((wigner_tiled::wigner_inv_tiled<32, 64>), dim3(wigner_tiled::grid_size(MW, nbatch), wigner_tiled::parts_synthesis(n2, nb)),
+                         dim3(512), 0, st, xh, Tq, S, n2, nb, b_in, nbatch);
   } else if (complex_out) {
     hipLaunchKernelGGL(so3_wigner_inv<true>, grid, dim3(16, 16), 0, st, xh, table, S, n2, nb, b_in, nbatch);
   } else {

@@ -8,7 +8,7 @@
 //
 // The table is consumed in a packed, zero-padded order that makes every chunk one contiguous block:
 //   analysis : Tp[part][mi][beta][n (32)][l (32)]        (pack_table_analysis)
-//   synthesis: Tq[part][mi][l (nb)][n (32)][beta (64)]   (pack_table_synthesis)
+//   synthesis: Tq[part][mi][l (nb)][n (32)][beta (64)]   (pack_table_synthesis; [n (16)][beta (32)] for small grids)
 // with zeros outside max(|m|, n) <= l < number of degrees, n < nb, beta < 2 b_grid.
 // A workgroup covers 32 values of n and 32 degrees (analysis) or 64 betas (synthesis); larger problems are cut
 // into parts, one more grid dimension: analysis (l0, n0) = (0,0), (32,0), (32,32) (n <= l), synthesis
@@ -50,6 +50,9 @@ inline int grid_size(int MW, long nbatch) {
 // parts of the analysis: degrees [l0, l0 + 32) x frequencies n in [n0, n0 + 32)
 __host__ __device__ inline int parts_analysis(int nb, int nl) { return nl <= 32 ? 1 : nb <= 32 ? 2 : 3; }
 __host__ __device__ inline void part_analysis(int part, int& l0, int& n0) { l0 = part >= 1 ? 32 : 0; n0 = part == 2 ? 32 : 0; }
+// The synthesis tile: 32 frequencies x 64 betas, or 16 x 32 where the whole problem fits that (b <= 16 on either side:
+// the grids of the reference's own models), so that lanes and accumulators are not spent on padding.
+__host__ __device__ inline bool small_synthesis(int n2, int nb) { return nb <= 16 && n2 <= 32; }
 // parts of the synthesis: n in [n0, n0 + 32) x betas [beta0, beta0 + 64)
 __host__ __device__ inline int parts_synthesis(int n2, int nb) { return (nb > 32 ? 2 : 1) * (n2 > 64 ? 2 : 1); }
 __host__ __device__ inline void part_synthesis(int part, int nb, int& n0, int& beta0) {
@@ -59,8 +62,11 @@ __host__ __device__ inline void part_synthesis(int part, int nb, int& n0, int& b
 
 __host__ __device__ inline size_t packed_floats_analysis_part(int n2, int nb) { return (size_t)(2 * nb - 1) * n2 * 1024; }
 __host__ __device__ inline size_t packed_floats_synthesis_part(int nb) { return (size_t)(2 * nb - 1) * nb * 32 * 64; }
+__host__ __device__ inline size_t packed_floats_synthesis_small(int nb) { return (size_t)(2 * nb - 1) * nb * 16 * 32; }
 __host__ __device__ inline size_t packed_floats_analysis(int n2, int nb, int nl) { return parts_analysis(nb, nl) * packed_floats_analysis_part(n2, nb); }
-__host__ __device__ inline size_t packed_floats_synthesis(int n2, int nb) { return parts_synthesis(n2, nb) * packed_floats_synthesis_part(nb); }
+__host__ __device__ inline size_t packed_floats_synthesis(int n2, int nb) {
+  return small_synthesis(n2, nb) ? packed_floats_synthesis_small(nb) : parts_synthesis(n2, nb) * packed_floats_synthesis_part(nb);
+}
 
 // one thread per packed element
 __global__ void pack_table_analysis(const float* __restrict__ T, float* __restrict__ Tp, int n2, int nb, int nl) {
@@ -81,14 +87,15 @@ __global__ void pack_table_analysis(const float* __restrict__ T, float* __restri
 }
 
 __global__ void pack_table_synthesis(const float* __restrict__ T, float* __restrict__ Tq, int n2, int nb, int b_spec) {
-  const size_t per_part = packed_floats_synthesis_part(nb), total = packed_floats_synthesis(n2, nb);
+  const bool small = small_synthesis(n2, nb);
+  const size_t per_part = small ? packed_floats_synthesis_small(nb) : packed_floats_synthesis_part(nb), total = packed_floats_synthesis(n2, nb);
   const long nspec = (long)b_spec * (4L * b_spec * b_spec - 1) / 3;
   for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
-    int n0, beta0;
-    part_synthesis((int)(i / per_part), nb, n0, beta0);
+    int n0 = 0, beta0 = 0;
+    if (!small) part_synthesis((int)(i / per_part), nb, n0, beta0);
     const size_t ip = i % per_part;
-    const int bt = beta0 + (int)(ip & 63), n = n0 + (int)((ip >> 6) & 31);
-    const size_t r = ip >> 11;
+    const int bt = beta0 + (int)(small ? ip & 31 : ip & 63), n = n0 + (int)(small ? (ip >> 5) & 15 : (ip >> 6) & 31);
+    const size_t r = small ? ip >> 9 : ip >> 11;
     const int l = (int)(r % nb), m = (int)(r / nb) - (nb - 1);
     const int am = m < 0 ? -m : m;
     float v = 0.f;
@@ -98,7 +105,9 @@ __global__ void pack_table_synthesis(const float* __restrict__ T, float* __restr
 }
 
 // ---------------------------------------------------------------------------------------------
-// analysis: 256 threads = 4 waves; wave w owns n = 8w .. 8w+7.  For each n the contraction
+// analysis: 256 threads = 4 waves; wave w owns n = w, w + 4, w + 8, ... (so that a part with fewer than 32
+// frequencies still occupies all four waves, and no wave spends matrix-core time on columns beyond the part).
+// For each n the contraction
 //   D_n[l, (z,c)] += sum_beta T[beta, n, l] * X[beta, z, n].c        (32 degrees x 16 z x (re,im))
 // is a 32x32 matrix-core tile with K = beta: v_mfma_f32_32x32x2_f32 takes two betas per instruction,
 // A = T (lane = l, half-wave = beta parity), B = X (lane = 2 z + c).  T is zero outside the valid
@@ -127,7 +136,7 @@ __global__ __launch_bounds__(256, 2) void wigner_fwd_tiled(const float2* __restr
   const int CW = NW - n0 < 32 ? NW - n0 : 32;   // columns of the part
 
   const int t = threadIdx.x;
-  const int lane = t & 63, wave = t >> 6;
+  const int lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const int l32 = lane & 31, h = lane >> 5;
   v16f acc[8];
 #pragma unroll
@@ -180,8 +189,8 @@ __global__ __launch_bounds__(256, 2) void wigner_fwd_tiled(const float2* __restr
 
   // operand addresses of this lane: A = Ts[(beta_local * 32 + n) * TLD + l], B = Xs[(beta_local * 16 + z) * XLD_M + n].c
   const float* Xf = reinterpret_cast<const float*>(Xs);
-  const int a_off = (h * 32 + 8 * wave) * TLD + l32;
-  const int b_off = ((h * ZT + (l32 >> 1)) * XLD_M + 8 * wave) * 2 + (l32 & 1);
+  const int a_off = (h * 32 + wave) * TLD + l32;
+  const int b_off = ((h * ZT + (l32 >> 1)) * XLD_M + wave) * 2 + (l32 & 1);
 
   load_chunk(0);
   for (int b0 = 0; b0 < n2; b0 += KB) {
@@ -207,8 +216,9 @@ __global__ __launch_bounds__(256, 2) void wigner_fwd_tiled(const float2* __restr
     for (int q = 0; q < KB / 2; ++q) {          // beta pair (2q, 2q+1) of the chunk
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        const float a = Ts[a_off + (2 * q * 32 + j) * TLD];
-        const float b = Xf[b_off + (2 * q * ZT * XLD_M + j) * 2];
+        if (4 * j + wave >= CW) continue;         // the same for the whole wave
+        const float a = Ts[a_off + (2 * q * 32 + 4 * j) * TLD];
+        const float b = Xf[b_off + (2 * q * ZT * XLD_M + 4 * j) * 2];
         acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[j], 0, 0, 0);
       }
     }
@@ -230,7 +240,7 @@ __global__ __launch_bounds__(256, 2) void wigner_fwd_tiled(const float2* __restr
     const int lbase = l * (4 * l * l - 1) / 3 + l * lcoef + l;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      const int n = n0 + 8 * wave + j;
+      const int n = n0 + 4 * j + wave;
       if (n >= NW || n > l || (n == 0 && m < 0)) continue;
       const float sg = (((m - n) & 1) ? -1.f : 1.f) * (c ? -1.f : 1.f);
       const int d = m * lcoef + n;
@@ -241,12 +251,21 @@ __global__ __launch_bounds__(256, 2) void wigner_fwd_tiled(const float2* __restr
 }
 
 // ---------------------------------------------------------------------------------------------
-// synthesis: 512 threads, thread = (n = t % 32, zq = (t / 32) % 8, beta half = t / 256)
+// synthesis: 512 threads, thread = (n = t % NP, zq = (t / NP) % 8, beta group = t / (8 NP)); the tile is NP
+// frequencies x BP betas x 16 batch items: (32, 64), or (16, 32) for small grids (small_synthesis).  A thread keeps
+// BP / (512 / (8 NP)) betas of two batch items.
 // ---------------------------------------------------------------------------------------------
+template <int NP, int BP>
 __global__ __launch_bounds__(512) void wigner_inv_tiled(const float2* __restrict__ xh, const float* __restrict__ Tq_g,
                                                         float2* __restrict__ S, int n2, int nb, int b_spec, long nbatch) {
+  constexpr int BH = 512 / (8 * NP);            // beta groups
+  constexpr int BPT = BP / BH;                  // betas per thread
+  constexpr int QL = BP + 4;                    // n stride (floats) of the T chunk
+  constexpr int DEG4 = NP * BP / 4;             // 16-byte words of one degree of the packed table
+  constexpr int TPT = LC * DEG4 / 512;          // words of a chunk per thread
+  static_assert(LC * DEG4 % 512 == 0 && BPT % 4 == 0, "tile shape");
   __shared__ __attribute__((aligned(16))) float2 xs[LC * ZT * SLD];
-  __shared__ __attribute__((aligned(16))) float Tq[LC * 32 * QLD];
+  __shared__ __attribute__((aligned(16))) float Tq[LC * NP * QL];
   const int MW = 2 * nb - 1, NW = nb;
   const int nzt = (int)((nbatch + ZT - 1) / ZT);
   int m, zt;
@@ -254,37 +273,42 @@ __global__ __launch_bounds__(512) void wigner_inv_tiled(const float2* __restrict
   const int mi = m + nb - 1;
   const long z0 = (long)zt * ZT;
   const int am = abs(m);
-  int n0, beta0;                                // this workgroup's part: frequencies n0 .. n0+31, betas beta0 .. beta0+63
-  part_synthesis(blockIdx.y, nb, n0, beta0);
+  int n0 = 0, beta0 = 0;                        // this workgroup's part: frequencies n0 .. n0+NP-1, betas beta0 .. beta0+BP-1
+  if constexpr (NP == 32) part_synthesis(blockIdx.y, nb, n0, beta0);
 
   const int t = threadIdx.x;
-  const int n = t & 31, zq = (t >> 5) & 7, bh = t >> 8;
-  float2 acc[32][2];
+  const int n = t & (NP - 1), zq = (t / NP) & 7, bh = t / (8 * NP);
+  float2 acc[BPT][2];
 #pragma unroll
-  for (int j = 0; j < 32; ++j) { acc[j][0] = make_float2(0.f, 0.f); acc[j][1] = make_float2(0.f, 0.f); }
+  for (int j = 0; j < BPT; ++j) { acc[j][0] = make_float2(0.f, 0.f); acc[j][1] = make_float2(0.f, 0.f); }
 
-  const int xz = t & 15, xn = n0 + (t >> 4);    // spectrum loader: z fastest (contiguous in memory), 32 values of n
+  const int xz = t & 15, xn = n0 + (t >> 4);    // spectrum loader: z fastest (contiguous in memory), t / 16 < NP values of n
+  const bool xload = (t >> 4) < NP;
   const float hs = ((m & 1) ? -0.5f : 0.5f);    // (-1)^(m-n)/2 = hs * (-1)^n
 
   // Unconditional (clamped) loads, next chunk fetched while the current one is consumed.
   float2 xa[LC], xb[LC];
-  float4 tq[LC];
-  // packed table: degree l of this m is 32*64 contiguous floats; slot i covers floats 4 t..+3 of degree l0 + i,
-  // i.e. n = t / 16, beta = 4 (t % 16)
-  const float4* tbase = reinterpret_cast<const float4*>(Tq_g + blockIdx.y * packed_floats_synthesis_part(nb) + (size_t)mi * nb * 2048);
-  const int tlds = (t >> 4) * QLD + 4 * (t & 15);
+  float4 tq[TPT];
+  // packed table: degree l of this m is NP*BP contiguous floats; a chunk of LC degrees is LC*DEG4 16-byte words, word
+  // e = t + 512 k of it is degree l0 + e / DEG4, n = (e % DEG4) / (BP / 4), beta = 4 (e % (BP / 4))
+  const size_t part_floats = NP == 32 ? packed_floats_synthesis_part(nb) : 0;
+  const float4* tbase = reinterpret_cast<const float4*>(Tq_g + blockIdx.y * part_floats + (size_t)mi * nb * (NP * BP));
   const long zc = z0 + xz < nbatch ? z0 + xz : nbatch - 1;
 
   auto load_chunk = [&](int l0) {
 #pragma unroll
     for (int i = 0; i < LC; ++i) {
       const int l = l0 + i;
-      const bool okx = (l < nb && l >= am && l >= xn && xn < NW);
+      const bool okx = (xload && l < nb && l >= am && l >= xn && xn < NW);
       const int ia = okx ? lmn_index(l, m, xn) : 0, ib = okx ? lmn_index(l, -m, -xn) : 0;
       xa[i] = xh[(size_t)ia * nbatch + zc];
       xb[i] = xh[(size_t)ib * nbatch + zc];
-      const float4 v = tbase[(size_t)(l < nb ? l : nb - 1) * 512 + t];
-      tq[i] = l < nb ? v : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+#pragma unroll
+    for (int k = 0; k < TPT; ++k) {
+      const int e = t + 512 * k, l = l0 + e / DEG4;
+      const float4 v = tbase[(size_t)(l < nb ? l : nb - 1) * DEG4 + e % DEG4];
+      tq[k] = l < nb ? v : make_float4(0.f, 0.f, 0.f, 0.f);
     }
   };
 
@@ -298,8 +322,12 @@ __global__ __launch_bounds__(512) void wigner_inv_tiled(const float2* __restrict
       const bool okx = (l < nb && l >= am && l >= xn && xn < NW && z0 + xz < nbatch);
       const float sg = (xn & 1) ? -hs : hs;
       const float2 a = xa[i], b = xb[i];
-      xs[(i * ZT + xz) * SLD + (t >> 4)] = okx ? make_float2(0.5f * a.x + sg * b.x, 0.5f * a.y - sg * b.y) : make_float2(0.f, 0.f);
-      *reinterpret_cast<float4*>(Tq + i * 32 * QLD + tlds) = tq[i];
+      if (xload) xs[(i * ZT + xz) * SLD + (t >> 4)] = okx ? make_float2(0.5f * a.x + sg * b.x, 0.5f * a.y - sg * b.y) : make_float2(0.f, 0.f);
+    }
+#pragma unroll
+    for (int k = 0; k < TPT; ++k) {
+      const int e = t + 512 * k, r = e % DEG4;
+      *reinterpret_cast<float4*>(Tq + ((e / DEG4) * NP + r / (BP / 4)) * QL + 4 * (r % (BP / 4))) = tq[k];
     }
     __syncthreads();
     if (l0 + LC < nb) load_chunk(l0 + LC);
@@ -308,9 +336,9 @@ __global__ __launch_bounds__(512) void wigner_inv_tiled(const float2* __restrict
       if (l0 + i < am || l0 + i >= nb) continue;
       const float2 x0 = xs[(i * ZT + 2 * zq) * SLD + n];
       const float2 x1 = xs[(i * ZT + 2 * zq + 1) * SLD + n];
-      const float4* tr = reinterpret_cast<const float4*>(Tq + (i * 32 + n) * QLD + 32 * bh);
+      const float4* tr = reinterpret_cast<const float4*>(Tq + (i * NP + n) * QL + BPT * bh);
 #pragma unroll
-      for (int b4 = 0; b4 < 8; ++b4) {
+      for (int b4 = 0; b4 < BPT / 4; ++b4) {
         const float4 tv = tr[b4];
         const float tt[4] = {tv.x, tv.y, tv.z, tv.w};
 #pragma unroll
@@ -330,8 +358,8 @@ __global__ __launch_bounds__(512) void wigner_inv_tiled(const float2* __restrict
     if (z >= nbatch) continue;
     float2* p = S + ((size_t)z * n2 * MW + mi) * NW + n0 + n;
 #pragma unroll
-    for (int j = 0; j < 32; ++j) {
-      const int bt = beta0 + 32 * bh + j;
+    for (int j = 0; j < BPT; ++j) {
+      const int bt = beta0 + BPT * bh + j;
       if (bt < n2) p[(size_t)bt * plane] = acc[j][zz];
     }
   }
