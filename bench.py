@@ -289,6 +289,11 @@ def measure_example_network(torch, name, steps, warmup, batch=32):
     out = {"workload": "%s training step (s2cnn_amd/harness.py), batch %d, synthetic data" % (name, batch),
            "ms_per_step": round(ms, 3), "samples_per_s": round(batch / (ms * 1e-3), 1), "first_loss": round(losses[0], 4),
            "last_loss": round(losses[-1], 4), "library_ms": round(sum(calls.values()), 3), "library_calls_ms": calls}
+    if name == "mnist":
+        # the same step captured into one HIP graph and replayed (the eager step is bound by its launches)
+        _, rlosses, rms = harness.train_steps_replayed(name, batch=batch, steps=max(steps, 20), warmup=3, lr=0.01)
+        out["graph_replay"] = {"ms_per_step": round(rms, 3), "samples_per_s": round(batch / (rms * 1e-3), 1),
+                               "first_loss": round(rlosses[0], 4), "last_loss": round(rlosses[-1], 4)}
     if name.startswith("shrec17"):
         # the same network with its BatchNorm3d + ReLU pairs evaluated inside the neighbouring transforms (same function)
         del model

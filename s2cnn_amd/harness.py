@@ -166,3 +166,46 @@ def train_steps(name, batch=32, steps=10, warmup=2, lr=0.05, device="cuda:0", se
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) / max(steps, 1) * 1e3
     return model, [float(l) for l in losses], ms
+
+
+def train_steps_replayed(name, batch=32, steps=10, warmup=3, lr=0.05, device="cuda:0", seed=0, model=None):
+    """The step of `train_steps` captured once into a HIP graph (torch.cuda.graph) and replayed `steps` times: nothing on
+    the path allocates through HIP, synchronises or records a memset, so the whole step (forward, loss, backward, SGD
+    update) is one graph launch; for the small networks, whose step is bound by launches, that is most of the time.
+    Returns (model, losses of the replayed steps, milliseconds per replayed step)."""
+    ctor, _, _, loss_fn = NETWORKS[name]
+    torch.manual_seed(seed)
+    if model is None:
+        model = ctor()
+    model = model.to(device)
+    model.train()
+    x, y = synthetic_batch(name, batch, device, seed)
+    opt = torch.optim.SGD(model.parameters(), lr=lr, momentum=0.9)
+
+    def step():
+        opt.zero_grad(set_to_none=True)
+        loss = loss_fn(model(x), y)
+        loss.backward()
+        opt.step()
+        return loss
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(max(warmup, 3)):     # tables, workspaces, momentum buffers and allocator pools exist before the capture
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    opt.zero_grad(set_to_none=True)
+    with torch.cuda.graph(graph):
+        static_loss = step()
+    losses = []
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        graph.replay()
+        losses.append(static_loss.detach().clone())
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / max(steps, 1) * 1e3
+    return model, [float(l) for l in losses], ms

@@ -96,3 +96,13 @@ def test_shape_networks_train_and_reload(hip, name, batch):
     twin.eval()
     with torch.no_grad():
         assert torch.equal(twin(x), want)
+
+
+@pytest.mark.gpu
+def test_digit_network_step_replayed_from_a_hip_graph(hip):
+    """The training step of the digit network captured into one HIP graph: the replayed steps continue the eager
+    warm-up steps with the losses an all-eager run of the same length gives."""
+    _, eager, _ = harness.train_steps("mnist", batch=16, steps=5, warmup=3, lr=0.05)
+    _, replayed, _ = harness.train_steps_replayed("mnist", batch=16, steps=5, warmup=3, lr=0.05)
+    print("eager", ["%.5f" % l for l in eager[3:]], "replayed", ["%.5f" % l for l in replayed], flush=True)
+    assert max(abs(a - b) for a, b in zip(eager[3:], replayed)) < 1e-5 * abs(eager[0])
