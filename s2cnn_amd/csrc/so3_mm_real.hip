@@ -60,6 +60,7 @@ template <bool KC, int EXT> struct TileShape {
 };
 
 template <int VEC> struct VecT { typedef float type; };
+template <> struct VecT<2> { typedef float2 type; };
 template <> struct VecT<4> { typedef float4 type; };
 
 // One operand's tile loader: global -> registers -> LDS.  EXT = tile extent along the free index,
@@ -102,6 +103,10 @@ struct TileLoader {
     if constexpr (VEC == 4) {
       const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, (int)so, 0);
       return make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
+    } else if constexpr (VEC == 2) {
+      typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+      const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(r, (int)voff, (int)so, 0);
+      return make_float2(__uint_as_float(v.x), __uint_as_float(v.y));
     } else {
       return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, (int)voff, (int)so, 0));
     }
@@ -433,9 +438,12 @@ int run(const float* a, const float* b, float* c, int nl, int RI, int CI, int KI
   if (grid < 1) return S2CNN_EINVAL;
   MmParams p{a, b, c, nl, RI, CI, KI};
   typedef Cfg<MODE> C_;
-  // four floats per access need the fast index of the operand to be a multiple of 4 and a 16-byte base
-  const bool a4 = (C_::A_KC ? KI : RI) % 4 == 0 && s2cnn::aligned16(a);
-  const bool b4 = (C_::B_KC ? KI : CI) % 4 == 0 && s2cnn::aligned16(b);
+  // four (two) floats per access need the fast index of the operand to be a multiple of 4 (2) and a 16-byte (8-byte) base
+  const int afast = C_::A_KC ? KI : RI, bfast = C_::B_KC ? KI : CI;
+  const bool a4 = afast % 4 == 0 && s2cnn::aligned16(a);
+  const bool b4 = bfast % 4 == 0 && s2cnn::aligned16(b);
+  const bool a2 = a4 || (afast % 2 == 0 && s2cnn::aligned8(a));
+  const bool b2 = b4 || (bfast % 2 == 0 && s2cnn::aligned8(b));
   hipStream_t st = static_cast<hipStream_t>(stream);
   // the fast loaders address a degree with 32-bit byte offsets
   const bool fast = a4 && b4 && (KI % TK == 0 || TK % KI == 0) && Lmax * Lmax * RI * KI < (1L << 30) && Lmax * Lmax * CI * KI < (1L << 30);
@@ -446,6 +454,9 @@ int run(const float* a, const float* b, float* c, int nl, int RI, int CI, int KI
   } while (0)
   if (fast) S2CNN_LAUNCH(4, 4, true);
   else if (a4 && b4) S2CNN_LAUNCH(4, 4, false);
+  else if (a4 && b2) S2CNN_LAUNCH(4, 2, false);
+  else if (a2 && b4) S2CNN_LAUNCH(2, 4, false);
+  else if (a2 && b2) S2CNN_LAUNCH(2, 2, false);      // even feature counts (50, 70, 350 in the reference's shape network)
   else if (a4) S2CNN_LAUNCH(4, 1, false);
   else if (b4) S2CNN_LAUNCH(1, 4, false);
   else S2CNN_LAUNCH(1, 1, false);

@@ -136,7 +136,9 @@ def test_basis_kernels_against_dense(hip, nl, cols):
                                         # several blocks per stage (8, 16), several stages per block (96, 128), ragged last stage
                                         (5, 8, 64, 32), (4, 4, 128, 64), (7, 32, 96, 32), (6, 16, 16, 8),
                                         # one operand with 16-byte accesses, the other with 4-byte ones
-                                        (5, 6, 20, 7), (4, 3, 7, 8), (7, 32, 100, 55)])
+                                        (5, 6, 20, 7), (4, 3, 7, 8), (7, 32, 100, 55),
+                                        # even sizes that are no multiples of four: 8-byte accesses, alone and beside 16-byte ones
+                                        (6, 2, 50, 70), (5, 6, 10, 14), (4, 16, 70, 350), (5, 4, 6, 20), (5, 2, 20, 6), (3, 6, 2, 2)])
 def test_so3_mm_real_forward_backward(hip, nl, B, Fi, Fo):
     import s2cnn_amd
     print(f"so3_mm_real nl={nl} B={B} Fi={Fi} Fo={Fo}", flush=True)
