@@ -259,6 +259,10 @@ int s2cnn_so3_analysis_real_masked_bits(const float *x, const void *bits, const 
  * nbatch must be a multiple of nfeature.  No counterpart in the reference.
  */
 int s2cnn_so3_analysis_prologue_available(int b_in, int b_out);
+/* the same function in the loads of the integral that ends the reference's networks (examples/shrec17/model.py:44-45 after
+ * the last BatchNorm3d + ReLU): out[z] = s2cnn_so3_integrate of max(a x + b, 0), params [2][nfeature] as above, any grid */
+int s2cnn_so3_integrate_affine_relu(const float *x, const float *params, int nfeature, const float *w, float *out,
+                                    int b, long n, void *stream);
 int s2cnn_volume_moments(const float *x, float *out, long nvol, long n, void *stream);
 int s2cnn_bn_relu_grad_moments(const float *g, const float *y, const float *params, int nfeature, float *out,
                                long nvol, long n, void *stream);

@@ -6,11 +6,18 @@
 
 namespace {
 
+// AFFINE: the integrand is max(a x + b, 0) with a = params[z % nfeature], b = params[nfeature + z % nfeature] of volume z
+template <bool AFFINE>
 __global__ __launch_bounds__(256) void so3_integrate_kernel(const float* __restrict__ x, const float* __restrict__ w,
-                                                            float* __restrict__ out, int n2) {
+                                                            float* __restrict__ out, int n2, const float* __restrict__ params,
+                                                            int nfeature) {
   __shared__ float part[256];
   const size_t plane = (size_t)n2 * n2;
   const float* xs = x + blockIdx.x * plane * n2;
+  float pa = 1.f, pb = 0.f;
+  if constexpr (AFFINE) { pa = params[blockIdx.x % nfeature]; pb = params[nfeature + blockIdx.x % nfeature]; }
+  auto f = [&](float v) { return AFFINE ? s2cnn::affine_relu(v, pa, pb) : v; };
+  auto f4 = [&](float4 v) { return AFFINE ? make_float4(f(v.x), f(v.y), f(v.z), f(v.w)) : v; };
   float acc = 0.f;
   if (plane % 4096 == 0 && (reinterpret_cast<uintptr_t>(x) & 15u) == 0) {
     // 16-byte loads, four in flight per thread (4 KB per workgroup and step)
@@ -20,7 +27,7 @@ __global__ __launch_bounds__(256) void so3_integrate_kernel(const float* __restr
       float4 s0 = make_float4(0.f, 0.f, 0.f, 0.f), s1 = s0, s2 = s0, s3 = s0;
       const float4* pl = x4 + bt * p4 + threadIdx.x;
       for (size_t i = 0; i < p4; i += 1024) {
-        const float4 v0 = pl[i], v1 = pl[i + 256], v2 = pl[i + 512], v3 = pl[i + 768];
+        const float4 v0 = f4(pl[i]), v1 = f4(pl[i + 256]), v2 = f4(pl[i + 512]), v3 = f4(pl[i + 768]);
         s0.x += v0.x; s0.y += v0.y; s0.z += v0.z; s0.w += v0.w;
         s1.x += v1.x; s1.y += v1.y; s1.z += v1.z; s1.w += v1.w;
         s2.x += v2.x; s2.y += v2.y; s2.z += v2.z; s2.w += v2.w;
@@ -36,8 +43,8 @@ __global__ __launch_bounds__(256) void so3_integrate_kernel(const float* __restr
       float4 s0 = make_float4(0.f, 0.f, 0.f, 0.f), s1 = s0;
       const float4* pl = x4 + (size_t)bt * p4;
       for (int i = threadIdx.x; i < p4; i += 512) {
-        const float4 v0 = pl[i];
-        const float4 v1 = i + 256 < p4 ? pl[i + 256] : make_float4(0.f, 0.f, 0.f, 0.f);
+        const float4 v0 = f4(pl[i]);
+        const float4 v1 = i + 256 < p4 ? f4(pl[i + 256]) : make_float4(0.f, 0.f, 0.f, 0.f);
         s0.x += v0.x; s0.y += v0.y; s0.z += v0.z; s0.w += v0.w;
         s1.x += v1.x; s1.y += v1.y; s1.z += v1.z; s1.w += v1.w;
       }
@@ -46,7 +53,7 @@ __global__ __launch_bounds__(256) void so3_integrate_kernel(const float* __restr
   } else {
     for (int bt = 0; bt < n2; ++bt) {
       float s = 0.f;
-      for (size_t i = threadIdx.x; i < plane; i += blockDim.x) s += xs[bt * plane + i];
+      for (size_t i = threadIdx.x; i < plane; i += blockDim.x) s += f(xs[bt * plane + i]);
       acc += w[bt] * s;
     }
   }
@@ -154,7 +161,16 @@ extern "C" int s2cnn_bn_relu_grad_moments(const float* g, const float* y, const 
 extern "C" int s2cnn_so3_integrate(const float* x, const float* w, float* out, int b, long n, void* stream) {
   s2cnn::clear_stale_error();
   if (!x || !w || !out || b < 1 || b > 1024 || n < 1 || n >= (1L << 31)) return S2CNN_EINVAL;
-  hipLaunchKernelGGL(so3_integrate_kernel, dim3((unsigned)n), dim3(256), 0, static_cast<hipStream_t>(stream), x, w, out, 2 * b);
+  hipLaunchKernelGGL(so3_integrate_kernel<false>, dim3((unsigned)n), dim3(256), 0, static_cast<hipStream_t>(stream), x, w, out, 2 * b, nullptr, 1);
+  return s2cnn::launch_status();
+}
+
+extern "C" int s2cnn_so3_integrate_affine_relu(const float* x, const float* params, int nfeature, const float* w, float* out, int b,
+                                               long n, void* stream) {
+  s2cnn::clear_stale_error();
+  if (!x || !params || !w || !out || b < 1 || b > 1024 || n < 1 || n >= (1L << 31) || nfeature < 1 || n % nfeature != 0) return S2CNN_EINVAL;
+  hipLaunchKernelGGL(so3_integrate_kernel<true>, dim3((unsigned)n), dim3(256), 0, static_cast<hipStream_t>(stream), x, w, out, 2 * b, params,
+                     nfeature);
   return s2cnn::launch_status();
 }
 

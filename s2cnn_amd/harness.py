@@ -79,8 +79,10 @@ class Shrec17Model(nn.Module):
         self.out_layer = nn.Linear(self.features[-2], self.features[-1])
 
     def forward(self, x):  # pylint: disable=W0221
-        x = run_sequence(self.sequential, x) if self.fused_norm else self.sequential(x)      # [batch, feature, beta, alpha, gamma]
-        x = so3_integrate(x)        # [batch, feature]
+        if self.fused_norm:
+            x = run_sequence(self.sequential, x, integrate=True)      # [batch, feature]
+        else:
+            x = so3_integrate(self.sequential(x))                     # [batch, feature, beta, alpha, gamma] -> [batch, feature]
         return F.log_softmax(self.out_layer(x), dim=1)
 
 
