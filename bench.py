@@ -274,6 +274,58 @@ def measure_network(torch, dev, steps, warmup):
             "separate_relu": {"ms_per_step": round(ms_sep, 3), "library_ms": round(sum(calls_sep.values()), 3)}}
 
 
+def measure_fft_floor(torch, dev, nvol=256, reps=10):
+    """What the plane pipeline of the per-volume 64^3 kernels costs without the Wigner contraction: the shipped kernels
+    with parts compiled out (s2cnn_so3_fft64_probe; the results of the stripped variants are meaningless), timed with
+    events on the launch stream at the size of benchmark config 2.  The passes between records and spectral rows are
+    timed from the full transforms (they are the difference between the transform and its kernel)."""
+    from s2cnn_amd import _hip
+    from s2cnn_amd.soft import so3_fft as PSO3
+    b = 32
+    x = torch.randn(nvol, 64, 64, 64, generator=torch.Generator().manual_seed(3)).to(dev)
+    y = torch.empty_like(x)
+    L = _hip.lib()
+    ws = _hip.workspace(L.s2cnn_so3_analysis_workspace(b, b, nvol, 0), x.device)
+    packed = {0: PSO3._setup_packed_wigner(b, b, True, False, x.device), 1: PSO3._setup_packed_wigner(b, b, False, True, x.device)}
+    spec = PSO3.so3_rfft(x)
+    out = {}
+    variants = [("analysis kernel", 0, 0), ("analysis kernel, no contraction multiply-adds", 0, 1),
+                ("analysis kernel, no contraction and no table loads", 0, 2),
+                ("synthesis kernel", 1, 0), ("synthesis kernel, no contraction multiply-adds", 1, 1)]
+    for name, direction, probe in variants:
+        def run():
+            _hip.check(L.s2cnn_so3_fft64_probe(_hip.ptr(x), _hip.ptr(y), _hip.ptr(packed[direction]), _hip.ptr(ws), ws.numel(), nvol,
+                                               direction, probe, _hip.stream_ptr()))
+        if direction == 1:
+            PSO3.so3_rifft(spec)                      # leaves the records of a real spectrum in the workspace
+        for _ in range(2):
+            run()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            run()
+        e1.record()
+        torch.cuda.synchronize()
+        out[name] = round(e0.elapsed_time(e1) / reps * 1e3, 1)
+    kt = _hip.KernelTimer()
+    with kt:
+        for _ in range(reps):
+            PSO3.so3_rifft(PSO3.so3_rfft(x))
+        torch.cuda.synchronize()
+    full = {k: sum(v) / len(v) * 1e3 for k, v in kt.summary().items()}
+    out["analysis, whole transform"] = round(full["s2cnn_so3_analysis"], 1)
+    out["synthesis, whole transform"] = round(full["s2cnn_so3_synthesis"], 1)
+    bytes_dir = so3_fft_bytes(b, b, nvol)
+    rows_a = full["s2cnn_so3_analysis"] - out["analysis kernel"]
+    rows_s = full["s2cnn_so3_synthesis"] - out["synthesis kernel"]
+    floor_us = (out["analysis kernel, no contraction and no table loads"] + rows_a) + (out["synthesis kernel, no contraction multiply-adds"] + rows_s)
+    return {"workload": "per-volume kernels of the 64^3 grid, %d volumes (benchmark config 2), microseconds per launch" % nvol,
+            "us": out,
+            "round_trip_without_contraction_us": round(floor_us, 1),
+            "frac_of_hbm_peak_without_contraction": round(2 * bytes_dir / (floor_us * 1e-6) / 1e9 / PEAK_HBM_GBS, 4),
+            "frac_of_hbm_peak_shipped": round(2 * bytes_dir / ((full["s2cnn_so3_analysis"] + full["s2cnn_so3_synthesis"]) * 1e-6) / 1e9 / PEAK_HBM_GBS, 4)}
+
+
 def measure_example_network(torch, name, steps, warmup, batch=32):
     """One of the reference's example networks (examples/mnist/run.py:55-98, examples/shrec17/model.py, model_original.py) in
     its training step (forward, loss, backward, SGD with momentum) on a fixed synthetic batch; time inside library calls
@@ -323,6 +375,8 @@ def main():
     ap.add_argument("--complex-product", action="store_true",
                     help="multiply complex spectra as the reference does instead of real-basis ones")
     ap.add_argument("--rows", action="store_true", help="also time every other op of the path (adds a `rows` object)")
+    ap.add_argument("--floor", action="store_true",
+                    help="also time the per-volume 64^3 kernels with their Wigner contraction compiled out (adds a `fft_floor` object)")
     ap.add_argument("--network", nargs="?", const="config5", default=None, choices=["config5", "mnist", "shrec17", "shrec17_original"],
                     help="also time a whole network, forward + backward (adds a `network` object): config5 = the SHREC17-shaped "
                          "network of benchmark config 5 (default); mnist, shrec17, shrec17_original = the reference's example "
@@ -437,6 +491,8 @@ def main():
         result["so3_mm"] = measure_so3_mm(torch, dev)
     if args.rows:
         result["rows"] = measure_rows(torch, dev, not args.no_cpu)
+    if args.floor:
+        result["fft_floor"] = measure_fft_floor(torch, dev)
     if args.network == "config5":
         result["network"] = measure_network(torch, dev, args.steps, args.warmup)
     elif args.network:

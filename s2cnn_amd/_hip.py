@@ -52,6 +52,7 @@ SIGNATURES = {
     "s2cnn_so3_relu_bits_bytes": (_size_t, [_int, _long]),
     "s2cnn_so3_synthesis_real_relu_bits": (_int, _FT3R_SIG[:4] + [_vp] + _FT3R_SIG[4:-1] + [_c_float_p, _int, _int, _vp]),
     "s2cnn_so3_analysis_real_masked_bits": (_int, [_c_float_p, _vp] + _FT3R_SIG[1:-1] + [_int, _vp]),
+    "s2cnn_so3_fft64_probe": (_int, [_c_float_p, _c_float_p, _c_float_p, _vp, _size_t, _long, _int, _int, _vp]),
     "s2cnn_so3_analysis_prologue_available": (_int, [_int, _int]),
     "s2cnn_so3_integrate_affine_relu": (_int, [_c_float_p, _c_float_p, _int, _c_float_p, _c_float_p, _int, _long, _vp]),
     "s2cnn_volume_moments": (_int, [_c_float_p, _c_float_p, _long, _long, _vp]),

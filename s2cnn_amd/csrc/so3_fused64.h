@@ -210,7 +210,10 @@ __device__ constexpr int table_slot(int it) { return it & 3; }
 // volume's feature z % nfeature in params [.][nfeature].
 constexpr int BITS_WORDS = N * N;      // 64-bit words per volume: [beta][alpha % 8][alpha / 8], bit = gamma
 __host__ __device__ inline size_t bits_index(long z, int beta, int d) { return ((size_t)z * N + beta) * N + 8 * d; }   // + alpha / 8
-template <int NA, int MASK>
+// PROBE (measurement only, results meaningless): 1: the Wigner contraction of an item reduced to one add per table
+// operand (table loads, LDS reads of the quads and everything else kept); 2: the table loads gone as well.  What is left
+// is the plane pipeline: loads, the 2-D transform through LDS with its barriers, the quad layout, the record.
+template <int NA, int MASK, int PROBE = 0>
 __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restrict__ x, const float* __restrict__ mask,
                                                            const float* __restrict__ Tf, float4* __restrict__ rec, long nbatch,
                                                            const float* __restrict__ params, int nfeature) {
@@ -291,6 +294,11 @@ __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restri
     for (int j1 = 2 * g; j1 < 2 * g + 2; ++j1) load_rows(j, j1);
   };
   auto load_table = [&](int j, int it) {
+    if constexpr (PROBE == 2) {
+      t1[table_slot(it)] = make_float4(1.f * j, 0.f, 0.f, 0.f);
+      t2[table_slot(it)] = make_float4(1.f * it, 0.f, 0.f, 0.f);
+      return;
+    }
     t1[table_slot(it)] = buf_load_f32x4(rt, toff, ((j * NIT + it) * 2 + 0) * (THREADS * 16));
     t2[table_slot(it)] = buf_load_f32x4(rt, toff, ((j * NIT + it) * 2 + 1) * (THREADS * 16));
   };
@@ -337,6 +345,10 @@ __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restri
     const float2 Pm = make_float2(zb.x + zb.z, zb.y - zb.w);
     const float2 Qm = make_float2(flip(zb.y + zb.w, sb), flip(zb.z - zb.x, sb));
     const float4 ta = t1[table_slot(it)], tb = t2[table_slot(it)];
+    if constexpr (PROBE != 0) {
+      accp[it][0].x += za.x + ta.x; accm[it][0].x += zb.x + tb.x;
+      return;
+    }
     const float a1[4] = {ta.x, ta.y, ta.z, ta.w};
     const float a2[4] = {tb.x, tb.y, tb.z, tb.w};
 #pragma unroll
@@ -685,7 +697,8 @@ __global__ __launch_bounds__(256) void spectrum_gather_real(const float* __restr
 // bias: NULL, or one value per feature added to every sample of volume z (feature = z % nfeature)
 // relu: nonzero = negative samples (after the bias) are stored as zero
 // NA as in analysis_kernel; CMAX: degree groups c < CMAX carry degrees of the input (6 for NA = 3, 7 for 5, 8 for 7)
-template <int NA, int CMAX>
+// PROBE (measurement only, results meaningless): 1: an item's share of a plane pair reduced to one add per table operand.
+template <int NA, int CMAX, int PROBE = 0>
 __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __restrict__ rec, const float* __restrict__ Tf,
                                                             float* __restrict__ y, long nbatch, const float* __restrict__ bias, int nfeature,
                                                             int relu, unsigned long long* __restrict__ bits) {
@@ -759,16 +772,20 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
     const float a1[4] = {ta.x, ta.y, ta.z, ta.w};
     const float a2[4] = {tb.x, tb.y, tb.z, tb.w};
     float2 Sp = make_float2(0.f, 0.f), Qp = make_float2(0.f, 0.f), Sm = make_float2(0.f, 0.f), Qm = make_float2(0.f, 0.f);
+    if constexpr (PROBE != 0) {
+      Sp.x = a1[0] + xp[it][0].x; Sm.x = a2[0] + xm[it][0].x;
+    } else {
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const float b1 = (u & 1) ? -a1[u] : a1[u], b2 = (u & 1) ? -a2[u] : a2[u];
-      Sp.x = fmaf(a1[u], xp[it][u].x, Sp.x); Sp.y = fmaf(a1[u], xp[it][u].y, Sp.y);
-      Qp.x = fmaf(b2, xp[it][u].x, Qp.x);    Qp.y = fmaf(b2, xp[it][u].y, Qp.y);
-      Sm.x = fmaf(a2[u], xm[it][u].x, Sm.x); Sm.y = fmaf(a2[u], xm[it][u].y, Sm.y);
-      Qm.x = fmaf(b1, xm[it][u].x, Qm.x);    Qm.y = fmaf(b1, xm[it][u].y, Qm.y);
+      for (int u = 0; u < 4; ++u) {
+        const float b1 = (u & 1) ? -a1[u] : a1[u], b2 = (u & 1) ? -a2[u] : a2[u];
+        Sp.x = fmaf(a1[u], xp[it][u].x, Sp.x); Sp.y = fmaf(a1[u], xp[it][u].y, Sp.y);
+        Qp.x = fmaf(b2, xp[it][u].x, Qp.x);    Qp.y = fmaf(b2, xp[it][u].y, Qp.y);
+        Sm.x = fmaf(a2[u], xm[it][u].x, Sm.x); Sm.y = fmaf(a2[u], xm[it][u].y, Sm.y);
+        Qm.x = fmaf(b1, xm[it][u].x, Qm.x);    Qm.y = fmaf(b1, xm[it][u].y, Qm.y);
+      }
+      const unsigned sb = ((sgn >> it) & 1u) << 31;
+      Qp.x = flip(Qp.x, sb); Qp.y = flip(Qp.y, sb); Qm.x = flip(Qm.x, sb); Qm.y = flip(Qm.y, sb);
     }
-    const unsigned sb = ((sgn >> it) & 1u) << 31;
-    Qp.x = flip(Qp.x, sb); Qp.y = flip(Qp.y, sb); Qm.x = flip(Qm.x, sb); Qm.y = flip(Qm.y, sb);
     const unsigned pos = it * THREADS + t + ((spad[it >> 2] >> (8 * (it & 3))) & 0xffu);
     stg_p[pos] = make_float4(Sp.x - Qp.y, Sp.y + Qp.x, Sp.x + Qp.y, Qp.x - Sp.y);
     stg_m[pos] = make_float4(Sm.x - Qm.y, Sm.y + Qm.x, Sm.x + Qm.y, Qm.x - Sm.y);
@@ -913,6 +930,19 @@ inline void launch_analysis(int nl, hipStream_t st, const s2cnn::Input& in, cons
     case s2cnn::PRO_AFFINE_RELU: launch_analysis_m<3>(nl, st, in, Tf, rec, nbatch); break;
     case s2cnn::PRO_BN_RELU_GRAD: launch_analysis_m<4>(nl, st, in, Tf, rec, nbatch); break;
     default: launch_analysis_m<0>(nl, st, in, Tf, rec, nbatch);
+  }
+}
+
+// The kernels with parts compiled out, for timing what the rest costs (see PROBE above); full spectra, no mask, no bias.
+inline void launch_probe(int direction, int probe, hipStream_t st, const float* x, float* y, const float* Tf, float4* rec, long nbatch) {
+  const dim3 grid(grid_size(nbatch)), block(THREADS);
+  if (direction == 0) {
+    if (probe == 1) hipLaunchKernelGGL((analysis_kernel<7, 0, 1>), grid, block, 0, st, x, nullptr, Tf, rec, nbatch, nullptr, 1);
+    else if (probe == 2) hipLaunchKernelGGL((analysis_kernel<7, 0, 2>), grid, block, 0, st, x, nullptr, Tf, rec, nbatch, nullptr, 1);
+    else hipLaunchKernelGGL((analysis_kernel<7, 0, 0>), grid, block, 0, st, x, nullptr, Tf, rec, nbatch, nullptr, 1);
+  } else {
+    if (probe == 1) hipLaunchKernelGGL((synthesis_kernel<7, 8, 1>), grid, block, 0, st, rec, Tf, y, nbatch, nullptr, 1, 0, nullptr);
+    else hipLaunchKernelGGL((synthesis_kernel<7, 8, 0>), grid, block, 0, st, rec, Tf, y, nbatch, nullptr, 1, 0, nullptr);
   }
 }
 
