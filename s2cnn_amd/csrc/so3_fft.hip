@@ -499,7 +499,10 @@ int analysis_impl(const s2cnn::Input& in, const float* table, const float* packe
       Tp = dst;
     }
     const int parts = wigner_tiled::parts_analysis(nb, b_out);
-    if (parts == 1)
+    if (wigner_tiled::small_analysis(nb, b_out))
+      hipLaunchKernelGGL((wigner_tiled::wigner_fwd_tiled<false, 16>), dim3(wigner_tiled::grid_size(MW, nbatch)), dim3(256), 0, st, X, Tp,
+                         reinterpret_cast<float2*>(out), n2, nb, b_out, nbatch);
+    else if (parts == 1)
       hipLaunchKernelGGL(wigner_tiled::wigner_fwd_tiled<false>, dim3(wigner_tiled::grid_size(MW, nbatch)), dim3(256), 0, st, X, Tp,
                          reinterpret_cast<float2*>(out), n2, nb, b_out, nbatch);
     else

@@ -7,7 +7,7 @@
 //              xs = (xhat[l,m,n] + (-1)^(m-n) conj xhat[l,-m,-n]) / 2
 //
 // The table is consumed in a packed, zero-padded order that makes every chunk one contiguous block:
-//   analysis : Tp[part][mi][beta][n (32)][l (32)]        (pack_table_analysis)
+//   analysis : Tp[part][mi][beta][n (32)][l (32)]        (pack_table_analysis; [n (16)][l (16)] for small problems)
 //   synthesis: Tq[part][mi][l (nb)][n (32)][beta (64)]   (pack_table_synthesis; [n (16)][beta (32)] for small grids)
 // with zeros outside max(|m|, n) <= l < number of degrees, n < nb, beta < 2 b_grid.
 // A workgroup covers 32 values of n and 32 degrees (analysis) or 64 betas (synthesis); larger problems are cut
@@ -61,23 +61,30 @@ __host__ __device__ inline void part_synthesis(int part, int nb, int& n0, int& b
 }
 
 __host__ __device__ inline size_t packed_floats_analysis_part(int n2, int nb) { return (size_t)(2 * nb - 1) * n2 * 1024; }
+// The analysis table tile: 32 frequencies x 32 degrees per beta, or 16 x 16 where the whole problem fits that (the padding
+// of the larger tile would be three quarters of all the table bytes a workgroup reads).
+__host__ __device__ inline bool small_analysis(int nb, int nl) { return nb <= 16 && nl <= 16; }
+__host__ __device__ inline size_t packed_floats_analysis_small(int n2, int nb) { return (size_t)(2 * nb - 1) * n2 * 256; }
 __host__ __device__ inline size_t packed_floats_synthesis_part(int nb) { return (size_t)(2 * nb - 1) * nb * 32 * 64; }
 __host__ __device__ inline size_t packed_floats_synthesis_small(int nb) { return (size_t)(2 * nb - 1) * nb * 16 * 32; }
-__host__ __device__ inline size_t packed_floats_analysis(int n2, int nb, int nl) { return parts_analysis(nb, nl) * packed_floats_analysis_part(n2, nb); }
+__host__ __device__ inline size_t packed_floats_analysis(int n2, int nb, int nl) {
+  return small_analysis(nb, nl) ? packed_floats_analysis_small(n2, nb) : parts_analysis(nb, nl) * packed_floats_analysis_part(n2, nb);
+}
 __host__ __device__ inline size_t packed_floats_synthesis(int n2, int nb) {
   return small_synthesis(n2, nb) ? packed_floats_synthesis_small(nb) : parts_synthesis(n2, nb) * packed_floats_synthesis_part(nb);
 }
 
 // one thread per packed element
 __global__ void pack_table_analysis(const float* __restrict__ T, float* __restrict__ Tp, int n2, int nb, int nl) {
-  const size_t per_part = packed_floats_analysis_part(n2, nb), total = packed_floats_analysis(n2, nb, nl);
+  const bool small = small_analysis(nb, nl);
+  const size_t per_part = small ? packed_floats_analysis_small(n2, nb) : packed_floats_analysis_part(n2, nb), total = packed_floats_analysis(n2, nb, nl);
   const long nspec = (long)nl * (4L * nl * nl - 1) / 3;
   for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
-    int l0, n0;
-    part_analysis((int)(i / per_part), l0, n0);
+    int l0 = 0, n0 = 0;
+    if (!small) part_analysis((int)(i / per_part), l0, n0);
     const size_t ip = i % per_part;
-    const int l = l0 + (int)(ip & 31), n = n0 + (int)((ip >> 5) & 31);
-    const size_t r = ip >> 10;
+    const int l = l0 + (int)(small ? ip & 15 : ip & 31), n = n0 + (int)(small ? (ip >> 4) & 15 : (ip >> 5) & 31);
+    const size_t r = small ? ip >> 8 : ip >> 10;
     const int bt = (int)(r % n2), m = (int)(r / n2) - (nb - 1);
     const int am = m < 0 ? -m : m;
     float v = 0.f;
@@ -117,8 +124,9 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 constexpr int XLD_M = 33;     // z stride (complex) of the X chunk: (z, c) lanes hit 32 distinct banks
 
 // PARTS = false: one part (nb, nl <= 32), the chunk of X is one contiguous run; true: the parts above, the chunk is
-// KB*16 row pieces.
-template <bool PARTS>
+// KB*16 row pieces.  TS: the packed table holds TS x TS values per beta (32, or 16 for small_analysis; the matrix-core
+// tile stays 32 x 32, its rows of degrees >= 16 read zeros).
+template <bool PARTS, int TS = 32>
 __global__ __launch_bounds__(256, 2) void wigner_fwd_tiled(const float2* __restrict__ X, const float* __restrict__ Tp,
                                                            float2* __restrict__ out, int n2, int nb, int nl, long nbatch) {
   __shared__ __attribute__((aligned(16))) float2 Xs[KB * ZT * XLD_M];
@@ -146,12 +154,16 @@ __global__ __launch_bounds__(256, 2) void wigner_fwd_tiled(const float2* __restr
 
   // Loads are unconditional (clamped addresses, values zeroed by select) so that all of a chunk's
   // loads are in flight together, and the next chunk is fetched while the current one is consumed.
+  static_assert(TS == 32 || (TS == 16 && !PARTS), "table tile");
+  constexpr int BW = TS * TS / 4;               // 16-byte words of one beta of the packed table
+  constexpr int TPT = KB * BW / 256;            // words of a chunk per thread
   float2 xr[KB * 2];
-  float4 tr_[KB];
-  // packed table: the chunk of KB betas is KB*1024 contiguous floats; slot i covers floats 4 (t + 256 i)..+3,
-  // i.e. beta_local = i, n = t / 8, l = 4 (t % 8)
-  const float4* tbase = reinterpret_cast<const float4*>(Tp + (PARTS ? blockIdx.y * packed_floats_analysis_part(n2, nb) : 0) + (size_t)mi * n2 * 1024);
-  const int tlds = (t >> 3) * TLD + 4 * (t & 7);
+  float4 tr_[TPT];
+  // packed table: the chunk of KB betas is KB * TS * TS contiguous floats; word e = t + 256 i of it is
+  // beta_local = e / BW, n = (e % BW) / (TS / 4), l = 4 (e % (TS / 4))
+  const float4* tbase = reinterpret_cast<const float4*>(Tp + (PARTS ? blockIdx.y * packed_floats_analysis_part(n2, nb) : 0) + (size_t)mi * n2 * (TS * TS));
+  if constexpr (TS < 32)                        // the rows of degrees >= TS are never written: they must read as zero
+    for (int i = t; i < KB * 32 * TLD; i += 256) Ts[i] = 0.f;
   // X is laid out [z tile][mi][beta][z % 16][n]: a chunk (KB betas) is KB*16 rows of NW complex numbers.
   // One part: the chunk is KB*16*NW contiguous numbers; thread slot i covers element e = t + 256 i of it.
   // Several parts: the part takes the CW columns from n0 of every row; a thread keeps one column (lc) and takes rows
@@ -180,10 +192,11 @@ __global__ __launch_bounds__(256, 2) void wigner_fwd_tiled(const float2* __restr
       }
     }
 #pragma unroll
-    for (int bt = 0; bt < KB; ++bt) {
+    for (int i = 0; i < TPT; ++i) {
+      const int e = t + 256 * i, bt = e / BW;
       const int bc = b0 + bt < n2 ? b0 + bt : n2 - 1;
-      const float4 v = tbase[(size_t)bc * 256 + t];
-      tr_[bt] = b0 + bt < n2 ? v : make_float4(0.f, 0.f, 0.f, 0.f);
+      const float4 v = tbase[(size_t)bc * BW + e % BW];
+      tr_[i] = b0 + bt < n2 ? v : make_float4(0.f, 0.f, 0.f, 0.f);
     }
   };
 
@@ -209,7 +222,10 @@ __global__ __launch_bounds__(256, 2) void wigner_fwd_tiled(const float2* __restr
       }
     }
 #pragma unroll
-    for (int bt = 0; bt < KB; ++bt) *reinterpret_cast<float4*>(Ts + bt * 32 * TLD + tlds) = tr_[bt];
+    for (int i = 0; i < TPT; ++i) {
+      const int e = t + 256 * i, r = e % BW;
+      *reinterpret_cast<float4*>(Ts + ((e / BW) * 32 + r / (TS / 4)) * TLD + 4 * (r % (TS / 4))) = tr_[i];
+    }
     __syncthreads();
     if (b0 + KB < n2) load_chunk(b0 + KB);
 #pragma unroll
