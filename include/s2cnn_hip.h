@@ -266,6 +266,18 @@ int s2cnn_so3_integrate_affine_relu(const float *x, const float *params, int nfe
 int s2cnn_volume_moments(const float *x, float *out, long nvol, long n, void *stream);
 int s2cnn_bn_relu_grad_moments(const float *g, const float *y, const float *params, int nfeature, float *out,
                                long nvol, long n, void *stream);
+/* the arithmetic between those calls, one small launch each instead of a chain of tensor operations (float64 inside):
+ * forward : moments [batch][nfeature][2] of s2cnn_volume_moments, count = samples per feature -> ab [2][nfeature] for the
+ *           analysis, stats [4][nfeature] = batch mean, biased batch variance, mean in use, 1/sqrt(var in use + eps)
+ *           (in use: the batch's when training != 0, else running_mean / running_var); when training and the running
+ *           buffers are given they move by `momentum` (unbiased variance), as nn.BatchNorm3d does; weight, bias: NULL = 1, 0
+ * backward: moments of s2cnn_bn_relu_grad_moments -> params [4][nfeature] for s2cnn_so3_analysis_real_bn_relu_grad and
+ *           gwb [2][nfeature] = the gradients of weight and bias */
+int s2cnn_bn_forward_from_moments(const float *moments, int batch, int nfeature, double count, const float *weight,
+                                  const float *bias, float *running_mean, float *running_var, double eps, double momentum,
+                                  int training, float *ab, float *stats, void *stream);
+int s2cnn_bn_backward_from_moments(const float *moments, int batch, int nfeature, double count, const float *ab,
+                                   const float *stats, int training, float *params, float *gwb, void *stream);
 int s2cnn_so3_analysis_real_affine_relu(const float *x, const float *params, int nfeature,
                                         const float *table, const float *packed_table, float *out,
                                         void *workspace, size_t workspace_bytes,

@@ -34,8 +34,13 @@ def _moments(name, n_per_volume, *operands):
     return out
 
 
-def _synthesis_and_statistics(ctx, zr, conv_bias, weight, bias, running_mean, running_var, b_grid, eps, training):
-    """y = synthesis(zr) + conv_bias, the batch statistics of y and the affine map (a, b) of the normalisation."""
+def _ptr_or_none(t):
+    return _hip.ptr(t) if t is not None else None
+
+
+def _synthesis_and_statistics(ctx, zr, conv_bias, weight, bias, running_mean, running_var, b_grid, eps, training, momentum):
+    """y = synthesis(zr) + conv_bias, the statistics of y and the affine map (a, b) of the normalisation; when training,
+    the running averages (if given) move by `momentum`."""
     nspec, batch, nf = zr.shape
     ctx.b_z = round((3 / 4 * nspec) ** (1 / 3))
     ctx.b_grid, ctx.training = b_grid, training
@@ -43,61 +48,50 @@ def _synthesis_and_statistics(ctx, zr, conv_bias, weight, bias, running_mean, ru
     y = so3_rifft_real_basis(zr, b_out=b_grid, bias=conv_bias)                       # [batch, feature, 2b, 2b, 2b]
     nvox = (2 * b_grid) ** 3
     ctx.count = batch * nvox
-    s = _moments("s2cnn_volume_moments", nvox, y).view(batch, nf, 2).double().sum(0)    # [feature, 2]
-    mean = s[:, 0] / ctx.count
-    var = (s[:, 1] / ctx.count - mean * mean).clamp_min(0.0)
-    use_mean, use_var = (mean, var) if training else (running_mean.double(), running_var.double())
-    invstd = torch.rsqrt(use_var + eps)
-    w = weight.double() if weight is not None else torch.ones_like(invstd)
-    a = w * invstd
-    b = (bias.double() if bias is not None else torch.zeros_like(a)) - use_mean * a
-    ab = torch.stack([a, b]).float()
-    ctx.save_for_backward(y, ab, use_mean, invstd)
+    mom = _moments("s2cnn_volume_moments", nvox, y)                                  # [batch * feature, 2]
+    ab = y.new_empty((2, nf))
+    stats = y.new_empty((4, nf))          # batch mean, biased batch variance, mean in use, 1 / sqrt(variance in use + eps)
+    for t in (weight, bias, running_mean, running_var):
+        if t is not None:
+            _hip.require_gpu_f32(t)
+            assert t.is_contiguous() and t.numel() == nf
+    _hip.call("s2cnn_bn_forward_from_moments", _hip.ptr(mom), batch, nf, float(ctx.count), _ptr_or_none(weight), _ptr_or_none(bias),
+              _ptr_or_none(running_mean), _ptr_or_none(running_var), float(eps), float(momentum), int(training), _hip.ptr(ab),
+              _hip.ptr(stats), _hip.stream_ptr())
+    ctx.save_for_backward(y, ab, stats)
     ctx.has_affine = (weight is not None, bias is not None)
-    mean_f, var_f = mean.float(), var.float()
-    ctx.mark_non_differentiable(mean_f, var_f)
-    return y, ab, mean_f, var_f
+    return y, ab
 
 
 def _gradients_from(ctx, g):
     """g: the gradient with respect to u = max(a y + b, 0).  Returns the gradients with respect to the spectrum zr, the
     bias of the layer, and the weight and bias of the normalisation."""
-    y, ab, mean, invstd = ctx.saved_tensors
+    y, ab, stats = ctx.saved_tensors
     batch, nf = y.shape[:2]
     nvox = (2 * ctx.b_grid) ** 3
-    d = _moments("s2cnn_bn_relu_grad_moments", nvox, g, y, ab, nf).view(batch, nf, 2).double().sum(0)
-    d1, d2 = d[:, 0], d[:, 1]                                                        # sum g m, sum g m y
-    a = ab[0].double()
-    gxhat = invstd * (d2 - mean * d1)                                                # sum g m (y - mean) / std
-    if ctx.training:
-        k2 = invstd * gxhat / ctx.count
-        p = -a * d1 / ctx.count + a * k2 * mean
-        q = -a * k2
-    else:
-        p = torch.zeros_like(a)
-        q = torch.zeros_like(a)
-    params = torch.stack([a, ab[1].double(), p, q]).float()
+    mom = _moments("s2cnn_bn_relu_grad_moments", nvox, g, y, ab, nf)                 # sum g m, sum g m y per volume
+    params = y.new_empty((4, nf))
+    gwb = y.new_empty((2, nf))
+    _hip.call("s2cnn_bn_backward_from_moments", _hip.ptr(mom), batch, nf, float(ctx.count), _hip.ptr(ab), _hip.ptr(stats),
+              int(ctx.training), _hip.ptr(params), _hip.ptr(gwb), _hip.stream_ptr())
     gz = so3_rfft_real_basis(g, for_grad=True, b_out=ctx.b_z, mask=LoadBNReLUGrad(y, params))
     g_conv_bias = gz[0].reshape(-1, nf).sum(0).reshape(ctx.bias_shape) if ctx.needs_input_grad[1] else None
-    g_weight = gxhat.to(gz.dtype) if ctx.has_affine[0] else None
-    g_bias = d1.to(gz.dtype) if ctx.has_affine[1] else None
-    return gz, g_conv_bias, g_weight, g_bias
+    return gz, g_conv_bias, (gwb[0] if ctx.has_affine[0] else None), (gwb[1] if ctx.has_affine[1] else None)
 
 
 class _SynthesisBNReLUAnalysis(torch.autograd.Function):
     """z_hat (real-basis spectrum [l m n, batch, feature]) of one layer -> the input spectrum of the next one.
-    Returns (x_hat, batch mean, biased batch variance); the statistics are not differentiable outputs (they feed the
-    running averages)."""
+    running_mean / running_var (buffers, may be None) are read in evaluation mode and updated in training mode."""
 
     @staticmethod
-    def forward(ctx, zr, conv_bias, weight, bias, running_mean, running_var, b_grid, b_next, eps, training):  # pylint: disable=W
-        y, ab, mean, var = _synthesis_and_statistics(ctx, zr, conv_bias, weight, bias, running_mean, running_var, b_grid, eps, training)
-        return so3_rfft_real_basis(y, b_out=b_next, mask=LoadAffineReLU(ab)), mean, var
+    def forward(ctx, zr, conv_bias, weight, bias, running_mean, running_var, b_grid, b_next, eps, training, momentum):  # pylint: disable=W
+        y, ab = _synthesis_and_statistics(ctx, zr, conv_bias, weight, bias, running_mean, running_var, b_grid, eps, training, momentum)
+        return so3_rfft_real_basis(y, b_out=b_next, mask=LoadAffineReLU(ab))
 
     @staticmethod
-    def backward(ctx, gxh, _gm, _gv):  # pylint: disable=W
+    def backward(ctx, gxh):  # pylint: disable=W
         g = so3_rifft_real_basis(gxh.contiguous(), for_grad=True, b_out=ctx.b_grid)      # gradient with respect to u
-        return (*_gradients_from(ctx, g), None, None, None, None, None, None)
+        return (*_gradients_from(ctx, g), None, None, None, None, None, None, None)
 
 
 class _SynthesisBNReLUIntegrate(torch.autograd.Function):
@@ -105,33 +99,35 @@ class _SynthesisBNReLUIntegrate(torch.autograd.Function):
     network (examples/shrec17/model.py:36-45).  The integral applies the normalisation and the activation in its loads."""
 
     @staticmethod
-    def forward(ctx, zr, conv_bias, weight, bias, running_mean, running_var, b_grid, eps, training):  # pylint: disable=W
-        y, ab, mean, var = _synthesis_and_statistics(ctx, zr, conv_bias, weight, bias, running_mean, running_var, b_grid, eps, training)
+    def forward(ctx, zr, conv_bias, weight, bias, running_mean, running_var, b_grid, eps, training, momentum):  # pylint: disable=W
+        y, ab = _synthesis_and_statistics(ctx, zr, conv_bias, weight, bias, running_mean, running_var, b_grid, eps, training, momentum)
         batch, nf = y.shape[:2]
         out = y.new_empty((batch, nf))
         _hip.call("s2cnn_so3_integrate_affine_relu", _hip.ptr(y), _hip.ptr(ab), nf, _hip.ptr(_setup_so3_integrate(b_grid, y.device)),
                   _hip.ptr(out), b_grid, batch * nf, _hip.stream_ptr())
-        return out, mean, var
+        return out
 
     @staticmethod
-    def backward(ctx, gout, _gm, _gv):  # pylint: disable=W
+    def backward(ctx, gout):  # pylint: disable=W
         y = ctx.saved_tensors[0]
         g = torch.empty_like(y)                                                          # gradient with respect to u: gout[z] w[beta]
         _hip.call("s2cnn_so3_integrate_grad", _hip.ptr(gout.contiguous()), _hip.ptr(_setup_so3_integrate(ctx.b_grid, y.device)), _hip.ptr(g),
                   ctx.b_grid, gout.numel(), _hip.stream_ptr())
-        return (*_gradients_from(ctx, g), None, None, None, None, None)
+        return (*_gradients_from(ctx, g), None, None, None, None, None, None)
 
 
-def _update_running_statistics(bn, mean, var_biased, count):
-    """What nn.BatchNorm3d does to its buffers in training mode (unbiased variance, momentum or cumulative average)."""
-    if not bn.track_running_stats or bn.running_mean is None:
-        return
-    with torch.no_grad():
-        bn.num_batches_tracked += 1
-        momentum = 1.0 / float(bn.num_batches_tracked) if bn.momentum is None else bn.momentum
-        unbiased = var_biased * (count / max(count - 1, 1))
-        bn.running_mean.mul_(1 - momentum).add_(mean.to(bn.running_mean.dtype), alpha=momentum)
-        bn.running_var.mul_(1 - momentum).add_(unbiased.to(bn.running_var.dtype), alpha=momentum)
+def _statistics_mode(bn):
+    """(training, momentum, running_mean, running_var) as nn.BatchNorm3d uses them, and its step counter moved on."""
+    training = bn.training or not bn.track_running_stats
+    momentum = 0.0
+    if bn.training and bn.track_running_stats and bn.running_mean is not None:
+        with torch.no_grad():
+            bn.num_batches_tracked += 1
+        momentum = 1.0 / float(bn.num_batches_tracked) if bn.momentum is None else bn.momentum     # None: cumulative average
+        return training, momentum, bn.running_mean, bn.running_var
+    if training:
+        return training, momentum, None, None
+    return training, momentum, bn.running_mean, bn.running_var
 
 
 def _normalised(conv, bn, act):
@@ -160,11 +156,8 @@ def run_sequence(sequence, x, integrate=False):
         bn, nxt = mods[i], mods[i + 2]
         if zr is None:
             zr = conv.product_spectrum(x)
-        training = bn.training or not bn.track_running_stats
-        xh, mean, var = _SynthesisBNReLUAnalysis.apply(zr, conv.bias, bn.weight, bn.bias, bn.running_mean, bn.running_var,
-                                                       conv.b_out, nxt.b_out, bn.eps, training)
-        if bn.training:
-            _update_running_statistics(bn, mean, var, x.size(0) * (2 * conv.b_out) ** 3)
+        training, momentum, rmean, rvar = _statistics_mode(bn)
+        xh = _SynthesisBNReLUAnalysis.apply(zr, conv.bias, bn.weight, bn.bias, rmean, rvar, conv.b_out, nxt.b_out, bn.eps, training, momentum)
         conv = nxt
         zr = conv.product_spectrum(None, xh)
         i += 3
@@ -172,12 +165,8 @@ def run_sequence(sequence, x, integrate=False):
         bn = mods[i]
         if zr is None:
             zr = conv.product_spectrum(x)
-        training = bn.training or not bn.track_running_stats
-        out, mean, var = _SynthesisBNReLUIntegrate.apply(zr, conv.bias, bn.weight, bn.bias, bn.running_mean, bn.running_var,
-                                                         conv.b_out, bn.eps, training)
-        if bn.training:
-            _update_running_statistics(bn, mean, var, x.size(0) * (2 * conv.b_out) ** 3)
-        return out
+        training, momentum, rmean, rvar = _statistics_mode(bn)
+        return _SynthesisBNReLUIntegrate.apply(zr, conv.bias, bn.weight, bn.bias, rmean, rvar, conv.b_out, bn.eps, training, momentum)
     y = conv(x) if zr is None else conv.from_spectrum(zr)
     for m in mods[i:]:
         y = m(y)

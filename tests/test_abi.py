@@ -44,7 +44,9 @@ def test_argument_rejection_without_gpu():
     assert lib.s2cnn_so3_analysis_workspace(32, 32, 256, 0) == 256 * 28 * 512 * 16 + packed   # one record per volume (7 items x 4 float4 x 512 threads), no intermediate planes
     assert lib.s2cnn_so3_synthesis_workspace(40, 32, 256, 0) == 256 * 28 * 512 * 16 + packed
     packed16 = lib.s2cnn_so3_packed_table_bytes(16, 16, 0)
-    assert packed16 == 31 * 32 * 1024 * 4
+    assert packed16 == 31 * 32 * 256 * 4                                            # small problems: 16 x 16 table values per beta
+    assert lib.s2cnn_so3_packed_table_bytes(16, 16, 1) == 31 * 16 * 16 * 32 * 4        # ... and a 16 x 32 tile per degree in the synthesis
+    assert lib.s2cnn_so3_packed_table_bytes(22, 22, 0) == 43 * 44 * 1024 * 4 and lib.s2cnn_so3_packed_table_bytes(22, 22, 1) == 43 * 22 * 2048 * 4
     assert lib.s2cnn_so3_analysis_workspace(16, 16, 256, 0) == 256 * 32 * 31 * 16 * 8 + packed16
     assert lib.s2cnn_so3_analysis(ctypes.c_void_p(0x1008), fake, fake, fake, null, 0, 32, 32, 1, 0, null) == -3   # 64^3 real input: 16-byte alignment
     assert lib.s2cnn_so3_synthesis_workspace(4, 6, 3, 1) == 16 * 12 * 7 * 7 * 8      # batch padded to the z tile, no fast path
