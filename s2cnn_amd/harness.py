@@ -80,7 +80,7 @@ class Shrec17Model(nn.Module):
 
     def forward(self, x):  # pylint: disable=W0221
         if self.fused_norm:
-            x = run_sequence(self.sequential, x, integrate=True)      # [batch, feature]
+            x = run_sequence(self.sequential, x, head="integrate")    # [batch, feature]
         else:
             x = so3_integrate(self.sequential(x))                     # [batch, feature, beta, alpha, gamma] -> [batch, feature]
         return F.log_softmax(self.out_layer(x), dim=1)
@@ -98,8 +98,11 @@ class Shrec17ModelOriginal(nn.Module):
         self.out_layer = nn.Sequential(nn.BatchNorm1d(self.features[-2], affine=False), nn.Linear(self.features[-2], self.features[-1]))
 
     def forward(self, x):  # pylint: disable=W0221
-        x = run_sequence(self.sequential, x) if self.fused_norm else self.sequential(x)
-        x = x.view(x.size(0), x.size(1), -1).max(-1)[0]
+        if self.fused_norm:
+            x = run_sequence(self.sequential, x, head="max")          # [batch, feature]
+        else:
+            x = self.sequential(x)
+            x = x.view(x.size(0), x.size(1), -1).max(-1)[0]
         return F.log_softmax(self.out_layer(x), dim=1)
 
 

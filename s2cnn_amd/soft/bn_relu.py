@@ -116,6 +116,32 @@ class _SynthesisBNReLUIntegrate(torch.autograd.Function):
         return (*_gradients_from(ctx, g), None, None, None, None, None, None)
 
 
+class _SynthesisBNReLUMax(torch.autograd.Function):
+    """z_hat of the last layer -> the maximum over the grid of max(batch_norm(y), 0), [batch, feature]: the end of the
+    reference's original shape network (examples/shrec17/model_original.py:36-47).  max(a y + b, 0) is monotone in y, so
+    its maximum sits at the largest (a >= 0) or smallest (a < 0) sample of y: the normalised tensor is never formed."""
+
+    @staticmethod
+    def forward(ctx, zr, conv_bias, weight, bias, running_mean, running_var, b_grid, eps, training, momentum):  # pylint: disable=W
+        y, ab = _synthesis_and_statistics(ctx, zr, conv_bias, weight, bias, running_mean, running_var, b_grid, eps, training, momentum)
+        batch, nf = y.shape[:2]
+        flat = y.view(batch, nf, -1)
+        hi, ihi = flat.max(-1)
+        lo, ilo = flat.min(-1)
+        a, b = ab[0].view(1, nf), ab[1].view(1, nf)
+        up = a >= 0
+        ctx.where = torch.where(up, ihi, ilo)                                            # [batch, feature]: the sample that carries the maximum
+        return torch.relu(a * torch.where(up, hi, lo) + b)
+
+    @staticmethod
+    def backward(ctx, gout):  # pylint: disable=W
+        y = ctx.saved_tensors[0]
+        batch, nf = y.shape[:2]
+        g = torch.zeros_like(y)                                                          # gradient with respect to u: one sample per volume
+        g.view(batch, nf, -1).scatter_(-1, ctx.where.unsqueeze(-1), gout.contiguous().unsqueeze(-1))
+        return (*_gradients_from(ctx, g), None, None, None, None, None, None)
+
+
 def _statistics_mode(bn):
     """(training, momentum, running_mean, running_var) as nn.BatchNorm3d uses them, and its step counter moved on."""
     training = bn.training or not bn.track_running_stats
@@ -140,15 +166,23 @@ def _fusable(conv, bn, act, nxt):
             and analysis_prologue_available(nxt.b_in, nxt.b_out))
 
 
-def run_sequence(sequence, x, integrate=False):
+def run_sequence(sequence, x, head=None):
     """`nn.Sequential(conv, [BatchNorm3d, ReLU, SO3Convolution] ..., ...)(x)` with every (BatchNorm3d, ReLU) that stands
     between two spectral layers evaluated inside the transforms of its neighbours.  Same function, same parameters, same
     buffer updates; whatever does not match the pattern runs as the module it is.
-    integrate: return so3_integrate of the result, [batch, feature]; a (BatchNorm3d, ReLU) that ends the sequence is then
-    evaluated in the loads of the integral."""
+    head: None, or what follows the sequence in the reference's networks, with a (BatchNorm3d, ReLU) that ends the sequence
+    evaluated inside it: "integrate" = so3_integrate of the result (the pair in the loads of the integral), "max" = the
+    maximum over the grid (taken on the samples before the pair); either returns [batch, feature]."""
+    assert head in (None, "integrate", "max"), head
+
+    def finish(y):
+        if head == "integrate":
+            return so3_integrate(y)
+        return y.view(y.size(0), y.size(1), -1).max(-1)[0] if head == "max" else y
+
     mods = list(sequence)
     if not mods or not hasattr(mods[0], "product_spectrum") or not x.is_cuda:
-        return so3_integrate(sequence(x)) if integrate else sequence(x)
+        return finish(sequence(x))
     conv = mods[0]
     zr = None
     i = 1
@@ -161,13 +195,14 @@ def run_sequence(sequence, x, integrate=False):
         conv = nxt
         zr = conv.product_spectrum(None, xh)
         i += 3
-    if integrate and len(mods) == i + 2 and _normalised(conv, mods[i], mods[i + 1]):
+    if head is not None and len(mods) == i + 2 and _normalised(conv, mods[i], mods[i + 1]):
         bn = mods[i]
         if zr is None:
             zr = conv.product_spectrum(x)
         training, momentum, rmean, rvar = _statistics_mode(bn)
-        return _SynthesisBNReLUIntegrate.apply(zr, conv.bias, bn.weight, bn.bias, rmean, rvar, conv.b_out, bn.eps, training, momentum)
+        last = _SynthesisBNReLUIntegrate if head == "integrate" else _SynthesisBNReLUMax
+        return last.apply(zr, conv.bias, bn.weight, bn.bias, rmean, rvar, conv.b_out, bn.eps, training, momentum)
     y = conv(x) if zr is None else conv.from_spectrum(zr)
     for m in mods[i:]:
         y = m(y)
-    return so3_integrate(y) if integrate else y
+    return finish(y)

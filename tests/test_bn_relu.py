@@ -109,13 +109,13 @@ def _sequence(sizes, feats, seed, **bn_kwargs):
     return seq
 
 
-@pytest.mark.parametrize("integrate", [False, True])       # True: so3_integrate after the sequence, the last pair in its loads
+@pytest.mark.parametrize("head", [None, "integrate", "max"])       # what follows the sequence, with the last pair inside it
 @pytest.mark.parametrize("sizes,feats,bn_kwargs", [
     ((12, 8, 6, 4), (2, 4, 5, 3), {}),                                       # small grids: folded plane kernels
     ((40, 32, 22, 7), (2, 3, 4, 3), {}),                                     # 64^3 and 44^3: per-volume kernels, truncated spectra
     ((12, 8, 6, 4), (2, 4, 5, 3), {"affine": False, "momentum": None}),      # no weights, cumulative running averages
     ((10, 8, 6), (2, 4, 5), {"track_running_stats": False})])                # batch statistics in evaluation mode as well
-def test_sequence_with_fused_normalisation(hip, sizes, feats, bn_kwargs, integrate):
+def test_sequence_with_fused_normalisation(hip, sizes, feats, bn_kwargs, head):
     import copy
     fus = _sequence(sizes, feats, 5, **bn_kwargs).cuda()
     ref = _as_checker(copy.deepcopy(fus))
@@ -142,8 +142,11 @@ def test_sequence_with_fused_normalisation(hip, sizes, feats, bn_kwargs, integra
         ref.train(mode == "train")
         fus.train(mode == "train")
         xa, xb = x.clone().requires_grad_(), x.clone().requires_grad_()
-        if integrate:
-            ya, yb = s2cnn_amd.so3_integrate(ref(xa)), bn_relu.run_sequence(fus, xb, integrate=True)
+        if head == "integrate":
+            ya, yb = s2cnn_amd.so3_integrate(ref(xa)), bn_relu.run_sequence(fus, xb, head=head)
+        elif head == "max":
+            out = ref(xa)
+            ya, yb = out.view(out.size(0), out.size(1), -1).max(-1)[0], bn_relu.run_sequence(fus, xb, head=head)
         else:
             ya, yb = ref(xa), bn_relu.run_sequence(fus, xb)
         assert _rel(yb, ya) < 1e-4, (mode, _rel(yb, ya))
