@@ -56,6 +56,19 @@ def test_argument_rejection_without_gpu():
     assert lib.s2cnn_so3_packed_table_bytes(70, 70, 0) == 0 and lib.s2cnn_so3_packed_table_bytes(70, 70, 1) == 0
     assert lib.s2cnn_so3_pack_table(fake, fake, 70, 70, 0, null) == -1
     assert b"workspace" in lib.s2cnn_strerror(-2)
+    # the normalisation inside the transforms: where the loads can do it, and what the entries refuse before any launch
+    assert lib.s2cnn_so3_analysis_prologue_available(32, 32) == 1 and lib.s2cnn_so3_analysis_prologue_available(22, 7) == 1
+    assert lib.s2cnn_so3_analysis_prologue_available(32, 40) == 0            # 64-point planes outside the per-volume kernels
+    assert lib.s2cnn_so3_analysis_real_affine_relu(fake, fake, 3, fake, null, fake, fake, 1 << 30, 32, 40, 3, 0, null) == -1
+    assert lib.s2cnn_so3_analysis_real_affine_relu(fake, fake, 3, fake, null, fake, fake, 1 << 30, 22, 22, 4, 0, null) == -1   # 4 volumes, 3 features
+    assert lib.s2cnn_so3_analysis_real_bn_relu_grad(fake, null, fake, 3, fake, null, fake, fake, 1 << 30, 22, 22, 3, 0, null) == -1   # no second tensor
+    assert lib.s2cnn_volume_moments(null, fake, 3, 8, null) == -1
+    assert lib.s2cnn_bn_relu_grad_moments(fake, fake, fake, 2, fake, 3, 8, null) == -1                  # 3 volumes, 2 features
+    assert lib.s2cnn_bn_forward_from_moments(fake, 2, 3, 16.0, null, null, null, null, 1e-5, 0.1, 0, fake, fake, null) == -1   # evaluation mode without running statistics
+    assert lib.s2cnn_bn_backward_from_moments(fake, 0, 3, 16.0, fake, fake, 1, fake, fake, null) == -1
+    assert lib.s2cnn_so3_integrate_affine_relu(fake, fake, 2, fake, fake, 4, 3, null) == -1              # 3 volumes, 2 features
+    assert lib.s2cnn_so3_fft64_probe(fake, fake, fake, fake, 1 << 30, 2, 1, 2, null) == -1               # the synthesis has no probe 2
+    assert lib.s2cnn_so3_fft64_probe(fake, fake, fake, fake, 0, 2, 0, 1, null) == -2                     # workspace too small
     # entry points of the real-basis path and the biased synthesis
     assert lib.s2cnn_s2_mm_real_fwd(null, null, null, 4, 2, 3, 5, null) == -1
     assert lib.s2cnn_s2_mm_real_gradx(fake, fake, fake, 4, 0, 3, 5, null) == -1                # empty batch
