@@ -361,6 +361,15 @@ def measure_example_network(torch, name, steps, warmup, batch=32):
         out["fused_norm"] = {"ms_per_step": round(fms, 3), "samples_per_s": round(batch / (fms * 1e-3), 1),
                              "first_loss": round(flosses[0], 4), "last_loss": round(flosses[-1], 4),
                              "library_ms": round(sum(fcalls.values()), 3), "library_calls_ms": fcalls}
+        # ... and that step captured into one HIP graph and replayed
+        del model
+        torch.cuda.empty_cache()
+        torch.manual_seed(0)
+        fused = harness.NETWORKS[name][0]()
+        fused.fused_norm = True
+        _, rlosses, rms = harness.train_steps_replayed(name, batch=batch, steps=steps, warmup=3, lr=0.01, model=fused)
+        out["fused_norm"]["graph_replay"] = {"ms_per_step": round(rms, 3), "samples_per_s": round(batch / (rms * 1e-3), 1),
+                                             "last_loss": round(rlosses[-1], 4)}
     return out
 
 

@@ -106,3 +106,20 @@ def test_digit_network_step_replayed_from_a_hip_graph(hip):
     _, replayed, _ = harness.train_steps_replayed("mnist", batch=16, steps=5, warmup=3, lr=0.05)
     print("eager", ["%.5f" % l for l in eager[3:]], "replayed", ["%.5f" % l for l in replayed], flush=True)
     assert max(abs(a - b) for a, b in zip(eager[3:], replayed)) < 1e-5 * abs(eager[0])
+
+
+@pytest.mark.gpu
+def test_shape_network_step_replayed_from_a_hip_graph(hip):
+    """The training step of the SHREC17 network with the normalisations inside the transforms, captured into one HIP
+    graph (statistics, running averages and the step counter of the BatchNorm3d modules included): the replayed steps
+    continue the eager ones with the same losses, and the buffers end where the all-eager run's do."""
+    torch.manual_seed(0)
+    eager_net = harness.Shrec17Model(55, fused_norm=True)
+    torch.manual_seed(0)
+    replay_net = harness.Shrec17Model(55, fused_norm=True)
+    _, eager, _ = harness.train_steps("shrec17", batch=4, steps=4, warmup=3, lr=0.02, model=eager_net)
+    _, replayed, _ = harness.train_steps_replayed("shrec17", batch=4, steps=4, warmup=3, lr=0.02, model=replay_net)
+    print("eager", ["%.5f" % l for l in eager[3:]], "replayed", ["%.5f" % l for l in replayed], flush=True)
+    assert max(abs(a - b) for a, b in zip(eager[3:], replayed)) < 1e-5 * abs(eager[0])
+    for (name, a), (_, b) in zip(eager_net.named_buffers(), replay_net.named_buffers()):
+        assert torch.allclose(a.float(), b.float(), rtol=1e-5, atol=1e-6), name
