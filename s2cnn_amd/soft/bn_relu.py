@@ -181,8 +181,8 @@ def run_sequence(sequence, x, head=None):
         return y.view(y.size(0), y.size(1), -1).max(-1)[0] if head == "max" else y
 
     mods = list(sequence)
-    if not mods or not hasattr(mods[0], "product_spectrum") or not x.is_cuda:
-        return finish(sequence(x))
+    if not mods or not hasattr(mods[0], "product_spectrum") or not x.is_cuda or x.size(0) == 0:
+        return finish(sequence(x))      # nothing to fuse (an empty batch behaves as the modules themselves do)
     conv = mods[0]
     zr = None
     i = 1
