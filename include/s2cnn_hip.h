@@ -266,17 +266,28 @@ int s2cnn_so3_integrate_affine_relu(const float *x, const float *params, int nfe
 int s2cnn_volume_moments(const float *x, float *out, long nvol, long n, void *stream);
 int s2cnn_bn_relu_grad_moments(const float *g, const float *y, const float *params, int nfeature, float *out,
                                long nvol, long n, void *stream);
+/* Where the synthesis that produces y (or the gradient g) stages whole planes in LDS it can form those sums itself, one
+ * pair per plane, and the separate read is not needed: s2cnn_so3_synthesis_moment_parts(b_in, b_out) = 2 b_out where
+ * s2cnn_so3_synthesis_real_moments can do that (real signals, complex spectrum; other arguments as
+ * s2cnn_so3_synthesis_real_bias), else 0.  moments [nbatch][2 b_out][2]; yref = NULL: (sum y, sum y^2) of the output;
+ * yref = the tensor y and params = ab: (sum g m, sum g m y) with the output as g. */
+int s2cnn_so3_synthesis_moment_parts(int b_in, int b_out);
+int s2cnn_so3_synthesis_real_moments(const float *xhat, const float *table, const float *packed_table, float *out,
+                                     void *workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
+                                     const float *bias, int nfeature, float *moments, const float *yref,
+                                     const float *params, void *stream);
 /* the arithmetic between those calls, one small launch each instead of a chain of tensor operations (float64 inside):
- * forward : moments [batch][nfeature][2] of s2cnn_volume_moments, count = samples per feature -> ab [2][nfeature] for the
+ * forward : moments [batch][nfeature][parts][2] (parts = 1 from s2cnn_volume_moments, 2 b from the synthesis above),
+ *           count = samples per feature -> ab [2][nfeature] for the
  *           analysis, stats [4][nfeature] = batch mean, biased batch variance, mean in use, 1/sqrt(var in use + eps)
  *           (in use: the batch's when training != 0, else running_mean / running_var); when training and the running
  *           buffers are given they move by `momentum` (unbiased variance), as nn.BatchNorm3d does; weight, bias: NULL = 1, 0
  * backward: moments of s2cnn_bn_relu_grad_moments -> params [4][nfeature] for s2cnn_so3_analysis_real_bn_relu_grad and
  *           gwb [2][nfeature] = the gradients of weight and bias */
-int s2cnn_bn_forward_from_moments(const float *moments, int batch, int nfeature, double count, const float *weight,
+int s2cnn_bn_forward_from_moments(const float *moments, int batch, int nfeature, int parts, double count, const float *weight,
                                   const float *bias, float *running_mean, float *running_var, double eps, double momentum,
                                   int training, float *ab, float *stats, void *stream);
-int s2cnn_bn_backward_from_moments(const float *moments, int batch, int nfeature, double count, const float *ab,
+int s2cnn_bn_backward_from_moments(const float *moments, int batch, int nfeature, int parts, double count, const float *ab,
                                    const float *stats, int training, float *params, float *gwb, void *stream);
 int s2cnn_so3_analysis_real_affine_relu(const float *x, const float *params, int nfeature,
                                         const float *table, const float *packed_table, float *out,

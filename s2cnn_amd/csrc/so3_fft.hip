@@ -518,10 +518,27 @@ int analysis_impl(const s2cnn::Input& in, const float* table, const float* packe
   return s2cnn::launch_status();
 }
 
+// Sums over the planes of the output that the synthesis can form where it stages whole planes in LDS (the folded plane
+// kernel in its one-round mode): see plane_real::plane_dft_inv.
+struct PlaneMoments {
+  float* out = nullptr;            // [nbatch * 2 b_out][2]
+  const float* yref = nullptr;
+  const float* params = nullptr;   // [2][nfeature]
+};
+
+// 2 b_out (the sums come per plane) where the real synthesis b_in -> b_out can form them, else 0
+int moment_parts(int b_in, int b_out) {
+  if (!sizes_ok(b_out, b_in, 1) || fused_path(b_out, b_in, 0, true) || 2 * b_out == 64) return 0;
+  const plane_real::Plan plan = plane_real::plan_inv(2 * b_out, b_in < b_out ? b_in : b_out, 2 * b_out);
+  return plan.pl > 0 && plan.alias ? 2 * b_out : 0;
+}
+
 int synthesis_impl(const float* xhat, const float* table, const float* packed_table, float* out, void* workspace,
                    size_t workspace_bytes, int b_in, int b_out, long nbatch, int complex_out, const float* bias, int nfeature,
-                   int relu, unsigned long long* bits, void* stream) {
+                   int relu, unsigned long long* bits, void* stream, const PlaneMoments& mom = PlaneMoments()) {
   if (!xhat || !table || !out || !sizes_ok(b_out, b_in, nbatch)) return S2CNN_EINVAL;
+  if (mom.out && (complex_out || moment_parts(b_in, b_out) == 0 || !s2cnn::aligned8(mom.out))) return S2CNN_EINVAL;
+  if (mom.yref && (!mom.params || nfeature < 1 || nbatch % nfeature != 0)) return S2CNN_EINVAL;
   if (bits && !fused_path(b_out, b_in, complex_out, true)) return S2CNN_EINVAL;
   if (bias && (complex_out || nfeature < 1 || nbatch % nfeature != 0)) return S2CNN_EINVAL;
   if (relu && complex_out) return S2CNN_EINVAL;
@@ -571,7 +588,8 @@ int synthesis_impl(const float* xhat, const float* table, const float* packed_ta
   } else if (plan.pl > 0) {
     if (plan.lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)plane_real::plane_dft_inv, hipFuncAttributeMaxDynamicSharedMemorySize, (int)plan.lds);
     hipLaunchKernelGGL(plane_real::plane_dft_inv, dim3((planes + plan.pl - 1) / plan.pl), dim3(plan.nt), plan.lds, st, S, out, n2, nb,
-                       (long)planes, plan.pl, plan.alias, relu, bias, bias ? nfeature : 1);
+                       (long)planes, plan.pl, plan.alias, relu, bias, (bias || mom.yref) ? nfeature : 1,
+                       reinterpret_cast<float2*>(mom.out), mom.yref, mom.params);
     return s2cnn::launch_status();
   } else {
     if (lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)so3_plane_dft_inv<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -670,6 +688,19 @@ extern "C" int s2cnn_so3_analysis_real_masked_bits(const float* x, const void* b
   if (s2cnn_so3_relu_bits_bytes(b_in, nbatch) == 0) return S2CNN_EINVAL;
   return analysis_prologue_impl(s2cnn::Input{x, static_cast<const float*>(bits), s2cnn::PRO_BITS}, table, packed_table, out, workspace,
                                 workspace_bytes, b_in, b_out, nbatch, real_basis, stream);
+}
+
+extern "C" int s2cnn_so3_synthesis_moment_parts(int b_in, int b_out) { return moment_parts(b_in, b_out); }
+
+extern "C" int s2cnn_so3_synthesis_real_moments(const float* xhat, const float* table, const float* packed_table, float* out,
+                                                void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
+                                                const float* bias, int nfeature, float* moments, const float* yref,
+                                                const float* params, void* stream) {
+  s2cnn::clear_stale_error();
+  if (!moments) return S2CNN_EINVAL;
+  PlaneMoments mom;
+  mom.out = moments; mom.yref = yref; mom.params = params;
+  return synthesis_impl(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, 0, bias, nfeature, 0, nullptr, stream, mom);
 }
 
 extern "C" int s2cnn_so3_analysis_prologue_available(int b_in, int b_out) { return prologue_path(b_in, b_out) ? 1 : 0; }

@@ -137,18 +137,37 @@ __global__ __launch_bounds__(256) void volume_moments_kernel(const float* __rest
   if (threadIdx.x == 0) out[z] = make_float2((float)part[0][0], (float)part[1][0]);
 }
 
-// The per-feature arithmetic of the normalisation on the sums of volume_moments_kernel, one thread per feature, float64:
-//   forward : mom [batch][F][2] = (sum y, sum y^2)  ->  mean, biased variance, 1/sqrt(var + eps) of the statistics in use
+// The per-feature arithmetic of the normalisation on the sums of volume_moments_kernel, one workgroup per feature, float64:
+//   forward : mom [batch][F][parts][2] = (sum y, sum y^2), `parts` partial sums per volume  ->  mean, biased variance, 1/sqrt(var + eps) of the statistics in use
 //             (the batch's when training, else the running ones), ab = (a, b) with a = weight / sqrt(var + eps),
 //             b = bias - mean a; when training, the running averages move by `momentum` (unbiased variance).
 //   backward: mom = (sum g m, sum g m y)  ->  params (a, b, p, q) of the load-time gradient, and the gradients of weight and bias.
-__global__ void bn_forward_kernel(const float2* __restrict__ mom, int batch, int nf, double count, const float* __restrict__ weight,
+// The two sums of feature f over its batch x parts partials, by one workgroup of 64 threads in a fixed order (float64).
+__device__ __forceinline__ void feature_sums(const float2* __restrict__ mom, int batch, int nf, int parts, int f, double& s1, double& s2) {
+  __shared__ double red[2][64];
+  double a1 = 0.0, a2 = 0.0;
+  const int total = batch * parts;
+  for (int i = threadIdx.x; i < total; i += 64) {
+    const int b = i / parts, p = i - b * parts;
+    const float2 v = mom[((size_t)b * nf + f) * parts + p];
+    a1 += v.x; a2 += v.y;
+  }
+  red[0][threadIdx.x] = a1; red[1][threadIdx.x] = a2;
+  __syncthreads();
+  for (int s = 32; s > 0; s >>= 1) {
+    if ((int)threadIdx.x < s) { red[0][threadIdx.x] += red[0][threadIdx.x + s]; red[1][threadIdx.x] += red[1][threadIdx.x + s]; }
+    __syncthreads();
+  }
+  s1 = red[0][0]; s2 = red[1][0];
+}
+
+__global__ void bn_forward_kernel(const float2* __restrict__ mom, int batch, int nf, int parts, double count, const float* __restrict__ weight,
                                   const float* __restrict__ bias, float* __restrict__ running_mean, float* __restrict__ running_var,
                                   double eps, double momentum, int training, float* __restrict__ ab, float* __restrict__ stats) {
-  const int f = blockIdx.x * blockDim.x + threadIdx.x;
-  if (f >= nf) return;
-  double s1 = 0.0, s2 = 0.0;
-  for (int b = 0; b < batch; ++b) { const float2 v = mom[(size_t)b * nf + f]; s1 += v.x; s2 += v.y; }
+  const int f = blockIdx.x;
+  double s1, s2;
+  feature_sums(mom, batch, nf, parts, f, s1, s2);
+  if (threadIdx.x != 0) return;
   const double mean = s1 / count;
   double var = s2 / count - mean * mean;
   var = var < 0.0 ? 0.0 : var;
@@ -168,12 +187,12 @@ __global__ void bn_forward_kernel(const float2* __restrict__ mom, int batch, int
   }
 }
 
-__global__ void bn_backward_kernel(const float2* __restrict__ mom, int batch, int nf, double count, const float* __restrict__ ab,
+__global__ void bn_backward_kernel(const float2* __restrict__ mom, int batch, int nf, int parts, double count, const float* __restrict__ ab,
                                    const float* __restrict__ stats, int training, float* __restrict__ params, float* __restrict__ gwb) {
-  const int f = blockIdx.x * blockDim.x + threadIdx.x;
-  if (f >= nf) return;
-  double d1 = 0.0, d2 = 0.0;
-  for (int b = 0; b < batch; ++b) { const float2 v = mom[(size_t)b * nf + f]; d1 += v.x; d2 += v.y; }
+  const int f = blockIdx.x;
+  double d1, d2;
+  feature_sums(mom, batch, nf, parts, f, d1, d2);
+  if (threadIdx.x != 0) return;
   const double mean = stats[2 * nf + f], invstd = stats[3 * nf + f], a = ab[f];
   const double gw = invstd * (d2 - mean * d1);          // sum g m (y - mean) / std
   double p = 0.0, q = 0.0;
@@ -192,26 +211,26 @@ __global__ void bn_backward_kernel(const float2* __restrict__ mom, int batch, in
 
 }  // namespace
 
-extern "C" int s2cnn_bn_forward_from_moments(const float* moments, int batch, int nfeature, double count, const float* weight,
+extern "C" int s2cnn_bn_forward_from_moments(const float* moments, int batch, int nfeature, int parts, double count, const float* weight,
                                              const float* bias, float* running_mean, float* running_var, double eps,
                                              double momentum, int training, float* ab, float* stats, void* stream) {
   s2cnn::clear_stale_error();
-  if (!moments || !ab || !stats || batch < 1 || nfeature < 1 || count < 1.0) return S2CNN_EINVAL;
+  if (!moments || !ab || !stats || batch < 1 || nfeature < 1 || parts < 1 || count < 1.0) return S2CNN_EINVAL;
   if (!training && (!running_mean || !running_var)) return S2CNN_EINVAL;
   if (!s2cnn::aligned8(moments)) return S2CNN_EALIGN;
-  hipLaunchKernelGGL(bn_forward_kernel, dim3((unsigned)((nfeature + 63) / 64)), dim3(64), 0, static_cast<hipStream_t>(stream),
-                     reinterpret_cast<const float2*>(moments), batch, nfeature, count, weight, bias, running_mean, running_var, eps, momentum,
+  hipLaunchKernelGGL(bn_forward_kernel, dim3((unsigned)nfeature), dim3(64), 0, static_cast<hipStream_t>(stream),
+                     reinterpret_cast<const float2*>(moments), batch, nfeature, parts, count, weight, bias, running_mean, running_var, eps, momentum,
                      training, ab, stats);
   return s2cnn::launch_status();
 }
 
-extern "C" int s2cnn_bn_backward_from_moments(const float* moments, int batch, int nfeature, double count, const float* ab,
+extern "C" int s2cnn_bn_backward_from_moments(const float* moments, int batch, int nfeature, int parts, double count, const float* ab,
                                               const float* stats, int training, float* params, float* gwb, void* stream) {
   s2cnn::clear_stale_error();
-  if (!moments || !ab || !stats || !params || !gwb || batch < 1 || nfeature < 1 || count < 1.0) return S2CNN_EINVAL;
+  if (!moments || !ab || !stats || !params || !gwb || batch < 1 || nfeature < 1 || parts < 1 || count < 1.0) return S2CNN_EINVAL;
   if (!s2cnn::aligned8(moments)) return S2CNN_EALIGN;
-  hipLaunchKernelGGL(bn_backward_kernel, dim3((unsigned)((nfeature + 63) / 64)), dim3(64), 0, static_cast<hipStream_t>(stream),
-                     reinterpret_cast<const float2*>(moments), batch, nfeature, count, ab, stats, training, params, gwb);
+  hipLaunchKernelGGL(bn_backward_kernel, dim3((unsigned)nfeature), dim3(64), 0, static_cast<hipStream_t>(stream),
+                     reinterpret_cast<const float2*>(moments), batch, nfeature, parts, count, ab, stats, training, params, gwb);
   return s2cnn::launch_status();
 }
 

@@ -296,9 +296,14 @@ __global__ __launch_bounds__(NT_MAX) void plane_dft_fwd(const float* __restrict_
 // ---------------------------------------------------------------------------------------------------
 // bias: NULL, or nfeature values; bias[z % nfeature] is added to every sample of volume z = plane / n2
 // relu: nonzero = negative samples (after the bias) are stored as zero
+// moments (alias mode only): NULL, or [nplanes] pairs of sums over each plane of the output v, formed from the staged
+// planes in a fixed order: yref == NULL: (sum v, sum v^2); else, with m = (a yref + b > 0), a = params[f],
+// b = params[nfeature + f] of the plane's feature f: (sum v m, sum v m yref): what a batch normalisation over the
+// volumes of a feature needs of its input, or (v being the gradient with respect to its activated output) of its gradient.
 __global__ __launch_bounds__(NT_MAX) void plane_dft_inv(const float2* __restrict__ S, float* __restrict__ y, int n2, int nb,
                                                         long nplanes, int PL, int alias, int relu, const float* __restrict__ bias,
-                                                        int nfeature) {
+                                                        int nfeature, float2* __restrict__ moments, const float* __restrict__ yref,
+                                                        const float* __restrict__ params) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
   const int h = n2 / 2, hp = pad(h + 1, 4), nb2 = pad(nb, 2), npp = pad(h + 1, 2);
   float2* tab = reinterpret_cast<float2*>(smem);                          // [nb][hp]
@@ -455,6 +460,27 @@ __global__ __launch_bounds__(NT_MAX) void plane_dft_inv(const float2* __restrict
     if (pv > PL) pv = PL;
     const int total = (int)pv * n2 * n2;                 // a multiple of 4
     float* dst = y + (size_t)plane0 * n2 * n2;
+    if (moments) {                                       // one wave per plane at a time, lanes stride over its samples
+      const int lane = t & 63, wave = t >> 6, nwave = NT >> 6, psize = n2 * n2;
+      for (int q = wave; q < (int)pv; q += nwave) {
+        const float* v = Ys + (size_t)q * psize;
+        float s1 = 0.f, s2 = 0.f;
+        if (yref) {
+          const int f = (int)(((plane0 + q) / n2) % nfeature);
+          const float a = params[f], b = params[nfeature + f];
+          const float* yr = yref + (size_t)(plane0 + q) * psize;
+          for (int i = lane; i < psize; i += 64) {
+            const float yv = yr[i], gm = s2cnn::relu_pass(v[i], fmaf(a, yv, b));
+            s1 += gm; s2 = fmaf(gm, yv, s2);
+          }
+        } else {
+          for (int i = lane; i < psize; i += 64) { const float x = v[i]; s1 += x; s2 = fmaf(x, x, s2); }
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) { s1 += __shfl_xor(s1, o); s2 += __shfl_xor(s2, o); }
+        if (lane == 0) moments[plane0 + q] = make_float2(s1, s2);
+      }
+    }
     if ((reinterpret_cast<uintptr_t>(y) & 15u) == 0) {
       for (int i = t; i < total / 4; i += NT) reinterpret_cast<float4*>(dst)[i] = reinterpret_cast<const float4*>(Ys)[i];
     } else {

@@ -21,7 +21,7 @@ from .. import _hip
 from .so3_conv import SO3Convolution
 from .so3_integrate import _setup_so3_integrate, so3_integrate
 from .so3_fft import (LoadAffineReLU, LoadBNReLUGrad, analysis_prologue_available, so3_rfft_real_basis,
-                      so3_rifft_real_basis)
+                      so3_rifft_real_basis, synthesis_moment_parts)
 
 
 def _moments(name, n_per_volume, *operands):
@@ -45,17 +45,23 @@ def _synthesis_and_statistics(ctx, zr, conv_bias, weight, bias, running_mean, ru
     ctx.b_z = round((3 / 4 * nspec) ** (1 / 3))
     ctx.b_grid, ctx.training = b_grid, training
     ctx.bias_shape = conv_bias.shape
-    y = so3_rifft_real_basis(zr, b_out=b_grid, bias=conv_bias)                       # [batch, feature, 2b, 2b, 2b]
     nvox = (2 * b_grid) ** 3
     ctx.count = batch * nvox
-    mom = _moments("s2cnn_volume_moments", nvox, y)                                  # [batch * feature, 2]
+    parts = synthesis_moment_parts(ctx.b_z, b_grid)                # > 0: the synthesis forms the sums itself, one pair per plane
+    if parts:
+        mom = zr.new_empty((batch * nf * parts, 2))
+        y = so3_rifft_real_basis(zr, b_out=b_grid, bias=conv_bias, moments=(mom, None, None))
+    else:
+        parts = 1
+        y = so3_rifft_real_basis(zr, b_out=b_grid, bias=conv_bias)                   # [batch, feature, 2b, 2b, 2b]
+        mom = _moments("s2cnn_volume_moments", nvox, y)                              # [batch * feature, 2]
     ab = y.new_empty((2, nf))
     stats = y.new_empty((4, nf))          # batch mean, biased batch variance, mean in use, 1 / sqrt(variance in use + eps)
     for t in (weight, bias, running_mean, running_var):
         if t is not None:
             _hip.require_gpu_f32(t)
             assert t.is_contiguous() and t.numel() == nf
-    _hip.call("s2cnn_bn_forward_from_moments", _hip.ptr(mom), batch, nf, float(ctx.count), _ptr_or_none(weight), _ptr_or_none(bias),
+    _hip.call("s2cnn_bn_forward_from_moments", _hip.ptr(mom), batch, nf, parts, float(ctx.count), _ptr_or_none(weight), _ptr_or_none(bias),
               _ptr_or_none(running_mean), _ptr_or_none(running_var), float(eps), float(momentum), int(training), _hip.ptr(ab),
               _hip.ptr(stats), _hip.stream_ptr())
     ctx.save_for_backward(y, ab, stats)
@@ -63,16 +69,18 @@ def _synthesis_and_statistics(ctx, zr, conv_bias, weight, bias, running_mean, ru
     return y, ab
 
 
-def _gradients_from(ctx, g):
-    """g: the gradient with respect to u = max(a y + b, 0).  Returns the gradients with respect to the spectrum zr, the
-    bias of the layer, and the weight and bias of the normalisation."""
+def _gradients_from(ctx, g, mom=None, parts=1):
+    """g: the gradient with respect to u = max(a y + b, 0); mom: its sums (sum g m, sum g m y), `parts` pairs per volume, if
+    the kernel that produced g has formed them.  Returns the gradients with respect to the spectrum zr, the bias of the
+    layer, and the weight and bias of the normalisation."""
     y, ab, stats = ctx.saved_tensors
     batch, nf = y.shape[:2]
     nvox = (2 * ctx.b_grid) ** 3
-    mom = _moments("s2cnn_bn_relu_grad_moments", nvox, g, y, ab, nf)                 # sum g m, sum g m y per volume
+    if mom is None:
+        mom = _moments("s2cnn_bn_relu_grad_moments", nvox, g, y, ab, nf)             # per volume
     params = y.new_empty((4, nf))
     gwb = y.new_empty((2, nf))
-    _hip.call("s2cnn_bn_backward_from_moments", _hip.ptr(mom), batch, nf, float(ctx.count), _hip.ptr(ab), _hip.ptr(stats),
+    _hip.call("s2cnn_bn_backward_from_moments", _hip.ptr(mom), batch, nf, parts, float(ctx.count), _hip.ptr(ab), _hip.ptr(stats),
               int(ctx.training), _hip.ptr(params), _hip.ptr(gwb), _hip.stream_ptr())
     gz = so3_rfft_real_basis(g, for_grad=True, b_out=ctx.b_z, mask=LoadBNReLUGrad(y, params))
     g_conv_bias = gz[0].reshape(-1, nf).sum(0).reshape(ctx.bias_shape) if ctx.needs_input_grad[1] else None
@@ -90,7 +98,15 @@ class _SynthesisBNReLUAnalysis(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, gxh):  # pylint: disable=W
-        g = so3_rifft_real_basis(gxh.contiguous(), for_grad=True, b_out=ctx.b_grid)      # gradient with respect to u
+        gxh = gxh.contiguous()
+        b_next = round((3 / 4 * gxh.size(0)) ** (1 / 3))
+        parts = synthesis_moment_parts(b_next, ctx.b_grid)
+        if parts:           # the synthesis that produces the gradient with respect to u forms its two sums as well
+            y, ab, _ = ctx.saved_tensors
+            mom = gxh.new_empty((y.size(0) * y.size(1) * parts, 2))
+            g = so3_rifft_real_basis(gxh, for_grad=True, b_out=ctx.b_grid, moments=(mom, y, ab))
+            return (*_gradients_from(ctx, g, mom, parts), None, None, None, None, None, None, None)
+        g = so3_rifft_real_basis(gxh, for_grad=True, b_out=ctx.b_grid)                   # gradient with respect to u
         return (*_gradients_from(ctx, g), None, None, None, None, None, None, None)
 
 

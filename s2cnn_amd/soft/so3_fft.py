@@ -144,8 +144,14 @@ def _analysis(x, b_in, b_out, batch_size, for_grad, complex_in, mask=None):
     return out
 
 
-def _synthesis(x, b_in, b_out, batch_size, for_grad, complex_out, bias=None, relu=False, bits=None):
-    """bits (with relu): an int64 tensor from `_relu_bits` that receives one bit per sample (the output is not <= 0)."""
+def synthesis_moment_parts(b_in, b_out):
+    """How many pairs of sums per volume the real synthesis b_in -> b_out can form while it writes its output (0: none)."""
+    return _hip.lib().s2cnn_so3_synthesis_moment_parts(b_in, b_out)
+
+
+def _synthesis(x, b_in, b_out, batch_size, for_grad, complex_out, bias=None, relu=False, bits=None, moments=None):
+    """bits (with relu): an int64 tensor from `_relu_bits` that receives one bit per sample (the output is not <= 0).
+    moments: None, or (out [volumes * parts, 2], yref or None, params or None) for s2cnn_so3_synthesis_real_moments."""
     _hip.require_gpu_f32(x)
     assert not (relu and complex_out)
     if complex_out and complex_via_real:
@@ -170,6 +176,14 @@ def _synthesis(x, b_in, b_out, batch_size, for_grad, complex_out, bias=None, rel
         _hip.require_gpu_f32(bias)
         bias = bias.reshape(-1).contiguous()
         assert len(batch_size) >= 1 and batch_size[-1] == bias.numel()
+    if moments is not None:
+        assert not relu and not complex_out
+        mom, yref, params = moments
+        nfeature = params.size(1) if params is not None else (1 if bias is None else bias.numel())
+        _hip.call("s2cnn_so3_synthesis_real_moments", _hip.ptr(x), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out), _hip.ptr(ws),
+                  ws.numel(), b_in, b_out, nbatch, _null_or_ptr(bias), nfeature, _hip.ptr(mom), _null_or_ptr(yref), _null_or_ptr(params),
+                  _hip.stream_ptr())
+        return out
     if relu and bits is not None:
         _hip.call("s2cnn_so3_synthesis_real_relu_bits", _hip.ptr(x), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out), _hip.ptr(bits),
                   _hip.ptr(ws), ws.numel(), b_in, b_out, nbatch, _null_or_ptr(bias), 1 if bias is None else bias.numel(), 0, _hip.stream_ptr())
@@ -240,7 +254,7 @@ def so3_ifft(x, for_grad=False, b_out=None):
     return _synthesis(x, b_in, b_out, batch_size, for_grad, 1)
 
 
-def so3_rifft(x, for_grad=False, b_out=None, bias=None, relu=False, bits=None):
+def so3_rifft(x, for_grad=False, b_out=None, bias=None, relu=False, bits=None, moments=None):
     '''
     :param x: [l * m * n, ..., complex]
     :param bias: None, or one value per entry of the last batch dimension, added to every sample of its volumes
@@ -249,7 +263,7 @@ def so3_rifft(x, for_grad=False, b_out=None, bias=None, relu=False, bits=None):
     :return: [..., beta, alpha, gamma]  (the real part of so3_ifft, whatever the symmetry of x)
     '''
     x, b_in, b_out, batch_size = _spectrum_args(x, b_out)
-    return _synthesis(x, b_in, b_out, batch_size, for_grad, 0, bias, relu, bits)
+    return _synthesis(x, b_in, b_out, batch_size, for_grad, 0, bias, relu, bits, moments)
 
 
 class SO3_fft_real(torch.autograd.Function):
@@ -344,7 +358,7 @@ def so3_rfft_real_basis(x, for_grad=False, b_out=None, mask=None):
     return out
 
 
-def so3_rifft_real_basis(r, for_grad=False, b_out=None, bias=None, relu=False, bits=None):
+def so3_rifft_real_basis(r, for_grad=False, b_out=None, bias=None, relu=False, bits=None, moments=None):
     '''
     :param r: [l * m * n, ...]  real-basis spectrum
     :param bias: None, or one value per entry of the last batch dimension, added to every sample of its volumes
@@ -358,7 +372,8 @@ def so3_rifft_real_basis(r, for_grad=False, b_out=None, bias=None, relu=False, b
         b_out = b_in
     if not (r.is_cuda and _real_basis_direct(b_in, b_out, True)):
         from ..so3_real import _convert
-        return so3_rifft(_convert("s2cnn_so3_spectrum_to_complex", r.contiguous(), (*r.shape, 2)), for_grad, b_out, bias, relu, bits)
+        return so3_rifft(_convert("s2cnn_so3_spectrum_to_complex", r.contiguous(), (*r.shape, 2)), for_grad, b_out, bias, relu, bits, moments)
+    assert moments is None, "sums per plane come from the two-stage synthesis only (synthesis_moment_parts)"
     _hip.require_gpu_f32(r)
     r = r.contiguous()
     batch_size = r.size()[1:]

@@ -64,8 +64,13 @@ def test_argument_rejection_without_gpu():
     assert lib.s2cnn_so3_analysis_real_bn_relu_grad(fake, null, fake, 3, fake, null, fake, fake, 1 << 30, 22, 22, 3, 0, null) == -1   # no second tensor
     assert lib.s2cnn_volume_moments(null, fake, 3, 8, null) == -1
     assert lib.s2cnn_bn_relu_grad_moments(fake, fake, fake, 2, fake, 3, 8, null) == -1                  # 3 volumes, 2 features
-    assert lib.s2cnn_bn_forward_from_moments(fake, 2, 3, 16.0, null, null, null, null, 1e-5, 0.1, 0, fake, fake, null) == -1   # evaluation mode without running statistics
-    assert lib.s2cnn_bn_backward_from_moments(fake, 0, 3, 16.0, fake, fake, 1, fake, fake, null) == -1
+    assert lib.s2cnn_bn_forward_from_moments(fake, 2, 3, 1, 16.0, null, null, null, null, 1e-5, 0.1, 0, fake, fake, null) == -1   # evaluation mode without running statistics
+    assert lib.s2cnn_bn_backward_from_moments(fake, 0, 3, 1, 16.0, fake, fake, 1, fake, fake, null) == -1
+    # sums per plane out of the synthesis: where it stages whole planes, not on the 64^3 grid
+    assert lib.s2cnn_so3_synthesis_moment_parts(22, 22) == 44 and lib.s2cnn_so3_synthesis_moment_parts(7, 22) == 44
+    assert lib.s2cnn_so3_synthesis_moment_parts(16, 16) == 32 and lib.s2cnn_so3_synthesis_moment_parts(32, 32) == 0
+    assert lib.s2cnn_so3_synthesis_real_moments(fake, fake, null, fake, fake, 1 << 30, 32, 32, 3, null, 1, fake, null, null, null) == -1
+    assert lib.s2cnn_so3_synthesis_real_moments(fake, fake, null, fake, fake, 1 << 30, 22, 22, 4, null, 3, fake, fake, fake, null) == -1   # 4 volumes, 3 features
     assert lib.s2cnn_so3_integrate_affine_relu(fake, fake, 2, fake, fake, 4, 3, null) == -1              # 3 volumes, 2 features
     assert lib.s2cnn_so3_fft64_probe(fake, fake, fake, fake, 1 << 30, 2, 1, 2, null) == -1               # the synthesis has no probe 2
     assert lib.s2cnn_so3_fft64_probe(fake, fake, fake, fake, 0, 2, 0, 1, null) == -2                     # workspace too small
