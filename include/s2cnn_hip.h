@@ -276,6 +276,11 @@ int s2cnn_so3_synthesis_real_moments(const float *xhat, const float *table, cons
                                      void *workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
                                      const float *bias, int nfeature, float *moments, const float *yref,
                                      const float *params, void *stream);
+/* On the 64^3 grid the per-volume synthesis kernel forms (sum y, sum y^2) of the volume it writes: moments [nbatch][2],
+ * other arguments as s2cnn_so3_synthesis_real_basis (real-basis spectrum; -1 where that entry point returns -1). */
+int s2cnn_so3_synthesis_real_basis_moments(const float *r, const float *table, const float *packed_table, float *out,
+                                           void *workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
+                                           const float *bias, int nfeature, float *moments, void *stream);
 /* the arithmetic between those calls, one small launch each instead of a chain of tensor operations (float64 inside):
  * forward : moments [batch][nfeature][parts][2] (parts = 1 from s2cnn_volume_moments, 2 b from the synthesis above),
  *           count = samples per feature -> ab [2][nfeature] for the

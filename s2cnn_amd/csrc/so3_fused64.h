@@ -698,12 +698,15 @@ __global__ __launch_bounds__(256) void spectrum_gather_real(const float* __restr
 // relu: nonzero = negative samples (after the bias) are stored as zero
 // NA as in analysis_kernel; CMAX: degree groups c < CMAX carry degrees of the input (6 for NA = 3, 7 for 5, 8 for 7)
 // PROBE (measurement only, results meaningless): 1: an item's share of a plane pair reduced to one add per table operand.
-template <int NA, int CMAX, int PROBE = 0>
+// MOM: the kernel also writes moments[z] = (sum, sum of squares) of the volume's output (bias included, before the
+// activation), summed in a fixed order: the statistics of a batch normalisation that follows, without a read of their own.
+template <int NA, int CMAX, int PROBE = 0, bool MOM = false>
 __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __restrict__ rec, const float* __restrict__ Tf,
                                                             float* __restrict__ y, long nbatch, const float* __restrict__ bias, int nfeature,
-                                                            int relu, unsigned long long* __restrict__ bits) {
+                                                            int relu, unsigned long long* __restrict__ bits, float2* __restrict__ moments) {
   using namespace fft64;
   __shared__ __attribute__((aligned(16))) float2 work[LDS_ELEMS];
+  float ms1 = 0.f, ms2 = 0.f;
   constexpr int STG_PADS = 144;                                              // one pad per row: sum of (4c+4) over the 8 degree groups
   __shared__ __attribute__((aligned(16))) float4 stg_p[NIT * THREADS + STG_PADS];   // item (c, a, n): its share of the bins [+a,n], [-a,-n]
   __shared__ __attribute__((aligned(16))) float4 stg_m[NIT * THREADS + STG_PADS];   //                                      [-a,n], [+a,-n]
@@ -830,6 +833,7 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
       float ra = v[k].x + bz, rb = v[k].y + bz;
+      if constexpr (MOM) { ms1 += ra + rb; ms2 = fmaf(ra, ra, fmaf(rb, rb, ms2)); }
       if (relu) { ra = s2cnn::relu_f(ra); rb = s2cnn::relu_f(rb); }
       buf_store_f32(ra, ry, yoff, (j * 4096 + k * 512) * 4);
       buf_store_f32(rb, ry, yoff, ((63 - j) * 4096 + k * 512) * 4);
@@ -908,6 +912,17 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
   fft_pass<true, 1>(work, twl); __syncthreads();
   fft_pass<true, 2>(work, twl); __syncthreads();
   stage_c2_store(NJ - 1);
+  if constexpr (MOM) {                              // the threads' partial sums through LDS, pairwise, always in the same order
+    __syncthreads();
+    float* red = reinterpret_cast<float*>(work);
+    red[t] = ms1; red[THREADS + t] = ms2;
+    __syncthreads();
+    for (int s = THREADS / 2; s > 0; s >>= 1) {
+      if (t < s) { red[t] += red[t + s]; red[THREADS + t] += red[THREADS + t + s]; }
+      __syncthreads();
+    }
+    if (t == 0) moments[z] = make_float2(red[0], red[THREADS]);
+  }
 }
 
 // item rounds that carry degrees below nl (the template argument NA of the kernels below)
@@ -941,18 +956,25 @@ inline void launch_probe(int direction, int probe, hipStream_t st, const float* 
     else if (probe == 2) hipLaunchKernelGGL((analysis_kernel<7, 0, 2>), grid, block, 0, st, x, nullptr, Tf, rec, nbatch, nullptr, 1);
     else hipLaunchKernelGGL((analysis_kernel<7, 0, 0>), grid, block, 0, st, x, nullptr, Tf, rec, nbatch, nullptr, 1);
   } else {
-    if (probe == 1) hipLaunchKernelGGL((synthesis_kernel<7, 8, 1>), grid, block, 0, st, rec, Tf, y, nbatch, nullptr, 1, 0, nullptr);
-    else hipLaunchKernelGGL((synthesis_kernel<7, 8, 0>), grid, block, 0, st, rec, Tf, y, nbatch, nullptr, 1, 0, nullptr);
+    if (probe == 1) hipLaunchKernelGGL((synthesis_kernel<7, 8, 1>), grid, block, 0, st, rec, Tf, y, nbatch, nullptr, 1, 0, nullptr, nullptr);
+    else hipLaunchKernelGGL((synthesis_kernel<7, 8, 0>), grid, block, 0, st, rec, Tf, y, nbatch, nullptr, 1, 0, nullptr, nullptr);
   }
 }
 
 // bits: NULL, or BITS_WORDS 64-bit words per volume that receive one bit per sample: the output is not <= 0
+// moments: NULL, or one (sum, sum of squares) per volume (see MOM)
 inline void launch_synthesis(int nl, hipStream_t st, const float4* rec, const float* Tf, float* y, long nbatch, const float* bias,
-                             int nfeature, int relu, unsigned long long* bits) {
+                             int nfeature, int relu, unsigned long long* bits, float2* moments = nullptr) {
   const dim3 grid(grid_size(nbatch)), block(THREADS);
-  if (nl <= 24) hipLaunchKernelGGL((synthesis_kernel<3, 6>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits);
-  else if (nl <= 28) hipLaunchKernelGGL((synthesis_kernel<5, 7>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits);
-  else hipLaunchKernelGGL((synthesis_kernel<7, 8>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits);
+  if (moments) {
+    if (nl <= 24) hipLaunchKernelGGL((synthesis_kernel<3, 6, 0, true>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments);
+    else if (nl <= 28) hipLaunchKernelGGL((synthesis_kernel<5, 7, 0, true>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments);
+    else hipLaunchKernelGGL((synthesis_kernel<7, 8, 0, true>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments);
+    return;
+  }
+  if (nl <= 24) hipLaunchKernelGGL((synthesis_kernel<3, 6>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, nullptr);
+  else if (nl <= 28) hipLaunchKernelGGL((synthesis_kernel<5, 7>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, nullptr);
+  else hipLaunchKernelGGL((synthesis_kernel<7, 8>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, nullptr);
 }
 
 }  // namespace fused64

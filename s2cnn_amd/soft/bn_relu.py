@@ -47,7 +47,7 @@ def _synthesis_and_statistics(ctx, zr, conv_bias, weight, bias, running_mean, ru
     ctx.bias_shape = conv_bias.shape
     nvox = (2 * b_grid) ** 3
     ctx.count = batch * nvox
-    parts = synthesis_moment_parts(ctx.b_z, b_grid)                # > 0: the synthesis forms the sums itself, one pair per plane
+    parts = synthesis_moment_parts(ctx.b_z, b_grid)                # > 0: the synthesis forms the sums itself, one pair per plane or volume
     if parts:
         mom = zr.new_empty((batch * nf * parts, 2))
         y = so3_rifft_real_basis(zr, b_out=b_grid, bias=conv_bias, moments=(mom, None, None))
@@ -100,7 +100,7 @@ class _SynthesisBNReLUAnalysis(torch.autograd.Function):
     def backward(ctx, gxh):  # pylint: disable=W
         gxh = gxh.contiguous()
         b_next = round((3 / 4 * gxh.size(0)) ** (1 / 3))
-        parts = synthesis_moment_parts(b_next, ctx.b_grid)
+        parts = synthesis_moment_parts(b_next, ctx.b_grid, grad=True)
         if parts:           # the synthesis that produces the gradient with respect to u forms its two sums as well
             y, ab, _ = ctx.saved_tensors
             mom = gxh.new_empty((y.size(0) * y.size(1) * parts, 2))

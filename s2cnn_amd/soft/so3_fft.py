@@ -144,8 +144,12 @@ def _analysis(x, b_in, b_out, batch_size, for_grad, complex_in, mask=None):
     return out
 
 
-def synthesis_moment_parts(b_in, b_out):
-    """How many pairs of sums per volume the real synthesis b_in -> b_out can form while it writes its output (0: none)."""
+def synthesis_moment_parts(b_in, b_out, grad=False):
+    """How many pairs of sums per volume the real synthesis b_in -> b_out of a real-basis spectrum can form while it
+    writes its output (0: none).  grad: the sums of the gradient of a normalisation (they need a second tensor) instead
+    of the output's own; the per-volume kernels of the 64^3 grid form only the latter, one pair per volume."""
+    if _real_basis_direct(b_in, b_out, True):
+        return 0 if grad else 1
     return _hip.lib().s2cnn_so3_synthesis_moment_parts(b_in, b_out)
 
 
@@ -373,7 +377,6 @@ def so3_rifft_real_basis(r, for_grad=False, b_out=None, bias=None, relu=False, b
     if not (r.is_cuda and _real_basis_direct(b_in, b_out, True)):
         from ..so3_real import _convert
         return so3_rifft(_convert("s2cnn_so3_spectrum_to_complex", r.contiguous(), (*r.shape, 2)), for_grad, b_out, bias, relu, bits, moments)
-    assert moments is None, "sums per plane come from the two-stage synthesis only (synthesis_moment_parts)"
     _hip.require_gpu_f32(r)
     r = r.contiguous()
     batch_size = r.size()[1:]
@@ -393,6 +396,12 @@ def so3_rifft_real_basis(r, for_grad=False, b_out=None, bias=None, relu=False, b
         bias = bias.reshape(-1).contiguous()
         nfeature = bias.numel()
         assert r.dim() >= 2 and r.size(-1) == nfeature
+    if moments is not None:
+        mom, yref, _ = moments
+        assert yref is None and not relu, "the per-volume kernels form the sums of their own output only (synthesis_moment_parts)"
+        _hip.call("s2cnn_so3_synthesis_real_basis_moments", _hip.ptr(r), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out), _hip.ptr(ws),
+                  ws.numel(), b_in, b_out, nbatch, _null_or_ptr(bias), nfeature, _hip.ptr(mom), _hip.stream_ptr())
+        return out
     if relu and bits is not None:
         _hip.call("s2cnn_so3_synthesis_real_relu_bits", _hip.ptr(r), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out), _hip.ptr(bits),
                   _hip.ptr(ws), ws.numel(), b_in, b_out, nbatch, _null_or_ptr(bias), nfeature, 1, _hip.stream_ptr())

@@ -41,6 +41,25 @@ def test_volume_moments(hip):
         assert (got - want).abs().max().item() < 2e-5 * want.abs().max().item(), n2    # a sample at the threshold may fall either way
 
 
+@pytest.mark.parametrize("b_in,b_out", [(32, 32), (22, 32), (26, 32), (22, 22), (7, 22), (6, 6)])
+def test_sums_formed_by_the_synthesis(hip, b_in, b_out):
+    """(sum y, sum y^2) per volume (64^3 grid) or per plane (two-stage path) written by the synthesis that produces y,
+    against float64 sums of that y; y itself bit for bit the output of the synthesis without the sums."""
+    parts = P.synthesis_moment_parts(b_in, b_out)
+    assert parts == (1 if b_out == 32 else 2 * b_out)
+    g = torch.Generator().manual_seed(b_in * 100 + b_out)
+    nspec = b_in * (4 * b_in ** 2 - 1) // 3
+    r = torch.randn(nspec, 2, 3, generator=g).cuda()
+    r[0] += 3.0                                                  # a mean well away from zero
+    bias = torch.tensor([0.5, -1.0, 2.0]).cuda()
+    mom = torch.full((6 * parts, 2), float("nan")).cuda()
+    y = P.so3_rifft_real_basis(r, b_out=b_out, bias=bias, moments=(mom, None, None))
+    assert torch.equal(y, P.so3_rifft_real_basis(r, b_out=b_out, bias=bias))
+    yd = y.double().view(6, parts, -1)
+    want = torch.stack([yd.sum(-1), (yd ** 2).sum(-1)], -1).view(-1, 2)
+    assert _rel(mom.double(), want) < 2e-6
+
+
 @pytest.mark.parametrize("b_in,b_out", PAIRS)
 def test_analysis_with_the_normalisation_in_its_loads(hip, b_in, b_out):
     """max(a y + b, 0) and a (a y + b > 0 ? g : 0) + p + q y formed by the loads of the analysis against the same
