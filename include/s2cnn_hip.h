@@ -276,11 +276,16 @@ int s2cnn_so3_synthesis_real_moments(const float *xhat, const float *table, cons
                                      void *workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
                                      const float *bias, int nfeature, float *moments, const float *yref,
                                      const float *params, void *stream);
-/* On the 64^3 grid the per-volume synthesis kernel forms (sum y, sum y^2) of the volume it writes: moments [nbatch][2],
- * other arguments as s2cnn_so3_synthesis_real_basis (real-basis spectrum; -1 where that entry point returns -1). */
+/* On the 64^3 grid the per-volume synthesis kernel forms the same sums over the volume it writes: moments [nbatch][2],
+ * yref and params as above (with yref: no bias, and spectra of at most 28 degrees, for which the kernel has registers to
+ * spare), other arguments as s2cnn_so3_synthesis_real_basis (real-basis spectrum).
+ * s2cnn_so3_synthesis_real_basis_moment_parts(b_in, b_out, grad = whether yref is given) = 1 where it can, else 0 (and
+ * the entry point returns -1). */
+int s2cnn_so3_synthesis_real_basis_moment_parts(int b_in, int b_out, int grad);
 int s2cnn_so3_synthesis_real_basis_moments(const float *r, const float *table, const float *packed_table, float *out,
                                            void *workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
-                                           const float *bias, int nfeature, float *moments, void *stream);
+                                           const float *bias, int nfeature, float *moments, const float *yref,
+                                           const float *params, void *stream);
 /* the arithmetic between those calls, one small launch each instead of a chain of tensor operations (float64 inside):
  * forward : moments [batch][nfeature][parts][2] (parts = 1 from s2cnn_volume_moments, 2 b from the synthesis above),
  *           count = samples per feature -> ab [2][nfeature] for the

@@ -61,7 +61,8 @@ SIGNATURES = {
     "s2cnn_bn_backward_from_moments": (_int, [_c_float_p, _int, _int, _int, ctypes.c_double, _c_float_p, _c_float_p, _int, _c_float_p, _c_float_p, _vp]),
     "s2cnn_so3_synthesis_moment_parts": (_int, [_int, _int]),
     "s2cnn_so3_synthesis_real_moments": (_int, _FT3R_SIG[:-1] + [_c_float_p, _int, _c_float_p, _c_float_p, _c_float_p, _vp]),
-    "s2cnn_so3_synthesis_real_basis_moments": (_int, _FT3R_SIG[:-1] + [_c_float_p, _int, _c_float_p, _vp]),
+    "s2cnn_so3_synthesis_real_basis_moment_parts": (_int, [_int, _int, _int]),
+    "s2cnn_so3_synthesis_real_basis_moments": (_int, _FT3R_SIG[:-1] + [_c_float_p, _int, _c_float_p, _c_float_p, _c_float_p, _vp]),
     "s2cnn_bn_relu_grad_moments": (_int, [_c_float_p, _c_float_p, _c_float_p, _int, _c_float_p, _long, _long, _vp]),
     "s2cnn_so3_analysis_real_affine_relu": (_int, [_c_float_p, _c_float_p, _int] + _FT3R_SIG[1:-1] + [_int, _vp]),
     "s2cnn_so3_analysis_real_bn_relu_grad": (_int, [_c_float_p, _c_float_p, _c_float_p, _int] + _FT3R_SIG[1:-1] + [_int, _vp]),

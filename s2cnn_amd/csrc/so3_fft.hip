@@ -352,8 +352,9 @@ int fused_analysis(const s2cnn::Input& in, const float* table, const float* pack
 
 int fused_synthesis(const float* xhat, const float* table, const float* packed_table, float* out, void* workspace,
                     size_t workspace_bytes, int b_in, long nbatch, bool real_basis, const float* bias, int nfeature, int relu,
-                    unsigned long long* bits, hipStream_t st, float* moments = nullptr) {
-  if (!s2cnn::aligned16(out) || !s2cnn::aligned16(bits) || !s2cnn::aligned8(moments)) return S2CNN_EALIGN;
+                    unsigned long long* bits, hipStream_t st, float* moments = nullptr, const float* yref = nullptr,
+                    const float* params = nullptr) {
+  if (!s2cnn::aligned16(out) || !s2cnn::aligned16(bits) || !s2cnn::aligned8(moments) || !s2cnn::aligned16(yref)) return S2CNN_EALIGN;
   const int nl = b_in < 32 ? b_in : 32;
   const size_t need = round256(fused64::scratch_bytes(nbatch)) + fused64::PACKED_FLOATS * sizeof(float);
   if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
@@ -370,7 +371,7 @@ int fused_synthesis(const float* xhat, const float* table, const float* packed_t
   else
     hipLaunchKernelGGL(fused64::spectrum_gather, dim3((unsigned)((nbatch + fused64::ZT - 1) / fused64::ZT), fused64::active_rounds(nl) * 16), dim3(256), 0, st,
                        reinterpret_cast<const float2*>(xhat), rec, nl, nbatch);
-  fused64::launch_synthesis(nl, st, rec, Tf, out, nbatch, bias, nfeature, relu, bits, reinterpret_cast<float2*>(moments));
+  fused64::launch_synthesis(nl, st, rec, Tf, out, nbatch, bias, nfeature, relu, bits, reinterpret_cast<float2*>(moments), yref, params);
   return s2cnn::launch_status();
 }
 
@@ -402,16 +403,23 @@ extern "C" int s2cnn_so3_synthesis_real_basis(const float* r, const float* table
                          nullptr, static_cast<hipStream_t>(stream));
 }
 
+extern "C" int s2cnn_so3_synthesis_real_basis_moment_parts(int b_in, int b_out, int grad) {
+  if (!sizes_ok(b_out, b_in, 1) || !fused_path(b_out, b_in, 0, true)) return 0;
+  return !grad || b_in <= fused64::GRAD_MOMENTS_MAX_NL ? 1 : 0;
+}
+
 extern "C" int s2cnn_so3_synthesis_real_basis_moments(const float* r, const float* table, const float* packed_table, float* out,
                                                       void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
-                                                      const float* bias, int nfeature, float* moments, void* stream) {
+                                                      const float* bias, int nfeature, float* moments, const float* yref,
+                                                      const float* params, void* stream) {
   s2cnn::clear_stale_error();
   if (!r || !table || !out || !moments || !sizes_ok(b_out, b_in, nbatch)) return S2CNN_EINVAL;
-  if (bias && (nfeature < 1 || nbatch % nfeature != 0)) return S2CNN_EINVAL;
-  if (!fused_path(b_out, b_in, 0, true)) return S2CNN_EINVAL;
+  if ((bias || yref) && (nfeature < 1 || nbatch % nfeature != 0)) return S2CNN_EINVAL;
+  if (yref && (!params || bias)) return S2CNN_EINVAL;
+  if (s2cnn_so3_synthesis_real_basis_moment_parts(b_in, b_out, yref != nullptr) == 0) return S2CNN_EINVAL;
   if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
-  return fused_synthesis(r, table, packed_table, out, workspace, workspace_bytes, b_in, nbatch, true, bias, bias ? nfeature : 1, 0,
-                         nullptr, static_cast<hipStream_t>(stream), moments);
+  return fused_synthesis(r, table, packed_table, out, workspace, workspace_bytes, b_in, nbatch, true, bias, bias || yref ? nfeature : 1, 0,
+                         nullptr, static_cast<hipStream_t>(stream), moments, yref, params);
 }
 
 extern "C" size_t s2cnn_so3_packed_table_bytes(int b_in, int b_out, int synthesis) {

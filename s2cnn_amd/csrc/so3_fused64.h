@@ -698,12 +698,17 @@ __global__ __launch_bounds__(256) void spectrum_gather_real(const float* __restr
 // relu: nonzero = negative samples (after the bias) are stored as zero
 // NA as in analysis_kernel; CMAX: degree groups c < CMAX carry degrees of the input (6 for NA = 3, 7 for 5, 8 for 7)
 // PROBE (measurement only, results meaningless): 1: an item's share of a plane pair reduced to one add per table operand.
-// MOM: the kernel also writes moments[z] = (sum, sum of squares) of the volume's output (bias included, before the
-// activation), summed in a fixed order: the statistics of a batch normalisation that follows, without a read of their own.
-template <int NA, int CMAX, int PROBE = 0, bool MOM = false>
+// MOM: the kernel also writes two sums over the volume it produces, formed in a fixed order, to moments[z]:
+//   1: (sum v, sum v^2) of the output v (bias included, before the activation): the statistics of a batch normalisation
+//      that follows, without a read of their own;
+//   2: (sum v m, sum v m w) with w = yref at the same sample and m = (a w + b > 0), a = params[f], b = params[nfeature + f],
+//      f = z % nfeature: the two reductions of the gradient of such a normalisation followed by max(., 0), with the
+//      output as the incoming gradient (s2cnn::bn_relu_grad).
+template <int NA, int CMAX, int PROBE = 0, int MOM = 0>
 __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __restrict__ rec, const float* __restrict__ Tf,
                                                             float* __restrict__ y, long nbatch, const float* __restrict__ bias, int nfeature,
-                                                            int relu, unsigned long long* __restrict__ bits, float2* __restrict__ moments) {
+                                                            int relu, unsigned long long* __restrict__ bits, float2* __restrict__ moments,
+                                                            const float* __restrict__ yref, const float* __restrict__ params) {
   using namespace fft64;
   __shared__ __attribute__((aligned(16))) float2 work[LDS_ELEMS];
   float ms1 = 0.f, ms2 = 0.f;
@@ -732,6 +737,9 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
   const __amdgpu_buffer_rsrc_t ry = make_rsrc(y + (size_t)z * (N * N * N), N * N * N * 4);
   const unsigned toff = t * 16;
   const unsigned yoff = (d * N + lo) * 4;          // + (beta * 4096 + k * 512) * 4: row alpha = d + 8 k, column gamma = lo
+  const __amdgpu_buffer_rsrc_t rw = make_rsrc(MOM == 2 ? yref + (size_t)z * (N * N * N) : y, MOM == 2 ? N * N * N * 4 : 0);
+  float mom_a = 0.f, mom_b = 0.f;
+  if constexpr (MOM == 2) { mom_a = params[z % nfeature]; mom_b = params[nfeature + z % nfeature]; }
 #pragma unroll
   for (int it = 0; it < NA; ++it) {
     int c, a, n;
@@ -825,6 +833,12 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
   // per wave and store.
   auto stage_c2_store = [&](int j) {
     float2 v[8];
+    [[maybe_unused]] float2 w[8];
+    if constexpr (MOM == 2) {
+#pragma unroll
+      for (int k = 0; k < 8; ++k)
+        w[k] = make_float2(buf_load_f32(rw, yoff, (j * 4096 + k * 512) * 4), buf_load_f32(rw, yoff, ((63 - j) * 4096 + k * 512) * 4));
+    }
     const float2* line = work + sigma(lo) + 8 * d * PITCH;
 #pragma unroll
     for (int k = 0; k < 8; ++k) v[k] = line[k * PITCH];
@@ -833,7 +847,11 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
       float ra = v[k].x + bz, rb = v[k].y + bz;
-      if constexpr (MOM) { ms1 += ra + rb; ms2 = fmaf(ra, ra, fmaf(rb, rb, ms2)); }
+      if constexpr (MOM == 1) { ms1 += ra + rb; ms2 = fmaf(ra, ra, fmaf(rb, rb, ms2)); }
+      if constexpr (MOM == 2) {
+        const float ga = s2cnn::relu_pass(ra, fmaf(mom_a, w[k].x, mom_b)), gb = s2cnn::relu_pass(rb, fmaf(mom_a, w[k].y, mom_b));
+        ms1 += ga + gb; ms2 = fmaf(ga, w[k].x, fmaf(gb, w[k].y, ms2));
+      }
       if (relu) { ra = s2cnn::relu_f(ra); rb = s2cnn::relu_f(rb); }
       buf_store_f32(ra, ry, yoff, (j * 4096 + k * 512) * 4);
       buf_store_f32(rb, ry, yoff, ((63 - j) * 4096 + k * 512) * 4);
@@ -912,7 +930,7 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
   fft_pass<true, 1>(work, twl); __syncthreads();
   fft_pass<true, 2>(work, twl); __syncthreads();
   stage_c2_store(NJ - 1);
-  if constexpr (MOM) {                              // the threads' partial sums through LDS, pairwise, always in the same order
+  if constexpr (MOM != 0) {                         // the threads' partial sums through LDS, pairwise, always in the same order
     __syncthreads();
     float* red = reinterpret_cast<float*>(work);
     red[t] = ms1; red[THREADS + t] = ms2;
@@ -956,25 +974,35 @@ inline void launch_probe(int direction, int probe, hipStream_t st, const float* 
     else if (probe == 2) hipLaunchKernelGGL((analysis_kernel<7, 0, 2>), grid, block, 0, st, x, nullptr, Tf, rec, nbatch, nullptr, 1);
     else hipLaunchKernelGGL((analysis_kernel<7, 0, 0>), grid, block, 0, st, x, nullptr, Tf, rec, nbatch, nullptr, 1);
   } else {
-    if (probe == 1) hipLaunchKernelGGL((synthesis_kernel<7, 8, 1>), grid, block, 0, st, rec, Tf, y, nbatch, nullptr, 1, 0, nullptr, nullptr);
-    else hipLaunchKernelGGL((synthesis_kernel<7, 8, 0>), grid, block, 0, st, rec, Tf, y, nbatch, nullptr, 1, 0, nullptr, nullptr);
+    if (probe == 1) hipLaunchKernelGGL((synthesis_kernel<7, 8, 1>), grid, block, 0, st, rec, Tf, y, nbatch, nullptr, 1, 0, nullptr, nullptr, nullptr, nullptr);
+    else hipLaunchKernelGGL((synthesis_kernel<7, 8, 0>), grid, block, 0, st, rec, Tf, y, nbatch, nullptr, 1, 0, nullptr, nullptr, nullptr, nullptr);
   }
 }
 
 // bits: NULL, or BITS_WORDS 64-bit words per volume that receive one bit per sample: the output is not <= 0
-// moments: NULL, or one (sum, sum of squares) per volume (see MOM)
+// degrees up to which the kernel has registers to spare for the second operand of the sums of MOM = 2
+constexpr int GRAD_MOMENTS_MAX_NL = 28;
+
+// moments: NULL, or two sums per volume (see MOM): those of the output, or, with yref and params (nl <= GRAD_MOMENTS_MAX_NL
+// only), those of the gradient of a normalisation
 inline void launch_synthesis(int nl, hipStream_t st, const float4* rec, const float* Tf, float* y, long nbatch, const float* bias,
-                             int nfeature, int relu, unsigned long long* bits, float2* moments = nullptr) {
+                             int nfeature, int relu, unsigned long long* bits, float2* moments = nullptr, const float* yref = nullptr,
+                             const float* params = nullptr) {
   const dim3 grid(grid_size(nbatch)), block(THREADS);
-  if (moments) {
-    if (nl <= 24) hipLaunchKernelGGL((synthesis_kernel<3, 6, 0, true>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments);
-    else if (nl <= 28) hipLaunchKernelGGL((synthesis_kernel<5, 7, 0, true>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments);
-    else hipLaunchKernelGGL((synthesis_kernel<7, 8, 0, true>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments);
+  if (moments && yref) {
+    if (nl <= 24) hipLaunchKernelGGL((synthesis_kernel<3, 6, 0, 2>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, yref, params);
+    else hipLaunchKernelGGL((synthesis_kernel<5, 7, 0, 2>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, yref, params);
     return;
   }
-  if (nl <= 24) hipLaunchKernelGGL((synthesis_kernel<3, 6>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, nullptr);
-  else if (nl <= 28) hipLaunchKernelGGL((synthesis_kernel<5, 7>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, nullptr);
-  else hipLaunchKernelGGL((synthesis_kernel<7, 8>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, nullptr);
+  if (moments) {
+    if (nl <= 24) hipLaunchKernelGGL((synthesis_kernel<3, 6, 0, 1>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, nullptr, nullptr);
+    else if (nl <= 28) hipLaunchKernelGGL((synthesis_kernel<5, 7, 0, 1>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, nullptr, nullptr);
+    else hipLaunchKernelGGL((synthesis_kernel<7, 8, 0, 1>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, nullptr, nullptr);
+    return;
+  }
+  if (nl <= 24) hipLaunchKernelGGL((synthesis_kernel<3, 6>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, nullptr, nullptr, nullptr);
+  else if (nl <= 28) hipLaunchKernelGGL((synthesis_kernel<5, 7>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, nullptr, nullptr, nullptr);
+  else hipLaunchKernelGGL((synthesis_kernel<7, 8>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, nullptr, nullptr, nullptr);
 }
 
 }  // namespace fused64

@@ -147,9 +147,9 @@ def _analysis(x, b_in, b_out, batch_size, for_grad, complex_in, mask=None):
 def synthesis_moment_parts(b_in, b_out, grad=False):
     """How many pairs of sums per volume the real synthesis b_in -> b_out of a real-basis spectrum can form while it
     writes its output (0: none).  grad: the sums of the gradient of a normalisation (they need a second tensor) instead
-    of the output's own; the per-volume kernels of the 64^3 grid form only the latter, one pair per volume."""
+    of the output's own (the per-volume kernels of the 64^3 grid form those for truncated spectra only)."""
     if _real_basis_direct(b_in, b_out, True):
-        return 0 if grad else 1
+        return _hip.lib().s2cnn_so3_synthesis_real_basis_moment_parts(b_in, b_out, int(grad))
     return _hip.lib().s2cnn_so3_synthesis_moment_parts(b_in, b_out)
 
 
@@ -397,10 +397,13 @@ def so3_rifft_real_basis(r, for_grad=False, b_out=None, bias=None, relu=False, b
         nfeature = bias.numel()
         assert r.dim() >= 2 and r.size(-1) == nfeature
     if moments is not None:
-        mom, yref, _ = moments
-        assert yref is None and not relu, "the per-volume kernels form the sums of their own output only (synthesis_moment_parts)"
+        mom, yref, params = moments
+        assert not relu
+        if params is not None:
+            nfeature = params.size(1)
         _hip.call("s2cnn_so3_synthesis_real_basis_moments", _hip.ptr(r), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out), _hip.ptr(ws),
-                  ws.numel(), b_in, b_out, nbatch, _null_or_ptr(bias), nfeature, _hip.ptr(mom), _hip.stream_ptr())
+                  ws.numel(), b_in, b_out, nbatch, _null_or_ptr(bias), nfeature, _hip.ptr(mom), _null_or_ptr(yref), _null_or_ptr(params),
+                  _hip.stream_ptr())
         return out
     if relu and bits is not None:
         _hip.call("s2cnn_so3_synthesis_real_relu_bits", _hip.ptr(r), _hip.ptr(table), _null_or_ptr(packed), _hip.ptr(out), _hip.ptr(bits),

@@ -71,8 +71,11 @@ def test_argument_rejection_without_gpu():
     assert lib.s2cnn_so3_synthesis_moment_parts(16, 16) == 32 and lib.s2cnn_so3_synthesis_moment_parts(32, 32) == 0
     assert lib.s2cnn_so3_synthesis_real_moments(fake, fake, null, fake, fake, 1 << 30, 32, 32, 3, null, 1, fake, null, null, null) == -1
     assert lib.s2cnn_so3_synthesis_real_moments(fake, fake, null, fake, fake, 1 << 30, 22, 22, 4, null, 3, fake, fake, fake, null) == -1   # 4 volumes, 3 features
-    assert lib.s2cnn_so3_synthesis_real_basis_moments(fake, fake, null, fake, fake, 1 << 30, 22, 22, 3, null, 1, fake, null) == -1    # not the 64^3 grid
-    assert lib.s2cnn_so3_synthesis_real_basis_moments(fake, fake, null, fake, fake, 1 << 30, 32, 32, 3, null, 1, null, null) == -1    # nowhere to write the sums
+    assert lib.s2cnn_so3_synthesis_real_basis_moment_parts(32, 32, 0) == 1 and lib.s2cnn_so3_synthesis_real_basis_moment_parts(32, 32, 1) == 0
+    assert lib.s2cnn_so3_synthesis_real_basis_moment_parts(22, 32, 1) == 1 and lib.s2cnn_so3_synthesis_real_basis_moment_parts(22, 22, 0) == 0
+    assert lib.s2cnn_so3_synthesis_real_basis_moments(fake, fake, null, fake, fake, 1 << 30, 22, 22, 3, null, 1, fake, null, null, null) == -1    # not the 64^3 grid
+    assert lib.s2cnn_so3_synthesis_real_basis_moments(fake, fake, null, fake, fake, 1 << 30, 32, 32, 3, null, 1, null, null, null, null) == -1    # nowhere to write the sums
+    assert lib.s2cnn_so3_synthesis_real_basis_moments(fake, fake, null, fake, fake, 1 << 30, 32, 32, 3, null, 3, fake, fake, fake, null) == -1    # all 32 degrees with a second tensor
     assert lib.s2cnn_so3_integrate_affine_relu(fake, fake, 2, fake, fake, 4, 3, null) == -1              # 3 volumes, 2 features
     assert lib.s2cnn_so3_fft64_probe(fake, fake, fake, fake, 1 << 30, 2, 1, 2, null) == -1               # the synthesis has no probe 2
     assert lib.s2cnn_so3_fft64_probe(fake, fake, fake, fake, 0, 2, 0, 1, null) == -2                     # workspace too small

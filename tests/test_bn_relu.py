@@ -60,6 +60,27 @@ def test_sums_formed_by_the_synthesis(hip, b_in, b_out):
     assert _rel(mom.double(), want) < 2e-6
 
 
+@pytest.mark.parametrize("b_in,b_out", [(22, 32), (26, 32), (28, 32), (22, 22), (7, 22), (6, 6)])
+def test_gradient_sums_formed_by_the_synthesis(hip, b_in, b_out):
+    """(sum g m, sum g m y), m = (a y + b > 0), with g the output of the synthesis and y a second tensor, per volume or per
+    plane, against float64 sums; none on the 64^3 grid for a spectrum of all 32 degrees."""
+    assert P.synthesis_moment_parts(32, 32, grad=True) == 0
+    parts = P.synthesis_moment_parts(b_in, b_out, grad=True)
+    assert parts == (1 if b_out == 32 else 2 * b_out)
+    gen = torch.Generator().manual_seed(b_in * 100 + b_out + 7)
+    nspec = b_in * (4 * b_in ** 2 - 1) // 3
+    r = torch.randn(nspec, 2, 3, generator=gen).cuda()
+    y = torch.randn(2, 3, 2 * b_out, 2 * b_out, 2 * b_out, generator=gen).cuda()
+    ab = torch.tensor([[0.7, 1.3, 2.0], [0.1, 0.4, -0.5]]).cuda()
+    mom = torch.full((6 * parts, 2), float("nan")).cuda()
+    g = P.so3_rifft_real_basis(r, for_grad=True, b_out=b_out, moments=(mom, y, ab))
+    assert torch.equal(g, P.so3_rifft_real_basis(r, for_grad=True, b_out=b_out))
+    m = ab[0].view(1, 3, 1, 1, 1) * y + ab[1].view(1, 3, 1, 1, 1) > 0
+    gm = (g * m).double().view(6, parts, -1)
+    want = torch.stack([gm.sum(-1), (gm * y.double().view(6, parts, -1)).sum(-1)], -1).view(-1, 2)
+    assert (mom.double() - want).abs().max().item() < 2e-5 * want.abs().max().item()      # a sample at the threshold may fall either way
+
+
 @pytest.mark.parametrize("b_in,b_out", PAIRS)
 def test_analysis_with_the_normalisation_in_its_loads(hip, b_in, b_out):
     """max(a y + b, 0) and a (a y + b > 0 ? g : 0) + p + q y formed by the loads of the analysis against the same
