@@ -276,11 +276,11 @@ int s2cnn_so3_synthesis_real_moments(const float *xhat, const float *table, cons
                                      void *workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
                                      const float *bias, int nfeature, float *moments, const float *yref,
                                      const float *params, void *stream);
-/* On the 64^3 grid the per-volume synthesis kernel forms the same sums over the volume it writes: moments [nbatch][2],
- * yref and params as above (with yref: no bias, and spectra of at most 28 degrees, for which the kernel has registers to
- * spare), other arguments as s2cnn_so3_synthesis_real_basis (real-basis spectrum).
- * s2cnn_so3_synthesis_real_basis_moment_parts(b_in, b_out, grad = whether yref is given) = 1 where it can, else 0 (and
- * the entry point returns -1). */
+/* The same with the spectrum in the real basis (other arguments as s2cnn_so3_synthesis_real_basis), and also on the 64^3
+ * grid, whose per-volume kernel forms the sums over the volume it writes: one pair per volume (with yref: no bias, and
+ * spectra of at most 28 degrees, for which the kernel has registers to spare).
+ * s2cnn_so3_synthesis_real_basis_moment_parts(b_in, b_out, grad = whether yref is given) = pairs per volume (1 on the
+ * 64^3 grid, 2 b_out elsewhere) where it can, else 0 (and the entry point returns -1); moments [nbatch][pairs][2]. */
 int s2cnn_so3_synthesis_real_basis_moment_parts(int b_in, int b_out, int grad);
 int s2cnn_so3_synthesis_real_basis_moments(const float *r, const float *table, const float *packed_table, float *out,
                                            void *workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
@@ -339,7 +339,8 @@ int s2cnn_so3_pack_table(const float *table, float *packed, int b_in, int b_out,
  * which saves the conversion pass and half of the spectrum traffic inside the convolution layer
  * (soft/so3_conv.py:36-56 has no such step: the reference keeps complex spectra throughout).
  * Available where s2cnn_so3_real_basis_transform_available(b_in, b_out, synthesis) returns 1
- * (a 64^3 grid on the signal side; S2CNN_EINVAL otherwise: compose the two calls instead).
+ * (analysis: a 64^3 grid on the signal side; synthesis: wherever s2cnn_so3_packed_table_bytes is not 0;
+ * S2CNN_EINVAL otherwise: compose the two calls instead).
  * Tables, packed tables and workspace exactly as for s2cnn_so3_analysis / s2cnn_so3_synthesis with
  * complex_in / complex_out = 0.
  * bias: NULL, or nfeature values; with the batch laid out [..., nfeature] (nbatch a multiple of nfeature),

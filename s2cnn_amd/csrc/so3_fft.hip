@@ -326,6 +326,12 @@ size_t packed_bytes(int b_grid, int b_spec, int cplx, bool synthesis) {
 
 size_t round256(size_t n) { return (n + 255) & ~(size_t)255; }
 
+// A synthesis of real signals that reads its spectrum in the real basis: the per-volume kernels of the 64^3 grid and the
+// tiled Wigner stage of the other grids.
+bool real_basis_synthesis(int b_in, int b_out) {
+  return b_in >= 1 && b_out >= 1 && (fused_path(b_out, b_in, 0, true) || packed_bytes(b_out, b_in, 0, true) != 0);
+}
+
 // Real signals on the 64^3 grid: per-volume kernel + the pass between its records and the spectral rows.
 // real_basis: the spectrum is stored in the real basis (one float per entry) instead of complex pairs.
 int fused_analysis(const s2cnn::Input& in, const float* table, const float* packed_table, float* out,
@@ -379,7 +385,7 @@ int fused_synthesis(const float* xhat, const float* table, const float* packed_t
 
 extern "C" int s2cnn_so3_real_basis_transform_available(int b_in, int b_out, int synthesis) {
   if (b_in < 1 || b_out < 1) return 0;
-  return synthesis ? fused_path(b_out, b_in, 0, true) : fused_path(b_in, b_out, 0, false);
+  return synthesis ? real_basis_synthesis(b_in, b_out) : fused_path(b_in, b_out, 0, false);
 }
 
 extern "C" int s2cnn_so3_analysis_real_basis(const float* x, const float* table, const float* packed_table, float* out,
@@ -389,37 +395,6 @@ extern "C" int s2cnn_so3_analysis_real_basis(const float* x, const float* table,
   if (!fused_path(b_in, b_out, 0, false)) return S2CNN_EINVAL;
   if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
   return fused_analysis(s2cnn::Input{x}, table, packed_table, out, workspace, workspace_bytes, b_out, nbatch, true, static_cast<hipStream_t>(stream));
-}
-
-extern "C" int s2cnn_so3_synthesis_real_basis(const float* r, const float* table, const float* packed_table, float* out,
-                                              void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
-                                              const float* bias, int nfeature, void* stream) {
-  s2cnn::clear_stale_error();
-  if (!r || !table || !out || !sizes_ok(b_out, b_in, nbatch)) return S2CNN_EINVAL;
-  if (bias && (nfeature < 1 || nbatch % nfeature != 0)) return S2CNN_EINVAL;
-  if (!fused_path(b_out, b_in, 0, true)) return S2CNN_EINVAL;
-  if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
-  return fused_synthesis(r, table, packed_table, out, workspace, workspace_bytes, b_in, nbatch, true, bias, bias ? nfeature : 1, 0,
-                         nullptr, static_cast<hipStream_t>(stream));
-}
-
-extern "C" int s2cnn_so3_synthesis_real_basis_moment_parts(int b_in, int b_out, int grad) {
-  if (!sizes_ok(b_out, b_in, 1) || !fused_path(b_out, b_in, 0, true)) return 0;
-  return !grad || b_in <= fused64::GRAD_MOMENTS_MAX_NL ? 1 : 0;
-}
-
-extern "C" int s2cnn_so3_synthesis_real_basis_moments(const float* r, const float* table, const float* packed_table, float* out,
-                                                      void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
-                                                      const float* bias, int nfeature, float* moments, const float* yref,
-                                                      const float* params, void* stream) {
-  s2cnn::clear_stale_error();
-  if (!r || !table || !out || !moments || !sizes_ok(b_out, b_in, nbatch)) return S2CNN_EINVAL;
-  if ((bias || yref) && (nfeature < 1 || nbatch % nfeature != 0)) return S2CNN_EINVAL;
-  if (yref && (!params || bias)) return S2CNN_EINVAL;
-  if (s2cnn_so3_synthesis_real_basis_moment_parts(b_in, b_out, yref != nullptr) == 0) return S2CNN_EINVAL;
-  if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
-  return fused_synthesis(r, table, packed_table, out, workspace, workspace_bytes, b_in, nbatch, true, bias, bias || yref ? nfeature : 1, 0,
-                         nullptr, static_cast<hipStream_t>(stream), moments, yref, params);
 }
 
 extern "C" size_t s2cnn_so3_packed_table_bytes(int b_in, int b_out, int synthesis) {
@@ -555,18 +530,20 @@ int moment_parts(int b_in, int b_out) {
 
 int synthesis_impl(const float* xhat, const float* table, const float* packed_table, float* out, void* workspace,
                    size_t workspace_bytes, int b_in, int b_out, long nbatch, int complex_out, const float* bias, int nfeature,
-                   int relu, unsigned long long* bits, void* stream, const PlaneMoments& mom = PlaneMoments()) {
+                   int relu, unsigned long long* bits, void* stream, const PlaneMoments& mom = PlaneMoments(), bool real_basis = false) {
   if (!xhat || !table || !out || !sizes_ok(b_out, b_in, nbatch)) return S2CNN_EINVAL;
+  if (real_basis && !real_basis_synthesis(b_in, b_out)) return S2CNN_EINVAL;
+  if (real_basis && fused_path(b_out, b_in, 0, true) && mom.out) return S2CNN_EINVAL;     // per volume: fused_synthesis, by its callers
   if (mom.out && (complex_out || moment_parts(b_in, b_out) == 0 || !s2cnn::aligned8(mom.out))) return S2CNN_EINVAL;
   if (mom.yref && (!mom.params || nfeature < 1 || nbatch % nfeature != 0)) return S2CNN_EINVAL;
   if (bits && !fused_path(b_out, b_in, complex_out, true)) return S2CNN_EINVAL;
   if (bias && (complex_out || nfeature < 1 || nbatch % nfeature != 0)) return S2CNN_EINVAL;
   if (relu && complex_out) return S2CNN_EINVAL;
-  if (!s2cnn::aligned8(xhat) || (complex_out && !s2cnn::aligned8(out))) return S2CNN_EALIGN;
+  if ((!real_basis && !s2cnn::aligned8(xhat)) || (complex_out && !s2cnn::aligned8(out))) return S2CNN_EALIGN;
   if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (fused_path(b_out, b_in, complex_out, true))
-    return fused_synthesis(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, nbatch, false, bias, bias ? nfeature : 1, relu, bits, st);
+    return fused_synthesis(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, nbatch, real_basis, bias, bias ? nfeature : 1, relu, bits, st);
   const size_t need = s2cnn_so3_synthesis_workspace(b_in, b_out, nbatch, complex_out);
   if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
   const int n2 = 2 * b_out, nb = b_in < b_out ? b_in : b_out;
@@ -585,12 +562,15 @@ int synthesis_impl(const float* xhat, const float* table, const float* packed_ta
       hipLaunchKernelGGL(wigner_tiled::pack_table_synthesis, dim3(2048), dim3(256), 0, st, table, dst, n2, nb, b_in);
       Tq = dst;
     }
-    if (wigner_tiled::small_synthesis(n2, nb))
-      hipLaunchKernelGGL((wigner_tiled::wigner_inv_tiled<16, 32>), dim3(wigner_tiled::grid_size(MW, nbatch)), dim3(512), 0, st, xh, Tq, S, n2, nb,
-                         b_in, nbatch);
-    else
-      hipLaunchKernelGGL((wigner_tiled::wigner_inv_tiled<32, 64>), dim3(wigner_tiled::grid_size(MW, nbatch), wigner_tiled::parts_synthesis(n2, nb)),
-                         dim3(512), 0, st, xh, Tq, S, n2, nb, b_in, nbatch);
+    const dim3 gs(wigner_tiled::grid_size(MW, nbatch)), gl(wigner_tiled::grid_size(MW, nbatch), wigner_tiled::parts_synthesis(n2, nb));
+    const void* spectrum = xhat;
+    if (wigner_tiled::small_synthesis(n2, nb)) {
+      if (real_basis) hipLaunchKernelGGL((wigner_tiled::wigner_inv_tiled<16, 32, true>), gs, dim3(512), 0, st, spectrum, Tq, S, n2, nb, b_in, nbatch);
+      else hipLaunchKernelGGL((wigner_tiled::wigner_inv_tiled<16, 32>), gs, dim3(512), 0, st, spectrum, Tq, S, n2, nb, b_in, nbatch);
+    } else {
+      if (real_basis) hipLaunchKernelGGL((wigner_tiled::wigner_inv_tiled<32, 64, true>), gl, dim3(512), 0, st, spectrum, Tq, S, n2, nb, b_in, nbatch);
+      else hipLaunchKernelGGL((wigner_tiled::wigner_inv_tiled<32, 64>), gl, dim3(512), 0, st, spectrum, Tq, S, n2, nb, b_in, nbatch);
+    }
   } else if (complex_out) {
     hipLaunchKernelGGL(so3_wigner_inv<true>, grid, dim3(16, 16), 0, st, xh, table, S, n2, nb, b_in, nbatch);
   } else {
@@ -648,14 +628,8 @@ namespace {
 int synthesis_relu_impl(const float* xhat, const float* table, const float* packed_table, float* out, unsigned long long* bits,
                         void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch, const float* bias, int nfeature,
                         int real_basis, void* stream) {
-  if (!real_basis)
-    return synthesis_impl(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, 0, bias, nfeature, 1, bits, stream);
-  if (!xhat || !table || !out || !sizes_ok(b_out, b_in, nbatch)) return S2CNN_EINVAL;
-  if (bias && (nfeature < 1 || nbatch % nfeature != 0)) return S2CNN_EINVAL;
-  if (!fused_path(b_out, b_in, 0, true)) return S2CNN_EINVAL;
-  if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
-  return fused_synthesis(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, nbatch, true, bias, bias ? nfeature : 1, 1,
-                         bits, static_cast<hipStream_t>(stream));
+  return synthesis_impl(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, 0, bias, nfeature, 1, bits, stream,
+                        PlaneMoments(), real_basis != 0);
 }
 
 int analysis_prologue_impl(const s2cnn::Input& in, const float* table, const float* packed_table, float* out,
@@ -721,6 +695,40 @@ extern "C" int s2cnn_so3_synthesis_real_moments(const float* xhat, const float* 
   PlaneMoments mom;
   mom.out = moments; mom.yref = yref; mom.params = params;
   return synthesis_impl(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, 0, bias, nfeature, 0, nullptr, stream, mom);
+}
+
+extern "C" int s2cnn_so3_synthesis_real_basis(const float* r, const float* table, const float* packed_table, float* out,
+                                              void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
+                                              const float* bias, int nfeature, void* stream) {
+  s2cnn::clear_stale_error();
+  return synthesis_impl(r, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, 0, bias, nfeature, 0, nullptr, stream,
+                        PlaneMoments(), true);
+}
+
+extern "C" int s2cnn_so3_synthesis_real_basis_moment_parts(int b_in, int b_out, int grad) {
+  if (!sizes_ok(b_out, b_in, 1) || !real_basis_synthesis(b_in, b_out)) return 0;
+  if (!fused_path(b_out, b_in, 0, true)) return moment_parts(b_in, b_out);
+  return !grad || b_in <= fused64::GRAD_MOMENTS_MAX_NL ? 1 : 0;
+}
+
+extern "C" int s2cnn_so3_synthesis_real_basis_moments(const float* r, const float* table, const float* packed_table, float* out,
+                                                      void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,
+                                                      const float* bias, int nfeature, float* moments, const float* yref,
+                                                      const float* params, void* stream) {
+  s2cnn::clear_stale_error();
+  if (!r || !table || !out || !moments || !sizes_ok(b_out, b_in, nbatch)) return S2CNN_EINVAL;
+  if ((bias || yref) && (nfeature < 1 || nbatch % nfeature != 0)) return S2CNN_EINVAL;
+  if (yref && !params) return S2CNN_EINVAL;
+  if (s2cnn_so3_synthesis_real_basis_moment_parts(b_in, b_out, yref != nullptr) == 0) return S2CNN_EINVAL;
+  if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
+  if (fused_path(b_out, b_in, 0, true)) {
+    if (yref && bias) return S2CNN_EINVAL;
+    return fused_synthesis(r, table, packed_table, out, workspace, workspace_bytes, b_in, nbatch, true, bias, bias || yref ? nfeature : 1, 0,
+                           nullptr, static_cast<hipStream_t>(stream), moments, yref, params);
+  }
+  PlaneMoments mom;
+  mom.out = moments; mom.yref = yref; mom.params = params;
+  return synthesis_impl(r, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, 0, bias, nfeature, 0, nullptr, stream, mom, true);
 }
 
 extern "C" int s2cnn_so3_analysis_prologue_available(int b_in, int b_out) { return prologue_path(b_in, b_out) ? 1 : 0; }

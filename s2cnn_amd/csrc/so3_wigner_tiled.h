@@ -270,10 +270,15 @@ __global__ __launch_bounds__(256, 2) void wigner_fwd_tiled(const float2* __restr
 // synthesis: 512 threads, thread = (n = t % NP, zq = (t / NP) % 8, beta group = t / (8 NP)); the tile is NP
 // frequencies x BP betas x 16 batch items: (32, 64), or (16, 32) for small grids (small_synthesis).  A thread keeps
 // BP / (512 / (8 NP)) betas of two batch items.
+// REAL: the spectrum comes in the real basis (float rows [lmn][nbatch]; the four entries (+-m, +-n) of a degree hold the
+// cos cos, cos sin, sin cos and sin sin coefficients, as s2cnn_so3_spectrum_to_real lays them out), and xs is the complex
+// coefficient at (m, n) that they stand for; else complex rows, symmetrised as above.
 // ---------------------------------------------------------------------------------------------
-template <int NP, int BP>
-__global__ __launch_bounds__(512) void wigner_inv_tiled(const float2* __restrict__ xh, const float* __restrict__ Tq_g,
+template <int NP, int BP, bool REAL = false>
+__global__ __launch_bounds__(512) void wigner_inv_tiled(const void* __restrict__ spectrum, const float* __restrict__ Tq_g,
                                                         float2* __restrict__ S, int n2, int nb, int b_spec, long nbatch) {
+  const float2* __restrict__ xh = static_cast<const float2*>(spectrum);
+  const float* __restrict__ xr = static_cast<const float*>(spectrum);
   constexpr int BH = 512 / (8 * NP);            // beta groups
   constexpr int BPT = BP / BH;                  // betas per thread
   constexpr int QL = BP + 4;                    // n stride (floats) of the T chunk
@@ -316,9 +321,16 @@ __global__ __launch_bounds__(512) void wigner_inv_tiled(const float2* __restrict
     for (int i = 0; i < LC; ++i) {
       const int l = l0 + i;
       const bool okx = (xload && l < nb && l >= am && l >= xn && xn < NW);
-      const int ia = okx ? lmn_index(l, m, xn) : 0, ib = okx ? lmn_index(l, -m, -xn) : 0;
-      xa[i] = xh[(size_t)ia * nbatch + zc];
-      xb[i] = xh[(size_t)ib * nbatch + zc];
+      if constexpr (REAL) {                       // xa = (r[+|m|, +n], r[-|m|, -n]), xb = (r[-|m|, +n], r[+|m|, -n])
+        const int ipp = okx ? lmn_index(l, am, xn) : 0, imm = okx ? lmn_index(l, -am, -xn) : 0;
+        const int imp = okx ? lmn_index(l, -am, xn) : 0, ipm = okx ? lmn_index(l, am, -xn) : 0;
+        xa[i] = make_float2(xr[(size_t)ipp * nbatch + zc], xr[(size_t)imm * nbatch + zc]);
+        xb[i] = make_float2(xr[(size_t)imp * nbatch + zc], xr[(size_t)ipm * nbatch + zc]);
+      } else {
+        const int ia = okx ? lmn_index(l, m, xn) : 0, ib = okx ? lmn_index(l, -m, -xn) : 0;
+        xa[i] = xh[(size_t)ia * nbatch + zc];
+        xb[i] = xh[(size_t)ib * nbatch + zc];
+      }
     }
 #pragma unroll
     for (int k = 0; k < TPT; ++k) {
@@ -338,7 +350,18 @@ __global__ __launch_bounds__(512) void wigner_inv_tiled(const float2* __restrict
       const bool okx = (l < nb && l >= am && l >= xn && xn < NW && z0 + xz < nbatch);
       const float sg = (xn & 1) ? -hs : hs;
       const float2 a = xa[i], b = xb[i];
-      if (xload) xs[(i * ZT + xz) * SLD + (t >> 4)] = okx ? make_float2(0.5f * a.x + sg * b.x, 0.5f * a.y - sg * b.y) : make_float2(0.f, 0.f);
+      float2 v;
+      if constexpr (REAL) {
+        const float pp = a.x, mm = a.y, mp = b.x, pm = b.y;
+        const float sm = (m & 1) ? -1.f : 1.f, r2 = 0.70710678118654752f;
+        if (am > 0 && xn > 0) v = m > 0 ? make_float2(0.5f * (pp + mm), 0.5f * (mp - pm)) : make_float2(sm * 0.5f * (pp - mm), -sm * 0.5f * (pm + mp));
+        else if (xn > 0) v = make_float2(r2 * pp, -r2 * pm);
+        else if (am > 0) v = m > 0 ? make_float2(r2 * pp, r2 * mp) : make_float2(sm * r2 * pp, -sm * r2 * mp);
+        else v = make_float2(pp, 0.f);
+      } else {
+        v = make_float2(0.5f * a.x + sg * b.x, 0.5f * a.y - sg * b.y);
+      }
+      if (xload) xs[(i * ZT + xz) * SLD + (t >> 4)] = okx ? v : make_float2(0.f, 0.f);
     }
 #pragma unroll
     for (int k = 0; k < TPT; ++k) {

@@ -72,8 +72,9 @@ def test_argument_rejection_without_gpu():
     assert lib.s2cnn_so3_synthesis_real_moments(fake, fake, null, fake, fake, 1 << 30, 32, 32, 3, null, 1, fake, null, null, null) == -1
     assert lib.s2cnn_so3_synthesis_real_moments(fake, fake, null, fake, fake, 1 << 30, 22, 22, 4, null, 3, fake, fake, fake, null) == -1   # 4 volumes, 3 features
     assert lib.s2cnn_so3_synthesis_real_basis_moment_parts(32, 32, 0) == 1 and lib.s2cnn_so3_synthesis_real_basis_moment_parts(32, 32, 1) == 0
-    assert lib.s2cnn_so3_synthesis_real_basis_moment_parts(22, 32, 1) == 1 and lib.s2cnn_so3_synthesis_real_basis_moment_parts(22, 22, 0) == 0
-    assert lib.s2cnn_so3_synthesis_real_basis_moments(fake, fake, null, fake, fake, 1 << 30, 22, 22, 3, null, 1, fake, null, null, null) == -1    # not the 64^3 grid
+    assert lib.s2cnn_so3_synthesis_real_basis_moment_parts(22, 32, 1) == 1 and lib.s2cnn_so3_synthesis_real_basis_moment_parts(22, 22, 0) == 44
+    assert lib.s2cnn_so3_synthesis_real_basis_moment_parts(70, 70, 0) == 0
+    assert lib.s2cnn_so3_synthesis_real_basis_moments(fake, fake, null, fake, fake, 1 << 30, 70, 70, 3, null, 1, fake, null, null, null) == -1    # no tiled stage at this size
     assert lib.s2cnn_so3_synthesis_real_basis_moments(fake, fake, null, fake, fake, 1 << 30, 32, 32, 3, null, 1, null, null, null, null) == -1    # nowhere to write the sums
     assert lib.s2cnn_so3_synthesis_real_basis_moments(fake, fake, null, fake, fake, 1 << 30, 32, 32, 3, null, 3, fake, fake, fake, null) == -1    # all 32 degrees with a second tensor
     assert lib.s2cnn_so3_integrate_affine_relu(fake, fake, 2, fake, fake, 4, 3, null) == -1              # 3 volumes, 2 features
@@ -86,13 +87,14 @@ def test_argument_rejection_without_gpu():
     assert lib.s2cnn_so3_mm_real_fwd(null, null, null, 4, 2, 3, 5, null) == -1
     assert lib.s2cnn_so3_synthesis_real_bias(null, null, null, null, null, 0, 4, 4, 1, null, 1, null) == -1
     assert lib.s2cnn_so3_synthesis_real_bias(fake, fake, null, fake, fake, 1 << 30, 4, 4, 6, fake, 4, null) == -1   # 6 volumes, 4 features
-    assert lib.s2cnn_so3_synthesis_real_basis(fake, fake, null, fake, fake, 1 << 30, 4, 4, 1, null, 1, null) == -1  # no direct kernel for this grid
+    assert lib.s2cnn_so3_synthesis_real_basis(fake, fake, null, fake, fake, 1 << 30, 70, 70, 1, null, 1, null) == -1  # no direct kernel for this grid
     assert lib.s2cnn_so3_real_basis_transform_available(32, 22, 0) == 1 and lib.s2cnn_so3_real_basis_transform_available(22, 22, 0) == 0
+    assert lib.s2cnn_so3_real_basis_transform_available(22, 22, 1) == 1 and lib.s2cnn_so3_real_basis_transform_available(70, 70, 1) == 0
     assert lib.s2cnn_so3_rft_expand_real(null, null, null, 4, 3, 8, null) == -1
     # relu in the epilogue of the synthesis, its mask in the loads of the analysis
     assert lib.s2cnn_so3_synthesis_real_relu(null, null, null, null, null, 0, 4, 4, 1, null, 1, 0, null) == -1
     assert lib.s2cnn_so3_synthesis_real_relu(fake, fake, null, fake, fake, 1 << 30, 4, 4, 6, fake, 4, 0, null) == -1    # 6 volumes, 4 features
-    assert lib.s2cnn_so3_synthesis_real_relu(fake, fake, null, fake, fake, 1 << 30, 4, 4, 1, null, 1, 1, null) == -1    # no real-basis kernel for this grid
+    assert lib.s2cnn_so3_synthesis_real_relu(fake, fake, null, fake, fake, 1 << 30, 70, 70, 1, null, 1, 1, null) == -1    # no real-basis kernel for this grid
     assert lib.s2cnn_so3_analysis_real_masked(fake, null, fake, null, fake, fake, 1 << 30, 4, 4, 1, 0, null) == -1      # no mask
     assert lib.s2cnn_so3_analysis_real_masked(fake, fake, fake, null, fake, fake, 1 << 30, 4, 4, 1, 1, null) == -1      # no real-basis kernel for this grid
     assert lib.s2cnn_so3_analysis_real_masked(fake, fake, fake, null, fake, null, 0, 4, 4, 1, 0, null) == -2            # no workspace
