@@ -339,7 +339,7 @@ int s2cnn_so3_pack_table(const float *table, float *packed, int b_in, int b_out,
  * which saves the conversion pass and half of the spectrum traffic inside the convolution layer
  * (soft/so3_conv.py:36-56 has no such step: the reference keeps complex spectra throughout).
  * Available where s2cnn_so3_real_basis_transform_available(b_in, b_out, synthesis) returns 1
- * (analysis: a 64^3 grid on the signal side; synthesis: wherever s2cnn_so3_packed_table_bytes is not 0;
+ * (wherever s2cnn_so3_packed_table_bytes is not 0, for the analysis with b_out <= 32 as well;
  * S2CNN_EINVAL otherwise: compose the two calls instead).
  * Tables, packed tables and workspace exactly as for s2cnn_so3_analysis / s2cnn_so3_synthesis with
  * complex_in / complex_out = 0.

@@ -331,6 +331,10 @@ size_t round256(size_t n) { return (n + 255) & ~(size_t)255; }
 bool real_basis_synthesis(int b_in, int b_out) {
   return b_in >= 1 && b_out >= 1 && (fused_path(b_out, b_in, 0, true) || packed_bytes(b_out, b_in, 0, true) != 0);
 }
+// The same for an analysis that writes the real basis: the tiled Wigner stage does where one part covers the spectrum.
+bool real_basis_analysis(int b_in, int b_out) {
+  return b_in >= 1 && b_out >= 1 && (fused_path(b_in, b_out, 0, false) || (packed_bytes(b_in, b_out, 0, false) != 0 && b_out <= 32));
+}
 
 // Real signals on the 64^3 grid: per-volume kernel + the pass between its records and the spectral rows.
 // real_basis: the spectrum is stored in the real basis (one float per entry) instead of complex pairs.
@@ -385,16 +389,7 @@ int fused_synthesis(const float* xhat, const float* table, const float* packed_t
 
 extern "C" int s2cnn_so3_real_basis_transform_available(int b_in, int b_out, int synthesis) {
   if (b_in < 1 || b_out < 1) return 0;
-  return synthesis ? real_basis_synthesis(b_in, b_out) : fused_path(b_in, b_out, 0, false);
-}
-
-extern "C" int s2cnn_so3_analysis_real_basis(const float* x, const float* table, const float* packed_table, float* out,
-                                             void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch, void* stream) {
-  s2cnn::clear_stale_error();
-  if (!x || !table || !out || !sizes_ok(b_in, b_out, nbatch)) return S2CNN_EINVAL;
-  if (!fused_path(b_in, b_out, 0, false)) return S2CNN_EINVAL;
-  if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
-  return fused_analysis(s2cnn::Input{x}, table, packed_table, out, workspace, workspace_bytes, b_out, nbatch, true, static_cast<hipStream_t>(stream));
+  return synthesis ? real_basis_synthesis(b_in, b_out) : real_basis_analysis(b_in, b_out);
 }
 
 extern "C" size_t s2cnn_so3_packed_table_bytes(int b_in, int b_out, int synthesis) {
@@ -441,19 +436,21 @@ bool prologue_path(int b_in, int b_out) {
 
 // in: the signal and what its loads do to it (real signals only for anything but PRO_NONE)
 int analysis_impl(const s2cnn::Input& in, const float* table, const float* packed_table, float* out,
-                  void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch, int complex_in, void* stream) {
+                  void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch, int complex_in, void* stream,
+                  bool real_basis = false) {
   const float* x = in.x;
+  if (real_basis && (complex_in || !real_basis_analysis(b_in, b_out))) return S2CNN_EINVAL;
   const float* mask = in.second_tensor() ? in.w : nullptr;
   if (!x || !table || !out || !sizes_ok(b_in, b_out, nbatch) || (in.kind != s2cnn::PRO_NONE && complex_in)) return S2CNN_EINVAL;
   if (in.kind != s2cnn::PRO_NONE && in.kind != s2cnn::PRO_AFFINE_RELU && !in.w) return S2CNN_EINVAL;
   if (in.kind == s2cnn::PRO_BITS && !fused_path(b_in, b_out, complex_in, false)) return S2CNN_EINVAL;
   if (in.kind >= s2cnn::PRO_AFFINE_RELU && (!in.params || in.nfeature < 1 || nbatch % in.nfeature != 0 || !prologue_path(b_in, b_out)))
     return S2CNN_EINVAL;
-  if (!s2cnn::aligned8(out) || (complex_in && !s2cnn::aligned8(x))) return S2CNN_EALIGN;
+  if ((!real_basis && !s2cnn::aligned8(out)) || (complex_in && !s2cnn::aligned8(x))) return S2CNN_EALIGN;
   if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (fused_path(b_in, b_out, complex_in, false))
-    return fused_analysis(in, table, packed_table, out, workspace, workspace_bytes, b_out, nbatch, false, st);
+    return fused_analysis(in, table, packed_table, out, workspace, workspace_bytes, b_out, nbatch, real_basis, st);
   const size_t need = s2cnn_so3_analysis_workspace(b_in, b_out, nbatch, complex_in);
   if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
   const int n2 = 2 * b_in, nb = b_in < b_out ? b_in : b_out;
@@ -462,6 +459,7 @@ int analysis_impl(const s2cnn::Input& in, const float* table, const float* packe
   const size_t lds = sizeof(float) * (2 * n2 + (complex_in ? 2 : 1) * n2 * n2 + 2 * n2 * NW);
   const unsigned planes = (unsigned)(nbatch * n2);
   const bool tiled = packed_bytes(b_in, b_out, complex_in, false) != 0;
+  const int ztile = !tiled ? 0 : real_basis ? wigner_tiled::ZH : wigner_tiled::ZT;   // batch items per tile of the intermediate
   const bool x16 = s2cnn::aligned16(x) && s2cnn::aligned16(mask);
   const plane_real::Plan plan = complex_in ? plane_real::Plan{0, 0, 0, 0} : plane_real::plan_fwd(n2, nb, planes);
   if (lds > 160 * 1024 && plan.pl == 0) return S2CNN_EINVAL;
@@ -471,19 +469,19 @@ int analysis_impl(const s2cnn::Input& in, const float* table, const float* packe
   } else if (n2 == 64 && x16) {
     const long npairs = nbatch * 32;
     hipLaunchKernelGGL(fft64::plane_fft64_fwd, dim3((unsigned)(npairs < 2048 ? npairs : 2048)), dim3(fft64::THREADS), 0, st, x, X, npairs, nb,
-                       tiled ? wigner_tiled::ZT : 0, mask);
+                       ztile, mask);
   } else if (plan.pl > 0) {
     if (plan.lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)plane_real::plane_dft_fwd, hipFuncAttributeMaxDynamicSharedMemorySize, (int)plan.lds);
     hipLaunchKernelGGL(plane_real::plane_dft_fwd, dim3((planes + plan.pl - 1) / plan.pl), dim3(plan.nt), plan.lds, st, x, X, n2, nb,
-                       tiled ? wigner_tiled::ZT : 0, (long)planes, plan.pl, plan.alias, mask, in.kind, in.params, in.nfeature);
+                       ztile, (long)planes, plan.pl, plan.alias, mask, in.kind, in.params, in.nfeature);
   } else {
     if (lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)so3_plane_dft_fwd<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    hipLaunchKernelGGL(so3_plane_dft_fwd<false>, dim3(planes), dim3(256), lds, st, x, X, n2, nb, tiled ? wigner_tiled::ZT : 0, mask);
+    hipLaunchKernelGGL(so3_plane_dft_fwd<false>, dim3(planes), dim3(256), lds, st, x, X, n2, nb, ztile, mask);
   }
   int rc = s2cnn::launch_status();
   if (rc) return rc;
   if (b_out > b_in) {  // entries with |m| or |n| >= b_in are never touched by stage 2
-    const size_t nfl = (size_t)s2cnn::so3_nspec(b_out) * nbatch * 2;
+    const size_t nfl = (size_t)s2cnn::so3_nspec(b_out) * nbatch * (real_basis ? 1 : 2);
     hipLaunchKernelGGL(fill_zero, dim3(1024), dim3(256), 0, st, out, nfl);
   }
   if (tiled) {
@@ -494,7 +492,13 @@ int analysis_impl(const s2cnn::Input& in, const float* table, const float* packe
       Tp = dst;
     }
     const int parts = wigner_tiled::parts_analysis(nb, b_out);
-    if (wigner_tiled::small_analysis(nb, b_out))
+    if (real_basis) {
+      const dim3 gh(wigner_tiled::grid_size_half(nb, nbatch), nb > wigner_tiled::NC ? 2 : 1);
+      if (wigner_tiled::small_analysis(nb, b_out))
+        hipLaunchKernelGGL((wigner_tiled::wigner_fwd_tiled_real<16>), gh, dim3(256), 0, st, X, Tp, out, n2, nb, b_out, nbatch);
+      else
+        hipLaunchKernelGGL((wigner_tiled::wigner_fwd_tiled_real<32>), gh, dim3(256), 0, st, X, Tp, out, n2, nb, b_out, nbatch);
+    } else if (wigner_tiled::small_analysis(nb, b_out))
       hipLaunchKernelGGL((wigner_tiled::wigner_fwd_tiled<false, 16>), dim3(wigner_tiled::grid_size(MW, nbatch)), dim3(256), 0, st, X, Tp,
                          reinterpret_cast<float2*>(out), n2, nb, b_out, nbatch);
     else if (parts == 1)
@@ -635,14 +639,7 @@ int synthesis_relu_impl(const float* xhat, const float* table, const float* pack
 int analysis_prologue_impl(const s2cnn::Input& in, const float* table, const float* packed_table, float* out,
                            void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch, int real_basis, void* stream) {
   if (in.kind == s2cnn::PRO_NONE) return S2CNN_EINVAL;
-  if (!real_basis)
-    return analysis_impl(in, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, 0, stream);
-  if (!in.x || !table || !out || !sizes_ok(b_in, b_out, nbatch)) return S2CNN_EINVAL;
-  if (in.kind != s2cnn::PRO_AFFINE_RELU && !in.w) return S2CNN_EINVAL;
-  if (in.kind >= s2cnn::PRO_AFFINE_RELU && (!in.params || in.nfeature < 1 || nbatch % in.nfeature != 0)) return S2CNN_EINVAL;
-  if (!fused_path(b_in, b_out, 0, false)) return S2CNN_EINVAL;
-  if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
-  return fused_analysis(in, table, packed_table, out, workspace, workspace_bytes, b_out, nbatch, true, static_cast<hipStream_t>(stream));
+  return analysis_impl(in, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, 0, stream, real_basis != 0);
 }
 }  // namespace
 
@@ -695,6 +692,12 @@ extern "C" int s2cnn_so3_synthesis_real_moments(const float* xhat, const float* 
   PlaneMoments mom;
   mom.out = moments; mom.yref = yref; mom.params = params;
   return synthesis_impl(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, 0, bias, nfeature, 0, nullptr, stream, mom);
+}
+
+extern "C" int s2cnn_so3_analysis_real_basis(const float* x, const float* table, const float* packed_table, float* out,
+                                             void* workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch, void* stream) {
+  s2cnn::clear_stale_error();
+  return analysis_impl(s2cnn::Input{x}, table, packed_table, out, workspace, workspace_bytes, b_in, b_out, nbatch, 0, stream, true);
 }
 
 extern "C" int s2cnn_so3_synthesis_real_basis(const float* r, const float* table, const float* packed_table, float* out,

@@ -29,23 +29,31 @@ constexpr int LC = 4;         // synthesis: degrees per chunk (LDS stays under 6
 
 __device__ __forceinline__ int lmn_index(int l, int m, int n) { return l * (4 * l * l - 1) / 3 + (l + m) * (2 * l + 1) + (l + n); }
 
-// Workgroup -> (m, z tile).  Consecutive workgroups go round-robin over the 8 XCDs; all workgroups
-// of one XCD that run together share m (and so the table slab in that XCD's L2).  Small |m| (long
-// degree ranges) first.  Returns false for padding workgroups.
-__device__ __forceinline__ bool decode_block(int MW, int nb, int nzt, int& m, int& zt) {
+// Workgroup -> item (o, zi) of no x nz.  Consecutive workgroups go round-robin over the 8 XCDs; the items, o-major,
+// are cut into 8 contiguous ranges of equal length, one per XCD: every XCD gets the same number of workgroups whatever
+// no is, and those of one XCD that run together share o (and so the table slab in that XCD's L2).  Returns false for
+// padding workgroups.
+__device__ __forceinline__ bool decode_item(int no, int nz, int& o, int& zi) {
   const int wid = blockIdx.x;
   const int xcd = wid & 7, slot = wid >> 3;
-  const int o = xcd + 8 * (slot / nzt);
-  zt = slot % nzt;
-  if (o >= MW) return false;
+  const int total = no * nz, per = (total + 7) >> 3;
+  const int item = xcd * per + slot;
+  if (item >= total) return false;
+  o = item / nz;
+  zi = item - o * nz;
+  return true;
+}
+inline int grid_items(int no, long nz) { return (int)(8L * ((no * nz + 7) / 8)); }
+
+// Workgroup -> (m, z tile); o = 0, 1, 2, ... is m = 0, 1, -1, 2, -2, ...
+__device__ __forceinline__ bool decode_block(int MW, int nb, int nzt, int& m, int& zt) {
+  int o;
+  if (!decode_item(MW, nzt, o, zt)) return false;
   m = (o & 1) ? (o + 1) / 2 : -(o / 2);
   return true;
 }
 
-inline int grid_size(int MW, long nbatch) {
-  const long nzt = (nbatch + ZT - 1) / ZT;
-  return (int)(8L * ((MW + 7) / 8) * nzt);
-}
+inline int grid_size(int MW, long nbatch) { return grid_items(MW, (nbatch + ZT - 1) / ZT); }
 
 // parts of the analysis: degrees [l0, l0 + 32) x frequencies n in [n0, n0 + 32)
 __host__ __device__ inline int parts_analysis(int nb, int nl) { return nl <= 32 ? 1 : nb <= 32 ? 2 : 3; }
@@ -157,7 +165,8 @@ __global__ __launch_bounds__(256, 2) void wigner_fwd_tiled(const float2* __restr
   static_assert(TS == 32 || (TS == 16 && !PARTS), "table tile");
   constexpr int BW = TS * TS / 4;               // 16-byte words of one beta of the packed table
   constexpr int TPT = KB * BW / 256;            // words of a chunk per thread
-  float2 xr[KB * 2];
+  constexpr int XPT = KB * ZT * TS / 256;     // numbers of a chunk of X per thread (NW <= TS)
+  float2 xr[XPT];
   float4 tr_[TPT];
   // packed table: the chunk of KB betas is KB * TS * TS contiguous floats; word e = t + 256 i of it is
   // beta_local = e / BW, n = (e % BW) / (TS / 4), l = 4 (e % (TS / 4))
@@ -179,7 +188,7 @@ __global__ __launch_bounds__(256, 2) void wigner_fwd_tiled(const float2* __restr
 
   auto load_chunk = [&](int b0) {
 #pragma unroll
-    for (int i = 0; i < KB * 2; ++i) {
+    for (int i = 0; i < XPT; ++i) {
       if constexpr (PARTS) {
         const int row = b0 * ZT + lr + 8 * i;                  // beta * 16 + z
         const bool ok = colok && row < nrows;
@@ -211,11 +220,11 @@ __global__ __launch_bounds__(256, 2) void wigner_fwd_tiled(const float2* __restr
     if constexpr (PARTS) {
       if (colok) {
 #pragma unroll
-        for (int i = 0; i < KB * 2; ++i) Xs[(lr + 8 * i) * XLD_M + lc] = xr[i];
+        for (int i = 0; i < XPT; ++i) Xs[(lr + 8 * i) * XLD_M + lc] = xr[i];
       }
     } else {
 #pragma unroll
-      for (int i = 0; i < KB * 2; ++i) {
+      for (int i = 0; i < XPT; ++i) {
         const int e = t + 256 * i;
         const int row = (int)(((float)e + 0.5f) * inv_nw);     // beta_local * 16 + z
         if (e < chunk_elems) Xs[row * XLD_M + (e - row * NW)] = xr[i];
@@ -262,6 +271,165 @@ __global__ __launch_bounds__(256, 2) void wigner_fwd_tiled(const float2* __restr
       const int d = m * lcoef + n;
       outf[(size_t)(lbase + d) * rowf] = acc[j][v];
       if (n > 0 || m > 0) outf[(size_t)(lbase - d) * rowf] = sg * acc[j][v];
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// analysis with the spectrum written in the real basis (float rows [lmn][nbatch]; the entries (+-m, +-n) of a degree hold
+// the cos cos, cos sin, sin cos and sin sin coefficients, as s2cnn_so3_spectrum_to_real lays them out).  One part only
+// (nb, nl <= 32).  Those four coefficients mix the complex ones of +m and -m at the same n >= 0:
+//   cc = A.x + sm C.x,  ss = A.x - sm C.x,  cs = -A.y - sm C.y,  sc = A.y - sm C.y,    A at (m, n), C at (-m, n), sm = (-1)^m
+// and the table of -m is that of +m read backwards in beta: T[2b-1-k; l,m,n] = (-1)^(l-n) T[k; l,-m,n].  So a workgroup owns
+// |m| and, instead of 16 batch items x (re, im), 8 batch items (X comes in tiles of 8) x four combinations of the two input rows,
+//   U1 = P.x + s0 Q.x, U2 = P.x - s0 Q.x, V1 = P.y + s0 Q.y, V2 = P.y - s0 Q.y,   P = X[k, m, n], Q = X[2b-1-k, -m, n],
+//   s0 = sm (-1)^n,
+// as 32 rows (combination x batch item) of a matrix-core tile whose 32 columns are the degrees, with the table of +m: an
+// even degree gets (cc, ss, -cs, sc) = T (U1, U2, V1, V2), an odd one (ss, cc, sc, -cs).  A lane then holds, for its degree,
+// four consecutive batch items of each combination: one 16-byte store per coefficient row.  Same matrix-core work as the complex kernel, no conversion pass, half
+// the bytes written.  Rows with m = 0 or n = 0 hold two coefficients (scaled by 1/sqrt 2, or 1/2 for the single one at
+// m = n = 0); the other columns are not written.
+// ---------------------------------------------------------------------------------------------
+constexpr int ZH = 8;         // batch items per workgroup of the real-basis analysis
+
+inline int grid_size_half(int nb, long nbatch) { return grid_items(nb, (nbatch + ZH - 1) / ZH); }
+
+// A workgroup takes 16 of the columns n (blockIdx.y picks the half when the table tile holds 32): four accumulator tiles per
+// wave and 28 to 36 KB of LDS leave room for three or four waves per SIMD.  TS: the packed table holds TS x TS values per beta; with
+// TS = 16 the rows of degrees >= 16 of the 32 x 32 matrix-core tile read whatever follows in LDS and are never written out.
+constexpr int NC = 16;        // columns n per workgroup of the real-basis analysis
+
+template <int TS = 32>
+__global__ __launch_bounds__(256, TS == 16 ? 4 : 3) void wigner_fwd_tiled_real(const float2* __restrict__ X, const float* __restrict__ Tp,
+                                                                float* __restrict__ out, int n2, int nb, int nl, long nbatch) {
+  constexpr int NJ = NC / 4;                    // columns n per wave
+  constexpr int XL = NC + 1;                    // n stride of the X chunk (float4): z stride = 4 banks, the 32 lanes of a beta read 32 banks
+  constexpr int TL = TS + 4;                    // n stride (floats) of the T chunk, 16-byte aligned rows of TS degrees
+  __shared__ __attribute__((aligned(16))) float4 Xs[KB * ZH * XL];       // [beta_local][z][n] of (U1, U2, V1, V2)
+  __shared__ __attribute__((aligned(16))) float Ts[KB * NC * TL + 32];   // [beta_local][n][l]
+  const int MW = 2 * nb - 1, NW = nb;
+  const int nzh = (int)((nbatch + ZH - 1) / ZH);
+  int am, zh;
+  if (!decode_item(nb, nzh, am, zh)) return;
+  const long z0 = (long)zh * ZH;
+  const int n0 = NC * blockIdx.y;               // this workgroup's columns: n0 .. n0 + 15
+  if (n0 >= NW) return;
+  const int CW = NW - n0 < NC ? NW - n0 : NC;
+
+  const int t = threadIdx.x;
+  const int lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int l32 = lane & 31, h = lane >> 5;
+  v16f acc[NJ];
+#pragma unroll
+  for (int j = 0; j < NJ; ++j)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
+
+  static_assert(TS == 32 || TS == 16, "table tile");
+  constexpr int BW = TS * TS / 4;               // 16-byte words of one beta of the packed table
+  constexpr int CWD = NC * TS / 4;              // of which this workgroup's columns are CWD contiguous ones
+  constexpr int TPT = KB * CWD / 256;           // words of a chunk per thread
+  constexpr int XPT = KB * ZH * NC / 256;       // numbers of a chunk of one input row per thread
+  float2 xp[XPT], xq[XPT];
+  float4 tr_[TPT];
+  const float4* tbase = reinterpret_cast<const float4*>(Tp + (size_t)(am + nb - 1) * n2 * (TS * TS)) + n0 * (TS / 4);
+  // LDS that no load fills (columns n >= CW, the rows of degrees >= TS) only reaches rows and columns of the tile that are
+  // never written out: it needs no clearing.
+  // X is laid out [z / 8][mi][beta][z % 8][n]: the two input rows of this workgroup are contiguous, 8 NW numbers per beta.
+  // A thread keeps one column (lc) and takes the rows (beta_local, z) = lr, lr + 16, ... of the chunk's KB * 8 (two betas
+  // per slot): offsets that advance by constants, nothing per slot to keep in registers.
+  const int lc = t & (NC - 1), lr = t / NC;
+  const bool colok = lc < CW;
+  const int lb = lr >> 3, lz = lr & 7;          // beta_local (of slot 0) and z of this thread's rows
+  const int bstep = ZH * NW;                    // numbers between two betas of X
+  const float2* xpb = X + (((size_t)zh * MW + (nb - 1 + am)) * n2 * ZH + lz) * NW + n0 + (colok ? lc : 0);
+  const float2* xqb = X + (((size_t)zh * MW + (nb - 1 - am)) * n2 * ZH + lz) * NW + n0 + (colok ? lc : 0);
+
+  auto load_chunk = [&](int b0) {
+#pragma unroll
+    for (int i = 0; i < XPT; ++i) {
+      const int bt = b0 + lb + 2 * i;
+      const bool ok = colok && bt < n2;
+      const float2 p = xpb[ok ? bt * bstep : 0];
+      const float2 q = xqb[ok ? (n2 - 1 - bt) * bstep : 0];
+      xp[i] = ok ? p : make_float2(0.f, 0.f);
+      xq[i] = ok ? q : make_float2(0.f, 0.f);
+    }
+#pragma unroll
+    for (int i = 0; i < TPT; ++i) {
+      const int e = t + 256 * i, bt = e / CWD;
+      const int bc = b0 + bt < n2 ? b0 + bt : n2 - 1;
+      const float4 v = tbase[(size_t)bc * BW + e % CWD];
+      tr_[i] = b0 + bt < n2 ? v : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+  };
+
+  // operand addresses of this lane: A (row l32 = 8 combination + z) = Xs[(beta_local * 8 + z) * XL + n][combination],
+  // B (column l32 = degree) = Ts[(beta_local * 16 + n) * TL + l]
+  const float* Xf = reinterpret_cast<const float*>(Xs);
+  const int a_off = ((h * ZH + (l32 & 7)) * XL + wave) * 4 + (l32 >> 3);
+  const int b_off = (h * NC + wave) * TL + l32;
+  const float s0 = ((am + lc) & 1) ? -1.f : 1.f;     // (-1)^(m + n) of this thread's column (n0 is even)
+
+  load_chunk(0);
+  for (int b0 = 0; b0 < n2; b0 += KB) {
+    __syncthreads();
+    if (colok) {
+#pragma unroll
+      for (int i = 0; i < XPT; ++i)
+        Xs[(lr + 16 * i) * XL + lc] = make_float4(fmaf(s0, xq[i].x, xp[i].x), fmaf(-s0, xq[i].x, xp[i].x), fmaf(s0, xq[i].y, xp[i].y), fmaf(-s0, xq[i].y, xp[i].y));
+    }
+#pragma unroll
+    for (int i = 0; i < TPT; ++i) {
+      const int e = t + 256 * i, r = e % CWD;
+      *reinterpret_cast<float4*>(Ts + ((e / CWD) * NC + r / (TS / 4)) * TL + 4 * (r % (TS / 4))) = tr_[i];
+    }
+    __syncthreads();
+    if (b0 + KB < n2) load_chunk(b0 + KB);
+#pragma unroll
+    for (int q = 0; q < KB / 2; ++q) {          // beta pair (2q, 2q+1) of the chunk
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        if (4 * j + wave >= CW) continue;         // the same for the whole wave
+        const float a = Xf[a_off + (2 * q * ZH * XL + 4 * j) * 4];
+        const float b = Ts[b_off + (2 * q * NC + 4 * j) * TL];
+        acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[j], 0, 0, 0);
+      }
+    }
+  }
+
+  // Accumulator register v of lane (l32 = degree l, h) holds combination v / 4 of batch item z0 + 4 h + v % 4.  A
+  // combination is one coefficient for even degrees and another for odd ones: 0 cc (+m,+n), 1 ss (-m,-n), 2 cs (+m,-n),
+  // 3 sc (-m,+n); even degrees: the combination's number, odd ones: that number with its last bit flipped.
+  const int l = l32;
+  if (l >= nl || l < am) return;
+  const long zq = z0 + 4 * h;
+  if (zq >= nbatch) return;
+  const bool vec = (nbatch & 3) == 0 && (reinterpret_cast<uintptr_t>(out) & 15u) == 0;   // then the four items exist and are aligned
+  const float f0 = am > 0 ? 0.70710678118654752f : 0.5f, f1 = am > 0 ? 1.f : 0.70710678118654752f;   // scale at n = 0, n > 0
+  const int lcoef = 2 * l + 1;
+  const int lbase = l * (4 * l * l - 1) / 3 + l * lcoef + l;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int kind = k ^ (l & 1);
+    const int row0 = lbase + ((kind == 0 || kind == 2) ? am : -am) * lcoef;      // column 0 of row +-m of degree l
+    const int nsg = (kind == 0 || kind == 3) ? 1 : -1;
+    const float sg = kind == 2 ? -1.f : 1.f;
+    const bool w0 = kind == 0 || (kind == 3 && am > 0), w1 = kind == 0 || kind == 2 || am > 0;   // the coefficient exists at n = 0, n > 0
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const int n = n0 + 4 * j + wave;            // the same for the whole wave
+      if (n >= NW) continue;
+      if (!(n <= l && (n > 0 ? w1 : w0))) continue;
+      const float g = sg * (n > 0 ? f1 : f0);
+      float* dst = out + (long)(row0 + nsg * n) * nbatch + zq;
+      if (vec) {
+        *reinterpret_cast<float4*>(dst) = make_float4(g * acc[j][4 * k], g * acc[j][4 * k + 1], g * acc[j][4 * k + 2], g * acc[j][4 * k + 3]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (zq + i < nbatch) dst[i] = g * acc[j][4 * k + i];
+      }
     }
   }
 }

@@ -88,7 +88,8 @@ def test_argument_rejection_without_gpu():
     assert lib.s2cnn_so3_synthesis_real_bias(null, null, null, null, null, 0, 4, 4, 1, null, 1, null) == -1
     assert lib.s2cnn_so3_synthesis_real_bias(fake, fake, null, fake, fake, 1 << 30, 4, 4, 6, fake, 4, null) == -1   # 6 volumes, 4 features
     assert lib.s2cnn_so3_synthesis_real_basis(fake, fake, null, fake, fake, 1 << 30, 70, 70, 1, null, 1, null) == -1  # no direct kernel for this grid
-    assert lib.s2cnn_so3_real_basis_transform_available(32, 22, 0) == 1 and lib.s2cnn_so3_real_basis_transform_available(22, 22, 0) == 0
+    assert lib.s2cnn_so3_real_basis_transform_available(32, 22, 0) == 1 and lib.s2cnn_so3_real_basis_transform_available(22, 22, 0) == 1
+    assert lib.s2cnn_so3_real_basis_transform_available(40, 36, 0) == 0          # a spectrum of more than 32 degrees: several parts
     assert lib.s2cnn_so3_real_basis_transform_available(22, 22, 1) == 1 and lib.s2cnn_so3_real_basis_transform_available(70, 70, 1) == 0
     assert lib.s2cnn_so3_rft_expand_real(null, null, null, 4, 3, 8, null) == -1
     # relu in the epilogue of the synthesis, its mask in the loads of the analysis
@@ -96,7 +97,7 @@ def test_argument_rejection_without_gpu():
     assert lib.s2cnn_so3_synthesis_real_relu(fake, fake, null, fake, fake, 1 << 30, 4, 4, 6, fake, 4, 0, null) == -1    # 6 volumes, 4 features
     assert lib.s2cnn_so3_synthesis_real_relu(fake, fake, null, fake, fake, 1 << 30, 70, 70, 1, null, 1, 1, null) == -1    # no real-basis kernel for this grid
     assert lib.s2cnn_so3_analysis_real_masked(fake, null, fake, null, fake, fake, 1 << 30, 4, 4, 1, 0, null) == -1      # no mask
-    assert lib.s2cnn_so3_analysis_real_masked(fake, fake, fake, null, fake, fake, 1 << 30, 4, 4, 1, 1, null) == -1      # no real-basis kernel for this grid
+    assert lib.s2cnn_so3_analysis_real_masked(fake, fake, fake, null, fake, fake, 1 << 30, 40, 36, 1, 1, null) == -1    # no real-basis kernel for this size
     assert lib.s2cnn_so3_analysis_real_masked(fake, fake, fake, null, fake, null, 0, 4, 4, 1, 0, null) == -2            # no workspace
 
 

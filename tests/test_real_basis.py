@@ -214,11 +214,11 @@ def test_convolution_real_and_complex_paths_agree(hip):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("b_in,b_out,nz", [(32, 32, 3), (32, 20, 33), (20, 32, 5), (6, 4, 2), (4, 6, 3), (22, 22, 17), (16, 16, 5),
-                                           (7, 22, 4), (36, 40, 2), (40, 36, 2)])
+                                           (7, 22, 4), (22, 7, 9), (36, 40, 2), (40, 36, 2), (40, 20, 2), (12, 30, 3), (10, 6, 24)])
 def test_transforms_in_the_real_basis(hip, b_in, b_out, nz):
-    """so3_rfft_real_basis / so3_rifft_real_basis against the two-step compositions they replace (direct
-    analysis kernels on the 64^3 grid, composed elsewhere; the synthesis reads the real basis wherever its Wigner stage is
-    the tiled one), for both tables, and the autograd pair by a dot-product test."""
+    """so3_rfft_real_basis / so3_rifft_real_basis against the two-step compositions they replace (per-volume
+    kernels on the 64^3 grid, elsewhere the tiled Wigner stage reads or writes the real basis; composed where that stage
+    does not apply: an analysis onto more than 32 degrees), for both tables, and the autograd pair by a dot-product test."""
     from s2cnn_amd.soft import so3_fft as P
     from s2cnn_amd.so3_real import so3_spectrum_to_complex, so3_spectrum_to_real
     g = torch.Generator().manual_seed(b_in * 100 + b_out)
