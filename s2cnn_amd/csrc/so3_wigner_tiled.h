@@ -20,8 +20,6 @@
 namespace wigner_tiled {
 
 constexpr int ZT = 16;        // batch items per workgroup
-constexpr int XLD = 36;       // analysis: z stride (complex) of the X chunk -> 2-way minimum on 8-byte reads
-constexpr int TLD = 36;       // analysis: n stride (floats) of the T chunk, 16-byte aligned rows of 32 degrees
 constexpr int KB = 8;         // analysis: betas per chunk
 constexpr int SLD = 33;       // synthesis: z stride (complex) of the spectrum chunk
 constexpr int QLD = 68;       // synthesis: n stride (floats) of the T chunk, 64 betas + pad
@@ -129,16 +127,19 @@ __global__ void pack_table_synthesis(const float* __restrict__ T, float* __restr
 // (l, n) range, so the padded rows cost matrix-core time but no correctness.
 // ---------------------------------------------------------------------------------------------
 typedef float v16f __attribute__((ext_vector_type(16)));
-constexpr int XLD_M = 33;     // z stride (complex) of the X chunk: (z, c) lanes hit 32 distinct banks
 
 // PARTS = false: one part (nb, nl <= 32), the chunk of X is one contiguous run; true: the parts above, the chunk is
-// KB*16 row pieces.  TS: the packed table holds TS x TS values per beta (32, or 16 for small_analysis; the matrix-core
-// tile stays 32 x 32, its rows of degrees >= 16 read zeros).
+// KB*16 row pieces.  TS: the packed table holds TS x TS values per beta (32, or 16 for small_analysis: half the columns, so
+// half the accumulators and a third of the LDS, twice the waves per SIMD; the matrix-core tile stays 32 x 32, its rows of
+// degrees >= 16 read whatever follows in LDS and are never written out).
 template <bool PARTS, int TS = 32>
-__global__ __launch_bounds__(256, 2) void wigner_fwd_tiled(const float2* __restrict__ X, const float* __restrict__ Tp,
-                                                           float2* __restrict__ out, int n2, int nb, int nl, long nbatch) {
+__global__ __launch_bounds__(256, TS == 16 ? 4 : 2) void wigner_fwd_tiled(const float2* __restrict__ X, const float* __restrict__ Tp,
+                                                                          float2* __restrict__ out, int n2, int nb, int nl, long nbatch) {
+  constexpr int NJ = TS / 4;                    // columns n per wave
+  constexpr int XLD_M = TS + 1;                 // z stride (complex) of the X chunk: (z, c) lanes hit 32 distinct banks
+  constexpr int TLD = TS + 4;                   // n stride (floats) of the T chunk, 16-byte aligned rows of TS degrees
   __shared__ __attribute__((aligned(16))) float2 Xs[KB * ZT * XLD_M];
-  __shared__ __attribute__((aligned(16))) float Ts[KB * 32 * TLD];
+  __shared__ __attribute__((aligned(16))) float Ts[KB * TS * TLD + 32];
   const int MW = 2 * nb - 1, NW = nb;
   const int nzt = (int)((nbatch + ZT - 1) / ZT);
   int m, zt;
@@ -154,9 +155,9 @@ __global__ __launch_bounds__(256, 2) void wigner_fwd_tiled(const float2* __restr
   const int t = threadIdx.x;
   const int lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const int l32 = lane & 31, h = lane >> 5;
-  v16f acc[8];
+  v16f acc[NJ];
 #pragma unroll
-  for (int j = 0; j < 8; ++j)
+  for (int j = 0; j < NJ; ++j)
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
 
@@ -171,8 +172,6 @@ __global__ __launch_bounds__(256, 2) void wigner_fwd_tiled(const float2* __restr
   // packed table: the chunk of KB betas is KB * TS * TS contiguous floats; word e = t + 256 i of it is
   // beta_local = e / BW, n = (e % BW) / (TS / 4), l = 4 (e % (TS / 4))
   const float4* tbase = reinterpret_cast<const float4*>(Tp + (PARTS ? blockIdx.y * packed_floats_analysis_part(n2, nb) : 0) + (size_t)mi * n2 * (TS * TS));
-  if constexpr (TS < 32)                        // the rows of degrees >= TS are never written: they must read as zero
-    for (int i = t; i < KB * 32 * TLD; i += 256) Ts[i] = 0.f;
   // X is laid out [z tile][mi][beta][z % 16][n]: a chunk (KB betas) is KB*16 rows of NW complex numbers.
   // One part: the chunk is KB*16*NW contiguous numbers; thread slot i covers element e = t + 256 i of it.
   // Several parts: the part takes the CW columns from n0 of every row; a thread keeps one column (lc) and takes rows
@@ -183,8 +182,8 @@ __global__ __launch_bounds__(256, 2) void wigner_fwd_tiled(const float2* __restr
   const int nrows = n2 * ZT;
   const int chunk_elems = KB * ZT * NW, n2elems = n2 * ZT * NW;
   const float inv_nw = 1.0f / (float)NW;         // e / NW for e < 4096, NW <= 32: (e + 0.5) * inv_nw truncates exactly
-  // columns n >= CW of the X chunk are never loaded: clear them once (T is zero there, but 0 * NaN is not)
-  for (int i = t; i < KB * ZT * XLD_M; i += 256) Xs[i] = make_float2(0.f, 0.f);
+  // LDS that no load fills (columns n >= CW of the X chunk, the rows of degrees >= TS of the T chunk) only reaches rows and
+  // columns of the tile that are skipped or never written out: it needs no clearing.
 
   auto load_chunk = [&](int b0) {
 #pragma unroll
@@ -211,7 +210,7 @@ __global__ __launch_bounds__(256, 2) void wigner_fwd_tiled(const float2* __restr
 
   // operand addresses of this lane: A = Ts[(beta_local * 32 + n) * TLD + l], B = Xs[(beta_local * 16 + z) * XLD_M + n].c
   const float* Xf = reinterpret_cast<const float*>(Xs);
-  const int a_off = (h * 32 + wave) * TLD + l32;
+  const int a_off = (h * TS + wave) * TLD + l32;
   const int b_off = ((h * ZT + (l32 >> 1)) * XLD_M + wave) * 2 + (l32 & 1);
 
   load_chunk(0);
@@ -233,16 +232,16 @@ __global__ __launch_bounds__(256, 2) void wigner_fwd_tiled(const float2* __restr
 #pragma unroll
     for (int i = 0; i < TPT; ++i) {
       const int e = t + 256 * i, r = e % BW;
-      *reinterpret_cast<float4*>(Ts + ((e / BW) * 32 + r / (TS / 4)) * TLD + 4 * (r % (TS / 4))) = tr_[i];
+      *reinterpret_cast<float4*>(Ts + ((e / BW) * TS + r / (TS / 4)) * TLD + 4 * (r % (TS / 4))) = tr_[i];
     }
     __syncthreads();
     if (b0 + KB < n2) load_chunk(b0 + KB);
 #pragma unroll
     for (int q = 0; q < KB / 2; ++q) {          // beta pair (2q, 2q+1) of the chunk
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
+      for (int j = 0; j < NJ; ++j) {
         if (4 * j + wave >= CW) continue;         // the same for the whole wave
-        const float a = Ts[a_off + (2 * q * 32 + 4 * j) * TLD];
+        const float a = Ts[a_off + (2 * q * TS + 4 * j) * TLD];
         const float b = Xf[b_off + (2 * q * ZT * XLD_M + 4 * j) * 2];
         acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[j], 0, 0, 0);
       }
@@ -264,7 +263,7 @@ __global__ __launch_bounds__(256, 2) void wigner_fwd_tiled(const float2* __restr
     const int lcoef = 2 * l + 1;
     const int lbase = l * (4 * l * l - 1) / 3 + l * lcoef + l;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < NJ; ++j) {
       const int n = n0 + 4 * j + wave;
       if (n >= NW || n > l || (n == 0 && m < 0)) continue;
       const float sg = (((m - n) & 1) ? -1.f : 1.f) * (c ? -1.f : 1.f);
