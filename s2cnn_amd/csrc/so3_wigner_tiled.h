@@ -489,8 +489,8 @@ __global__ __launch_bounds__(512) void wigner_inv_tiled(const void* __restrict__
       const int l = l0 + i;
       const bool okx = (xload && l < nb && l >= am && l >= xn && xn < NW);
       if constexpr (REAL) {                       // xa = (r[+|m|, +n], r[-|m|, -n]), xb = (r[-|m|, +n], r[+|m|, -n])
-        const int ipp = okx ? lmn_index(l, am, xn) : 0, imm = okx ? lmn_index(l, -am, -xn) : 0;
-        const int imp = okx ? lmn_index(l, -am, xn) : 0, ipm = okx ? lmn_index(l, am, -xn) : 0;
+        const int rp = lmn_index(l, am, 0), rm = rp - 2 * am * (2 * l + 1);      // column 0 of the rows +|m| and -|m|
+        const int ipp = okx ? rp + xn : 0, imm = okx ? rm - xn : 0, imp = okx ? rm + xn : 0, ipm = okx ? rp - xn : 0;
         xa[i] = make_float2(xr[(size_t)ipp * nbatch + zc], xr[(size_t)imm * nbatch + zc]);
         xb[i] = make_float2(xr[(size_t)imp * nbatch + zc], xr[(size_t)ipm * nbatch + zc]);
       } else {
