@@ -214,7 +214,8 @@ def test_convolution_real_and_complex_paths_agree(hip):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("b_in,b_out,nz", [(32, 32, 3), (32, 20, 33), (20, 32, 5), (6, 4, 2), (4, 6, 3), (22, 22, 17), (16, 16, 5),
-                                           (7, 22, 4), (22, 7, 9), (36, 40, 2), (40, 36, 2), (40, 20, 2), (12, 30, 3), (10, 6, 24)])
+                                           (7, 22, 4), (22, 7, 9), (36, 40, 2), (40, 36, 2), (40, 20, 2), (12, 30, 3), (10, 6, 24),
+                                           (1, 1, 3), (17, 17, 9), (25, 16, 13), (16, 25, 3), (33, 20, 2), (20, 33, 1)])
 def test_transforms_in_the_real_basis(hip, b_in, b_out, nz):
     """so3_rfft_real_basis / so3_rifft_real_basis against the two-step compositions they replace (per-volume
     kernels on the 64^3 grid, elsewhere the tiled Wigner stage reads or writes the real basis; composed where that stage
