@@ -137,56 +137,54 @@ __global__ __launch_bounds__(NT_MAX) void plane_dft_fwd(const float* __restrict_
   // fold gamma; rows go to slots so that the pair (a, n2-a) is adjacent: 0 -> 0, h -> 1, a -> 2a, n2-a -> 2a+1.
   // The planes of a workgroup are one contiguous run of rows; LOADS of them are issued before the first is used.
   {
-    const int hg = h + 1, total = PL * n2 * hg;
+    const int hg = h + 1;
     const long rows_valid = (nplanes - plane0) * n2;
     const float* src = x + (size_t)plane0 * n2 * n2;
     const float* msk = mask ? mask + (size_t)plane0 * n2 * n2 : nullptr;
     const float inv_n2 = 1.0f / (float)n2;
-    // one copy of the loop per case, so that the batched loads of the plain case stay one run of loads
+    // one copy of the loop per case, so that the batched loads of the plain case stay one run of loads.
+    // A thread keeps one column g (and its mirror n2 - g) and walks down the rows of the workgroup's planes in steps of
+    // RS = NT / hg rows: the loads of a wave are runs of hg consecutive floats of consecutive rows, and per element there
+    // is no more index arithmetic than the plane and the slot of its row.
     auto fold_rows = [&](auto kind_c) {
       constexpr int KIND = decltype(kind_c)::value;
       constexpr bool SECOND = KIND == 1 || KIND == 4;
-      Walk2 wk;
-      wk.init(t, NT, hg);
-      for (int e = t; e < total; e += LOADS * NT) {
+      const int RS = NT / hg;
+      const int g = t % hg, r0 = t / hg;
+      const bool lane_on = r0 < RS;
+      const bool paired = g > 0 && g < h;
+      const int g2 = paired ? n2 - g : g;
+      const int nrows = PL * n2;
+      for (int Rb = r0; Rb - r0 < nrows; Rb += LOADS * RS) {      // the same number of rounds for every thread
         float v1[LOADS], v2[LOADS], m1[LOADS], m2[LOADS];
-        int dst[LOADS], pln[LOADS];
-        unsigned pmask = 0, vmask = 0;
 #pragma unroll
         for (int u = 0; u < LOADS; ++u) {
-          const int R = wk.row, g = wk.col;
-          const bool live = e + u * NT < total;
-          const bool valid = live && R < rows_valid;
-          const bool paired = g > 0 && g < h;
-          const int o1 = valid ? R * n2 + g : 0;
-          const int o2 = valid && paired ? R * n2 + n2 - g : o1;
-          v1[u] = src[o1];
-          v2[u] = src[o2];
-          if constexpr (SECOND) { m1[u] = msk[o1]; m2[u] = msk[o2]; }
-          if (valid) vmask |= 1u << u;
-          if (paired) pmask |= 1u << u;
-          const int q = (int)(((float)R + 0.5f) * inv_n2), a = R - q * n2;
-          pln[u] = live ? q : 0;
-          const int slot = a == 0 ? 0 : a == h ? 1 : a < h ? 2 * a : 2 * (n2 - a) + 1;
-          dst[u] = live ? (q * hg + g) * ns + slot : -1;
-          wk.step();
+          const int R = Rb + u * RS;
+          const bool valid = lane_on && R < nrows && R < rows_valid;
+          const int o = valid ? R * n2 : 0;
+          v1[u] = src[o + g];
+          v2[u] = src[o + g2];
+          if constexpr (SECOND) { m1[u] = msk[o + g]; m2[u] = msk[o + g2]; }
         }
 #pragma unroll
         for (int u = 0; u < LOADS; ++u) {
-          float a = v1[u], b = v2[u];
-          if constexpr (KIND == 1) { a = s2cnn::relu_pass(a, m1[u]); b = s2cnn::relu_pass(b, m2[u]); }
+          const int R = Rb + u * RS;
+          if (!(lane_on && R < nrows)) continue;
+          const int q = (int)(((float)R + 0.5f) * inv_n2), a = R - q * n2;     // plane of the workgroup, row of the plane
+          float va = v1[u], vb = v2[u];
+          if constexpr (KIND == 1) { va = s2cnn::relu_pass(va, m1[u]); vb = s2cnn::relu_pass(vb, m2[u]); }
           if constexpr (KIND == 3) {
-            const float4 c = par[pln[u]];
-            a = s2cnn::affine_relu(a, c.x, c.y); b = s2cnn::affine_relu(b, c.x, c.y);
+            const float4 c = par[q];
+            va = s2cnn::affine_relu(va, c.x, c.y); vb = s2cnn::affine_relu(vb, c.x, c.y);
           }
           if constexpr (KIND == 4) {
-            const float4 c = par[pln[u]];
-            a = s2cnn::bn_relu_grad(a, m1[u], c.x, c.y, c.z, c.w); b = s2cnn::bn_relu_grad(b, m2[u], c.x, c.y, c.z, c.w);
+            const float4 c = par[q];
+            va = s2cnn::bn_relu_grad(va, m1[u], c.x, c.y, c.z, c.w); vb = s2cnn::bn_relu_grad(vb, m2[u], c.x, c.y, c.z, c.w);
           }
-          if (!((vmask >> u) & 1u)) a = b = 0.f;
-          const bool paired = (pmask >> u) & 1u;
-          if (!paired) b = 0.f;
-          if (dst[u] >= 0) EO[dst[u]] = make_float2(a + b, paired ? a - b : 0.f);
+          if (R >= rows_valid) va = vb = 0.f;
+          int slot = a < h ? 2 * a : 2 * (n2 - a) + 1;
+          slot = a == 0 ? 0 : a == h ? 1 : slot;
+          EO[(q * hg + g) * ns + slot] = make_float2(paired ? va + vb : va, paired ? va - vb : 0.f);
         }
       }
     };
