@@ -124,6 +124,9 @@ __global__ __launch_bounds__(NT_MAX) void plane_dft_fwd(const float* __restrict_
   float4* Yf = reinterpret_cast<float4*>(alias ? EO : EO + (size_t)PL * (h + 1) * ns);   // [PL][h+1][nbp]
   const long plane0 = (long)blockIdx.x * PL;
   const int t = threadIdx.x, NT = blockDim.x;
+  // volume and beta of the workgroup's first plane, once (plane counts fit 32 bits: the host refuses more than 2^31 planes)
+  const unsigned vol0 = (unsigned)plane0 / (unsigned)n2, beta0 = (unsigned)plane0 - vol0 * n2;
+  const float inv_n2f = 1.0f / (float)n2;
 
   for (int i = t; i < (h + 1) * nbp; i += NT) {
     const int j = i / nbp, k = i - j * nbp;
@@ -188,10 +191,72 @@ __global__ __launch_bounds__(NT_MAX) void plane_dft_fwd(const float* __restrict_
         }
       }
     };
-    if (kind == 1) fold_rows(std::integral_constant<int, 1>{});
-    else if (kind == 3) fold_rows(std::integral_constant<int, 3>{});
-    else if (kind == 4) fold_rows(std::integral_constant<int, 4>{});
-    else fold_rows(std::integral_constant<int, 0>{});
+    // The same for four columns g0 .. g0 + 3 per thread and step (n2 >= 8): two 16-byte loads per tensor, the row's
+    // plane and slot worked out once for four numbers.  The mirror columns n2 - g0 - j come as the run
+    // [n2 - g0 - 3, n2 - g0]; for g0 = 0, whose column 0 has no mirror, as [n2 - 4, n2 - 1] (the run never leaves the row).
+    auto fold_quads = [&](auto kind_c) {
+      constexpr int KIND = decltype(kind_c)::value;
+      constexpr bool SECOND = KIND == 1 || KIND == 4;
+      constexpr int QL = SECOND ? LOADS / 4 : LOADS / 2;      // 16-byte loads per tensor in flight: the registers of LOADS numbers
+      const int GQ = (hg + 3) / 4;
+      const int RS = NT / GQ;
+      const int g0 = 4 * (t % GQ), r0 = t / GQ;
+      const bool lane_on = r0 < RS;
+      const int gm = g0 == 0 ? n2 - 4 : n2 - g0 - 3;       // where the run of mirror columns starts
+      const int nrows = PL * n2;
+      auto ld4 = [](const float* p) { return make_float4(p[0], p[1], p[2], p[3]); };
+      for (int Rb = r0; Rb - r0 < nrows; Rb += QL * RS) {      // the same number of rounds for every thread
+        float4 v1[QL], v2[QL], m1[QL], m2[QL];
+#pragma unroll
+        for (int u = 0; u < QL; ++u) {
+          const int R = Rb + u * RS;
+          const bool valid = lane_on && R < nrows && R < rows_valid;
+          const int o = valid ? R * n2 : 0;
+          v1[u] = ld4(src + o + g0);
+          v2[u] = ld4(src + o + gm);
+          if constexpr (SECOND) { m1[u] = ld4(msk + o + g0); m2[u] = ld4(msk + o + gm); }
+        }
+#pragma unroll
+        for (int u = 0; u < QL; ++u) {
+          const int R = Rb + u * RS;
+          if (!(lane_on && R < nrows)) continue;
+          const int q = (int)(((float)R + 0.5f) * inv_n2), a = R - q * n2;     // plane of the workgroup, row of the plane
+          int slot = a < h ? 2 * a : 2 * (n2 - a) + 1;
+          slot = a == 0 ? 0 : a == h ? 1 : slot;
+          const bool zero = R >= rows_valid;
+          [[maybe_unused]] float4 c = make_float4(0.f, 0.f, 0.f, 0.f);
+          if constexpr (KIND >= 3) c = par[q];
+          const float xa[4] = {v1[u].x, v1[u].y, v1[u].z, v1[u].w}, ma[4] = {m1[u].x, m1[u].y, m1[u].z, m1[u].w};
+          // mirror of column g0 + j: element 3 - j of the run, or 4 - j of the run that starts one later (g0 = 0, j >= 1)
+          const float xr[4] = {v2[u].x, v2[u].y, v2[u].z, v2[u].w}, mr[4] = {m2[u].x, m2[u].y, m2[u].z, m2[u].w};
+          float2* dst = EO + (q * hg + g0) * ns + slot;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int g = g0 + j;
+            if (g > h) continue;
+            const bool paired = g > 0 && g < h;
+            float va = xa[j], vb = g0 == 0 ? xr[(4 - j) & 3] : xr[3 - j];
+            [[maybe_unused]] const float wa = ma[j], wb = g0 == 0 ? mr[(4 - j) & 3] : mr[3 - j];
+            if constexpr (KIND == 1) { va = s2cnn::relu_pass(va, wa); vb = s2cnn::relu_pass(vb, wb); }
+            if constexpr (KIND == 3) { va = s2cnn::affine_relu(va, c.x, c.y); vb = s2cnn::affine_relu(vb, c.x, c.y); }
+            if constexpr (KIND == 4) { va = s2cnn::bn_relu_grad(va, wa, c.x, c.y, c.z, c.w); vb = s2cnn::bn_relu_grad(vb, wb, c.x, c.y, c.z, c.w); }
+            if (zero) va = vb = 0.f;
+            dst[j * ns] = make_float2(paired ? va + vb : va, paired ? va - vb : 0.f);
+          }
+        }
+      }
+    };
+    if (n2 >= 8) {
+      if (kind == 1) fold_quads(std::integral_constant<int, 1>{});
+      else if (kind == 3) fold_quads(std::integral_constant<int, 3>{});
+      else if (kind == 4) fold_quads(std::integral_constant<int, 4>{});
+      else fold_quads(std::integral_constant<int, 0>{});
+    } else {
+      if (kind == 1) fold_rows(std::integral_constant<int, 1>{});
+      else if (kind == 3) fold_rows(std::integral_constant<int, 3>{});
+      else if (kind == 4) fold_rows(std::integral_constant<int, 4>{});
+      else fold_rows(std::integral_constant<int, 0>{});
+    }
     if (ns > n2)   // n2 = 2 mod 4: two empty slots
       for (int i = t; i < PL * hg * (ns - n2); i += NT) EO[(i / (ns - n2)) * ns + n2 + i % (ns - n2)] = make_float2(0.f, 0.f);
   }
@@ -269,9 +334,11 @@ __global__ __launch_bounds__(NT_MAX) void plane_dft_fwd(const float* __restrict_
     if (pl >= nplanes) continue;
     float2* dst = X + (size_t)pl * ((2 * nb - 1) * nb);
     size_t mstride = nb;
-    if (ztile > 0) {
-      const size_t z = pl / n2, beta = pl % n2;
-      dst = X + ((z / ztile) * (2 * nb - 1) * n2 + beta) * ztile * nb + (z % ztile) * nb;
+    if (ztile > 0) {              // volume and beta of the plane, tile and place in the tile of the volume: 32-bit arithmetic
+      const unsigned bq = beta0 + q, dz = (unsigned)(((float)bq + 0.5f) * inv_n2f);
+      const unsigned beta = bq - dz * n2, z = vol0 + dz;
+      const unsigned zt = z / (unsigned)ztile, zr = z - zt * ztile;
+      dst = X + ((size_t)zt * (2 * nb - 1) * n2 + beta) * ztile * nb + zr * nb;
       mstride = (size_t)n2 * ztile * nb;
     }
 #pragma unroll
@@ -309,44 +376,75 @@ __global__ __launch_bounds__(NT_MAX) void plane_dft_inv(const float2* __restrict
   float4* UU = alias ? AB : AB + (size_t)PL * nb * nb2;                   // [PL][nb][npp]
   const long plane0 = (long)blockIdx.x * PL;
   const int t = threadIdx.x, NT = blockDim.x;
+  // volume and beta of the workgroup's first plane, once (plane counts fit 32 bits: the host refuses more than 2^31 planes)
+  const unsigned vol0 = (unsigned)plane0 / (unsigned)n2, beta0 = (unsigned)plane0 - vol0 * n2;
+  const float inv_n2f = 1.0f / (float)n2;
 
   for (int i = t; i < nb * hp; i += NT) {
     const int k = i / hp, j = i - k * hp;
     tab[i] = j <= h ? cs_entry(j, k, n2) : make_float2(0.f, 0.f);
   }
-  // A, B from the rows +m and -m of S; LOADS pairs of rows are in flight per thread
+  // A, B from the rows +m and -m of S; LOADS pairs of rows are in flight per thread.  A thread keeps one column n (two
+  // adjacent ones where nb is even: 16-byte loads and LDS stores) and walks down the rows R = q nb + m of the workgroup's
+  // planes in steps of RS rows: per element nothing but the plane and the frequency of its row is worked out.
   {
-    const int total = PL * nb * nb2, srow = (2 * nb - 1) * nb;
+    const int srow = (2 * nb - 1) * nb, nrows = PL * nb;
     const float2* src = S + (size_t)plane0 * srow;
     const long planes_valid = nplanes - plane0;
     const float inv_nb = 1.0f / (float)nb;
-    Walk2 wk;
-    wk.init(t, NT, nb2);
-    for (int e = t; e < total; e += LOADS * NT) {
-      float2 sp[LOADS], sm[LOADS];
-      unsigned keep = 0, both = 0;
+    auto combine = [](float2 p, float2 m, bool both) {
+      return both ? make_float4(p.x + m.x, p.y + m.y, m.y - p.y, p.x - m.x) : make_float4(p.x, p.y, 0.f, 0.f);
+    };
+    if ((nb & 1) == 0) {
+      const int CP = nb / 2, RS = NT / CP;
+      const int n = 2 * (t % CP), r0 = t / CP;
+      const bool lane_on = r0 < RS;
+      constexpr int QL = LOADS / 2;
+      for (int Rb = r0; Rb - r0 < nrows; Rb += QL * RS) {
+        float4 sp[QL], sm[QL];
 #pragma unroll
-      for (int u = 0; u < LOADS; ++u) {
-        const int R = wk.row, n = wk.col;                      // R = q nb + m
-        const int q = (int)(((float)R + 0.5f) * inv_nb), m = R - q * nb;
-        const bool live = e + u * NT < total;
-        const bool valid = live && n < nb && q < planes_valid;
-        const int o1 = valid ? q * srow + (nb - 1 + m) * nb + n : 0;
-        sp[u] = src[o1];
-        sm[u] = src[valid ? q * srow + (nb - 1 - m) * nb + n : 0];
-        if (valid) keep |= 1u << u;
-        if (m > 0) both |= 1u << u;
-        wk.step();
+        for (int u = 0; u < QL; ++u) {
+          const int R = Rb + u * RS;
+          const int q = (int)(((float)R + 0.5f) * inv_nb), m = R - q * nb;
+          const bool valid = lane_on && R < nrows && q < planes_valid;
+          sp[u] = *reinterpret_cast<const float4*>(src + (valid ? q * srow + (nb - 1 + m) * nb + n : 0));
+          sm[u] = *reinterpret_cast<const float4*>(src + (valid ? q * srow + (nb - 1 - m) * nb + n : 0));
+        }
+#pragma unroll
+        for (int u = 0; u < QL; ++u) {
+          const int R = Rb + u * RS;
+          if (!(lane_on && R < nrows)) continue;
+          const int q = (int)(((float)R + 0.5f) * inv_nb), m = R - q * nb;
+          float4 a0 = make_float4(0.f, 0.f, 0.f, 0.f), a1 = a0;
+          if (q < planes_valid) {
+            a0 = combine(make_float2(sp[u].x, sp[u].y), make_float2(sm[u].x, sm[u].y), m > 0);
+            a1 = combine(make_float2(sp[u].z, sp[u].w), make_float2(sm[u].z, sm[u].w), m > 0);
+          }
+          AB[R * nb2 + n] = a0;
+          AB[R * nb2 + n + 1] = a1;
+        }
       }
+    } else {
+      const int RS = NT / nb2;
+      const int n = t % nb2, r0 = t / nb2;
+      const bool lane_on = r0 < RS;
+      for (int Rb = r0; Rb - r0 < nrows; Rb += LOADS * RS) {
+        float2 sp[LOADS], sm[LOADS];
 #pragma unroll
-      for (int u = 0; u < LOADS; ++u) {
-        const int i = e + u * NT;
-        if (i >= total) continue;
-        float4 ab = make_float4(0.f, 0.f, 0.f, 0.f);
-        if ((keep >> u) & 1u)
-          ab = (both >> u) & 1u ? make_float4(sp[u].x + sm[u].x, sp[u].y + sm[u].y, sm[u].y - sp[u].y, sp[u].x - sm[u].x)
-                                : make_float4(sp[u].x, sp[u].y, 0.f, 0.f);
-        AB[i] = ab;
+        for (int u = 0; u < LOADS; ++u) {
+          const int R = Rb + u * RS;
+          const int q = (int)(((float)R + 0.5f) * inv_nb), m = R - q * nb;
+          const bool valid = lane_on && R < nrows && n < nb && q < planes_valid;
+          sp[u] = src[valid ? q * srow + (nb - 1 + m) * nb + n : 0];
+          sm[u] = src[valid ? q * srow + (nb - 1 - m) * nb + n : 0];
+        }
+#pragma unroll
+        for (int u = 0; u < LOADS; ++u) {
+          const int R = Rb + u * RS;
+          if (!(lane_on && R < nrows)) continue;
+          const int q = (int)(((float)R + 0.5f) * inv_nb), m = R - q * nb;
+          AB[R * nb2 + n] = n < nb && q < planes_valid ? combine(sp[u], sm[u], m > 0) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
       }
     }
   }
@@ -427,7 +525,7 @@ __global__ __launch_bounds__(NT_MAX) void plane_dft_inv(const float2* __restrict
       dst = y + (size_t)pl * n2 * n2;
     }
     if (!active || pl >= nplanes) continue;
-    const float bz = bias ? bias[(int)(pl / n2) % nfeature] : 0.f;
+    const float bz = bias ? bias[(vol0 + (unsigned)(((float)(beta0 + q) + 0.5f) * inv_n2f)) % (unsigned)nfeature] : 0.f;
     auto act = [relu](float v) { return relu ? s2cnn::relu_f(v) : v; };
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
