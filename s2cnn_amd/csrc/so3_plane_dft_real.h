@@ -378,6 +378,7 @@ __global__ __launch_bounds__(NT_MAX) void plane_dft_inv(const float2* __restrict
   const int t = threadIdx.x, NT = blockDim.x;
   // volume and beta of the workgroup's first plane, once (plane counts fit 32 bits: the host refuses more than 2^31 planes)
   const unsigned vol0 = (unsigned)plane0 / (unsigned)n2, beta0 = (unsigned)plane0 - vol0 * n2;
+  const unsigned feat0 = nfeature > 1 ? vol0 % (unsigned)nfeature : 0u;     // feature of that volume
   const float inv_n2f = 1.0f / (float)n2;
 
   for (int i = t; i < nb * hp; i += NT) {
@@ -517,37 +518,47 @@ __global__ __launch_bounds__(NT_MAX) void plane_dft_inv(const float2* __restrict
       }
     }
     // staged mode (one round): y goes to LDS over the consumed spectra and leaves as one contiguous run below
-    float* dst;
-    if (alias) {
-      __syncthreads();
-      dst = Ys + (size_t)q * n2 * n2;
-    } else {
-      dst = y + (size_t)pl * n2 * n2;
-    }
+    if (alias) __syncthreads();
     if (!active || pl >= nplanes) continue;
-    const float bz = bias ? bias[(vol0 + (unsigned)(((float)(beta0 + q) + 0.5f) * inv_n2f)) % (unsigned)nfeature] : 0.f;
-    auto act = [relu](float v) { return relu ? s2cnn::relu_f(v) : v; };
+    float bz = 0.f;
+    if (bias) {                   // the feature of the plane's volume, without a division per item
+      unsigned f = feat0 + (unsigned)(((float)(beta0 + q) + 0.5f) * inv_n2f);
+      while (f >= (unsigned)nfeature) f -= nfeature;
+      bz = bias[f];
+    }
+    const float lo = relu ? 0.f : -INFINITY;             // v < lo ? lo : v  is max(v, 0) that keeps a NaN, or v
+    // one copy per address space, so that the staged mode writes LDS with immediate offsets
+    auto emit = [&](float* dst) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int a = 2 * pb + i;
-      if (a > h) continue;
-      const bool mirror_a = a > 0 && a < h;
+      for (int i = 0; i < 2; ++i) {
+        const int a = 2 * pb + i;
+        if (a > h) continue;
+        const bool mirror_a = a > 0 && a < h;
+        float* r0 = dst + a * n2 + 4 * gb;               // columns g = 4 gb + k
+        float* r1 = dst + a * n2 + n2 - 4 * gb;          // columns n2 - g
+        float* r2 = dst + (n2 - a) * n2 + 4 * gb;
+        float* r3 = dst + (n2 - a) * n2 + n2 - 4 * gb;
 #pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        const int g = 4 * gb + k;
-        if (g > h) continue;
-        const bool mirror_g = g > 0 && g < h;
-        cc[i][k] += bz;
-        const float yc = cc[i][k] + sc[i][k], ys = cs[i][k] + ss[i][k];
-        dst[a * n2 + g] = act(yc - ys);
-        if (mirror_g) dst[a * n2 + n2 - g] = act(yc + ys);
-        if (mirror_a) {
-          const float zc = cc[i][k] - sc[i][k], zs = cs[i][k] - ss[i][k];
-          dst[(n2 - a) * n2 + g] = act(zc - zs);
-          if (mirror_g) dst[(n2 - a) * n2 + n2 - g] = act(zc + zs);
+        for (int k = 0; k < 4; ++k) {
+          const int g = 4 * gb + k;
+          if (g > h) continue;
+          const bool mirror_g = g > 0 && g < h;
+          const float c0 = cc[i][k] + bz;
+          const float yc = c0 + sc[i][k], ys = cs[i][k] + ss[i][k];
+          float v = yc - ys;
+          r0[k] = v < lo ? lo : v;
+          if (mirror_g) { v = yc + ys; r1[-k] = v < lo ? lo : v; }
+          if (mirror_a) {
+            const float zc = c0 - sc[i][k], zs = cs[i][k] - ss[i][k];
+            v = zc - zs;
+            r2[k] = v < lo ? lo : v;
+            if (mirror_g) { v = zc + zs; r3[-k] = v < lo ? lo : v; }
+          }
         }
       }
-    }
+    };
+    if (alias) emit(Ys + (size_t)q * n2 * n2);
+    else emit(y + (size_t)pl * n2 * n2);
   }
   if (!alias) return;
   __syncthreads();
