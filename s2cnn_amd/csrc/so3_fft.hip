@@ -566,7 +566,7 @@ int synthesis_impl(const float* xhat, const float* table, const float* packed_ta
       hipLaunchKernelGGL(wigner_tiled::pack_table_synthesis, dim3(2048), dim3(256), 0, st, table, dst, n2, nb, b_in);
       Tq = dst;
     }
-    const dim3 gs(wigner_tiled::grid_size(MW, nbatch)), gl(wigner_tiled::grid_size(MW, nbatch), wigner_tiled::parts_synthesis(n2, nb));
+    const dim3 gs(wigner_tiled::grid_size_by_weight(MW, nbatch)), gl(wigner_tiled::grid_size_by_weight(MW, nbatch), wigner_tiled::parts_synthesis(n2, nb));
     const void* spectrum = xhat;
     if (wigner_tiled::small_synthesis(n2, nb)) {
       if (real_basis) hipLaunchKernelGGL((wigner_tiled::wigner_inv_tiled<16, 32, true>), gs, dim3(512), 0, st, spectrum, Tq, S, n2, nb, b_in, nbatch);

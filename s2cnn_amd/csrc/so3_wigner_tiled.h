@@ -53,6 +53,22 @@ __device__ __forceinline__ bool decode_block(int MW, int nb, int nzt, int& m, in
 
 inline int grid_size(int MW, long nbatch) { return grid_items(MW, (nbatch + ZT - 1) / ZT); }
 
+// The same for the synthesis, whose work per workgroup falls with |m| (no degree below |m| contributes): equal counts
+// of consecutive o would give the first XCD all the long ones.  Whole frequencies are dealt to the XCDs instead, in the
+// order o = 0, 1, 2, ... of falling work, back and forth (XCD 0 .. 7, then 7 .. 0, ...): every XCD gets long and short
+// ones, and an uneven last round holds the shortest.
+__device__ __forceinline__ bool decode_block_by_weight(int MW, int nzt, int& m, int& zt) {
+  const int wid = blockIdx.x;
+  const int xcd = wid & 7, slot = wid >> 3;
+  const int round = slot / nzt;
+  zt = slot - round * nzt;
+  const int o = 8 * round + ((round & 1) ? 7 - xcd : xcd);
+  if (o >= MW) return false;
+  m = (o & 1) ? (o + 1) / 2 : -(o / 2);
+  return true;
+}
+inline int grid_size_by_weight(int MW, long nbatch) { return (int)(8L * ((MW + 7) / 8) * ((nbatch + ZT - 1) / ZT)); }
+
 // parts of the analysis: degrees [l0, l0 + 32) x frequencies n in [n0, n0 + 32)
 __host__ __device__ inline int parts_analysis(int nb, int nl) { return nl <= 32 ? 1 : nb <= 32 ? 2 : 3; }
 __host__ __device__ inline void part_analysis(int part, int& l0, int& n0) { l0 = part >= 1 ? 32 : 0; n0 = part == 2 ? 32 : 0; }
@@ -457,7 +473,7 @@ __global__ __launch_bounds__(512) void wigner_inv_tiled(const void* __restrict__
   const int MW = 2 * nb - 1, NW = nb;
   const int nzt = (int)((nbatch + ZT - 1) / ZT);
   int m, zt;
-  if (!decode_block(MW, nb, nzt, m, zt)) return;
+  if (!decode_block_by_weight(MW, nzt, m, zt)) return;
   const int mi = m + nb - 1;
   const long z0 = (long)zt * ZT;
   const int am = abs(m);
