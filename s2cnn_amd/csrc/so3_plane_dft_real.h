@@ -576,12 +576,31 @@ __global__ __launch_bounds__(NT_MAX) void plane_dft_inv(const float2* __restrict
           const int f = (int)(((plane0 + q) / n2) % nfeature);
           const float a = params[f], b = params[nfeature + f];
           const float* yr = yref + (size_t)(plane0 + q) * psize;
-          for (int i = lane; i < psize; i += 64) {
-            const float yv = yr[i], gm = s2cnn::relu_pass(v[i], fmaf(a, yv, b));
-            s1 += gm; s2 = fmaf(gm, yv, s2);
+          if ((reinterpret_cast<uintptr_t>(yr) & 15u) == 0) {       // four samples per load, four loads in flight (n2 is even)
+            const float4* yr4 = reinterpret_cast<const float4*>(yr);
+            const float4* v4 = reinterpret_cast<const float4*>(v);
+#pragma unroll 4
+            for (int i = lane; i < psize / 4; i += 64) {
+              const float4 yv = yr4[i], g = v4[i];
+              const float g0 = s2cnn::relu_pass(g.x, fmaf(a, yv.x, b)), g1 = s2cnn::relu_pass(g.y, fmaf(a, yv.y, b));
+              const float g2 = s2cnn::relu_pass(g.z, fmaf(a, yv.z, b)), g3 = s2cnn::relu_pass(g.w, fmaf(a, yv.w, b));
+              s1 += (g0 + g1) + (g2 + g3);
+              s2 = fmaf(g0, yv.x, fmaf(g1, yv.y, fmaf(g2, yv.z, fmaf(g3, yv.w, s2))));
+            }
+          } else {
+            for (int i = lane; i < psize; i += 64) {
+              const float yv = yr[i], gm = s2cnn::relu_pass(v[i], fmaf(a, yv, b));
+              s1 += gm; s2 = fmaf(gm, yv, s2);
+            }
           }
         } else {
-          for (int i = lane; i < psize; i += 64) { const float x = v[i]; s1 += x; s2 = fmaf(x, x, s2); }
+          const float4* v4 = reinterpret_cast<const float4*>(v);
+#pragma unroll 4
+          for (int i = lane; i < psize / 4; i += 64) {
+            const float4 x = v4[i];
+            s1 += (x.x + x.y) + (x.z + x.w);
+            s2 = fmaf(x.x, x.x, fmaf(x.y, x.y, fmaf(x.z, x.z, fmaf(x.w, x.w, s2))));
+          }
         }
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) { s1 += __shfl_xor(s1, o); s2 += __shfl_xor(s2, o); }
