@@ -35,7 +35,6 @@ namespace plane_real {
 
 using dft_common::pad;
 using dft_common::cs_entry;
-using dft_common::Walk2;
 
 constexpr int NT_MAX = 1024;
 constexpr int PL_MAX = 64;                  // planes per workgroup
