@@ -166,6 +166,17 @@ def measure_rows(torch, dev, with_cpu):
     t = cpu_s(lambda: O.so3_ifft(sc[:, :1].cpu()))
     add("so3_ifft complex b=32 N=16", gpu_ms(lambda: PSO3.so3_ifft(sc)), byc, "B", t, 1 / 16, "1 volume of 16")
     del xc, sc
+    # --- real SO(3) transforms on the grids below 64^3, spectrum in the real basis as inside the layers: the 44^3 grid of
+    # config 5 (b = 22, 32 x 100 volumes) and the 32^3 grid of the reference's SHREC17 model (b = 16, 32 x 100 volumes)
+    for bs, nv in ((22, 3200), (16, 3200)):
+        xs = torch.randn(nv, 2 * bs, 2 * bs, 2 * bs, device=dev)
+        rs = PSO3.so3_rfft_real_basis(xs)
+        bys = 4.0 * xs.numel() + 4.0 * rs.numel()
+        t = cpu_s(lambda: O.so3_rfft(xs[:4].cpu()))
+        add("so3 analysis real b=%d N=%d" % (bs, nv), gpu_ms(lambda: PSO3.so3_rfft_real_basis(xs)), bys, "B", t, 4 / nv, "4 volumes of %d" % nv)
+        t = cpu_s(lambda: O.so3_rifft(O.so3_rfft(xs[:4].cpu())))
+        add("so3 synthesis real b=%d N=%d" % (bs, nv), gpu_ms(lambda: PSO3.so3_rifft_real_basis(rs)), bys, "B", t, 4 / nv, "4 volumes of %d (with their analysis)" % nv)
+        del xs, rs
     # --- kernel -> spectrum at config-4 size: [64, 64, 192] -> [43680, 64, 64, 2]
     grid = s2cnn_amd.so3_near_identity_grid()
     kk = torch.randn(64, 64, len(grid), device=dev)
