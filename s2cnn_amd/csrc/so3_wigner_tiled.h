@@ -56,13 +56,13 @@ inline int grid_size(int MW, long nbatch) { return grid_items(MW, (nbatch + ZT -
 // The same for the synthesis, whose work per workgroup falls with |m| (no degree below |m| contributes): equal counts
 // of consecutive o would give the first XCD all the long ones.  Whole frequencies are dealt to the XCDs instead, in the
 // order o = 0, 1, 2, ... of falling work, back and forth (XCD 0 .. 7, then 7 .. 0, ...): every XCD gets long and short
-// ones, and an uneven last round holds the shortest.
+// ones, and an uneven last sweep holds the shortest.
 __device__ __forceinline__ bool decode_block_by_weight(int MW, int nzt, int& m, int& zt) {
   const int wid = blockIdx.x;
   const int xcd = wid & 7, slot = wid >> 3;
-  const int round = slot / nzt;
-  zt = slot - round * nzt;
-  const int o = 8 * round + ((round & 1) ? 7 - xcd : xcd);
+  const int sweep = slot / nzt;
+  zt = slot - sweep * nzt;
+  const int o = 8 * sweep + ((sweep & 1) ? 7 - xcd : xcd);
   if (o >= MW) return false;
   m = (o & 1) ? (o + 1) / 2 : -(o / 2);
   return true;
