@@ -28,6 +28,12 @@ template <> struct Pack<1> {
   static __device__ __forceinline__ void fma(float a, float b, float& c) { c = fmaf(a, b, c); }
   static __device__ __forceinline__ float dot(float a, float b) { return a * b; }
 };
+template <> struct Pack<2> {
+  typedef float2 type;
+  static __device__ __forceinline__ float2 zero() { return make_float2(0.f, 0.f); }
+  static __device__ __forceinline__ void fma(float a, float2 b, float2& c) { c.x = fmaf(a, b.x, c.x); c.y = fmaf(a, b.y, c.y); }
+  static __device__ __forceinline__ float dot(float2 a, float2 b) { return fmaf(a.x, b.x, a.y * b.y); }
+};
 template <> struct Pack<4> {
   typedef float4 type;
   static __device__ __forceinline__ float4 zero() { return make_float4(0.f, 0.f, 0.f, 0.f); }
@@ -199,9 +205,12 @@ int check(const void* a, const void* b, const void* c, int nl, int nbatch, int f
   return S2CNN_OK;
 }
 
-// 16-byte accesses need rows of z, y that start on 16-byte boundaries
+// 16-byte (8-byte) accesses need rows of z, y that start on 16-byte (8-byte) boundaries
 bool vec4(const void* a, const void* b, const void* c, int fo) {
   return fo % 4 == 0 && s2cnn::aligned16(a) && s2cnn::aligned16(b) && s2cnn::aligned16(c);
+}
+bool vec2(const void* a, const void* b, const void* c, int fo) {
+  return fo % 2 == 0 && s2cnn::aligned8(a) && s2cnn::aligned8(b) && s2cnn::aligned8(c);
 }
 
 }  // namespace
@@ -214,6 +223,9 @@ extern "C" int s2cnn_s2_mm_real_fwd(const float* x, const float* y, float* z, in
   if (vec4(y, z, z, f_out)) {
     const dim3 grid(nl * nl, NSPLIT, (unsigned)(((long)npair * (f_out / 4) + 255) / 256));
     hipLaunchKernelGGL(s2_mm_real_fwd_kernel<4>, grid, dim3(256), 0, st, x, y, z, nl, nbatch, f_in, f_out);
+  } else if (vec2(y, z, z, f_out)) {
+    const dim3 grid(nl * nl, NSPLIT, (unsigned)(((long)npair * (f_out / 2) + 255) / 256));
+    hipLaunchKernelGGL(s2_mm_real_fwd_kernel<2>, grid, dim3(256), 0, st, x, y, z, nl, nbatch, f_in, f_out);
   } else {
     const dim3 grid(nl * nl, NSPLIT, (unsigned)(((long)npair * f_out + 255) / 256));
     hipLaunchKernelGGL(s2_mm_real_fwd_kernel<1>, grid, dim3(256), 0, st, x, y, z, nl, nbatch, f_in, f_out);
@@ -228,6 +240,8 @@ extern "C" int s2cnn_s2_mm_real_gradx(const float* gz, const float* y, float* gx
   const dim3 grid(nl * nl, (nbatch + IB - 1) / IB, (f_in + KC - 1) / KC);
   if (vec4(gz, y, y, f_out))
     hipLaunchKernelGGL(s2_mm_real_gradx_kernel<4>, grid, dim3(256), 0, st, gz, y, gx, nl, nbatch, f_in, f_out);
+  else if (vec2(gz, y, y, f_out))
+    hipLaunchKernelGGL(s2_mm_real_gradx_kernel<2>, grid, dim3(256), 0, st, gz, y, gx, nl, nbatch, f_in, f_out);
   else
     hipLaunchKernelGGL(s2_mm_real_gradx_kernel<1>, grid, dim3(256), 0, st, gz, y, gx, nl, nbatch, f_in, f_out);
   return s2cnn::launch_status();
@@ -240,6 +254,9 @@ extern "C" int s2cnn_s2_mm_real_grady(const float* gz, const float* x, float* gy
   if (vec4(gz, gz, gy, f_out)) {
     const dim3 grid(nl * nl, (f_out / 4 + 15) / 16, (f_in + KC - 1) / KC);
     hipLaunchKernelGGL((s2_mm_real_grady_kernel<4, 16>), grid, dim3(256), 0, st, gz, x, gy, nl, nbatch, f_in, f_out);
+  } else if (vec2(gz, gz, gy, f_out)) {
+    const dim3 grid(nl * nl, (f_out / 2 + 31) / 32, (f_in + KC - 1) / KC);
+    hipLaunchKernelGGL((s2_mm_real_grady_kernel<2, 32>), grid, dim3(256), 0, st, gz, x, gy, nl, nbatch, f_in, f_out);
   } else {
     const dim3 grid(nl * nl, (f_out + 63) / 64, (f_in + KC - 1) / KC);
     hipLaunchKernelGGL((s2_mm_real_grady_kernel<1, 64>), grid, dim3(256), 0, st, gz, x, gy, nl, nbatch, f_in, f_out);

@@ -347,9 +347,9 @@ def test_factorised_kernel_transform_matches_dense(hip):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("nl,B,Fi,Fo", [(4, 2, 3, 5), (10, 32, 1, 20), (7, 5, 6, 9), (6, 16, 12, 16), (5, 3, 6, 100), (3, 1, 1, 1),
-                                        (4, 7, 20, 8), (2, 2, 3, 1028)])
+                                        (4, 7, 20, 8), (2, 2, 3, 1028), (6, 16, 6, 50), (5, 3, 9, 2), (3, 4, 2, 70)])
 def test_s2_mm_real_forward_backward(hip, nl, B, Fi, Fo):
-    """The real outer product against numpy: odd sizes (4-byte accesses), multiples of four (16-byte accesses), more
+    """The real outer product against numpy: odd sizes (4-byte accesses), even ones (8-byte), multiples of four (16-byte accesses), more
     input features than one register pass, an odd batch, rows longer than a workgroup."""
     import s2cnn_amd
     print(f"s2_mm_real nl={nl} B={B} Fi={Fi} Fo={Fo}", flush=True)
