@@ -145,8 +145,16 @@ extern "C" int s2cnn_s2_analysis(const float* x, const float* table, float* out,
     const s2_real::Plan plan = s2_real::plan_fwd(n2, nb);
     if (plan.rb > 0) {
       if (plan.lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)s2_real::analysis_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)plan.lds);
-      hipLaunchKernelGGL(s2_real::analysis_kernel, dim3((unsigned)nbatch), dim3(s2_real::NT), plan.lds, st, x, table,
-                         reinterpret_cast<float2*>(out), n2, nb, nbatch, plan.rb);
+      // few signals: split along beta, partial spectra in the workspace, added up in a fixed order
+      int nsplit = s2_real::splits_for(n2, plan.rb, nbatch);
+      const size_t nout = (size_t)nb * nb * nbatch;
+      if (nsplit > 1 && nsplit * nout * sizeof(float2) > workspace_bytes) nsplit = 1;
+      float2* dst = nsplit > 1 ? static_cast<float2*>(workspace) : reinterpret_cast<float2*>(out);
+      hipLaunchKernelGGL(s2_real::analysis_kernel, dim3((unsigned)nbatch, nsplit), dim3(s2_real::NT), plan.lds, st, x, table,
+                         dst, n2, nb, nbatch, plan.rb);
+      if (nsplit > 1)
+        hipLaunchKernelGGL(s2_real::reduce_splits, dim3((unsigned)((nout + 255) / 256 < 1024 ? (nout + 255) / 256 : 1024)), dim3(256), 0, st,
+                           dst, reinterpret_cast<float2*>(out), (long)nout, nsplit);
       return s2cnn::launch_status();
     }
   }
@@ -174,7 +182,7 @@ extern "C" int s2cnn_s2_synthesis(const float* xhat, const float* table, float* 
     const s2_real::Plan plan = s2_real::plan_inv(n2, nb);
     if (plan.rb > 0) {
       if (plan.lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)s2_real::synthesis_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)plan.lds);
-      hipLaunchKernelGGL(s2_real::synthesis_kernel, dim3((unsigned)nbatch), dim3(s2_real::NT), plan.lds, st,
+      hipLaunchKernelGGL(s2_real::synthesis_kernel, dim3((unsigned)nbatch, s2_real::splits_for(n2, 64, nbatch)), dim3(s2_real::NT), plan.lds, st,
                          reinterpret_cast<const float2*>(xhat), table, out, n2, nb, nbatch);
       return s2cnn::launch_status();
     }

@@ -12,6 +12,8 @@
 //     Yc[alpha] = sum_m A[m] c[m alpha], Ys[alpha] = sum_m B[m] s[m alpha], y[alpha] = Yc - Ys, y[n2-alpha] = Yc + Ys.
 //
 // The signal is processed in chunks of RB rows (betas); the next chunk's loads are in flight while one is transformed.
+// A batch too small to fill the chip with one workgroup per signal is split along beta (grid.y = split): the synthesis
+// needs nothing more, the analysis writes one partial spectrum per split and reduce_splits adds them in a fixed order.
 #pragma once
 #include <hip/hip_runtime.h>
 #include "dft_common.h"
@@ -61,7 +63,33 @@ __device__ __forceinline__ int isqrt_floor(int v) {
   return l;
 }
 
+// chunks of RB rows per split, for `nsplit` splits of n2 rows
+__host__ __device__ inline int rows_per_split(int n2, int RB, int nsplit) {
+  const int nchunk = (n2 + RB - 1) / RB;
+  return RB * ((nchunk + nsplit - 1) / nsplit);
+}
+
+// How many splits along beta a batch of nbatch signals gets: enough workgroups for four per CU (the kernels are bound by
+// what one CU issues, so the work has to spread evenly over all of them), whole chunks per split.
+inline int splits_for(int n2, int RB, long nbatch) {
+  const int nchunk = (n2 + RB - 1) / RB;
+  long want = (1024 + nbatch - 1) / nbatch;
+  if (want > nchunk) want = nchunk;
+  if (want > 8) want = 8;
+  return want < 1 ? 1 : (int)want;
+}
+
+// out[e][z] = sum over the splits of partial[s][e][z], in the order of s
+__global__ void reduce_splits(const float2* __restrict__ partial, float2* __restrict__ out, long n, int nsplit) {
+  for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+    float2 v = partial[i];
+    for (int s = 1; s < nsplit; ++s) { const float2 p = partial[(size_t)s * n + i]; v.x += p.x; v.y += p.y; }
+    out[i] = v;
+  }
+}
+
 // x [nbatch][n2][n2] -> out [nb^2][nbatch] complex;  T [n2][nb^2]
+// grid.y > 1: split blockIdx.y takes its share of the rows and writes out + blockIdx.y * nb^2 * nbatch (partial spectra)
 __global__ __launch_bounds__(NT) void analysis_kernel(const float* __restrict__ x, const float* __restrict__ T,
                                                       float2* __restrict__ out, int n2, int nb, long nbatch, int RB) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
@@ -72,6 +100,9 @@ __global__ __launch_bounds__(NT) void analysis_kernel(const float* __restrict__ 
   const long z = blockIdx.x;
   const int t = threadIdx.x;
   const float* xs = x + (size_t)z * n2 * n2;
+  const int rps = rows_per_split(n2, RB, gridDim.y);
+  const int rbeg = blockIdx.y * rps, rend = rbeg + rps < n2 ? rbeg + rps : n2;       // this workgroup's rows
+  out += (size_t)blockIdx.y * nspec * nbatch;
 
   for (int i = t; i < hg * nbp; i += NT) {
     const int j = i / nbp, k = i - j * nbp;
@@ -96,7 +127,7 @@ __global__ __launch_bounds__(NT) void analysis_kernel(const float* __restrict__ 
 #pragma unroll
     for (int u = 0; u < PF; ++u) {
       const int r = row0 + wk.row, a = wk.col;
-      const bool ok = t + u * NT < per_chunk && r < n2;
+      const bool ok = t + u * NT < per_chunk && r < rend;
       const bool paired = a > 0 && a < h;
       const int o = ok ? r * n2 + a : 0;
       v1[u] = xs[o];
@@ -105,8 +136,8 @@ __global__ __launch_bounds__(NT) void analysis_kernel(const float* __restrict__ 
       wk.step();
     }
   };
-  prefetch(0);
-  for (int row0 = 0; row0 < n2; row0 += RB) {
+  prefetch(rbeg);
+  for (int row0 = rbeg; row0 < rend; row0 += RB) {
     {   // registers -> folded rows in LDS
       Walk2 wk;
       wk.init(t, NT, hg);
@@ -121,7 +152,7 @@ __global__ __launch_bounds__(NT) void analysis_kernel(const float* __restrict__ 
       }
     }
     __syncthreads();
-    if (row0 + RB < n2) prefetch(row0 + RB);
+    if (row0 + RB < rend) prefetch(row0 + RB);
     // row transform: 2 rows x 2 frequencies per thread
     const int nmp = nbp / 2, items = RB / 2 * nmp;
     for (int it = t; it < items; it += NT) {
@@ -142,7 +173,7 @@ __global__ __launch_bounds__(NT) void analysis_kernel(const float* __restrict__ 
     }
     __syncthreads();
     // table contraction over the rows of this chunk
-    const int nrow = n2 - row0 < RB ? n2 - row0 : RB;
+    const int nrow = rend - row0 < RB ? rend - row0 : RB;
 #pragma unroll
     for (int q = 0; q < 2; ++q) {
       if (!eok[q]) continue;
@@ -165,7 +196,7 @@ __global__ __launch_bounds__(NT) void analysis_kernel(const float* __restrict__ 
     if (eok[q]) out[(size_t)(t + q * NT) * nbatch + z] = acc[q];
 }
 
-// xhat [nb^2][nbatch] complex -> y [nbatch][n2][n2];  T [n2][nb^2]
+// xhat [nb^2][nbatch] complex -> y [nbatch][n2][n2];  T [n2][nb^2]; grid.y splits the rows
 __global__ __launch_bounds__(NT) void synthesis_kernel(const float2* __restrict__ xhat, const float* __restrict__ T,
                                                        float* __restrict__ y, int n2, int nb, long nbatch) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
@@ -184,8 +215,10 @@ __global__ __launch_bounds__(NT) void synthesis_kernel(const float2* __restrict_
   }
   for (int e = t; e < nspec; e += NT) xh[e] = xhat[(size_t)e * nbatch + z];
   __syncthreads();
+  const int rps = rows_per_split(n2, RB, gridDim.y);
+  const int rbeg = blockIdx.y * rps, rend = rbeg + rps < n2 ? rbeg + rps : n2;
 
-  for (int row0 = 0; row0 < n2; row0 += RB) {
+  for (int row0 = rbeg; row0 < rend; row0 += RB) {
     // A, B of the rows of this chunk: thread = (row, m >= 0), sum over l >= m
     for (int it = t; it < RB * nb; it += NT) {
       const int r = it / nb, m = it - r * nb;
