@@ -121,9 +121,9 @@ def _analysis(x, b_in, b_out, batch_size, for_grad, complex_in, mask=None):
     assert mask is None or not complex_in
     if complex_in and complex_via_real:
         # the transform is linear over the complex numbers: analysis(x) = analysis(Re x) + i analysis(Im x), and the
-        # kernels for real signals are the tuned ones
-        A = _analysis(x[..., 0].contiguous(), b_in, b_out, batch_size, for_grad, 0)
-        B = _analysis(x[..., 1].contiguous(), b_in, b_out, batch_size, for_grad, 0)
+        # kernels for real signals are the tuned ones; both parts go through them as one batch of twice the volumes
+        AB = _analysis(torch.stack((x[..., 0], x[..., 1]), 0), b_in, b_out, (2, *batch_size), for_grad, 0)
+        A, B = AB[:, 0], AB[:, 1]
         return torch.stack((A[..., 0] - B[..., 1], A[..., 1] + B[..., 0]), -1)
     if x.data_ptr() % 16:
         x = x.clone()
@@ -160,10 +160,10 @@ def _synthesis(x, b_in, b_out, batch_size, for_grad, complex_out, bias=None, rel
     assert not (relu and complex_out)
     if complex_out and complex_via_real:
         # y = synthesis(x) is complex-linear in x and the real-output kernels return Re y for ANY spectrum:
-        # Re y = real_synthesis(x), Im y = Re(-i y) = real_synthesis(-i x)
-        re = _synthesis(x, b_in, b_out, batch_size, for_grad, 0)
-        im = _synthesis(torch.stack((x[..., 1], -x[..., 0]), -1), b_in, b_out, batch_size, for_grad, 0)
-        return torch.stack((re, im), -1)
+        # Re y = real_synthesis(x), Im y = Re(-i y) = real_synthesis(-i x): one batch of twice the volumes
+        both = torch.stack((x, torch.stack((x[..., 1], -x[..., 0]), -1)), 1)          # [nspec, 2, ..., 2]
+        y = _synthesis(both, b_in, b_out, (2, *batch_size), for_grad, 0)
+        return torch.stack((y[0], y[1]), -1)
     L = _hip.lib()
     nbatch = 1
     for d in batch_size:
