@@ -35,17 +35,31 @@ def sum_of_squares(t):
     forward and one elementwise pass backward over the 1 GiB output.  (Autograd through out * out or
     vector_norm(out)**2 is the same function with three to five passes, none of them the layer's.)"""
     import torch
+    from s2cnn_amd import _hip
+
+    def timed(name, fn):
+        """fn() between two events on the launch stream while a KernelTimer is active: the loss is the harness's own
+        work, and its time is reported under its own keys beside the library's calls."""
+        timer = _hip.KernelTimer.active
+        if timer is None or not torch.cuda.is_available():
+            return fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        out = fn()
+        e1.record()
+        timer.records.append((name, e0, e1))
+        return out
 
     class _SumOfSquares(torch.autograd.Function):
         @staticmethod
         def forward(ctx, x):
             ctx.save_for_backward(x)
-            return torch.linalg.vector_norm(x).square()
+            return timed("harness_loss_forward", lambda: torch.linalg.vector_norm(x).square())
 
         @staticmethod
         def backward(ctx, g):
             (x,) = ctx.saved_tensors
-            return x * (2.0 * g)
+            return timed("harness_loss_backward", lambda: x * (2.0 * g))
 
     return _SumOfSquares.apply(t)
 
@@ -58,7 +72,7 @@ def mm_flops(nl, B, Fi, Fo, real=True):
     """Algorithmic flops of one block product: B Fi Fo sum_l (2l+1)^3 = B Fi Fo nl^2 (2 nl^2 - 1) multiply-adds,
     real (2 flops each) in the real basis the layer uses, complex (8 flops each) in so3_mm proper.  The complex kernels
     form a complex product from three real ones, so the matrix cores execute 6 flops per complex multiply-add: their
-    rows also give `mfma_executed_frac` = 3/4 of the algorithmic fraction."""
+    `frac` is that executed fraction, and `algorithmic_frac` (4/3 of it) the textbook count."""
     return (2.0 if real else 8.0) * B * Fi * Fo * nl * nl * (2 * nl * nl - 1)
 
 
@@ -149,8 +163,9 @@ def measure_rows(torch, dev, with_cpu):
     t = cpu_s(lambda: O.so3_mm(xm[:, :1], ymg.detach().cpu()))
     add("so3_mm fwd nl=32 B=16 64->64", gpu_ms(lambda: s2cnn_amd.so3_mm(xmg, ymg)), fl, "F", t, 1 / 16, "batch 1 of 16")
     add("so3_mm grad (x and y)", gpu_ms(lambda: torch.autograd.grad(zm, (xmg, ymg), gzm, retain_graph=True)), 2 * fl, "F", None, 1, "")
-    for k in ("so3_mm fwd nl=32 B=16 64->64", "so3_mm grad (x and y)"):
-        rows[k]["mfma_executed_frac"] = round(0.75 * rows[k]["frac"], 4)
+    for k in ("so3_mm fwd nl=32 B=16 64->64", "so3_mm grad (x and y)"):   # three real products per complex one: see measure_so3_mm
+        rows[k]["algorithmic_frac"] = rows[k]["frac"]
+        rows[k]["frac"] = round(0.75 * rows[k]["frac"], 4)
     del xm, xmg, ymg, zm, gzm
     # --- Haar integral at config-4 output size [16, 64, 64, 64, 64]
     xi = torch.randn(16, 64, 64, 64, 64, device=dev)
@@ -193,9 +208,10 @@ def measure_rows(torch, dev, with_cpu):
 
 def measure_so3_mm(torch, dev, reps=5):
     """Benchmark config 3: the complex block product alone, x [43680, 16, 64, 2], y [43680, 64, 64, 2] with entries
-    N(0, 1/64), forward and the gradients with respect to x and y, each timed with events on the launch stream.  `frac` is
-    algorithmic flops (8 per complex multiply-add) over the fp32 matrix peak; the kernels form a complex product from three
-    real ones, so the matrix cores execute 3/4 of that: `mfma_executed_frac`."""
+    N(0, 1/64), forward and the gradients with respect to x and y, each timed with events on the launch stream.  The kernels
+    form a complex product from three real ones (6 flops per complex multiply-add on the matrix cores instead of 8), so
+    `frac` = EXECUTED flops over the fp32 matrix peak (what the roofline bounds); `algorithmic_frac` counts the 8 flops of
+    the textbook complex multiply-add and can exceed 1."""
     import s2cnn_amd
     from s2cnn_amd import _hip
     nl, B, Fi, Fo = 32, 16, 64, 64
@@ -218,20 +234,20 @@ def measure_so3_mm(torch, dev, reps=5):
     pc = {k: sum(v) / len(v) for k, v in kt.summary().items()}
     fl = mm_flops(nl, B, Fi, Fo, real=False)
     out = {"workload": "so3_mm fwd + grad x + grad y, x [43680,16,64,2], y [43680,64,64,2] (benchmark config 3)", "bound": "mfma",
-           "flop_per_launch": fl, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s"}
+           "flop_per_launch": fl, "executed_flop_per_launch": 0.75 * fl, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s"}
     total = 0.0
     for name in ("s2cnn_so3_mm_fwd", "s2cnn_so3_mm_gradx", "s2cnn_so3_mm_grady"):
         ach = fl / (pc[name] * 1e-3) / 1e12
         total += pc[name]
-        out[name] = {"ms": round(pc[name], 3), "achieved": round(ach, 2), "frac": round(ach / PEAK_FP32_MFMA_TFLOPS, 4),
-                     "mfma_executed_frac": round(0.75 * ach / PEAK_FP32_MFMA_TFLOPS, 4)}
+        out[name] = {"ms": round(pc[name], 3), "achieved": round(0.75 * ach, 2), "frac": round(0.75 * ach / PEAK_FP32_MFMA_TFLOPS, 4),
+                     "algorithmic_tflops": round(ach, 2), "algorithmic_frac": round(ach / PEAK_FP32_MFMA_TFLOPS, 4)}
     out["ms_fwd_bwd"] = round(total, 3)
     del x, y, gz
     torch.cuda.empty_cache()
     return out
 
 
-def measure_network(torch, dev, steps, warmup):
+def measure_network(torch, dev, steps, warmup, separate_relu=True):
     """The SHREC17-shaped network of benchmark config 5 (S2Conv 6->100 b 128->32, ReLU, SO3Conv 100->100 b 32->22, ReLU,
     SO3Conv 100->55 b 22->7, so3_integrate; batch 32, near-identity grids scaled by the bandwidth ratio), forward and
     backward with respect to the weights, timed like the headline step; time inside library calls listed beside it.
@@ -278,16 +294,63 @@ def measure_network(torch, dev, steps, warmup):
         return ms, calls
 
     ms, calls = timed("relu")
-    ms_sep, calls_sep = timed(None)
-    return {"workload": "S2Conv 6->100 (b 128->32), SO3Conv 100->100 (32->22), SO3Conv 100->55 (22->7), integrate; batch 32, fwd+bwd (benchmark config 5)",
-            "ms_per_step": round(ms, 3), "samples_per_s": round(32 / (ms * 1e-3), 1),
-            "library_ms": round(sum(calls.values()), 3), "library_calls_ms": calls,
-            "separate_relu": {"ms_per_step": round(ms_sep, 3), "library_ms": round(sum(calls_sep.values()), 3)}}
+    out = {"workload": "S2Conv 6->100 (b 128->32), SO3Conv 100->100 (32->22), SO3Conv 100->55 (22->7), integrate; batch 32, fwd+bwd (benchmark config 5)",
+           "steps": steps, "ms_per_step": round(ms, 3), "samples_per_s": round(32 / (ms * 1e-3), 1),
+           "library_ms": round(sum(v for k, v in calls.items() if k.startswith("s2cnn_")), 3), "library_calls_ms": calls}
+    if separate_relu:
+        ms_sep, calls_sep = timed(None)
+        out["separate_relu"] = {"ms_per_step": round(ms_sep, 3),
+                                "library_ms": round(sum(v for k, v in calls_sep.items() if k.startswith("s2cnn_")), 3)}
+    return out
+
+
+def measure_config1(torch, dev, reps=50):
+    """Benchmark config 1: the digit network of examples/mnist/run.py:55-98 (S2Conv 1->20 b 30->10, ReLU, SO3Conv 20->40
+    b 10->6, ReLU, so3_integrate, Linear 40->10), forward only, batch 32, input uniform in [0, 1) with 70 % zeros.  Timed
+    eagerly (bound by its launches) and as one HIP graph replayed (nothing on the path allocates through HIP, synchronises or
+    records a memset)."""
+    from s2cnn_amd import _hip, harness
+    torch.manual_seed(0)
+    net = harness.S2ConvNet_original().to(dev).eval()
+    g = torch.Generator().manual_seed(1)
+    x = (torch.rand(32, 1, 60, 60, generator=g) * (torch.rand(32, 1, 60, 60, generator=g) < 0.3)).to(dev)
+
+    def wall_ms(fn):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / reps * 1e3
+
+    with torch.no_grad():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                net(x)                                  # tables, workspaces and allocator pools exist before the capture
+        torch.cuda.current_stream().wait_stream(side)
+        eager = wall_ms(lambda: net(x))
+        with _hip.KernelTimer() as kt:
+            net(x)
+            torch.cuda.synchronize()
+        library = sum(sum(v) for k, v in kt.summary().items())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            static_y = net(x)
+        replay = wall_ms(graph.replay)
+        same = bool(torch.equal(static_y, net(x)))
+    return {"workload": "S2Conv 1->20 (b 30->10), ReLU, SO3Conv 20->40 (b 10->6), ReLU, integrate, Linear 40->10; batch 32, forward "
+                        "(benchmark config 1)",
+            "eager_ms": round(eager, 4), "eager_samples_per_s": round(32 / (eager * 1e-3), 1), "library_ms": round(library, 4),
+            "graph_replay_ms": round(replay, 4), "graph_replay_samples_per_s": round(32 / (replay * 1e-3), 1),
+            "replay_equals_eager": same}
 
 
 def measure_fft_floor(torch, dev, nvol=256, reps=10):
     """What the plane pipeline of the per-volume 64^3 kernels costs without the Wigner contraction: the shipped kernels
-    with parts compiled out (s2cnn_so3_fft64_probe; the results of the stripped variants are meaningless), timed with
+    with parts compiled out (s2cnn_so3_fft64_probe of the measurement library libs2cnn_probe.so, built by
+    `python -m s2cnn_amd.csrc.build --probes`; the results of the stripped variants are meaningless), timed with
     events on the launch stream at the size of benchmark config 2.  The passes between records and spectral rows are
     timed from the full transforms (they are the difference between the transform and its kernel)."""
     from s2cnn_amd import _hip
@@ -296,6 +359,7 @@ def measure_fft_floor(torch, dev, nvol=256, reps=10):
     x = torch.randn(nvol, 64, 64, 64, generator=torch.Generator().manual_seed(3)).to(dev)
     y = torch.empty_like(x)
     L = _hip.lib()
+    P = _hip.probe_lib()
     ws = _hip.workspace(L.s2cnn_so3_analysis_workspace(b, b, nvol, 0), x.device)
     packed = {0: PSO3._setup_packed_wigner(b, b, True, False, x.device), 1: PSO3._setup_packed_wigner(b, b, False, True, x.device)}
     spec = PSO3.so3_rfft(x)
@@ -305,7 +369,7 @@ def measure_fft_floor(torch, dev, nvol=256, reps=10):
                 ("synthesis kernel", 1, 0), ("synthesis kernel, no contraction multiply-adds", 1, 1)]
     for name, direction, probe in variants:
         def run():
-            _hip.check(L.s2cnn_so3_fft64_probe(_hip.ptr(x), _hip.ptr(y), _hip.ptr(packed[direction]), _hip.ptr(ws), ws.numel(), nvol,
+            _hip.check(P.s2cnn_so3_fft64_probe(_hip.ptr(x), _hip.ptr(y), _hip.ptr(packed[direction]), _hip.ptr(ws), ws.numel(), nvol,
                                                direction, probe, _hip.stream_ptr()))
         if direction == 1:
             PSO3.so3_rifft(spec)                      # leaves the records of a real spectrum in the workspace
@@ -392,6 +456,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-fft", action="store_true", help="skip the standalone FFT round trip")
     ap.add_argument("--no-mm", action="store_true", help="skip the standalone complex so3_mm (benchmark config 3)")
+    ap.add_argument("--no-networks", action="store_true", help="skip benchmark configs 1 and 5 (the `config1` and `config5` objects)")
     ap.add_argument("--complex-product", action="store_true",
                     help="multiply complex spectra as the reference does instead of real-basis ones")
     ap.add_argument("--rows", action="store_true", help="also time every other op of the path (adds a `rows` object)")
@@ -463,7 +528,10 @@ def main():
                                   "this workload; not re-measured in this run)",
                 "flop_per_launch": flops, "ms_per_launch": round(per_call[dominant], 3)}
     if "_real_" not in dominant:   # three real products per complex one: the matrix cores execute 3/4 of the algorithmic flops
-        roofline["mfma_executed_frac"] = round(0.75 * roofline["frac"], 4)
+        roofline["algorithmic_frac"] = roofline["frac"]
+        roofline["achieved"] = round(0.75 * ach, 2)
+        roofline["frac"] = round(0.75 * roofline["frac"], 4)
+        roofline["flop_per_launch"] = 0.75 * flops
     kernels = {n: {"ms": round(ms, 3)} for n, ms in per_call.items()}
     for n in mm_names:
         kernels[n]["tflops"] = round(flops_of[n] / (per_call[n] * 1e-3) / 1e12, 2)
@@ -472,6 +540,16 @@ def main():
             nbytes = so3_fft_bytes(b, b, B * F) - (4 * nspec(b) * B * F if n.endswith("_real_basis") else 0)
             kernels[n]["gbs"] = round(nbytes / (per_call[n] * 1e-3) / 1e9, 1)
 
+    # where the step goes: the library's calls (the layer), the loss of the benchmark configuration (the harness's own two
+    # passes over the output) and what is left (the two small library GEMMs of the kernel spectrum, launches, gaps)
+    sums = {k: sum(v) / args.steps for k, v in timer.summary().items()}
+    library_ms = sum(v for k, v in sums.items() if k.startswith("s2cnn_"))
+    loss_ms = sum(v for k, v in sums.items() if k.startswith("harness_loss"))
+    breakdown = {"library_calls_ms": round(library_ms, 3), "harness_loss_ms": round(loss_ms, 3),
+                 "other_ms": round(ms_per_step - library_ms - loss_ms, 3),
+                 "layer_share_of_step": round(1.0 - loss_ms / ms_per_step, 4),
+                 "samples_per_s_without_harness_loss": round(B / ((ms_per_step - loss_ms) * 1e-3), 1)}
+
     result = {
         "metric": "SO3Conv fwd+bwd samples/s (b=32, 64->64 ch); SO(3) FFT achieved HBM GB/s",
         "value": round(value, 2), "unit": "samples/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -479,7 +557,7 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "SO3Convolution fwd+bwd, batch %d, %d->%d features, b_in=b_out=%d, 192-point "
                                "near-identity grid, loss=sum(out^2) (benchmark config 4)" % (B, F, F, b)},
-        "roofline": roofline, "kernels": kernels,
+        "roofline": roofline, "step_breakdown": breakdown, "kernels": kernels,
     }
 
     # ---- standalone SO(3) FFT round trip (benchmark config 2: [256, 64, 64, 64] -> [43680, 256, 2] -> back)
@@ -509,6 +587,10 @@ def main():
 
     if not args.no_mm:
         result["so3_mm"] = measure_so3_mm(torch, dev)
+    if not args.no_networks:
+        result["config1"] = measure_config1(torch, dev)
+        if args.network != "config5":
+            result["config5"] = measure_network(torch, dev, min(args.steps, 5), 2, separate_relu=False)
     if args.rows:
         result["rows"] = measure_rows(torch, dev, not args.no_cpu)
     if args.floor:

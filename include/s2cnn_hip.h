@@ -308,17 +308,6 @@ int s2cnn_so3_analysis_real_bn_relu_grad(const float *g, const float *y, const f
                                          void *workspace, size_t workspace_bytes,
                                          int b_in, int b_out, long nbatch, int real_basis, void *stream);
 
-/* ---- timing probe (not part of the drop-in path) --------------------------------------
- * The per-volume kernel of the 64^3 grid alone (direction 0: analysis, x -> records in the workspace; 1: synthesis,
- * records -> y), full spectra, with parts compiled out: probe 0 the kernel as shipped, 1 without the multiply-adds of the
- * Wigner contraction, 2 (analysis) without its table loads as well.  With probe != 0 the results are meaningless: the
- * entry exists so that `bench.py --floor` can time what the plane pipeline alone costs.  packed_table: the packed table
- * of s2cnn_so3_pack_table(32, 32, direction); workspace: s2cnn_so3_analysis_workspace(32, 32, nbatch, 0) bytes.
- * No counterpart in the reference.
- */
-int s2cnn_so3_fft64_probe(const float *x, float *y, const float *packed_table, void *workspace, size_t workspace_bytes,
-                          long nbatch, int direction, int probe, void *stream);
-
 /* ---- table repacking for the real-signal fast path of the two transforms above ------
  * The reference uploads its Wigner table once per (b, nl, weighted, device) and reuses it
  * (soft/so3_fft.py:205-209); a caller of this library does the same with the packed copy:

@@ -52,7 +52,6 @@ SIGNATURES = {
     "s2cnn_so3_relu_bits_bytes": (_size_t, [_int, _long]),
     "s2cnn_so3_synthesis_real_relu_bits": (_int, _FT3R_SIG[:4] + [_vp] + _FT3R_SIG[4:-1] + [_c_float_p, _int, _int, _vp]),
     "s2cnn_so3_analysis_real_masked_bits": (_int, [_c_float_p, _vp] + _FT3R_SIG[1:-1] + [_int, _vp]),
-    "s2cnn_so3_fft64_probe": (_int, [_c_float_p, _c_float_p, _c_float_p, _vp, _size_t, _long, _int, _int, _vp]),
     "s2cnn_so3_analysis_prologue_available": (_int, [_int, _int]),
     "s2cnn_so3_integrate_affine_relu": (_int, [_c_float_p, _c_float_p, _int, _c_float_p, _c_float_p, _int, _long, _vp]),
     "s2cnn_volume_moments": (_int, [_c_float_p, _c_float_p, _long, _long, _vp]),
@@ -91,6 +90,21 @@ def lib():
         fn = getattr(handle, name)
         fn.restype = res
         fn.argtypes = args
+    return handle
+
+
+PROBE_LIB_PATH = os.path.join(_HERE, "csrc", "libs2cnn_probe.so")
+
+
+@lru_cache(maxsize=1)
+def probe_lib():
+    """The measurement library (include/s2cnn_hip_probe.h): kernels with parts compiled out, for `bench.py --floor` only.
+    Built on request (`python -m s2cnn_amd.csrc.build --probes`); nothing in the package calls it."""
+    if not os.path.exists(PROBE_LIB_PATH):
+        raise RuntimeError("libs2cnn_probe.so is not built (%s); run `python -m s2cnn_amd.csrc.build --probes`" % PROBE_LIB_PATH)
+    handle = ctypes.CDLL(PROBE_LIB_PATH)
+    handle.s2cnn_so3_fft64_probe.restype = _int
+    handle.s2cnn_so3_fft64_probe.argtypes = [_c_float_p, _c_float_p, _c_float_p, _vp, _size_t, _long, _int, _int, _vp]
     return handle
 
 

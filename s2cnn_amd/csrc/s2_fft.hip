@@ -130,7 +130,19 @@ bool sizes_ok(int b_grid, int b_spec, long nbatch) {
 
 }  // namespace
 
-extern "C" size_t s2cnn_s2_analysis_workspace(int b_in, int b_out, long nbatch, int) { return ws_bytes(b_in, b_out, nbatch); }
+// The analysis of few real signals is split along beta and writes one partial spectrum per split into the workspace:
+// the size covers them (complex_in = 0), so that a split is never dropped for want of room.
+extern "C" size_t s2cnn_s2_analysis_workspace(int b_in, int b_out, long nbatch, int complex_in) {
+  size_t need = ws_bytes(b_in, b_out, nbatch);
+  if (need && !complex_in && b_out <= b_in) {
+    const s2_real::Plan plan = s2_real::plan_fwd(2 * b_in, b_out);
+    if (plan.rb > 0) {
+      const size_t split = (size_t)s2_real::splits_for(2 * b_in, plan.rb, nbatch) * b_out * b_out * nbatch * sizeof(float2);
+      if (split > need) need = split;
+    }
+  }
+  return need;
+}
 extern "C" size_t s2cnn_s2_synthesis_workspace(int b_in, int b_out, long nbatch, int) { return ws_bytes(b_out, b_in, nbatch); }
 
 extern "C" int s2cnn_s2_analysis(const float* x, const float* table, float* out, void* workspace, size_t workspace_bytes,
@@ -148,7 +160,9 @@ extern "C" int s2cnn_s2_analysis(const float* x, const float* table, float* out,
       // few signals: split along beta, partial spectra in the workspace, added up in a fixed order
       int nsplit = s2_real::splits_for(n2, plan.rb, nbatch);
       const size_t nout = (size_t)nb * nb * nbatch;
-      if (nsplit > 1 && nsplit * nout * sizeof(float2) > workspace_bytes) nsplit = 1;
+      if (nsplit > 1 && nsplit * nout * sizeof(float2) > workspace_bytes)      // a workspace sized for the two-kernel path only:
+        nsplit = (int)(workspace_bytes / (nout * sizeof(float2)));              // as many splits as it holds
+      if (nsplit < 2) nsplit = 1;
       float2* dst = nsplit > 1 ? static_cast<float2*>(workspace) : reinterpret_cast<float2*>(out);
       hipLaunchKernelGGL(s2_real::analysis_kernel, dim3((unsigned)nbatch, nsplit), dim3(s2_real::NT), plan.lds, st, x, table,
                          dst, n2, nb, nbatch, plan.rb);

@@ -753,21 +753,6 @@ extern "C" int s2cnn_so3_analysis_real_bn_relu_grad(const float* g, const float*
 }
 
 // ---------------------------------------------------------------------------------------------
-// Timing probe: the per-volume kernel of one direction on the 64^3 grid (without the pass between records and spectral
-// rows) with parts of it compiled out.  Not part of the drop-in path: with probe != 0 the results are meaningless.
-// ---------------------------------------------------------------------------------------------
-extern "C" int s2cnn_so3_fft64_probe(const float* x, float* y, const float* packed_table, void* workspace, size_t workspace_bytes,
-                                     long nbatch, int direction, int probe, void* stream) {
-  s2cnn::clear_stale_error();
-  if (!packed_table || nbatch < 1 || direction < 0 || direction > 1 || probe < 0 || probe > (direction == 0 ? 2 : 1)) return S2CNN_EINVAL;
-  if ((direction == 0 && !x) || (direction == 1 && !y)) return S2CNN_EINVAL;
-  if (!s2cnn::aligned16(x) || !s2cnn::aligned16(y) || !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
-  if (!workspace || workspace_bytes < fused64::scratch_bytes(nbatch) || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
-  fused64::launch_probe(direction, probe, static_cast<hipStream_t>(stream), x, y, packed_table, static_cast<float4*>(workspace), nbatch);
-  return s2cnn::launch_status();
-}
-
-// ---------------------------------------------------------------------------------------------
 // s2cnn_so3_analysis for callers that cannot allocate: the scratch is a buffer of the library's own.
 // `scratch` below is the host-side stand-in of the device array, not a device address: host code uses the
 // address that hipGetSymbolAddress returns for the current device (every GPU holds its own copy).

@@ -966,19 +966,6 @@ inline void launch_analysis(int nl, hipStream_t st, const s2cnn::Input& in, cons
   }
 }
 
-// The kernels with parts compiled out, for timing what the rest costs (see PROBE above); full spectra, no mask, no bias.
-inline void launch_probe(int direction, int probe, hipStream_t st, const float* x, float* y, const float* Tf, float4* rec, long nbatch) {
-  const dim3 grid(grid_size(nbatch)), block(THREADS);
-  if (direction == 0) {
-    if (probe == 1) hipLaunchKernelGGL((analysis_kernel<7, 0, 1>), grid, block, 0, st, x, nullptr, Tf, rec, nbatch, nullptr, 1);
-    else if (probe == 2) hipLaunchKernelGGL((analysis_kernel<7, 0, 2>), grid, block, 0, st, x, nullptr, Tf, rec, nbatch, nullptr, 1);
-    else hipLaunchKernelGGL((analysis_kernel<7, 0, 0>), grid, block, 0, st, x, nullptr, Tf, rec, nbatch, nullptr, 1);
-  } else {
-    if (probe == 1) hipLaunchKernelGGL((synthesis_kernel<7, 8, 1>), grid, block, 0, st, rec, Tf, y, nbatch, nullptr, 1, 0, nullptr, nullptr, nullptr, nullptr);
-    else hipLaunchKernelGGL((synthesis_kernel<7, 8, 0>), grid, block, 0, st, rec, Tf, y, nbatch, nullptr, 1, 0, nullptr, nullptr, nullptr, nullptr);
-  }
-}
-
 // bits: NULL, or BITS_WORDS 64-bit words per volume that receive one bit per sample: the output is not <= 0
 // degrees up to which the kernel has registers to spare for the second operand of the sums of MOM = 2
 constexpr int GRAD_MOMENTS_MAX_NL = 28;

@@ -165,7 +165,14 @@ def _statistics_mode(bn):
     if bn.training and bn.track_running_stats and bn.running_mean is not None:
         with torch.no_grad():
             bn.num_batches_tracked += 1
-        momentum = 1.0 / float(bn.num_batches_tracked) if bn.momentum is None else bn.momentum     # None: cumulative average
+        if bn.momentum is None:                           # cumulative average: the factor 1 / n is read on the host
+            if torch.cuda.is_current_stream_capturing():
+                raise RuntimeError("BatchNorm3d(momentum=None) cannot be recorded into a HIP graph: its averaging factor 1 / "
+                                   "num_batches_tracked is read on the host and would be frozen at the value of the capture; "
+                                   "give the module a numeric momentum, or run this step eagerly")
+            momentum = 1.0 / float(bn.num_batches_tracked)
+        else:
+            momentum = bn.momentum
         return training, momentum, bn.running_mean, bn.running_var
     if training:
         return training, momentum, None, None

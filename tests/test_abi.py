@@ -26,6 +26,24 @@ def test_library_exports_every_declared_symbol():
     assert lib.s2cnn_abi_version() == 1
 
 
+def test_measurement_entry_is_not_in_the_product_library():
+    """Kernels with parts compiled out live in a library of their own (include/s2cnn_hip_probe.h) that only
+    `bench.py --floor` loads: the drop-in boundary exports nothing of it."""
+    from s2cnn_amd import _hip
+    lib = _hip.lib()
+    text = open(os.path.join(ROOT, "include", "s2cnn_hip_probe.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = sorted(set(re.findall(r"\b(s2cnn_[a-z0-9_]+)\s*\(", text)))
+    assert names == ["s2cnn_so3_fft64_probe"]
+    for n in names:
+        assert not hasattr(lib, n) and n not in _hip.SIGNATURES
+    if os.path.exists(_hip.PROBE_LIB_PATH):
+        probe = _hip.probe_lib()
+        fake, null = ctypes.c_void_p(0x1000), ctypes.c_void_p(0)
+        assert probe.s2cnn_so3_fft64_probe(fake, fake, fake, fake, 1 << 30, 2, 1, 2, null) == -1     # the synthesis has no probe 2
+        assert probe.s2cnn_so3_fft64_probe(fake, fake, fake, fake, 0, 2, 0, 1, null) == -2           # workspace too small
+
+
 def test_argument_rejection_without_gpu():
     from s2cnn_amd import _hip
     lib = _hip.lib()
@@ -78,8 +96,6 @@ def test_argument_rejection_without_gpu():
     assert lib.s2cnn_so3_synthesis_real_basis_moments(fake, fake, null, fake, fake, 1 << 30, 32, 32, 3, null, 1, null, null, null, null) == -1    # nowhere to write the sums
     assert lib.s2cnn_so3_synthesis_real_basis_moments(fake, fake, null, fake, fake, 1 << 30, 32, 32, 3, null, 3, fake, fake, fake, null) == -1    # all 32 degrees with a second tensor
     assert lib.s2cnn_so3_integrate_affine_relu(fake, fake, 2, fake, fake, 4, 3, null) == -1              # 3 volumes, 2 features
-    assert lib.s2cnn_so3_fft64_probe(fake, fake, fake, fake, 1 << 30, 2, 1, 2, null) == -1               # the synthesis has no probe 2
-    assert lib.s2cnn_so3_fft64_probe(fake, fake, fake, fake, 0, 2, 0, 1, null) == -2                     # workspace too small
     # entry points of the real-basis path and the biased synthesis
     assert lib.s2cnn_s2_mm_real_fwd(null, null, null, 4, 2, 3, 5, null) == -1
     assert lib.s2cnn_s2_mm_real_gradx(fake, fake, fake, 4, 0, 3, 5, null) == -1                # empty batch

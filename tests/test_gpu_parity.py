@@ -214,6 +214,28 @@ def test_s2_transforms(hip, b_in, b_out, for_grad):
     close(PS2.s2_rifft(s.cuda(), for_grad, b_in), O.s2_ifft(s.double(), for_grad, b_in)[..., 0], "s2_rifft")
 
 
+@pytest.mark.parametrize("b,nbatch", [(12, 5), (32, 100), (20, 1)])
+def test_s2_analysis_of_few_signals_at_full_bandwidth(hip, b, nbatch):
+    """b_out = b_in with few signals: the analysis is split along beta and the partial spectra go through the workspace
+    (s2cnn_s2_analysis_workspace covers them).  Checked against the oracle, and through the raw C ABI with a workspace of
+    the two-kernel path's size only, where the library must run with as many splits as fit and give the same spectrum."""
+    import ctypes
+    x = rnd((nbatch, 2 * b, 2 * b), 33 + b)
+    want = O.s2_fft(O.as_complex(x.double()), False, b)
+    got = PS2.s2_rfft(x.cuda(), False, b)
+    close(got, want, f"s2_rfft b={b}, {nbatch} signals")
+    xg = x.cuda()
+    table = PS2._setup_wigner(b, b, True, xg.device)
+    small = nbatch * 2 * b * (2 * b - 1) * 8
+    assert hip.s2cnn_s2_analysis_workspace(b, b, nbatch, 0) >= small
+    ws = torch.empty(small, dtype=torch.uint8, device=xg.device)
+    out = torch.full_like(got, float("nan"))
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    rc = hip.s2cnn_s2_analysis(p(xg), p(table), p(out), p(ws), small, b, b, nbatch, 0, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0
+    close(out, want, "the same with the smaller workspace")
+
+
 def test_so3_integrate(hip):
     for b in (1, 3, 6, 16, 32):                     # 32: the 16-byte-load path (planes of 4096 samples)
         x = rnd((2, 5, 2 * b, 2 * b, 2 * b), 40 + b)

@@ -46,6 +46,43 @@ def test_static_scratch_analysis_equals_workspace_analysis(hip, b_in, b_out, n_f
             assert torch.equal(ref, out), (b_in, b_out, n, use_packed)
 
 
+def test_static_scratch_analysis_allocates_nothing(hip):
+    """The defining property: after a first call on the device (which resolves the address of the library's buffer), a
+    call leaves the free device memory as it found it, and it can be recorded into a HIP graph (a hipMalloc during a
+    capture fails) whose replays give the eager result."""
+    from s2cnn_amd.soft import so3_fft as PSO3
+    dev = torch.device("cuda:0")
+    b = 32
+    table = PSO3._setup_wigner(b, b, True, dev)
+    packed = PSO3._setup_packed_wigner(b, b, True, False, dev)
+    x = torch.randn(6, 2 * b, 2 * b, 2 * b, generator=torch.Generator().manual_seed(7)).to(dev)
+    out = torch.empty(_nspec(b), 6, 2, device=dev)
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+
+    def run(stream):
+        return hip.s2cnn_so3_analysis_static(p(x), p(table), p(packed), p(out), b, b, 6, 0, ctypes.c_void_p(stream.cuda_stream))
+
+    assert run(torch.cuda.current_stream()) == 0
+    torch.cuda.synchronize()
+    want = out.clone()
+    free_before = torch.cuda.mem_get_info(dev)[0]
+    for _ in range(3):
+        assert run(torch.cuda.current_stream()) == 0
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info(dev)[0] == free_before            # hipMemGetInfo: no device memory was taken
+    assert torch.equal(out, want)
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.graph(graph, stream=side):
+        assert run(torch.cuda.current_stream()) == 0                 # the capture stream
+    for _ in range(2):
+        out.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want)
+
+
 def test_static_scratch_rejects_what_does_not_fit(hip):
     dev = torch.device("cuda:0")
     fake = ctypes.c_void_p(torch.empty(64, device=dev).data_ptr())
