@@ -22,8 +22,8 @@ extern "C" int s2cnn_so3_fft64_probe(const float* x, float* y, const float* pack
     else if (probe == 2) hipLaunchKernelGGL((analysis_kernel<7, 0, 2>), grid, block, 0, st, x, nullptr, packed_table, rec, nbatch, nullptr, 1);
     else hipLaunchKernelGGL((analysis_kernel<7, 0, 0>), grid, block, 0, st, x, nullptr, packed_table, rec, nbatch, nullptr, 1);
   } else {
-    if (probe == 1) hipLaunchKernelGGL((synthesis_kernel<7, 8, 1>), grid, block, 0, st, rec, packed_table, y, nbatch, nullptr, 1, 0, nullptr, nullptr, nullptr, nullptr);
-    else hipLaunchKernelGGL((synthesis_kernel<7, 8, 0>), grid, block, 0, st, rec, packed_table, y, nbatch, nullptr, 1, 0, nullptr, nullptr, nullptr, nullptr);
+    if (probe == 1) hipLaunchKernelGGL((synthesis_kernel<7, 1>), grid, block, 0, st, rec, packed_table, y, nbatch, nullptr, 1, 0, nullptr, nullptr, nullptr, nullptr);
+    else hipLaunchKernelGGL((synthesis_kernel<7, 0>), grid, block, 0, st, rec, packed_table, y, nbatch, nullptr, 1, 0, nullptr, nullptr, nullptr, nullptr);
   }
   return s2cnn::launch_status();
 }

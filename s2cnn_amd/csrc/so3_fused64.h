@@ -10,7 +10,11 @@
 //
 // Work decomposition: an ITEM is (c, a, n) = four consecutive degrees l = 4c..4c+3 of the two columns
 // (m = +a, n) and (m = -a, n), 0 <= a, n <= 4c+3.  There are sum_c (4c+4)^2 = 3264 items for c < 8;
-// thread t owns items t, t+512, ..., t+6*512, i.e. 7 x 4 x 2 complex values in registers.
+// a thread owns 7 of them (one per ROUND), i.e. 7 x 4 x 2 complex values in registers.  Which ones is a table
+// (so3_fused64_items.h, written by gen_fused64_items.py): consecutive rounds of a thread hold the same column (a, n)
+// where they can, because the bins of a column are then read (analysis) or written (synthesis) once for the whole
+// RUN of rounds instead of once per item, and items of low degree sit in the first rounds, so that a truncated
+// spectrum skips the later ones.  Nothing below depends on the assignment beyond what the table says.
 // With P = plane of beta_j, P' = plane of beta_{63-j}, t1 = T[j,l,+a,n], t2 = T[j,l,-a,n], s = (-1)^(l-n):
 //   analysis : X[l,+a,n] += t1 P[+a,n] + s t2 P'[+a,n]      X[l,-a,n] += t2 P[-a,n] + s t1 P'[-a,n]
 //   synthesis: S[+a,n] = sum_l t1 xs[l,+a,n]   S'[+a,n] = sum_l s t2 xs[l,+a,n]   (and -a with t1 <-> t2)
@@ -26,6 +30,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include "so3_plane_fft64.h"
+#include "so3_fused64_items.h"
 
 namespace fused64 {
 
@@ -66,25 +71,16 @@ __device__ __forceinline__ float flip(float x, unsigned signbit) { return __uint
 
 __host__ __device__ inline int lmn_index(int l, int m, int n) { return l * (4 * l * l - 1) / 3 + (l + m) * (2 * l + 1) + (l + n); }
 
-// item index -> (c, a, n); false for the padding slots behind the last item
-__host__ __device__ inline bool decode_item(int i, int& c, int& a, int& n) {
-  c = 0; a = 0; n = 0;
-  if (i >= NITEMS) return false;
-  int off = 0;
-  for (int cc = 0; cc < 8; ++cc) {
-    const int s = 4 * cc + 4;
-    if (i < off + s * s) {
-      const int r = i - off;
-      c = cc; a = r / s; n = r - a * s;
-      return true;
-    }
-    off += s * s;
-  }
-  return false;
+// place i = round * THREADS + thread -> its item (c, a, n); false for a place without an item (a, n then name the
+// column of the neighbouring round, so that the place starts no run of its own)
+__device__ __forceinline__ bool decode_item(int i, int& c, int& a, int& n) {
+  const unsigned e = ITEM_TABLE[i];
+  n = (int)(e & 31u); a = (int)((e >> 5) & 31u); c = (int)((e >> 10) & 7u);
+  return (e >> 13) & 1u;
 }
 
 // Packed table: float index ((((j*NIT + it)*2 + h)*THREADS + t)*4 + u) holds
-//   0.5 * T[j, l = 4c+u, m = (h ? -a : +a), n]   for item (c, a, n) = it*THREADS + t,
+//   0.5 * T[j, l = 4c+u, m = (h ? -a : +a), n]   for the item (c, a, n) of place it*THREADS + t,
 // zero where l < max(a, n), l >= nl, or the slot is padding.  T is [64][nspec_stride].
 __global__ void pack_table(const float* __restrict__ T, float* __restrict__ Tf, long nspec_stride, int nl) {
   for (size_t e = blockIdx.x * (size_t)blockDim.x + threadIdx.x; e < PACKED_FLOATS; e += (size_t)gridDim.x * blockDim.x) {
@@ -202,8 +198,9 @@ __host__ __device__ constexpr int quad_row(int a) { return a * QPITCH + 2 * (a >
 //   after item 0, 1, 2: items 4, 5, 6 of the same plane pair;  after 3, 4, 5, 6: items 3, 0, 1, 2 of the next pair
 __device__ constexpr int table_slot(int it) { return it & 3; }
 
-// NA: item rounds that carry degrees below the output bandwidth (items are ordered by degree group, so a truncated
-// spectrum leaves the later rounds without work: NA = 3 covers l < 24, 5 covers l < 28, 7 everything).
+// NA: item rounds that carry degrees below the output bandwidth (the item table puts the low degree groups into the
+// first rounds, so a truncated spectrum leaves the later rounds without work: NA = 3 covers l < 24, 6 covers l < 28, 7
+// everything).
 // MASK: what is done to x as it is loaded, one of s2cnn::Prologue: 0: nothing; 1: x where mask > 0 and zero elsewhere
 // (mask: a tensor of the shape of x); 2: the same with `mask` holding one BIT per sample instead (bits_index below), as
 // the synthesis writes them; 3: max(a x + b, 0); 4: a (a mask + b > 0 ? x : 0) + p + q mask, with a, b, p, q of the
@@ -244,6 +241,7 @@ __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restri
     decode_item(it * THREADS + t, c, a, n);
     adr[it] = (unsigned)(quad_row(a) + 4 * n) | ((unsigned)(n & 1) << 31);
   }
+
   // where this thread's outputs of the last gamma stage go: row slot lo holds m = sigma(lo)
   const int m = sigma(lo);
   // quad[a][n] = { Z[+a,n], Z[-a,-n], Z[-a,n], Z[+a,-n] }; +0 and -0 are the same frequency, so
@@ -334,18 +332,24 @@ __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restri
     for (int k2 = 4; k2 < 8; ++k2) q[qa + 4 * (64 - d - 8 * k2) + pos_hi] = v[k2];   // n = 32 (d = 0, k2 = 4) lands in the pad of the row
     q[extra] = v[0];
   };
-  auto accumulate = [&](const float2* q, int it) {
-    const float4* src = reinterpret_cast<const float4*>(q + (adr[it] & 0x7fffffffu));
-    const float4 za = src[0], zb = src[1];              // Z[+a,n], Z[-a,-n] | Z[-a,n], Z[+a,-n]
-    const unsigned sb = adr[it] & 0x80000000u;
-    // twice the separated planes (the table carries the factor 1/2):
-    // P = Z[m,n] + conj Z[-m,-n],  P' = (Z[m,n] - conj Z[-m,-n]) / i, the latter times (-1)^n
-    const float2 Pp = make_float2(za.x + za.z, za.y - za.w);
-    const float2 Qp = make_float2(flip(za.y + za.w, sb), flip(za.z - za.x, sb));
-    const float2 Pm = make_float2(zb.x + zb.z, zb.y - zb.w);
-    const float2 Qm = make_float2(flip(zb.y + zb.w, sb), flip(zb.z - zb.x, sb));
+  // fresh: the rounds in which some thread of this half of the workgroup starts another column (FRESH_LO, FRESH_HI of the
+  // item table, compile-time): the quad is read and separated there and serves the rounds that follow
+  float2 Pp, Qp, Pm, Qm;          // the separated bins of the column of the current run
+  auto accumulate = [&](const float2* q, int it, unsigned fresh) {
+    if (it == 0 || ((fresh >> it) & 1u)) {
+      const float4* src = reinterpret_cast<const float4*>(q + (adr[it] & 0x7fffffffu));
+      const float4 za = src[0], zb = src[1];              // Z[+a,n], Z[-a,-n] | Z[-a,n], Z[+a,-n]
+      const unsigned sb = adr[it] & 0x80000000u;
+      // twice the separated planes (the table carries the factor 1/2):
+      // P = Z[m,n] + conj Z[-m,-n],  P' = (Z[m,n] - conj Z[-m,-n]) / i, the latter times (-1)^n
+      Pp = make_float2(za.x + za.z, za.y - za.w);
+      Qp = make_float2(flip(za.y + za.w, sb), flip(za.z - za.x, sb));
+      Pm = make_float2(zb.x + zb.z, zb.y - zb.w);
+      Qm = make_float2(flip(zb.y + zb.w, sb), flip(zb.z - zb.x, sb));
+    }
     const float4 ta = t1[table_slot(it)], tb = t2[table_slot(it)];
-    if constexpr (PROBE != 0) {
+    if constexpr (PROBE == 1 || PROBE == 2) {
+      const float4 za = make_float4(Pp.x, Pp.y, Qp.x, Qp.y), zb = make_float4(Pm.x, Pm.y, Qm.x, Qm.y);
       accp[it][0].x += za.x + ta.x; accm[it][0].x += zb.x + tb.x;
       return;
     }
@@ -383,7 +387,7 @@ __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restri
   // memory instructions are spread over the step so that their queue never fills up
 #define S2CNN_ACC(k, jl, il)                                                                             \
   if constexpr ((k) < NA) {                                                                              \
-    accumulate(cur, k); S2CNN_FENCE();                                                                   \
+    accumulate(cur, k, FR); S2CNN_FENCE();                                                               \
     if constexpr ((k) + 4 < NA) load_table(j, (k) + 4); else load_table(j + 1, (k) & 3);                 \
     S2CNN_FENCE();                                                                                       \
   }
@@ -391,6 +395,7 @@ __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restri
   // Waves d < 4 transform first and contract second, waves d >= 4 the other way round: each SIMD holds one
   // wave of either kind, so its LDS-bound and its FMA-bound half of a stage overlap.
   if (d < 4) {
+    constexpr unsigned FR = FRESH_LO;
     for (int j = 0; j < NJ - 1; ++j) {
       const float2* cur = quad[j & 1];
       float2* nxt = quad[(j + 1) & 1];
@@ -409,6 +414,7 @@ __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restri
       __syncthreads();
     }
   } else {
+    constexpr unsigned FR = FRESH_HI;
     for (int j = 0; j < NJ - 1; ++j) {
       const float2* cur = quad[j & 1];
       float2* nxt = quad[(j + 1) & 1];
@@ -440,7 +446,7 @@ __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restri
     const float2* cur = quad[(NJ - 1) & 1];
 #define S2CNN_LAST(k)                                                                                    \
   if constexpr ((k) < NA) {                                                                              \
-    accumulate(cur, k);                                                                                  \
+    accumulate(cur, k, FRESH_LO | FRESH_HI);                                                             \
     if constexpr ((k) + 4 < NA) { S2CNN_FENCE(); load_table(NJ - 1, (k) + 4); S2CNN_FENCE(); }           \
   }
     S2CNN_LAST(0) S2CNN_LAST(1) S2CNN_LAST(2) S2CNN_LAST(3) S2CNN_LAST(4) S2CNN_LAST(5) S2CNN_LAST(6)
@@ -690,13 +696,15 @@ __global__ __launch_bounds__(256) void spectrum_gather_real(const float* __restr
 // synthesis: records of the symmetrised spectrum -> y [nbatch][64][64][64] real
 //
 // While plane pair j is transformed in `work` (two gamma stages, two alpha stages, the last one
-// straight into the global stores), every item puts its share of the bins of pair j+1 into a staging
-// area; a reduction over the (up to 8) items of a column then fills `work` for the next step.
+// straight into the global stores), the shares of the items in the bins of pair j+1 are summed in registers
+// over each RUN of rounds that hold the same column, and leave for a staging area when the run ends.  The
+// item table cuts a column into at most two runs; the staging area has one place per column and run, and
+// a reduction over the two places fills `work` for the next step.
 // Sums are formed in a fixed order: results are reproducible bit for bit.
 // ---------------------------------------------------------------------------------------------
 // bias: NULL, or one value per feature added to every sample of volume z (feature = z % nfeature)
 // relu: nonzero = negative samples (after the bias) are stored as zero
-// NA as in analysis_kernel; CMAX: degree groups c < CMAX carry degrees of the input (6 for NA = 3, 7 for 5, 8 for 7)
+// NA as in analysis_kernel
 // PROBE (measurement only, results meaningless): 1: an item's share of a plane pair reduced to one add per table operand.
 // MOM: the kernel also writes two sums over the volume it produces, formed in a fixed order, to moments[z]:
 //   1: (sum v, sum v^2) of the output v (bias included, before the activation): the statistics of a batch normalisation
@@ -704,7 +712,7 @@ __global__ __launch_bounds__(256) void spectrum_gather_real(const float* __restr
 //   2: (sum v m, sum v m w) with w = yref at the same sample and m = (a w + b > 0), a = params[f], b = params[nfeature + f],
 //      f = z % nfeature: the two reductions of the gradient of such a normalisation followed by max(., 0), with the
 //      output as the incoming gradient (s2cnn::bn_relu_grad).
-template <int NA, int CMAX, int PROBE = 0, int MOM = 0>
+template <int NA, int PROBE = 0, int MOM = 0>
 __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __restrict__ rec, const float* __restrict__ Tf,
                                                             float* __restrict__ y, long nbatch, const float* __restrict__ bias, int nfeature,
                                                             int relu, unsigned long long* __restrict__ bits, float2* __restrict__ moments,
@@ -712,9 +720,9 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
   using namespace fft64;
   __shared__ __attribute__((aligned(16))) float2 work[LDS_ELEMS];
   float ms1 = 0.f, ms2 = 0.f;
-  constexpr int STG_PADS = 144;                                              // one pad per row: sum of (4c+4) over the 8 degree groups
-  __shared__ __attribute__((aligned(16))) float4 stg_p[NIT * THREADS + STG_PADS];   // item (c, a, n): its share of the bins [+a,n], [-a,-n]
-  __shared__ __attribute__((aligned(16))) float4 stg_m[NIT * THREADS + STG_PADS];   //                                      [-a,n], [+a,-n]
+  constexpr int NCOL = 32 * 32;                                               // columns (a, n), a, n < 32
+  __shared__ __attribute__((aligned(16))) float4 stg_p[2 * NCOL];             // [run of the column][32 a + n]: the run's share of the bins [+a,n], [-a,-n]
+  __shared__ __attribute__((aligned(16))) float4 stg_m[2 * NCOL];             //                                                            [-a,n], [+a,-n]
   const long z = volume_of_block(nbatch);
   if (z < 0) return;
   const int t = threadIdx.x;
@@ -723,15 +731,16 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
   Twiddles twl;
   make_twiddles<true>(twl);
   for (int i = t; i < LDS_ELEMS; i += THREADS) work[i] = make_float2(0.f, 0.f);   // bins of m = 32 and n = 32 stay zero ... until a transform overwrites them: cleared again in reduce()
+  // places of the staging area that no run writes (the second place of a column with one run, the columns beyond a
+  // truncated spectrum) are read by reduce() all the same: they stay zero
+  for (int i = t; i < 2 * NCOL; i += THREADS) { stg_p[i] = make_float4(0.f, 0.f, 0.f, 0.f); stg_m[i] = make_float4(0.f, 0.f, 0.f, 0.f); }
 
   float2 xp[NIT][4], xm[NIT][4];
-  unsigned sgn = 0;                 // bit it = n odd for item it
-  // Where an item's share goes in the staging area: the rows of degree group c are (4c+5) entries apart (one pad per
-  // row), so that the threads of reduce() that walk down a column hit different banks.  Kept as the number of pads in
-  // front of the item (at most 144), four of them per word.
-  unsigned spad[(NIT + 3) / 4];
+  // the table entries of this thread's places, two per word: bits 0-9 the column 32 a + n (bit 0 = n odd), bit 14 which of
+  // the column's two runs this one is, bit 15 the run ends with this round
+  unsigned ent[(NIT + 1) / 2];
 #pragma unroll
-  for (int w = 0; w < (NIT + 3) / 4; ++w) spad[w] = 0;
+  for (int w = 0; w < (NIT + 1) / 2; ++w) ent[w] = 0;
   const __amdgpu_buffer_rsrc_t rr = make_rsrc(rec + (size_t)z * REC_F4, (unsigned)REC_BYTES);
   const __amdgpu_buffer_rsrc_t rt = make_rsrc(Tf, (unsigned)(PACKED_FLOATS * 4));
   const __amdgpu_buffer_rsrc_t ry = make_rsrc(y + (size_t)z * (N * N * N), N * N * N * 4);
@@ -742,14 +751,7 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
   if constexpr (MOM == 2) { mom_a = params[z % nfeature]; mom_b = params[nfeature + z % nfeature]; }
 #pragma unroll
   for (int it = 0; it < NA; ++it) {
-    int c, a, n;
-    const bool item = decode_item(it * THREADS + t, c, a, n);
-    sgn |= (unsigned)(n & 1) << it;
-    {
-      constexpr int PADC[8] = {0, 4, 12, 24, 40, 60, 84, 112};      // pads in front of degree group c
-      const unsigned pad = item ? (unsigned)(a + PADC[c]) : (unsigned)STG_PADS;   // padding slots land behind the last item
-      spad[it >> 2] |= pad << (8 * (it & 3));
-    }
+    ent[it >> 1] |= (unsigned)ITEM_TABLE[it * THREADS + t] << (16 * (it & 1));
     const float4 v0 = buf_load_f32x4(rr, toff, (it * 4 + 0) * (THREADS * 16)), v1 = buf_load_f32x4(rr, toff, (it * 4 + 1) * (THREADS * 16));
     const float4 v2 = buf_load_f32x4(rr, toff, (it * 4 + 2) * (THREADS * 16)), v3 = buf_load_f32x4(rr, toff, (it * 4 + 3) * (THREADS * 16));
     xp[it][0] = make_float2(v0.x, v0.y); xp[it][1] = make_float2(v0.z, v0.w);
@@ -757,20 +759,6 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
     xm[it][0] = make_float2(v2.x, v2.y); xm[it][1] = make_float2(v2.z, v2.w);
     xm[it][2] = make_float2(v3.x, v3.y); xm[it][3] = make_float2(v3.z, v3.w);
   }
-  // the two columns (a, n) this thread reduces: shell order q -> k = max(a, n), (k, 0..k) then (0..k-1, k);
-  // q = t and 1023 - t, so that the lanes of a wave have the same number of items per column
-  int ca[2], cn[2];
-#pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    const int q = h ? 1023 - t : t;
-    int k = (int)sqrtf((float)q);
-    if (k * k > q) --k;
-    if ((k + 1) * (k + 1) <= q) ++k;
-    const int rr = q - k * k;
-    ca[h] = rr <= k ? k : rr - k - 1;
-    cn[h] = rr <= k ? rr : k;
-  }
-
   float4 t1[4], t2[4];
   auto load_table = [&](int j, int it) {
     t1[table_slot(it)] = buf_load_f32x4(rt, toff, ((j * NIT + it) * 2 + 0) * (THREADS * 16));
@@ -778,13 +766,15 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
   };
   // the item's share of a plane pair: S = sum_l t1 xs, S' = sum_l s t2 xs at (+a, n), t1 <-> t2 at (-a, n);
   // complex plane Z = S + i S' at [m,n], its Hermitian partner conj S + i conj S' at [-m,-n]
-  auto contribute = [&](int it) {
+  // the sums of the current run: S = sum_l t1 xs, S' = sum_l s t2 xs at (+a, n), t1 <-> t2 at (-a, n)
+  float2 Sp = make_float2(0.f, 0.f), Qp = make_float2(0.f, 0.f), Sm = make_float2(0.f, 0.f), Qm = make_float2(0.f, 0.f);
+  // fresh: as in analysis_kernel; a run can only end in front of a round that starts one, or in the last round
+  auto contribute = [&](int it, unsigned fresh) {
     const float4 ta = t1[table_slot(it)], tb = t2[table_slot(it)];
     const float a1[4] = {ta.x, ta.y, ta.z, ta.w};
     const float a2[4] = {tb.x, tb.y, tb.z, tb.w};
-    float2 Sp = make_float2(0.f, 0.f), Qp = make_float2(0.f, 0.f), Sm = make_float2(0.f, 0.f), Qm = make_float2(0.f, 0.f);
     if constexpr (PROBE != 0) {
-      Sp.x = a1[0] + xp[it][0].x; Sm.x = a2[0] + xm[it][0].x;
+      Sp.x += a1[0] + xp[it][0].x; Sm.x += a2[0] + xm[it][0].x;
     } else {
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
@@ -794,30 +784,29 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
         Sm.x = fmaf(a2[u], xm[it][u].x, Sm.x); Sm.y = fmaf(a2[u], xm[it][u].y, Sm.y);
         Qm.x = fmaf(b1, xm[it][u].x, Qm.x);    Qm.y = fmaf(b1, xm[it][u].y, Qm.y);
       }
-      const unsigned sb = ((sgn >> it) & 1u) << 31;
-      Qp.x = flip(Qp.x, sb); Qp.y = flip(Qp.y, sb); Qm.x = flip(Qm.x, sb); Qm.y = flip(Qm.y, sb);
     }
-    const unsigned pos = it * THREADS + t + ((spad[it >> 2] >> (8 * (it & 3))) & 0xffu);
-    stg_p[pos] = make_float4(Sp.x - Qp.y, Sp.y + Qp.x, Sp.x + Qp.y, Qp.x - Sp.y);
-    stg_m[pos] = make_float4(Sm.x - Qm.y, Sm.y + Qm.x, Sm.x + Qm.y, Qm.x - Sm.y);
+    // the run ends here (in the last round every run does): complex plane Z = S + i S' at [m,n], its Hermitian partner
+    // conj S + i conj S' at [-m,-n], the factor (-1)^n of S' in the sign bit; then the sums start again
+    if (it != NA - 1 && !((fresh >> (it + 1)) & 1u)) return;
+    const unsigned e = (ent[it >> 1] >> (16 * (it & 1))) & 0xffffu;
+    if (it == NA - 1 || (e >> 15)) {
+      const unsigned sb = (e & 1u) << 31;
+      const float qpx = flip(Qp.x, sb), qpy = flip(Qp.y, sb), qmx = flip(Qm.x, sb), qmy = flip(Qm.y, sb);
+      const unsigned pos = ((e >> 4) & 0x400u) | (e & 0x3ffu);
+      stg_p[pos] = make_float4(Sp.x - qpy, Sp.y + qpx, Sp.x + qpy, qpx - Sp.y);
+      stg_m[pos] = make_float4(Sm.x - qmy, Sm.y + qmx, Sm.x + qmy, qmx - Sm.y);
+      Sp = make_float2(0.f, 0.f); Qp = Sp; Sm = Sp; Qm = Sp;
+    }
   };
-  // staging -> work (natural order): sum over the items c = max(a,n)/4 .. 7 of each column, in that order
+  // staging -> work (natural order): the two runs of each column, in that order; thread t takes the columns t and t + 512
   auto reduce = [&]() {
-    constexpr int OFF[8] = {0, 20, 92, 248, 520, 940, 1540, 2352};    // sum of (4c'+4)(4c'+5) over c' < c
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-      const int a = ca[h], n = cn[h];
-      const int cmin = (a > n ? a : n) >> 2;
-      float4 s0 = make_float4(0.f, 0.f, 0.f, 0.f), s1 = s0;
-#pragma unroll
-      for (int c = 0; c < 8; ++c) {
-        if (c >= cmin && c < CMAX) {
-          const int i = OFF[c] + a * (4 * c + 5) + n;
-          const float4 u0 = stg_p[i], u1 = stg_m[i];
-          s0.x += u0.x; s0.y += u0.y; s0.z += u0.z; s0.w += u0.w;
-          s1.x += u1.x; s1.y += u1.y; s1.z += u1.z; s1.w += u1.w;
-        }
-      }
+      const int col = t + h * THREADS;
+      const int a = col >> 5, n = col & 31;
+      const float4 u0 = stg_p[col], v0 = stg_p[NCOL + col], u1 = stg_m[col], v1 = stg_m[NCOL + col];
+      const float4 s0 = make_float4(u0.x + v0.x, u0.y + v0.y, u0.z + v0.z, u0.w + v0.w);
+      const float4 s1 = make_float4(u1.x + v1.x, u1.y + v1.y, u1.z + v1.z, u1.w + v1.w);
       const int rp = a * PITCH, rm = ((64 - a) & 63) * PITCH;
       work[rp + n] = make_float2(s0.x, s0.y);
       if (n > 0) work[rm + 64 - n] = make_float2(s0.z, s0.w);
@@ -871,7 +860,7 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
   // (pair P being contributed; the slot then takes item k + 4 of the same pair or item k % 4 of the next one)
 #define S2CNN_CON(k, P)                                                                                  \
   if constexpr ((k) < NA) {                                                                              \
-    contribute(k); S2CNN_FENCE();                                                                        \
+    contribute(k, FR); S2CNN_FENCE();                                                                    \
     if constexpr ((k) + 4 < NA) load_table((P) < NJ ? (P) : NJ - 1, (k) + 4);                            \
     else load_table((P) + 1 < NJ ? (P) + 1 : NJ - 1, (k) & 3);                                           \
     S2CNN_FENCE();                                                                                       \
@@ -881,7 +870,10 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
   if constexpr (NA > 2) load_table(0, 2);
   if constexpr (NA > 3) load_table(0, 3);
   __syncthreads();
-  S2CNN_CON(0, 0) S2CNN_CON(1, 0) S2CNN_CON(2, 0) S2CNN_CON(3, 0) S2CNN_CON(4, 0) S2CNN_CON(5, 0) S2CNN_CON(6, 0)
+  {
+    constexpr unsigned FR = FRESH_LO | FRESH_HI;
+    S2CNN_CON(0, 0) S2CNN_CON(1, 0) S2CNN_CON(2, 0) S2CNN_CON(3, 0) S2CNN_CON(4, 0) S2CNN_CON(5, 0) S2CNN_CON(6, 0)
+  }
   __syncthreads();
   reduce();
   __syncthreads();
@@ -890,6 +882,7 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
   // Waves d < 4 transform first, waves d >= 4 last: each SIMD holds one wave of either kind, so the LDS-bound
   // and the FMA-bound half of a stage overlap.
   if (d < 4) {
+    constexpr unsigned FR = FRESH_LO;
     for (int j = 0; j < NJ - 1; ++j) {
       fft_pass<true, 0>(work, twl); S2CNN_FENCE();
       S2CNN_CON(0, j + 1) S2CNN_CON(1, j + 1)
@@ -907,6 +900,7 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
       __syncthreads();
     }
   } else {
+    constexpr unsigned FR = FRESH_HI;
     for (int j = 0; j < NJ - 1; ++j) {
       S2CNN_CON(0, j + 1) S2CNN_CON(1, j + 1)
       fft_pass<true, 0>(work, twl);
@@ -944,14 +938,14 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
 }
 
 // item rounds that carry degrees below nl (the template argument NA of the kernels below)
-inline int active_rounds(int nl) { return nl <= 24 ? 3 : nl <= 28 ? 5 : NIT; }
+inline int active_rounds(int nl) { return nl <= 24 ? 3 : nl <= 28 ? 6 : NIT; }
 
 // Launchers: the instantiation whose item rounds cover the nl degrees present.
 template <int MASK>
 inline void launch_analysis_m(int nl, hipStream_t st, const s2cnn::Input& in, const float* Tf, float4* rec, long nbatch) {
   const dim3 grid(grid_size(nbatch)), block(THREADS);
   if (nl <= 24) hipLaunchKernelGGL((analysis_kernel<3, MASK>), grid, block, 0, st, in.x, in.w, Tf, rec, nbatch, in.params, in.nfeature);
-  else if (nl <= 28) hipLaunchKernelGGL((analysis_kernel<5, MASK>), grid, block, 0, st, in.x, in.w, Tf, rec, nbatch, in.params, in.nfeature);
+  else if (nl <= 28) hipLaunchKernelGGL((analysis_kernel<6, MASK>), grid, block, 0, st, in.x, in.w, Tf, rec, nbatch, in.params, in.nfeature);
   else hipLaunchKernelGGL((analysis_kernel<7, MASK>), grid, block, 0, st, in.x, in.w, Tf, rec, nbatch, in.params, in.nfeature);
 }
 
@@ -977,19 +971,19 @@ inline void launch_synthesis(int nl, hipStream_t st, const float4* rec, const fl
                              const float* params = nullptr) {
   const dim3 grid(grid_size(nbatch)), block(THREADS);
   if (moments && yref) {
-    if (nl <= 24) hipLaunchKernelGGL((synthesis_kernel<3, 6, 0, 2>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, yref, params);
-    else hipLaunchKernelGGL((synthesis_kernel<5, 7, 0, 2>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, yref, params);
+    if (nl <= 24) hipLaunchKernelGGL((synthesis_kernel<3, 0, 2>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, yref, params);
+    else hipLaunchKernelGGL((synthesis_kernel<6, 0, 2>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, yref, params);
     return;
   }
   if (moments) {
-    if (nl <= 24) hipLaunchKernelGGL((synthesis_kernel<3, 6, 0, 1>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, nullptr, nullptr);
-    else if (nl <= 28) hipLaunchKernelGGL((synthesis_kernel<5, 7, 0, 1>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, nullptr, nullptr);
-    else hipLaunchKernelGGL((synthesis_kernel<7, 8, 0, 1>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, nullptr, nullptr);
+    if (nl <= 24) hipLaunchKernelGGL((synthesis_kernel<3, 0, 1>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, nullptr, nullptr);
+    else if (nl <= 28) hipLaunchKernelGGL((synthesis_kernel<6, 0, 1>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, nullptr, nullptr);
+    else hipLaunchKernelGGL((synthesis_kernel<7, 0, 1>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, nullptr, nullptr);
     return;
   }
-  if (nl <= 24) hipLaunchKernelGGL((synthesis_kernel<3, 6>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, nullptr, nullptr, nullptr);
-  else if (nl <= 28) hipLaunchKernelGGL((synthesis_kernel<5, 7>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, nullptr, nullptr, nullptr);
-  else hipLaunchKernelGGL((synthesis_kernel<7, 8>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, nullptr, nullptr, nullptr);
+  if (nl <= 24) hipLaunchKernelGGL((synthesis_kernel<3>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, nullptr, nullptr, nullptr);
+  else if (nl <= 28) hipLaunchKernelGGL((synthesis_kernel<6>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, nullptr, nullptr, nullptr);
+  else hipLaunchKernelGGL((synthesis_kernel<7>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, nullptr, nullptr, nullptr);
 }
 
 }  // namespace fused64
