@@ -74,7 +74,13 @@ template <> struct VecT<4> { typedef float4 type; };
 // init, the stage advances by a wave-uniform step (scalar arithmetic), rows outside the matrix are clamped
 // to a valid row (their products land in accumulators that are never stored) and only a ragged LAST stage
 // (TK a multiple of KI, odd number of blocks) is masked: the loop body is loads and LDS writes, nothing else.
-template <bool KC, bool MNMAJ, int EXT, int VEC, bool FAST>
+//
+// FAST = 2: KI >= TK but not a multiple of it (100 features), KI a multiple of VEC.  A stage then starts anywhere inside
+// a block and may run over ONE block boundary.  Where the stage starts is still uniform (scalar offset, scalar
+// bookkeeping); a thread only has to know whether ITS contraction steps lie behind the boundary, which is one compare
+// with a uniform value and the (uniform) distance between the end of a block and the start of the next added to its
+// offset: the same loop body as FAST = 1 plus a compare, a select and an add per slot.
+template <bool KC, bool MNMAJ, int EXT, int VEC, int FAST>
 struct TileLoader {
   static constexpr int NSLOT = EXT * TK / (NT * VEC);
   static constexpr int LD = TileShape<KC, EXT>::LD;
@@ -97,6 +103,10 @@ struct TileLoader {
   int sub, nsub, step_in, step_cross;
   int stage_i, last_ragged;     // last_ragged: index of the one masked stage, or -1
   unsigned tail_ok;             // bit q: slot q lies inside the matrix in that stage
+  // FAST = 2 only
+  int kin_s;                    // uniform: position inside its block at which the current stage starts
+  int kk0;                      // this thread's first contraction step inside a stage
+  unsigned cross_bytes;         // uniform: what a step behind the block boundary adds to the offset
 
   typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
   static __device__ __forceinline__ vec_t buffer_load(__amdgpu_buffer_rsrc_t r, unsigned voff, unsigned so) {
@@ -123,7 +133,8 @@ struct TileLoader {
       const int K = L * KI, nstage = (K + TK - 1) / TK, ktail = K - (nstage - 1) * TK;
       rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base_l), 0, 4 * L * L * MNI * KI, 0x00020000);
       soff = 0; sub = 0; stage_i = 0;
-      if (KI >= TK) { nsub = KI / TK; step_in = TK * unit; step_cross = blk_k_stride - (KI - TK) * unit; }
+      if (FAST == 2) { nsub = 1; step_in = TK * unit; step_cross = 0; kin_s = 0; cross_bytes = 4u * (unsigned)(blk_k_stride - KI * unit); }
+      else if (KI >= TK) { nsub = KI / TK; step_in = TK * unit; step_cross = blk_k_stride - (KI - TK) * unit; }
       else { nsub = 1; step_in = 0; step_cross = (TK / KI) * blk_k_stride; }
       last_ragged = ktail < TK ? nstage - 1 : -1;
       tail_ok = 0;
@@ -133,6 +144,7 @@ struct TileLoader {
         const int kk = (t % TPR) * VEC, r0 = t / TPR;
         const int kbl = KI >= TK ? 0 : kk / KI, kin = kk - kbl * KI;
         lds_off = r0 * LD + kk;
+        kk0 = kk;
 #pragma unroll
         for (int q = 0; q < NSLOT; ++q) {
           int row = tile0 + r0 + q * (NT / TPR);
@@ -147,6 +159,7 @@ struct TileLoader {
         mn = mn > last ? 0 : mn;
         const int kk = t / TPR;
         lds_off = kk * LD + (t % TPR) * VEC;
+        kk0 = kk;
         const int mb = mn / MNI, mi = mn - mb * MNI;
 #pragma unroll
         for (int q = 0; q < NSLOT; ++q) {
@@ -187,6 +200,28 @@ struct TileLoader {
 
   // clamped address + select instead of a predicated load: all loads of a stage are in flight together
   __device__ __forceinline__ void load() {
+    if (FAST == 2) {
+      const int room = KI - kin_s;                     // contraction steps of this stage that still lie in the current block
+      if (stage_i == last_ragged) {
+#pragma unroll
+        for (int q = 0; q < NSLOT; ++q) {
+          const int k = KC ? kk0 : kk0 + q * KSTEP;
+          const vec_t v = buffer_load(rsrc, foff[q] + (k >= room ? cross_bytes : 0u), soff);
+          reg[q] = ((tail_ok >> q) & 1u) ? v : vec_t{};
+        }
+      } else {
+#pragma unroll
+        for (int q = 0; q < NSLOT; ++q) {
+          const int k = KC ? kk0 : kk0 + q * KSTEP;    // KC: a thread's VEC steps never straddle a block (KI is a multiple of VEC)
+          reg[q] = buffer_load(rsrc, foff[q] + (k >= room ? cross_bytes : 0u), soff);
+        }
+      }
+      ++stage_i;
+      kin_s += TK;
+      soff += 4u * (unsigned)step_in;
+      if (kin_s >= KI) { kin_s -= KI; soff += cross_bytes; }
+      return;
+    }
     if (FAST) {
       if (stage_i == last_ragged) {
 #pragma unroll
@@ -321,7 +356,7 @@ __host__ __device__ inline void tile_counts(int L, int RI, int CI, int TN, int& 
   slots = tm * tn;
 }
 
-template <int MODE, int VA, int VB, bool FAST, int NCB>
+template <int MODE, int VA, int VB, int FAST, int NCB>
 __global__ __launch_bounds__(NT) void so3_block_mm_real_kernel(MmParams p) {
   typedef Cfg<MODE> C_;
   constexpr int TN = 64 * NCB;
@@ -446,20 +481,23 @@ int run(const float* a, const float* b, float* c, int nl, int RI, int CI, int KI
   const bool b2 = b4 || (bfast % 2 == 0 && s2cnn::aligned8(b));
   hipStream_t st = static_cast<hipStream_t>(stream);
   // the fast loaders address a degree with 32-bit byte offsets
-  const bool fast = a4 && b4 && (KI % TK == 0 || TK % KI == 0) && Lmax * Lmax * RI * KI < (1L << 30) && Lmax * Lmax * CI * KI < (1L << 30);
+  const bool small = Lmax * Lmax * RI * KI < (1L << 30) && Lmax * Lmax * CI * KI < (1L << 30);
+  const bool fast = a4 && b4 && (KI % TK == 0 || TK % KI == 0) && small;
+  const bool fast2 = a4 && b4 && !fast && KI > TK && KI % 4 == 0 && small;     // 100 features: stages that run over a block boundary
 #define S2CNN_LAUNCH(VA, VB, FAST)                                                                                    \
   do {                                                                                                                \
     if (narrow) hipLaunchKernelGGL((so3_block_mm_real_kernel<MODE, VA, VB, FAST, 1>), dim3(grid), dim3(NT), 0, st, p); \
     else hipLaunchKernelGGL((so3_block_mm_real_kernel<MODE, VA, VB, FAST, 2>), dim3(grid), dim3(NT), 0, st, p);        \
   } while (0)
-  if (fast) S2CNN_LAUNCH(4, 4, true);
-  else if (a4 && b4) S2CNN_LAUNCH(4, 4, false);
-  else if (a4 && b2) S2CNN_LAUNCH(4, 2, false);
-  else if (a2 && b4) S2CNN_LAUNCH(2, 4, false);
-  else if (a2 && b2) S2CNN_LAUNCH(2, 2, false);      // even feature counts (50, 70, 350 in the reference's shape network)
-  else if (a4) S2CNN_LAUNCH(4, 1, false);
-  else if (b4) S2CNN_LAUNCH(1, 4, false);
-  else S2CNN_LAUNCH(1, 1, false);
+  if (fast) S2CNN_LAUNCH(4, 4, 1);
+  else if (fast2) S2CNN_LAUNCH(4, 4, 2);
+  else if (a4 && b4) S2CNN_LAUNCH(4, 4, 0);
+  else if (a4 && b2) S2CNN_LAUNCH(4, 2, 0);
+  else if (a2 && b4) S2CNN_LAUNCH(2, 4, 0);
+  else if (a2 && b2) S2CNN_LAUNCH(2, 2, 0);      // even feature counts (50, 70, 350 in the reference's shape network)
+  else if (a4) S2CNN_LAUNCH(4, 1, 0);
+  else if (b4) S2CNN_LAUNCH(1, 4, 0);
+  else S2CNN_LAUNCH(1, 1, 0);
 #undef S2CNN_LAUNCH
   return s2cnn::launch_status();
 }
