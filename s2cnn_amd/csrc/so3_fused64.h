@@ -189,11 +189,19 @@ inline size_t scratch_bytes(long nbatch) { return (size_t)nbatch * REC_BYTES; }
 // Z[+a,n], Z[-a,-n], Z[-a,n], Z[+a,-n], side by side at quad[a][n][0..3].  Meanwhile pair j is
 // contracted out of the other quad buffer, two items per stage.
 // ---------------------------------------------------------------------------------------------
-constexpr int QPITCH = 32 * 4 + 14;             // complex numbers per a-row of the quad layout: 33 quads (the unused n = 32 included) + room for the skew
-constexpr int QUAD_ELEMS = 33 * QPITCH;         // row 32 takes the unused m = 32
+// NR: frequencies 0 <= a, n < NR are kept.  32 in general; a spectrum truncated below degree 24 (NA = 3 item rounds) needs
+// 24 only, which lets the two quad buffers and the plane of such a kernel fit the LDS of a CU twice: two workgroups (two
+// volumes in different phases of their steps) per CU.
+constexpr int rows_kept(int NA) { return NA <= 3 ? 24 : 32; }
+// waves per SIMD the kernels are compiled for: 4 (two workgroups per CU) where the registers of the truncated kernel allow
+// it without spilling more than a few values: `lean` = the variant loads no second tensor / forms no sums
+constexpr int waves_per_simd(int NA, bool lean) { return NA <= 3 && lean ? 4 : 2; }
+// complex numbers per a-row of the quad layout: NR quads + one more (the unused n = NR) + room for the skew
+constexpr int quad_pitch(int NR) { return NR * 4 + 14; }
+constexpr int quad_elems(int NR) { return (NR + 1) * quad_pitch(NR); }     // row NR takes what is not kept (the dump row)
 // Row a starts 2 (a / 8) complex numbers late.  The last gamma stage writes the rows 8r + s (r = lane % 8) at once; a pitch
 // that keeps rows 16-byte aligned puts rows 8 apart into the same banks, the skew moves them 4 banks apart instead.
-__host__ __device__ constexpr int quad_row(int a) { return a * QPITCH + 2 * (a >> 3); }
+template <int NR> __host__ __device__ constexpr int quad_row(int a) { return a * quad_pitch(NR) + 2 * (a >> 3); }
 // table registers: four slots, item it in slot it % 4; a slot is refilled right after its item has been used:
 //   after item 0, 1, 2: items 4, 5, 6 of the same plane pair;  after 3, 4, 5, 6: items 3, 0, 1, 2 of the next pair
 __device__ constexpr int table_slot(int it) { return it & 3; }
@@ -211,12 +219,13 @@ __host__ __device__ inline size_t bits_index(long z, int beta, int d) { return (
 // operand (table loads, LDS reads of the quads and everything else kept); 2: the table loads gone as well.  What is left
 // is the plane pipeline: loads, the 2-D transform through LDS with its barriers, the quad layout, the record.
 template <int NA, int MASK, int PROBE = 0>
-__global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restrict__ x, const float* __restrict__ mask,
+__global__ __launch_bounds__(THREADS, waves_per_simd(NA, MASK == 0 || MASK == 2 || MASK == 3)) void analysis_kernel(const float* __restrict__ x, const float* __restrict__ mask,
                                                            const float* __restrict__ Tf, float4* __restrict__ rec, long nbatch,
                                                            const float* __restrict__ params, int nfeature) {
   constexpr bool MASKED = MASK == 1 || MASK == 4;      // a second tensor is loaded beside x
   using namespace fft64;
   __shared__ __attribute__((aligned(16))) float2 work[LDS_ELEMS];
+  constexpr int NR = rows_kept(NA), QUAD_ELEMS = quad_elems(NR);
   __shared__ __attribute__((aligned(16))) float2 quad[2][QUAD_ELEMS];
   const long z = volume_of_block(nbatch);
   if (z < 0) return;
@@ -239,7 +248,7 @@ __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restri
   for (int it = 0; it < NIT; ++it) {
     int c, a, n;
     decode_item(it * THREADS + t, c, a, n);
-    adr[it] = (unsigned)(quad_row(a) + 4 * n) | ((unsigned)(n & 1) << 31);
+    adr[it] = it < NA ? (unsigned)(quad_row<NR>(a) + 4 * n) | ((unsigned)(n & 1) << 31) : 0u;   // active rounds hold a, n < NR
   }
 
   // where this thread's outputs of the last gamma stage go: row slot lo holds m = sigma(lo)
@@ -247,10 +256,15 @@ __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restri
   // quad[a][n] = { Z[+a,n], Z[-a,-n], Z[-a,n], Z[+a,-n] }; +0 and -0 are the same frequency, so
   //   m = 0 counts as -0 when n < 0 (the item (0, n) then finds Z[0,n], Z[0,-n] in its first two places) and
   //   n = 0 is written to the place of -0 as well (the one extra store below, by the wave d = 0).
-  const int qa = quad_row(m <= 32 ? m : 64 - m);      // m = 32: the dump row
+  const int am = m <= 32 ? m : 64 - m;
+  // Rows that are not kept (am >= NR; m = 32 always) go to the dump row, every lane to places of its own there whatever
+  // the column is (nmul = 0): no branch, and no two lanes at the same address.
+  const bool keep = am < NR;
+  const int qa = keep ? quad_row<NR>(am) : quad_row<NR>(NR) + 4 * (am - NR);
+  const int nmul = keep ? 4 : 0;
   const int pos_lo = m > 32 ? 2 : 0;                  // place of an output with n >= 0
   const int pos_hi = (m > 32 || m == 0) ? 1 : 3;      // place of an output with n < 0
-  const int extra = d == 0 ? qa + pos_hi : 32 * QPITCH + 130;   // n = 0 again as -0; other waves: the dump row
+  const int extra = d == 0 ? qa + pos_hi : quad_row<NR>(NR) + 4 * NR + 2;   // n = 0 again as -0; other waves: the pad of the dump row
 
   float2 accp[NIT][4], accm[NIT][4];
 #pragma unroll
@@ -326,10 +340,15 @@ __global__ __launch_bounds__(THREADS) void analysis_kernel(const float* __restri
 #pragma unroll
     for (int j2 = 0; j2 < 8; ++j2) v[j2] = line[j2];
     fft8<false>(v);
+    // outputs n = d + 8 k2 >= 0 and n' = 64 - d - 8 k2 > 0 (the bins -n'); those that are not kept are not written (d is
+    // uniform over the wave); n' = NR lands in the pad of the row
+    // (which outputs are kept is known at compile time: d + 8 k2 < NR for every d < 8, or for none)
 #pragma unroll
-    for (int k2 = 0; k2 < 4; ++k2) q[qa + 4 * (d + 8 * k2) + pos_lo] = v[k2];
+    for (int k2 = 0; k2 < 4; ++k2)
+      if (8 * k2 + 7 < NR) q[qa + nmul * (d + 8 * k2) + pos_lo] = v[k2];
 #pragma unroll
-    for (int k2 = 4; k2 < 8; ++k2) q[qa + 4 * (64 - d - 8 * k2) + pos_hi] = v[k2];   // n = 32 (d = 0, k2 = 4) lands in the pad of the row
+    for (int k2 = 4; k2 < 8; ++k2)
+      if (64 - 8 * k2 <= NR) q[qa + nmul * (64 - d - 8 * k2) + pos_hi] = v[k2];
     q[extra] = v[0];
   };
   // fresh: the rounds in which some thread of this half of the workgroup starts another column (FRESH_LO, FRESH_HI of the
@@ -713,15 +732,16 @@ __global__ __launch_bounds__(256) void spectrum_gather_real(const float* __restr
 //      f = z % nfeature: the two reductions of the gradient of such a normalisation followed by max(., 0), with the
 //      output as the incoming gradient (s2cnn::bn_relu_grad).
 template <int NA, int PROBE = 0, int MOM = 0>
-__global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __restrict__ rec, const float* __restrict__ Tf,
+__global__ __launch_bounds__(THREADS, waves_per_simd(NA, MOM == 0)) void synthesis_kernel(const float4* __restrict__ rec, const float* __restrict__ Tf,
                                                             float* __restrict__ y, long nbatch, const float* __restrict__ bias, int nfeature,
                                                             int relu, unsigned long long* __restrict__ bits, float2* __restrict__ moments,
                                                             const float* __restrict__ yref, const float* __restrict__ params) {
   using namespace fft64;
   __shared__ __attribute__((aligned(16))) float2 work[LDS_ELEMS];
   float ms1 = 0.f, ms2 = 0.f;
-  constexpr int NCOL = 32 * 32;                                               // columns (a, n), a, n < 32
-  __shared__ __attribute__((aligned(16))) float4 stg_p[2 * NCOL];             // [run of the column][32 a + n]: the run's share of the bins [+a,n], [-a,-n]
+  constexpr int NR = rows_kept(NA);                                           // frequencies a, n < NR carry degrees of the input (see analysis_kernel)
+  constexpr int NCOL = NR * NR;                                               // columns (a, n)
+  __shared__ __attribute__((aligned(16))) float4 stg_p[2 * NCOL];             // [run of the column][NR a + n]: the run's share of the bins [+a,n], [-a,-n]
   __shared__ __attribute__((aligned(16))) float4 stg_m[2 * NCOL];             //                                                            [-a,n], [+a,-n]
   const long z = volume_of_block(nbatch);
   if (z < 0) return;
@@ -792,7 +812,8 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
     if (it == NA - 1 || (e >> 15)) {
       const unsigned sb = (e & 1u) << 31;
       const float qpx = flip(Qp.x, sb), qpy = flip(Qp.y, sb), qmx = flip(Qm.x, sb), qmy = flip(Qm.y, sb);
-      const unsigned pos = ((e >> 4) & 0x400u) | (e & 0x3ffu);
+      const unsigned col32 = e & 0x3ffu;                                        // 32 a + n
+      const unsigned pos = ((e >> 14) & 1u) * NCOL + col32 - (32 - NR) * (col32 >> 5);
       stg_p[pos] = make_float4(Sp.x - qpy, Sp.y + qpx, Sp.x + qpy, qpx - Sp.y);
       stg_m[pos] = make_float4(Sm.x - qmy, Sm.y + qmx, Sm.x + qmy, qmx - Sm.y);
       Sp = make_float2(0.f, 0.f); Qp = Sp; Sm = Sp; Qm = Sp;
@@ -803,7 +824,8 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const int col = t + h * THREADS;
-      const int a = col >> 5, n = col & 31;
+      if (NCOL < 2 * THREADS && col >= NCOL) break;
+      const int a = col / NR, n = col - a * NR;
       const float4 u0 = stg_p[col], v0 = stg_p[NCOL + col], u1 = stg_m[col], v1 = stg_m[NCOL + col];
       const float4 s0 = make_float4(u0.x + v0.x, u0.y + v0.y, u0.z + v0.z, u0.w + v0.w);
       const float4 s1 = make_float4(u1.x + v1.x, u1.y + v1.y, u1.z + v1.z, u1.w + v1.w);
@@ -815,7 +837,17 @@ __global__ __launch_bounds__(THREADS) void synthesis_kernel(const float4* __rest
         if (n > 0) work[rp + 64 - n] = make_float2(s1.z, s1.w);
       }
     }
-    if (t < 64) { work[32 * PITCH + t] = make_float2(0.f, 0.f); work[t * PITCH + 32] = make_float2(0.f, 0.f); }
+    // the bins that no column fills hold what the last transform left there: cleared again
+    if constexpr (NR == 32) {
+      if (t < 64) { work[32 * PITCH + t] = make_float2(0.f, 0.f); work[t * PITCH + 32] = make_float2(0.f, 0.f); }
+    } else {
+      constexpr int GAP = 64 - 2 * NR + 1;                  // frequencies NR .. 64 - NR on either axis
+      for (int i = t; i < GAP * 64; i += THREADS) work[(NR + (i >> 6)) * PITCH + (i & 63)] = make_float2(0.f, 0.f);
+      for (int i = t; i < (64 - GAP) * GAP; i += THREADS) {
+        const int rr = i / GAP, c = NR + (i - rr * GAP);
+        work[(rr < NR ? rr : rr + GAP) * PITCH + c] = make_float2(0.f, 0.f);
+      }
+    }
   };
   // second alpha stage: lane lo takes the column slot sigma(lo), i.e. column gamma = lo; inputs at row slots
   // 8 d + j, outputs rows alpha = d + 8 k.  Real part -> plane j, imaginary part -> plane 63-j, one whole 256-byte row
