@@ -347,6 +347,52 @@ def measure_config1(torch, dev, reps=50):
             "replay_equals_eager": same}
 
 
+def measure_overlap(torch, dev, reps=6):
+    """Can the transforms (bound by vector instructions and latency) and the products (bound by the matrix cores) of the
+    headline layer share the chip?  Half of the layer's batch each: the analysis of 512 volumes of 64^3 and the real-basis
+    product at batch 8 (64 -> 64 features, 32 degrees), first one after the other on one stream, then at the same time on two
+    streams of equal priority.  A compute unit cannot hold a workgroup of both kernels at once (registers and LDS, see
+    profiles/), so the two can only divide the CUs between them."""
+    import s2cnn_amd
+    from s2cnn_amd.soft import so3_fft as PSO3
+    nl, B, F = 32, 8, 64
+    x = torch.randn(B * F, 64, 64, 64, device=dev)
+    xs = torch.randn(nspec(nl), B, F, device=dev)
+    ys = torch.randn(nspec(nl), F, F, device=dev) * 0.125
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+
+    def both(parallel):
+        a, b = (s1, s2) if parallel else (s1, s1)
+        with torch.cuda.stream(a):
+            PSO3.so3_rfft_real_basis(x)
+        with torch.cuda.stream(b):
+            s2cnn_amd.so3_mm_real(xs, ys)
+
+    def timed(fn):
+        for _ in range(2):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / reps * 1e3
+
+    def only_fft():
+        with torch.cuda.stream(s1):
+            PSO3.so3_rfft_real_basis(x)
+
+    def only_mm():
+        with torch.cuda.stream(s1):
+            s2cnn_amd.so3_mm_real(xs, ys)
+
+    out = {"workload": "analysis of 512 volumes of 64^3 and so3_mm_real forward at batch 8 (64->64, 32 degrees): half of the headline layer's batch each",
+           "analysis_alone_ms": round(timed(only_fft), 4), "product_alone_ms": round(timed(only_mm), 4),
+           "one_stream_ms": round(timed(lambda: both(False)), 4), "two_streams_ms": round(timed(lambda: both(True)), 4)}
+    out["gain_of_two_streams"] = round(1.0 - out["two_streams_ms"] / out["one_stream_ms"], 4)
+    return out
+
+
 def measure_fft_floor(torch, dev, nvol=256, reps=10):
     """What the plane pipeline of the per-volume 64^3 kernels costs without the Wigner contraction: the shipped kernels
     with parts compiled out (s2cnn_so3_fft64_probe of the measurement library libs2cnn_probe.so, built by
@@ -462,6 +508,8 @@ def main():
     ap.add_argument("--rows", action="store_true", help="also time every other op of the path (adds a `rows` object)")
     ap.add_argument("--floor", action="store_true",
                     help="also time the per-volume 64^3 kernels with their Wigner contraction compiled out (adds a `fft_floor` object)")
+    ap.add_argument("--overlap", action="store_true",
+                    help="also time a transform and a product of half the layer's batch on one stream and on two (adds an `overlap` object)")
     ap.add_argument("--network", nargs="?", const="config5", default=None, choices=["config5", "mnist", "shrec17", "shrec17_original"],
                     help="also time a whole network, forward + backward (adds a `network` object): config5 = the SHREC17-shaped "
                          "network of benchmark config 5 (default); mnist, shrec17, shrec17_original = the reference's example "
@@ -595,6 +643,8 @@ def main():
         result["rows"] = measure_rows(torch, dev, not args.no_cpu)
     if args.floor:
         result["fft_floor"] = measure_fft_floor(torch, dev)
+    if args.overlap:
+        result["overlap"] = measure_overlap(torch, dev)
     if args.network == "config5":
         result["network"] = measure_network(torch, dev, args.steps, args.warmup)
     elif args.network:

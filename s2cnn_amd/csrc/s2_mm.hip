@@ -59,94 +59,144 @@ __global__ __launch_bounds__(256) void s2_mm_fwd_kernel(const float2* __restrict
   }
 }
 
-// ---- grad x: grid.x = nl^2 (l,m), grid.y = batch item i, grid.z = feature pass.  Lanes run along j, every wave takes
-// the n = wave, wave + nwaves, ...; each lane accumulates KC features, then lanes and waves are reduced.
+// CV complex numbers per lane along j: 2 (16-byte accesses) when F_out is even and the rows start on 16-byte boundaries
+template <int CV> struct CPack;
+template <> struct CPack<1> {
+  typedef float2 type;
+  static __device__ __forceinline__ float2 zero() { return make_float2(0.f, 0.f); }
+  // acc += sum over the lane's entries of a * b (complex)
+  static __device__ __forceinline__ void dot(float2 a, float2 b, float2& acc) {
+    acc.x = fmaf(a.x, b.x, fmaf(-a.y, b.y, acc.x));
+    acc.y = fmaf(a.x, b.y, fmaf(a.y, b.x, acc.y));
+  }
+  // acc[entry] += conj(a[entry]) * s for a complex scalar s
+  static __device__ __forceinline__ void conj_axpy(float2 a, float2 s, float2& acc) {
+    acc.x = fmaf(a.x, s.x, fmaf(a.y, s.y, acc.x));
+    acc.y = fmaf(a.x, s.y, fmaf(-a.y, s.x, acc.y));
+  }
+};
+template <> struct CPack<2> {
+  typedef float4 type;
+  static __device__ __forceinline__ float4 zero() { return make_float4(0.f, 0.f, 0.f, 0.f); }
+  static __device__ __forceinline__ void dot(float4 a, float4 b, float2& acc) {
+    acc.x = fmaf(a.x, b.x, fmaf(-a.y, b.y, fmaf(a.z, b.z, fmaf(-a.w, b.w, acc.x))));
+    acc.y = fmaf(a.x, b.y, fmaf(a.y, b.x, fmaf(a.z, b.w, fmaf(a.w, b.z, acc.y))));
+  }
+  static __device__ __forceinline__ void conj_axpy(float4 a, float2 s, float4& acc) {
+    acc.x = fmaf(a.x, s.x, fmaf(a.y, s.y, acc.x));
+    acc.y = fmaf(a.x, s.y, fmaf(-a.y, s.x, acc.y));
+    acc.z = fmaf(a.z, s.x, fmaf(a.w, s.y, acc.z));
+    acc.w = fmaf(a.z, s.y, fmaf(-a.w, s.x, acc.w));
+  }
+};
+
+constexpr int IB = 4;   // grad x: batch items per workgroup
+
+// ---- grad x.  grid.x = nl^2 (l, m), grid.y = group of IB batch items, grid.z = feature pass.  The (n, j group) pairs of
+// the row block gz[l,m,:,i,:] are spread over the threads (consecutive threads read consecutive 8 CV bytes of a row); a
+// thread accumulates IB x KC partial sums (one piece of y serves the IB items), then lanes and waves are reduced.
+template <int CV>
 __global__ __launch_bounds__(256) void s2_mm_gradx_kernel(const float2* __restrict__ gz, const float2* __restrict__ y,
                                                           float2* __restrict__ gx, int nl, int nbatch, int fi, int fo) {
-  __shared__ float2 part[4][KC];
-  const int lm = blockIdx.x, i = blockIdx.y, k0 = blockIdx.z * KC;
+  typedef typename CPack<CV>::type vec_t;
+  __shared__ float2 part[4][IB][KC];
+  const int lm = blockIdx.x, i0 = blockIdx.y * IB, k0 = blockIdx.z * KC;
   const int l = isqrt_floor(lm), m = lm - l * l - l;
   const int L = 2 * l + 1;
   const size_t base = (size_t)l * (4 * l * l - 1) / 3 + (size_t)(l + m) * L;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  float2 acc[KC];
+  const int fov = fo / CV;
+  float2 acc[IB][KC];
 #pragma unroll
-  for (int u = 0; u < KC; ++u) acc[u] = make_float2(0.f, 0.f);
-  for (int nn = wave; nn < L; nn += 4) {
-    const float2* g = gz + ((base + nn) * nbatch + i) * fo;
-    const float2* yy = y + (size_t)(l * l + nn) * fi * fo;
-    for (int j = lane; j < fo; j += 64) {
-      const float2 a = g[j];
+  for (int q = 0; q < IB; ++q)
 #pragma unroll
-      for (int u = 0; u < KC; ++u) {
-        if (k0 + u < fi) {
-          const float2 b = yy[(size_t)(k0 + u) * fo + j];
-          acc[u].x += a.x * b.x - a.y * b.y;
-          acc[u].y += a.x * b.y + a.y * b.x;
-        }
+    for (int u = 0; u < KC; ++u) acc[q][u] = make_float2(0.f, 0.f);
+  int nn = threadIdx.x / fov, jv = threadIdx.x - nn * fov;          // walks (n, jv) with stride 256
+  const int dn = 256 / fov, dj = 256 - dn * fov;
+  for (; nn < L; ) {
+    const vec_t* g = reinterpret_cast<const vec_t*>(gz + ((base + nn) * nbatch + i0) * fo) + jv;
+    vec_t a[IB];
+#pragma unroll
+    for (int q = 0; q < IB; ++q) a[q] = i0 + q < nbatch ? g[(size_t)q * fov] : CPack<CV>::zero();
+    const vec_t* yy = reinterpret_cast<const vec_t*>(y + ((size_t)(l * l + nn) * fi + k0) * fo) + jv;
+#pragma unroll
+    for (int u = 0; u < KC; ++u) {
+      if (k0 + u < fi) {
+        const vec_t b = yy[(size_t)u * fov];
+#pragma unroll
+        for (int q = 0; q < IB; ++q) CPack<CV>::dot(a[q], b, acc[q][u]);
       }
     }
+    nn += dn; jv += dj;
+    if (jv >= fov) { jv -= fov; ++nn; }
   }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
-  for (int u = 0; u < KC; ++u) {
+  for (int q = 0; q < IB; ++q)
 #pragma unroll
-    for (int s = 32; s > 0; s >>= 1) {
-      acc[u].x += __shfl_down(acc[u].x, s, 64);
-      acc[u].y += __shfl_down(acc[u].y, s, 64);
+    for (int u = 0; u < KC; ++u) {
+      float2 v = acc[q][u];
+#pragma unroll
+      for (int sh = 32; sh > 0; sh >>= 1) { v.x += __shfl_down(v.x, sh, 64); v.y += __shfl_down(v.y, sh, 64); }
+      if (lane == 0) part[wave][q][u] = v;
     }
-    if (lane == 0) part[wave][u] = acc[u];
-  }
   __syncthreads();
-  if (threadIdx.x < KC && k0 + (int)threadIdx.x < fi) {
-    const int u = threadIdx.x;
-    const float2 a = part[0][u], b = part[1][u], c = part[2][u], d = part[3][u];
-    gx[((size_t)lm * nbatch + i) * fi + k0 + u] = make_float2(a.x + b.x + c.x + d.x, a.y + b.y + c.y + d.y);
+  if (threadIdx.x < IB * KC) {
+    const int q = threadIdx.x / KC, u = threadIdx.x - q * KC;
+    if (i0 + q < nbatch && k0 + u < fi) {
+      const float2 a = part[0][q][u], b = part[1][q][u], c = part[2][q][u], d = part[3][q][u];
+      gx[((size_t)lm * nbatch + i0 + q) * fi + k0 + u] = make_float2((a.x + b.x) + (c.x + d.x), (a.y + b.y) + (c.y + d.y));
+    }
   }
 }
 
-// ---- grad y: grid.x = nl^2 (l,n), grid.y = tiles of 64 output features j, grid.z = feature pass.  Lane = j; the four
-// waves split the (m, i) reduction; each lane accumulates KC input features (x is wave-uniform), then waves are reduced.
+// ---- grad y.  grid.x = nl^2 (l, n), grid.y = tile of JT j groups, grid.z = feature pass.  The threads form
+// SL = 256 / JT slices of JT lanes; slice q takes the (m, i) pairs q, q + SL, ...; a lane accumulates KC pieces (x is
+// uniform over a slice), then the slices are reduced through LDS in a fixed order.
+template <int CV, int JT>
 __global__ __launch_bounds__(256) void s2_mm_grady_kernel(const float2* __restrict__ gz, const float2* __restrict__ x,
                                                           float2* __restrict__ gy, int nl, int nbatch, int fi, int fo) {
-  __shared__ float2 part[4][KC][64];
+  typedef typename CPack<CV>::type vec_t;
+  constexpr int SL = 256 / JT;
+  __shared__ float2 part[SL][KC][JT * CV];
   const int ln = blockIdx.x, k0 = blockIdx.z * KC;
   const int l = isqrt_floor(ln), n = ln - l * l - l;
   const int L = 2 * l + 1;
   const size_t base = (size_t)l * (4 * l * l - 1) / 3 + (size_t)(l + n);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int j = blockIdx.y * 64 + lane;
-  float2 acc[KC];
+  const int fov = fo / CV;
+  const int slice = threadIdx.x / JT, jl = threadIdx.x - slice * JT;
+  const int jv = blockIdx.y * JT + jl;
+  vec_t acc[KC];
 #pragma unroll
-  for (int u = 0; u < KC; ++u) acc[u] = make_float2(0.f, 0.f);
-  const int total = L * nbatch;                       // (m, i) pairs
-  for (int r = wave; r < total; r += 4) {
-    const int mm = r / nbatch, i = r - mm * nbatch;
-    const float2 a = j < fo ? gz[((base + (size_t)mm * L) * nbatch + i) * fo + j] : make_float2(0.f, 0.f);
+  for (int u = 0; u < KC; ++u) acc[u] = CPack<CV>::zero();
+  const int total = L * nbatch;                                    // (m, i) pairs
+  int mm = slice / nbatch, i = slice - mm * nbatch;                // walks the pairs with stride SL
+  const int dm = SL / nbatch, di = SL - dm * nbatch;
+  for (int p = slice; p < total; p += SL) {
+    const vec_t a = jv < fov ? reinterpret_cast<const vec_t*>(gz + ((base + (size_t)mm * L) * nbatch + i) * fo)[jv] : CPack<CV>::zero();
     const float2* xx = x + ((size_t)(l * l + mm) * nbatch + i) * fi + k0;
 #pragma unroll
-    for (int u = 0; u < KC; ++u) {
-      if (k0 + u < fi) {
-        const float2 b = xx[u];
-        acc[u].x += a.x * b.x + a.y * b.y;            // conj(a) * b
-        acc[u].y += a.x * b.y - a.y * b.x;
-      }
-    }
+    for (int u = 0; u < KC; ++u)
+      if (k0 + u < fi) CPack<CV>::conj_axpy(a, xx[u], acc[u]);
+    mm += dm; i += di;
+    if (i >= nbatch) { i -= nbatch; ++mm; }
   }
 #pragma unroll
-  for (int u = 0; u < KC; ++u) part[wave][u][lane] = acc[u];
+  for (int u = 0; u < KC; ++u) reinterpret_cast<vec_t*>(&part[slice][u][0])[jl] = acc[u];
   __syncthreads();
-  for (int o = threadIdx.x; o < KC * 64; o += 256) {
-    const int u = o >> 6, jj = o & 63;
-    const int jg = blockIdx.y * 64 + jj;
-    if (k0 + u < fi && jg < fo) {
-      const float2 a = part[0][u][jj], b = part[1][u][jj], c = part[2][u][jj], d = part[3][u][jj];
-      gy[((size_t)ln * fi + k0 + u) * fo + jg] = make_float2(a.x + b.x + c.x + d.x, a.y + b.y + c.y + d.y);
+  for (int o = threadIdx.x; o < KC * JT * CV; o += 256) {
+    const int u = o / (JT * CV), jj = o - u * (JT * CV);
+    const int j = blockIdx.y * JT * CV + jj;
+    if (k0 + u < fi && j < fo) {
+      float2 v = make_float2(0.f, 0.f);
+#pragma unroll
+      for (int q = 0; q < SL; ++q) { v.x += part[q][u][jj].x; v.y += part[q][u][jj].y; }
+      gy[((size_t)ln * fi + k0 + u) * fo + j] = v;
     }
   }
 }
 
 int check(const void* a, const void* b, const void* c, int nl, int nbatch, int fi, int fo) {
-  if (!a || !b || !c || nl < 1 || nl > 255 || nbatch < 1 || nbatch > 65535 || fi < 1 || fo < 1) return S2CNN_EINVAL;
+  if (!a || !b || !c || nl < 1 || nl > 255 || nbatch < 1 || nbatch > 65535 || fi < 1 || fo < 1) return S2CNN_EINVAL;   // grid.y of grad x: ceil(nbatch / IB)
   if ((long)nbatch * fo >= (1L << 31) || (long)nbatch * fi >= (1L << 31) || (long)fi * fo >= (1L << 31)) return S2CNN_EINVAL;
   if ((fi + KC - 1) / KC > 65535 || (fo + 63) / 64 > 65535 || ((long)nbatch * fo + 255) / 256 > 65535) return S2CNN_EINVAL;
   if (!s2cnn::aligned8(a) || !s2cnn::aligned8(b) || !s2cnn::aligned8(c)) return S2CNN_EALIGN;
@@ -168,17 +218,27 @@ extern "C" int s2cnn_s2_mm_fwd(const float* x, const float* y, float* z, int nl,
 extern "C" int s2cnn_s2_mm_gradx(const float* gz, const float* y, float* gx, int nl, int nbatch, int f_in, int f_out, void* stream) {
   s2cnn::clear_stale_error();
   if (int rc = check(gz, y, gx, nl, nbatch, f_in, f_out)) return rc;
-  hipLaunchKernelGGL(s2_mm_gradx_kernel, dim3(nl * nl, nbatch, (f_in + KC - 1) / KC), dim3(256), 0, static_cast<hipStream_t>(stream),
-                     reinterpret_cast<const float2*>(gz), reinterpret_cast<const float2*>(y), reinterpret_cast<float2*>(gx),
-                     nl, nbatch, f_in, f_out);
+  const dim3 grid(nl * nl, (nbatch + IB - 1) / IB, (f_in + KC - 1) / KC);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const float2 *g2 = reinterpret_cast<const float2*>(gz), *y2 = reinterpret_cast<const float2*>(y);
+  if (f_out % 2 == 0 && s2cnn::aligned16(gz) && s2cnn::aligned16(y))
+    hipLaunchKernelGGL(s2_mm_gradx_kernel<2>, grid, dim3(256), 0, st, g2, y2, reinterpret_cast<float2*>(gx), nl, nbatch, f_in, f_out);
+  else
+    hipLaunchKernelGGL(s2_mm_gradx_kernel<1>, grid, dim3(256), 0, st, g2, y2, reinterpret_cast<float2*>(gx), nl, nbatch, f_in, f_out);
   return s2cnn::launch_status();
 }
 
 extern "C" int s2cnn_s2_mm_grady(const float* gz, const float* x, float* gy, int nl, int nbatch, int f_in, int f_out, void* stream) {
   s2cnn::clear_stale_error();
   if (int rc = check(gz, x, gy, nl, nbatch, f_in, f_out)) return rc;
-  hipLaunchKernelGGL(s2_mm_grady_kernel, dim3(nl * nl, (f_out + 63) / 64, (f_in + KC - 1) / KC), dim3(256), 0,
-                     static_cast<hipStream_t>(stream), reinterpret_cast<const float2*>(gz), reinterpret_cast<const float2*>(x),
-                     reinterpret_cast<float2*>(gy), nl, nbatch, f_in, f_out);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const float2 *g2 = reinterpret_cast<const float2*>(gz), *x2 = reinterpret_cast<const float2*>(x);
+  if (f_out % 2 == 0 && s2cnn::aligned16(gz) && s2cnn::aligned16(gy)) {
+    const dim3 grid(nl * nl, (f_out / 2 + 15) / 16, (f_in + KC - 1) / KC);
+    hipLaunchKernelGGL((s2_mm_grady_kernel<2, 16>), grid, dim3(256), 0, st, g2, x2, reinterpret_cast<float2*>(gy), nl, nbatch, f_in, f_out);
+  } else {
+    const dim3 grid(nl * nl, (f_out + 31) / 32, (f_in + KC - 1) / KC);
+    hipLaunchKernelGGL((s2_mm_grady_kernel<1, 32>), grid, dim3(256), 0, st, g2, x2, reinterpret_cast<float2*>(gy), nl, nbatch, f_in, f_out);
+  }
   return s2cnn::launch_status();
 }

@@ -56,7 +56,8 @@ def test_so3_mm_forward_backward(hip, nl, B, Fi, Fo):
     close(gyg, gyo, "gy")
 
 
-@pytest.mark.parametrize("nl,B,Fi,Fo", [(4, 2, 3, 5), (10, 32, 1, 20), (7, 5, 6, 9), (6, 16, 12, 15)])
+@pytest.mark.parametrize("nl,B,Fi,Fo", [(4, 2, 3, 5), (10, 32, 1, 20), (7, 5, 6, 9), (6, 16, 12, 15),
+                                        (5, 3, 10, 6), (8, 7, 6, 100)])      # even F_out: 16-byte accesses in the gradients
 def test_s2_mm_forward_backward(hip, nl, B, Fi, Fo):
     print(f"s2_mm nl={nl} B={B} Fi={Fi} Fo={Fo}", flush=True)
     x = rnd((nl * nl, B, Fi, 2), 6)
