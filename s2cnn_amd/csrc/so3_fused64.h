@@ -726,8 +726,10 @@ __global__ __launch_bounds__(256) void spectrum_gather_real(const float* __restr
 // NA as in analysis_kernel
 // PROBE (measurement only, results meaningless): 1: an item's share of a plane pair reduced to one add per table operand.
 // MOM: the kernel also writes two sums over the volume it produces, formed in a fixed order, to moments[z]:
-//   1: (sum v, sum v^2) of the output v (bias included, before the activation): the statistics of a batch normalisation
-//      that follows, without a read of their own;
+//   1: (sum v, sum (v - mean of the volume)^2) of the output v (bias included, before the activation): the statistics of
+//      a batch normalisation that follows, without a read of their own.  Every thread sums its squares around a pivot (its
+//      first sample); the threads' sums are moved to their means and merged pairwise in float64, so a mean that is large
+//      against the spread costs the variance no digits;
 //   2: (sum v m, sum v m w) with w = yref at the same sample and m = (a w + b > 0), a = params[f], b = params[nfeature + f],
 //      f = z % nfeature: the two reductions of the gradient of such a normalisation followed by max(., 0), with the
 //      output as the incoming gradient (s2cnn::bn_relu_grad).
@@ -739,6 +741,7 @@ __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MOM == 0)) void synthes
   using namespace fft64;
   __shared__ __attribute__((aligned(16))) float2 work[LDS_ELEMS];
   float ms1 = 0.f, ms2 = 0.f;
+  [[maybe_unused]] float mpivot = 0.f;
   constexpr int NR = rows_kept(NA);                                           // frequencies a, n < NR carry degrees of the input (see analysis_kernel)
   constexpr int NCOL = NR * NR;                                               // columns (a, n)
   __shared__ __attribute__((aligned(16))) float4 stg_p[2 * NCOL];             // [run of the column][NR a + n]: the run's share of the bins [+a,n], [-a,-n]
@@ -868,7 +871,11 @@ __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MOM == 0)) void synthes
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
       float ra = v[k].x + bz, rb = v[k].y + bz;
-      if constexpr (MOM == 1) { ms1 += ra + rb; ms2 = fmaf(ra, ra, fmaf(rb, rb, ms2)); }
+      if constexpr (MOM == 1) {
+        if (j == 0 && k == 0) mpivot = ra;
+        const float da = ra - mpivot, db = rb - mpivot;
+        ms1 += da + db; ms2 = fmaf(da, da, fmaf(db, db, ms2));
+      }
       if constexpr (MOM == 2) {
         const float ga = s2cnn::relu_pass(ra, fmaf(mom_a, w[k].x, mom_b)), gb = s2cnn::relu_pass(rb, fmaf(mom_a, w[k].y, mom_b));
         ms1 += ga + gb; ms2 = fmaf(ga, w[k].x, fmaf(gb, w[k].y, ms2));
@@ -956,7 +963,26 @@ __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MOM == 0)) void synthes
   fft_pass<true, 1>(work, twl); __syncthreads();
   fft_pass<true, 2>(work, twl); __syncthreads();
   stage_c2_store(NJ - 1);
-  if constexpr (MOM != 0) {                         // the threads' partial sums through LDS, pairwise, always in the same order
+  if constexpr (MOM == 1) {                         // (mean, squared deviations) of every thread's 2 x 8 x 32 samples, merged pairwise in float64
+    __syncthreads();
+    double* red = reinterpret_cast<double*>(work);
+    constexpr double NT_SAMPLES = 2.0 * 8.0 * NJ;
+    red[t] = (double)mpivot + (double)ms1 / NT_SAMPLES;
+    red[THREADS + t] = (double)ms2 - (double)ms1 * (double)ms1 / NT_SAMPLES;
+    __syncthreads();
+    double cnt = NT_SAMPLES;                        // samples behind each entry at this level
+    for (int s = THREADS / 2; s > 0; s >>= 1) {
+      if (t < s) {
+        const double dm = red[t + s] - red[t];
+        red[THREADS + t] += red[THREADS + t + s] + dm * dm * (0.5 * cnt);
+        red[t] = 0.5 * (red[t] + red[t + s]);
+      }
+      cnt *= 2.0;
+      __syncthreads();
+    }
+    if (t == 0) moments[z] = make_float2((float)(red[0] * cnt), (float)red[THREADS]);
+  }
+  if constexpr (MOM == 2) {                         // the threads' partial sums through LDS, pairwise, always in the same order
     __syncthreads();
     float* red = reinterpret_cast<float*>(work);
     red[t] = ms1; red[THREADS + t] = ms2;

@@ -89,7 +89,9 @@ __global__ __launch_bounds__(256) void so3_integrate_grad_kernel(const float* __
 
 // Two sums per volume in one read, in a fixed order (bit-reproducible): what a batch normalisation over the volumes
 // of a feature needs of them.
-//   GRAD = false: out[z] = (sum x, sum x^2)
+//   GRAD = false: out[z] = (sum x, sum (x - mean_z)^2), mean_z the mean of the volume.  The squares are summed around a
+//                 pivot (the volume's first sample) and moved to the mean in float64, so a mean that is large against the
+//                 spread costs the variance no digits (E[x^2] - mean^2 in float32 would).
 //   GRAD = true : out[z] = (sum g m, sum g m y) with m = (a y + b > 0), a = params[z % F], b = params[F + z % F]
 template <bool GRAD>
 __global__ __launch_bounds__(256) void volume_moments_kernel(const float* __restrict__ x, const float* __restrict__ y,
@@ -101,12 +103,14 @@ __global__ __launch_bounds__(256) void volume_moments_kernel(const float* __rest
   const float* ys = GRAD ? y + z * n : nullptr;
   float a = 0.f, b = 0.f;
   if constexpr (GRAD) { a = params[z % nfeature]; b = params[nfeature + z % nfeature]; }
+  const float pivot = GRAD ? 0.f : xs[0];
   auto term = [&](float xv, float yv, float& s1, float& s2) {
     if constexpr (GRAD) {
       const float gm = s2cnn::relu_pass(xv, fmaf(a, yv, b));
       s1 += gm; s2 = fmaf(gm, yv, s2);
     } else {
-      s1 += xv; s2 = fmaf(xv, xv, s2);
+      const float dv = xv - pivot;
+      s1 += dv; s2 = fmaf(dv, dv, s2);
     }
   };
   float s1[4] = {0.f, 0.f, 0.f, 0.f}, s2[4] = {0.f, 0.f, 0.f, 0.f};
@@ -134,11 +138,14 @@ __global__ __launch_bounds__(256) void volume_moments_kernel(const float* __rest
     }
     __syncthreads();
   }
-  if (threadIdx.x == 0) out[z] = make_float2((float)part[0][0], (float)part[1][0]);
+  if (threadIdx.x == 0) {
+    if constexpr (GRAD) out[z] = make_float2((float)part[0][0], (float)part[1][0]);
+    else out[z] = make_float2((float)(part[0][0] + (double)n * (double)pivot), (float)(part[1][0] - part[0][0] * part[0][0] / (double)n));
+  }
 }
 
 // The per-feature arithmetic of the normalisation on the sums of volume_moments_kernel, one workgroup per feature, float64:
-//   forward : mom [batch][F][parts][2] = (sum y, sum y^2), `parts` partial sums per volume  ->  mean, biased variance, 1/sqrt(var + eps) of the statistics in use
+//   forward : mom [batch][F][parts][2] = (sum y, sum (y - mean of the part)^2), `parts` partial sums per volume of equal counts  ->  mean, biased variance, 1/sqrt(var + eps) of the statistics in use
 //             (the batch's when training, else the running ones), ab = (a, b) with a = weight / sqrt(var + eps),
 //             b = bias - mean a; when training, the running averages move by `momentum` (unbiased variance).
 //   backward: mom = (sum g m, sum g m y)  ->  params (a, b, p, q) of the load-time gradient, and the gradients of weight and bias.
@@ -166,10 +173,25 @@ __global__ void bn_forward_kernel(const float2* __restrict__ mom, int batch, int
                                   double eps, double momentum, int training, float* __restrict__ ab, float* __restrict__ stats) {
   const int f = blockIdx.x;
   double s1, s2;
-  feature_sums(mom, batch, nf, parts, f, s1, s2);
-  if (threadIdx.x != 0) return;
+  feature_sums(mom, batch, nf, parts, f, s1, s2);          // sum of the samples, sum of the parts' squared deviations from their own means
   const double mean = s1 / count;
-  double var = s2 / count - mean * mean;
+  // ... plus what the parts' means deviate from the mean of all: sum over the parts of n_part (mean_part - mean)^2
+  const double npart = count / ((double)batch * parts);
+  __shared__ double spread[64];
+  double d2 = 0.0;
+  for (int i = threadIdx.x; i < batch * parts; i += 64) {
+    const int b = i / parts, p = i - b * parts;
+    const double dm = (double)mom[((size_t)b * nf + f) * parts + p].x / npart - mean;
+    d2 += dm * dm;
+  }
+  spread[threadIdx.x] = d2;
+  __syncthreads();
+  for (int s = 32; s > 0; s >>= 1) {
+    if ((int)threadIdx.x < s) spread[threadIdx.x] += spread[threadIdx.x + s];
+    __syncthreads();
+  }
+  if (threadIdx.x != 0) return;
+  double var = (s2 + npart * spread[0]) / count;
   var = var < 0.0 ? 0.0 : var;
   double use_mean = mean, use_var = var;
   if (!training) { use_mean = running_mean[f]; use_var = running_var[f]; }

@@ -361,7 +361,8 @@ __global__ __launch_bounds__(NT_MAX) void plane_dft_fwd(const float* __restrict_
 // bias: NULL, or nfeature values; bias[z % nfeature] is added to every sample of volume z = plane / n2
 // relu: nonzero = negative samples (after the bias) are stored as zero
 // moments (alias mode only): NULL, or [nplanes] pairs of sums over each plane of the output v, formed from the staged
-// planes in a fixed order: yref == NULL: (sum v, sum v^2); else, with m = (a yref + b > 0), a = params[f],
+// planes in a fixed order: yref == NULL: (sum v, sum (v - mean of the plane)^2), the squares summed around a pivot so that
+// a large mean costs no digits; else, with m = (a yref + b > 0), a = params[f],
 // b = params[nfeature + f] of the plane's feature f: (sum v m, sum v m yref): what a batch normalisation over the
 // volumes of a feature needs of its input, or (v being the gradient with respect to its activated output) of its gradient.
 __global__ __launch_bounds__(NT_MAX) void plane_dft_inv(const float2* __restrict__ S, float* __restrict__ y, int n2, int nb,
@@ -592,14 +593,20 @@ __global__ __launch_bounds__(NT_MAX) void plane_dft_inv(const float2* __restrict
               s1 += gm; s2 = fmaf(gm, yv, s2);
             }
           }
-        } else {
+        } else {                                         // squares around a pivot (the plane's first sample), moved to the plane's mean below
           const float4* v4 = reinterpret_cast<const float4*>(v);
+          const float pivot = v[0];
 #pragma unroll 4
           for (int i = lane; i < psize / 4; i += 64) {
             const float4 x = v4[i];
-            s1 += (x.x + x.y) + (x.z + x.w);
-            s2 = fmaf(x.x, x.x, fmaf(x.y, x.y, fmaf(x.z, x.z, fmaf(x.w, x.w, s2))));
+            const float d0 = x.x - pivot, d1 = x.y - pivot, d2 = x.z - pivot, d3 = x.w - pivot;
+            s1 += (d0 + d1) + (d2 + d3);
+            s2 = fmaf(d0, d0, fmaf(d1, d1, fmaf(d2, d2, fmaf(d3, d3, s2))));
           }
+#pragma unroll
+          for (int o = 32; o > 0; o >>= 1) { s1 += __shfl_xor(s1, o); s2 += __shfl_xor(s2, o); }
+          if (lane == 0) moments[plane0 + q] = make_float2(fmaf((float)psize, pivot, s1), s2 - s1 * s1 / (float)psize);   // (sum v, sum (v - mean)^2)
+          continue;
         }
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) { s1 += __shfl_xor(s1, o); s2 += __shfl_xor(s2, o); }

@@ -21,12 +21,18 @@ def _rel(got, want):
     return (got - want).abs().max().item() / max(want.abs().max().item(), 1e-30)
 
 
+def _sum_and_squared_deviations(v):
+    """[parts, samples] float64 -> [parts, 2]: (sum v, sum (v - mean of the part)^2), what the library's sums of a
+    normalisation's input are."""
+    return torch.stack([v.sum(-1), ((v - v.mean(-1, keepdim=True)) ** 2).sum(-1)], -1)
+
+
 def test_volume_moments(hip):
     g = torch.Generator().manual_seed(1)
     for n2, nvol in ((64, 6), (44, 4), (14, 9), (6, 5)):
         x = (torch.randn(nvol, n2, n2, n2, generator=g) + 0.5).cuda()
         got = bn_relu._moments("s2cnn_volume_moments", n2 ** 3, x).double()
-        want = torch.stack([x.double().sum((1, 2, 3)), (x.double() ** 2).sum((1, 2, 3))], 1)
+        want = _sum_and_squared_deviations(x.double().view(nvol, -1))
         assert _rel(got, want) < 2e-6, n2
         # the sums of the backward pass: sum g m and sum g m y with m = (a y + b > 0), feature = volume % 3
         y = torch.randn(nvol // 3 * 3, n2, n2, n2, generator=g).cuda()
@@ -43,8 +49,8 @@ def test_volume_moments(hip):
 
 @pytest.mark.parametrize("b_in,b_out", [(32, 32), (22, 32), (26, 32), (22, 22), (7, 22), (6, 6)])
 def test_sums_formed_by_the_synthesis(hip, b_in, b_out):
-    """(sum y, sum y^2) per volume (64^3 grid) or per plane (two-stage path) written by the synthesis that produces y,
-    against float64 sums of that y; y itself bit for bit the output of the synthesis without the sums."""
+    """(sum y, sum (y - mean)^2) per volume (64^3 grid) or per plane (two-stage path) written by the synthesis that produces
+    y, against float64 sums of that y; y itself bit for bit the output of the synthesis without the sums."""
     parts = P.synthesis_moment_parts(b_in, b_out)
     assert parts == (1 if b_out == 32 else 2 * b_out)
     g = torch.Generator().manual_seed(b_in * 100 + b_out)
@@ -55,9 +61,37 @@ def test_sums_formed_by_the_synthesis(hip, b_in, b_out):
     mom = torch.full((6 * parts, 2), float("nan")).cuda()
     y = P.so3_rifft_real_basis(r, b_out=b_out, bias=bias, moments=(mom, None, None))
     assert torch.equal(y, P.so3_rifft_real_basis(r, b_out=b_out, bias=bias))
-    yd = y.double().view(6, parts, -1)
-    want = torch.stack([yd.sum(-1), (yd ** 2).sum(-1)], -1).view(-1, 2)
-    assert _rel(mom.double(), want) < 2e-6
+    yd = y.double().view(6 * parts, -1)
+    want = _sum_and_squared_deviations(yd)
+    # the mean each part's sum stands for, against the spread of the part (what a normalisation divides by), and the spread itself
+    mean_err = ((mom.double()[:, 0] - want[:, 0]) / yd.size(1)).abs() / yd.std(-1)
+    assert mean_err.max().item() < 1e-6 and _rel(mom.double()[:, 1], want[:, 1]) < 2e-5
+
+
+@pytest.mark.parametrize("ratio", [100.0, 1000.0])
+@pytest.mark.parametrize("b_in,b_out", [(32, 32), (22, 22), (6, 6)])
+def test_statistics_of_a_signal_with_a_large_mean(hip, b_in, b_out, ratio):
+    """A mean `ratio` times the standard deviation: the batch variance that the normalisation forms from the library's sums
+    (the synthesis's own, and s2cnn_volume_moments) must keep its digits, as nn.BatchNorm3d's does; E[y^2] - mean^2 from
+    float32 sums would be off by 10 % at a ratio of 1000."""
+    g = torch.Generator().manual_seed(int(ratio) + b_in)
+    nspec = b_in * (4 * b_in ** 2 - 1) // 3
+    nb, nf = 2, 3
+    r = torch.randn(nspec, nb, nf, generator=g).cuda()
+    y0 = P.so3_rifft_real_basis(r, b_out=b_out)
+    bias = (ratio * y0.std()).item() * torch.tensor([1.0, -1.0, 0.5]).cuda()      # the layer's bias carries the mean
+    parts = P.synthesis_moment_parts(b_in, b_out)
+    nvox = (2 * b_out) ** 3
+    mom = torch.full((nb * nf * parts, 2), float("nan")).cuda()
+    y = P.so3_rifft_real_basis(r, b_out=b_out, bias=bias, moments=(mom, None, None))
+    want_var = y.double().transpose(0, 1).reshape(nf, -1).var(1, unbiased=False)
+    for sums, nparts in ((mom, parts), (bn_relu._moments("s2cnn_volume_moments", nvox, y), 1)):
+        ab, stats = torch.empty(2, nf).cuda(), torch.empty(4, nf).cuda()
+        from s2cnn_amd import _hip
+        _hip.call("s2cnn_bn_forward_from_moments", _hip.ptr(sums), nb, nf, nparts, float(nb * nvox), None, None, None, None, 1e-5, 0.1, 1,
+                  _hip.ptr(ab), _hip.ptr(stats), _hip.stream_ptr())
+        got_var = stats[1].double()
+        assert _rel(got_var, want_var) < 1e-3, (nparts, got_var, want_var)
 
 
 @pytest.mark.parametrize("b_in,b_out", [(22, 32), (26, 32), (28, 32), (22, 22), (7, 22), (6, 6)])
