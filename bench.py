@@ -167,6 +167,29 @@ def measure_rows(torch, dev, with_cpu):
         rows[k]["algorithmic_frac"] = rows[k]["frac"]
         rows[k]["frac"] = round(0.75 * rows[k]["frac"], 4)
     del xm, xmg, ymg, zm, gzm
+    # --- the real-basis product at the sizes of the second layer of config 5 (22 degrees, batch 32, 100 -> 100 features: blocks
+    # of 100 do not divide the contraction stage of 32) and of the headline layer, one row per product
+    from s2cnn_amd import so3_real
+    for (nlr, Br, Fr) in ((22, 32, 100), (32, 16, 64)):
+        xr = torch.randn(nspec(nlr), Br, Fr, device=dev).requires_grad_()
+        yr = (torch.randn(nspec(nlr), Fr, Fr, device=dev) * 0.125).requires_grad_()
+        gzr = torch.randn(nspec(nlr), Br, Fr, device=dev)
+
+        def prod_step():
+            zz = so3_real.so3_mm_real(xr, yr)
+            torch.autograd.grad(zz, (xr, yr), gzr)
+
+        for _ in range(2):
+            prod_step()
+        torch.cuda.synchronize()
+        with _hip.KernelTimer() as kt:
+            for _ in range(5):
+                prod_step()
+            torch.cuda.synchronize()
+        flr = mm_flops(nlr, Br, Fr, Fr, real=True)
+        for name, v in kt.summary().items():
+            add("%s nl=%d B=%d %d->%d" % (name.replace("s2cnn_", ""), nlr, Br, Fr, Fr), sum(v) / len(v), flr, "F", None, 1, "")
+        del xr, yr, gzr
     # --- Haar integral at config-4 output size [16, 64, 64, 64, 64]
     xi = torch.randn(16, 64, 64, 64, 64, device=dev)
     t = cpu_s(lambda: O.so3_integrate(xi[:2].cpu()))
