@@ -244,8 +244,10 @@ int s2cnn_so3_analysis_real_masked_bits(const float *x, const void *bits, const 
  * model_original.py:28-35): three passes over the activations forward and five backward.  Here the next layer's analysis
  * applies the normalisation and the activation as it loads the previous layer's output y, and the backward analysis of
  * the previous layer forms the gradient with respect to y as it loads the incoming gradient:
- *   s2cnn_volume_moments            out[z] = (sum y, sum y^2) of each of the nvol volumes of n samples: the batch
- *                                   statistics of a feature are sums of these over the batch
+ *   s2cnn_volume_moments            out[z] = (sum y, sum (y - mean_z)^2), mean_z the mean of the volume, for each of the nvol
+ *                                   volumes of n samples (squares summed around a pivot and moved to the mean in float64: a
+ *                                   mean far above the spread costs no digits); s2cnn_bn_forward_from_moments merges the
+ *                                   volumes of a feature into its batch statistics
  *   s2cnn_so3_analysis_real_affine_relu     the analysis of max(a y + b, 0), a = params[z % nfeature],
  *                                   b = params[nfeature + z % nfeature]  (a = weight / sqrt(var + eps), b = bias - mean a)
  *   s2cnn_bn_relu_grad_moments      out[z] = (sum g m, sum g m y), m = (a y + b > 0): the two reductions of the backward
@@ -269,7 +271,7 @@ int s2cnn_bn_relu_grad_moments(const float *g, const float *y, const float *para
 /* Where the synthesis that produces y (or the gradient g) stages whole planes in LDS it can form those sums itself, one
  * pair per plane, and the separate read is not needed: s2cnn_so3_synthesis_moment_parts(b_in, b_out) = 2 b_out where
  * s2cnn_so3_synthesis_real_moments can do that (real signals, complex spectrum; other arguments as
- * s2cnn_so3_synthesis_real_bias), else 0.  moments [nbatch][2 b_out][2]; yref = NULL: (sum y, sum y^2) of the output;
+ * s2cnn_so3_synthesis_real_bias), else 0.  moments [nbatch][2 b_out][2]; yref = NULL: (sum y, sum (y - mean of the plane)^2) of the output;
  * yref = the tensor y and params = ab: (sum g m, sum g m y) with the output as g. */
 int s2cnn_so3_synthesis_moment_parts(int b_in, int b_out);
 int s2cnn_so3_synthesis_real_moments(const float *xhat, const float *table, const float *packed_table, float *out,
@@ -287,7 +289,8 @@ int s2cnn_so3_synthesis_real_basis_moments(const float *r, const float *table, c
                                            const float *bias, int nfeature, float *moments, const float *yref,
                                            const float *params, void *stream);
 /* the arithmetic between those calls, one small launch each instead of a chain of tensor operations (float64 inside):
- * forward : moments [batch][nfeature][parts][2] (parts = 1 from s2cnn_volume_moments, 2 b from the synthesis above),
+ * forward : moments [batch][nfeature][parts][2] (parts = 1 from s2cnn_volume_moments, 2 b from the synthesis above; per
+ *           part the sum and the squared deviations from the part's own mean, all parts of equal size),
  *           count = samples per feature -> ab [2][nfeature] for the
  *           analysis, stats [4][nfeature] = batch mean, biased batch variance, mean in use, 1/sqrt(var in use + eps)
  *           (in use: the batch's when training != 0, else running_mean / running_var); when training and the running
