@@ -20,6 +20,7 @@
 #include "so3_plane_fft64.h"
 #include "so3_wigner_tiled.h"
 #include "so3_fused64.h"
+#include "so3_fused32.h"
 #include "so3_plane_dft_real.h"
 #include <mutex>
 
@@ -295,15 +296,28 @@ __global__ void add_bias_kernel(float* __restrict__ y, const float* __restrict__
   }
 }
 
-// Real signals on the 64^3 grid go through the per-volume kernels of so3_fused64.h (the planes never leave the CU).
-bool fused_path(int b_grid, int b_spec, int cplx, bool synthesis) {
-  return !cplx && b_grid == 32 && (synthesis || b_spec <= 32);
+// Real signals on the 64^3 and 32^3 grids go through the per-volume kernels of so3_fused64.h / so3_fused32.h (the planes
+// never leave the CU).
+enum FusedKind { FUSED_NONE = 0, FUSED_64, FUSED_32 };
+FusedKind fused_kind(int b_grid, int b_spec, int cplx, bool synthesis) {
+  if (cplx) return FUSED_NONE;
+  if (b_grid == 32 && (synthesis || b_spec <= 32)) return FUSED_64;
+  if (b_grid == 16 && (synthesis || b_spec <= 16)) return FUSED_32;
+  return FUSED_NONE;
+}
+bool fused_path(int b_grid, int b_spec, int cplx, bool synthesis) { return fused_kind(b_grid, b_spec, cplx, synthesis) != FUSED_NONE; }
+size_t fused_scratch_bytes(FusedKind k, long nbatch) { return k == FUSED_64 ? fused64::scratch_bytes(nbatch) : fused32::scratch_bytes(nbatch); }
+size_t fused_packed_floats(FusedKind k) { return k == FUSED_64 ? fused64::PACKED_FLOATS : fused32::PACKED_FLOATS; }
+// table [2 b_grid][nspec(b_spec)] -> the packed table of the per-volume kernels, degrees below nl
+void fused_pack_table(FusedKind k, hipStream_t st, const float* table, float* packed, int b_spec, int nl) {
+  if (k == FUSED_64) hipLaunchKernelGGL(fused64::pack_table, dim3(1024), dim3(256), 0, st, table, packed, s2cnn::so3_nspec(b_spec), nl);
+  else hipLaunchKernelGGL(fused32::pack_table, dim3(256), dim3(256), 0, st, table, packed, s2cnn::so3_nspec(b_spec), nl);
 }
 
 // Bytes of the intermediate; batch items padded to the z tile of the tiled Wigner kernels.
 size_t ws_bytes(int b_grid, int b_spec, long nbatch, int cplx, bool synthesis) {
   if (b_grid < 1 || b_spec < 1 || nbatch < 1) return 0;
-  if (fused_path(b_grid, b_spec, cplx, synthesis)) return fused64::scratch_bytes(nbatch);
+  if (const FusedKind k = fused_kind(b_grid, b_spec, cplx, synthesis)) return fused_scratch_bytes(k, nbatch);
   const long nb = b_grid < b_spec ? b_grid : b_spec;
   const long MW = 2 * nb - 1, NW = cplx ? MW : nb;
   const long zpad = (nbatch + wigner_tiled::ZT - 1) / wigner_tiled::ZT * wigner_tiled::ZT;
@@ -317,7 +331,7 @@ bool sizes_ok(int b_grid, int b_spec, long nbatch) {
 
 // Bytes of the packed table of the tiled fast path; 0 when that path does not apply.
 size_t packed_bytes(int b_grid, int b_spec, int cplx, bool synthesis) {
-  if (fused_path(b_grid, b_spec, cplx, synthesis)) return fused64::PACKED_FLOATS * sizeof(float);
+  if (const FusedKind k = fused_kind(b_grid, b_spec, cplx, synthesis)) return fused_packed_floats(k) * sizeof(float);
   const int nb = b_grid < b_spec ? b_grid : b_spec;
   if (cplx || nb > 64) return 0;
   if (synthesis) return 2 * b_grid <= 128 ? wigner_tiled::packed_floats_synthesis(2 * b_grid, nb) * sizeof(float) : 0;
@@ -336,52 +350,69 @@ bool real_basis_analysis(int b_in, int b_out) {
   return b_in >= 1 && b_out >= 1 && (fused_path(b_in, b_out, 0, false) || (packed_bytes(b_in, b_out, 0, false) != 0 && b_out <= 32));
 }
 
-// Real signals on the 64^3 grid: per-volume kernel + the pass between its records and the spectral rows.
+// Real signals on the 64^3 or 32^3 grid: per-volume kernel + the pass between its records and the spectral rows.
 // real_basis: the spectrum is stored in the real basis (one float per entry) instead of complex pairs.
-int fused_analysis(const s2cnn::Input& in, const float* table, const float* packed_table, float* out,
+int fused_analysis(FusedKind kind, const s2cnn::Input& in, const float* table, const float* packed_table, float* out,
                    void* workspace, size_t workspace_bytes, int b_out, long nbatch, bool real_basis, hipStream_t st) {
   if (!s2cnn::aligned16(in.x) || !s2cnn::aligned16(in.w)) return S2CNN_EALIGN;
-  const size_t need = round256(fused64::scratch_bytes(nbatch)) + fused64::PACKED_FLOATS * sizeof(float);
+  const size_t need = round256(fused_scratch_bytes(kind, nbatch)) + fused_packed_floats(kind) * sizeof(float);
   if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
   float4* rec = static_cast<float4*>(workspace);
   const float* Tf = packed_table;
   if (!Tf) {  // pack behind the records on every call
-    float* dst = reinterpret_cast<float*>(static_cast<char*>(workspace) + round256(fused64::scratch_bytes(nbatch)));
-    hipLaunchKernelGGL(fused64::pack_table, dim3(1024), dim3(256), 0, st, table, dst, s2cnn::so3_nspec(b_out), b_out);
+    float* dst = reinterpret_cast<float*>(static_cast<char*>(workspace) + round256(fused_scratch_bytes(kind, nbatch)));
+    fused_pack_table(kind, st, table, dst, b_out, b_out);
     Tf = dst;
   }
-  fused64::launch_analysis(b_out, st, in, Tf, rec, nbatch);
-  if (real_basis)
-    hipLaunchKernelGGL(fused64::spectrum_scatter_real, dim3((unsigned)((nbatch + fused64::ZR - 1) / fused64::ZR), fused64::active_rounds(b_out) * 32), dim3(256), 0, st,
-                       rec, out, b_out, nbatch);
-  else
-    hipLaunchKernelGGL(fused64::spectrum_scatter, dim3((unsigned)((nbatch + fused64::ZT - 1) / fused64::ZT), fused64::active_rounds(b_out) * 16), dim3(256), 0, st,
-                       rec, reinterpret_cast<float2*>(out), b_out, nbatch);
+  const unsigned tiles_r = (unsigned)((nbatch + fused64::ZR - 1) / fused64::ZR), tiles_c = (unsigned)((nbatch + fused64::ZT - 1) / fused64::ZT);
+  float2* outc = reinterpret_cast<float2*>(out);
+  if (kind == FUSED_64) {
+    const int rounds = fused64::active_rounds(b_out);
+    fused64::launch_analysis(b_out, st, in, Tf, rec, nbatch);
+    if (real_basis) hipLaunchKernelGGL(fused64::spectrum_scatter_real<>, dim3(tiles_r, rounds * 32), dim3(256), 0, st, rec, out, b_out, nbatch);
+    else hipLaunchKernelGGL(fused64::spectrum_scatter<>, dim3(tiles_c, rounds * 16), dim3(256), 0, st, rec, outc, b_out, nbatch);
+  } else {
+    const int rounds = fused32::active_rounds(b_out);
+    fused32::launch_analysis(b_out, st, in, Tf, rec, nbatch);
+    if (real_basis)
+      hipLaunchKernelGGL(fused64::spectrum_scatter_real<fused32::Geometry>, dim3(tiles_r, rounds * 16), dim3(256), 0, st, rec, out, b_out, nbatch);
+    else
+      hipLaunchKernelGGL(fused64::spectrum_scatter<fused32::Geometry>, dim3(tiles_c, rounds * 8), dim3(256), 0, st, rec, outc, b_out, nbatch);
+  }
   return s2cnn::launch_status();
 }
 
-int fused_synthesis(const float* xhat, const float* table, const float* packed_table, float* out, void* workspace,
+int fused_synthesis(FusedKind kind, const float* xhat, const float* table, const float* packed_table, float* out, void* workspace,
                     size_t workspace_bytes, int b_in, long nbatch, bool real_basis, const float* bias, int nfeature, int relu,
                     unsigned long long* bits, hipStream_t st, float* moments = nullptr, const float* yref = nullptr,
                     const float* params = nullptr) {
   if (!s2cnn::aligned16(out) || !s2cnn::aligned16(bits) || !s2cnn::aligned8(moments) || !s2cnn::aligned16(yref)) return S2CNN_EALIGN;
-  const int nl = b_in < 32 ? b_in : 32;
-  const size_t need = round256(fused64::scratch_bytes(nbatch)) + fused64::PACKED_FLOATS * sizeof(float);
+  if (bits && kind != FUSED_64) return S2CNN_EINVAL;
+  const int b_grid = kind == FUSED_64 ? 32 : 16;
+  const int nl = b_in < b_grid ? b_in : b_grid;
+  const size_t need = round256(fused_scratch_bytes(kind, nbatch)) + fused_packed_floats(kind) * sizeof(float);
   if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
   float4* rec = static_cast<float4*>(workspace);
   const float* Tf = packed_table;
   if (!Tf) {
-    float* dst = reinterpret_cast<float*>(static_cast<char*>(workspace) + round256(fused64::scratch_bytes(nbatch)));
-    hipLaunchKernelGGL(fused64::pack_table, dim3(1024), dim3(256), 0, st, table, dst, s2cnn::so3_nspec(b_in), nl);
+    float* dst = reinterpret_cast<float*>(static_cast<char*>(workspace) + round256(fused_scratch_bytes(kind, nbatch)));
+    fused_pack_table(kind, st, table, dst, b_in, nl);
     Tf = dst;
   }
-  if (real_basis)
-    hipLaunchKernelGGL(fused64::spectrum_gather_real, dim3((unsigned)((nbatch + fused64::ZR - 1) / fused64::ZR), fused64::active_rounds(nl) * 32), dim3(256), 0, st,
-                       xhat, rec, nl, nbatch);
-  else
-    hipLaunchKernelGGL(fused64::spectrum_gather, dim3((unsigned)((nbatch + fused64::ZT - 1) / fused64::ZT), fused64::active_rounds(nl) * 16), dim3(256), 0, st,
-                       reinterpret_cast<const float2*>(xhat), rec, nl, nbatch);
-  fused64::launch_synthesis(nl, st, rec, Tf, out, nbatch, bias, nfeature, relu, bits, reinterpret_cast<float2*>(moments), yref, params);
+  const unsigned tiles_r = (unsigned)((nbatch + fused64::ZR - 1) / fused64::ZR), tiles_c = (unsigned)((nbatch + fused64::ZT - 1) / fused64::ZT);
+  const float2* xc = reinterpret_cast<const float2*>(xhat);
+  float2* mom = reinterpret_cast<float2*>(moments);
+  if (kind == FUSED_64) {
+    const int rounds = fused64::active_rounds(nl);
+    if (real_basis) hipLaunchKernelGGL(fused64::spectrum_gather_real<>, dim3(tiles_r, rounds * 32), dim3(256), 0, st, xhat, rec, nl, nbatch);
+    else hipLaunchKernelGGL(fused64::spectrum_gather<>, dim3(tiles_c, rounds * 16), dim3(256), 0, st, xc, rec, nl, nbatch);
+    fused64::launch_synthesis(nl, st, rec, Tf, out, nbatch, bias, nfeature, relu, bits, mom, yref, params);
+  } else {
+    const int rounds = fused32::active_rounds(nl);
+    if (real_basis) hipLaunchKernelGGL(fused64::spectrum_gather_real<fused32::Geometry>, dim3(tiles_r, rounds * 16), dim3(256), 0, st, xhat, rec, nl, nbatch);
+    else hipLaunchKernelGGL(fused64::spectrum_gather<fused32::Geometry>, dim3(tiles_c, rounds * 8), dim3(256), 0, st, xc, rec, nl, nbatch);
+    fused32::launch_synthesis(nl, st, rec, Tf, out, nbatch, bias, nfeature, relu, mom, yref, params);
+  }
   return s2cnn::launch_status();
 }
 
@@ -404,9 +435,9 @@ extern "C" int s2cnn_so3_pack_table(const float* table, float* packed, int b_in,
   if (!s2cnn::aligned16(packed)) return S2CNN_EALIGN;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int nb = b_in < b_out ? b_in : b_out;
-  if (fused_path(synthesis ? b_out : b_in, synthesis ? b_in : b_out, 0, synthesis != 0)) {
-    const int b_spec = synthesis ? b_in : b_out;
-    hipLaunchKernelGGL(fused64::pack_table, dim3(1024), dim3(256), 0, st, table, packed, s2cnn::so3_nspec(b_spec), b_spec < 32 ? b_spec : 32);
+  if (const FusedKind k = fused_kind(synthesis ? b_out : b_in, synthesis ? b_in : b_out, 0, synthesis != 0)) {
+    const int b_spec = synthesis ? b_in : b_out, b_grid = synthesis ? b_out : b_in;
+    fused_pack_table(k, st, table, packed, b_spec, b_spec < b_grid ? b_spec : b_grid);
   } else if (synthesis) {
     hipLaunchKernelGGL(wigner_tiled::pack_table_synthesis, dim3(2048), dim3(256), 0, st, table, packed, 2 * b_out, nb, b_in);
   } else {
@@ -443,14 +474,14 @@ int analysis_impl(const s2cnn::Input& in, const float* table, const float* packe
   const float* mask = in.second_tensor() ? in.w : nullptr;
   if (!x || !table || !out || !sizes_ok(b_in, b_out, nbatch) || (in.kind != s2cnn::PRO_NONE && complex_in)) return S2CNN_EINVAL;
   if (in.kind != s2cnn::PRO_NONE && in.kind != s2cnn::PRO_AFFINE_RELU && !in.w) return S2CNN_EINVAL;
-  if (in.kind == s2cnn::PRO_BITS && !fused_path(b_in, b_out, complex_in, false)) return S2CNN_EINVAL;
+  if (in.kind == s2cnn::PRO_BITS && fused_kind(b_in, b_out, complex_in, false) != FUSED_64) return S2CNN_EINVAL;
   if (in.kind >= s2cnn::PRO_AFFINE_RELU && (!in.params || in.nfeature < 1 || nbatch % in.nfeature != 0 || !prologue_path(b_in, b_out)))
     return S2CNN_EINVAL;
   if ((!real_basis && !s2cnn::aligned8(out)) || (complex_in && !s2cnn::aligned8(x))) return S2CNN_EALIGN;
   if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (fused_path(b_in, b_out, complex_in, false))
-    return fused_analysis(in, table, packed_table, out, workspace, workspace_bytes, b_out, nbatch, real_basis, st);
+  if (const FusedKind k = fused_kind(b_in, b_out, complex_in, false))
+    return fused_analysis(k, in, table, packed_table, out, workspace, workspace_bytes, b_out, nbatch, real_basis, st);
   const size_t need = s2cnn_so3_analysis_workspace(b_in, b_out, nbatch, complex_in);
   if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
   const int n2 = 2 * b_in, nb = b_in < b_out ? b_in : b_out;
@@ -540,14 +571,14 @@ int synthesis_impl(const float* xhat, const float* table, const float* packed_ta
   if (real_basis && fused_path(b_out, b_in, 0, true) && mom.out) return S2CNN_EINVAL;     // per volume: fused_synthesis, by its callers
   if (mom.out && (complex_out || moment_parts(b_in, b_out) == 0 || !s2cnn::aligned8(mom.out))) return S2CNN_EINVAL;
   if (mom.yref && (!mom.params || nfeature < 1 || nbatch % nfeature != 0)) return S2CNN_EINVAL;
-  if (bits && !fused_path(b_out, b_in, complex_out, true)) return S2CNN_EINVAL;
+  if (bits && fused_kind(b_out, b_in, complex_out, true) != FUSED_64) return S2CNN_EINVAL;
   if (bias && (complex_out || nfeature < 1 || nbatch % nfeature != 0)) return S2CNN_EINVAL;
   if (relu && complex_out) return S2CNN_EINVAL;
   if ((!real_basis && !s2cnn::aligned8(xhat)) || (complex_out && !s2cnn::aligned8(out))) return S2CNN_EALIGN;
   if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (fused_path(b_out, b_in, complex_out, true))
-    return fused_synthesis(xhat, table, packed_table, out, workspace, workspace_bytes, b_in, nbatch, real_basis, bias, bias ? nfeature : 1, relu, bits, st);
+  if (const FusedKind k = fused_kind(b_out, b_in, complex_out, true))
+    return fused_synthesis(k, xhat, table, packed_table, out, workspace, workspace_bytes, b_in, nbatch, real_basis, bias, bias ? nfeature : 1, relu, bits, st);
   const size_t need = s2cnn_so3_synthesis_workspace(b_in, b_out, nbatch, complex_out);
   if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
   const int n2 = 2 * b_out, nb = b_in < b_out ? b_in : b_out;
@@ -651,7 +682,7 @@ extern "C" int s2cnn_so3_synthesis_real_relu(const float* xhat, const float* tab
 }
 
 extern "C" size_t s2cnn_so3_relu_bits_bytes(int b_grid, long nbatch) {
-  if (nbatch < 1 || !fused_path(b_grid, b_grid, 0, true)) return 0;
+  if (nbatch < 1 || fused_kind(b_grid, b_grid, 0, true) != FUSED_64) return 0;      // the kernels of the 64^3 grid write them
   return (size_t)nbatch * fused64::BITS_WORDS * sizeof(unsigned long long);
 }
 
@@ -710,8 +741,9 @@ extern "C" int s2cnn_so3_synthesis_real_basis(const float* r, const float* table
 
 extern "C" int s2cnn_so3_synthesis_real_basis_moment_parts(int b_in, int b_out, int grad) {
   if (!sizes_ok(b_out, b_in, 1) || !real_basis_synthesis(b_in, b_out)) return 0;
-  if (!fused_path(b_out, b_in, 0, true)) return moment_parts(b_in, b_out);
-  return !grad || b_in <= fused64::GRAD_MOMENTS_MAX_NL ? 1 : 0;
+  const FusedKind k = fused_kind(b_out, b_in, 0, true);
+  if (k == FUSED_NONE) return moment_parts(b_in, b_out);
+  return !grad || k == FUSED_32 || b_in <= fused64::GRAD_MOMENTS_MAX_NL ? 1 : 0;
 }
 
 extern "C" int s2cnn_so3_synthesis_real_basis_moments(const float* r, const float* table, const float* packed_table, float* out,
@@ -724,9 +756,9 @@ extern "C" int s2cnn_so3_synthesis_real_basis_moments(const float* r, const floa
   if (yref && !params) return S2CNN_EINVAL;
   if (s2cnn_so3_synthesis_real_basis_moment_parts(b_in, b_out, yref != nullptr) == 0) return S2CNN_EINVAL;
   if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
-  if (fused_path(b_out, b_in, 0, true)) {
+  if (const FusedKind k = fused_kind(b_out, b_in, 0, true)) {
     if (yref && bias) return S2CNN_EINVAL;
-    return fused_synthesis(r, table, packed_table, out, workspace, workspace_bytes, b_in, nbatch, true, bias, bias || yref ? nfeature : 1, 0,
+    return fused_synthesis(k, r, table, packed_table, out, workspace, workspace_bytes, b_in, nbatch, true, bias, bias || yref ? nfeature : 1, 0,
                            nullptr, static_cast<hipStream_t>(stream), moments, yref, params);
   }
   PlaneMoments mom;

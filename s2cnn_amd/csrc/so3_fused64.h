@@ -487,16 +487,25 @@ __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MASK == 0 || MASK == 2 
 
 // ---------------------------------------------------------------------------------------------
 // records <-> spectral rows, for a tile of 16 volumes and 32 items per workgroup (256 threads).
-// grid (ceil(nbatch / 16), NIT * 16).  Row kinds of an item and degree: 0 (+a, n)  1 (-a, n)
+// grid (ceil(nbatch / 16), rounds * G::THREADS / 32).  Row kinds of an item and degree: 0 (+a, n)  1 (-a, n)
 // 2 (-a,-n)  3 (+a,-n); kinds 2, 3 are (-1)^(a-n) conj of kinds 0, 1 in a spectrum of a real signal.
 // ---------------------------------------------------------------------------------------------
 constexpr int ZT = 16;              // volumes per tile: one 128-byte piece of a spectral row
 constexpr int IT_TILE = 32;         // items per tile
 constexpr int VLD = 16 * ZT + 1;    // LDS floats per item: 16 components x 16 volumes, padded
 
+// What these passes need to know of the kernels whose records they read and write: threads per volume, the size of a
+// record and the item of every place.  The per-volume kernels of another grid (so3_fused32.h) bring their own.
+struct Geometry {
+  static constexpr int THREADS = fused64::THREADS;
+  static constexpr int REC_F4 = fused64::REC_F4;
+  static __device__ __forceinline__ bool decode(int i, int& c, int& a, int& n) { return decode_item(i, c, a, n); }
+};
+
+template <class G>
 __device__ __forceinline__ int pack_item_info(int i) {
   int c, a, n;
-  const bool ok = decode_item(i, c, a, n);
+  const bool ok = G::decode(i, c, a, n);
   return c | (a << 8) | (n << 16) | (ok ? 1 << 24 : 0);
 }
 
@@ -511,13 +520,15 @@ __device__ __forceinline__ int row_index(int info, int u, int kind, int nl) {
   return lmn_index(l, m, kind >= 2 ? -n : n);
 }
 
+template <class G = Geometry>
 __global__ __launch_bounds__(256) void spectrum_scatter(const float4* __restrict__ rec, float2* __restrict__ out, int nl, long nbatch) {
+  constexpr int THREADS = G::THREADS, REC_F4 = G::REC_F4, TILES = THREADS / IT_TILE;
   __shared__ float vals[IT_TILE * VLD];
   __shared__ int info[IT_TILE];
   const int th = threadIdx.x;
   const long z0 = (long)blockIdx.x * ZT;
-  const int it = blockIdx.y >> 4, t0 = (blockIdx.y & 15) * IT_TILE;
-  if (th < IT_TILE) info[th] = pack_item_info(it * THREADS + t0 + th);
+  const int it = blockIdx.y / TILES, t0 = (blockIdx.y % TILES) * IT_TILE;
+  if (th < IT_TILE) info[th] = pack_item_info<G>(it * THREADS + t0 + th);
 #pragma unroll
   for (int r = 0; r < 8; ++r) {
     const int e = th + 256 * r;
@@ -547,13 +558,15 @@ __global__ __launch_bounds__(256) void spectrum_scatter(const float4* __restrict
 // xh [nspec][nbatch] complex (any symmetry) -> records of the symmetrised spectrum
 //   xs[l,m,n] = xh[l,m,n] + (-1)^(m-n) conj xh[l,-m,-n]   (twice the Hermitian part: the table carries 1/2),
 // zero where there is no such degree; the (-a) half of items with a = 0 is zero (it is the (+a) half).
+template <class G = Geometry>
 __global__ __launch_bounds__(256) void spectrum_gather(const float2* __restrict__ xh, float4* __restrict__ rec, int nl, long nbatch) {
+  constexpr int THREADS = G::THREADS, REC_F4 = G::REC_F4, TILES = THREADS / IT_TILE;
   __shared__ float vals[IT_TILE * VLD];
   __shared__ int info[IT_TILE];
   const int th = threadIdx.x;
   const long z0 = (long)blockIdx.x * ZT;
-  const int it = blockIdx.y >> 4, t0 = (blockIdx.y & 15) * IT_TILE;
-  if (th < IT_TILE) info[th] = pack_item_info(it * THREADS + t0 + th);
+  const int it = blockIdx.y / TILES, t0 = (blockIdx.y % TILES) * IT_TILE;
+  if (th < IT_TILE) info[th] = pack_item_info<G>(it * THREADS + t0 + th);
   __syncthreads();
   {
     const int zz = th & 15, u = (th >> 4) & 3, pm = (th >> 6) & 1, sub = th >> 7;
@@ -595,7 +608,7 @@ __global__ __launch_bounds__(256) void spectrum_gather(const float2* __restrict_
 // and backwards (records hold twice the complex value, the table carries 1/2):
 //     2 A = (cc + ss, sc - cs)   2 C = s (cc - ss, -(cs + sc))   with cc, cs, sc, ss = R[+a,+n], R[+a,-n], R[-a,+n], R[-a,-n]
 //     a = 0: sqrt2 (cc, -cs), C unused     n = 0: sqrt2 (cc, sc), s sqrt2 (cc, -sc)     a = n = 0: (2 cc, 0)
-// Tiles of 32 volumes (128-byte pieces of a row) and 16 items; grid (ceil(nbatch / 32), NIT * 32).
+// Tiles of 32 volumes (128-byte pieces of a row) and 16 items; grid (ceil(nbatch / 32), rounds * G::THREADS / 16).
 // ---------------------------------------------------------------------------------------------
 constexpr int ZR = 32;
 constexpr int IT_TILE_R = 16;
@@ -623,13 +636,15 @@ __device__ __forceinline__ RowRule row_rule(int inf, int rs, int nl) {
   return r;
 }
 
+template <class G = Geometry>
 __global__ __launch_bounds__(256) void spectrum_scatter_real(const float4* __restrict__ rec, float* __restrict__ out, int nl, long nbatch) {
+  constexpr int THREADS = G::THREADS, REC_F4 = G::REC_F4, TILES = THREADS / IT_TILE_R;
   __shared__ float vals[IT_TILE_R * VLD_R];
   __shared__ RowRule rules[IT_TILE_R * 16];
   const int th = threadIdx.x;
   const long z0 = (long)blockIdx.x * ZR;
-  const int it = blockIdx.y >> 5, t0 = (blockIdx.y & 31) * IT_TILE_R;
-  rules[th] = row_rule(pack_item_info(it * THREADS + t0 + (th >> 4)), th & 15, nl);   // 16 items x 16 row slots: one per thread
+  const int it = blockIdx.y / TILES, t0 = (blockIdx.y % TILES) * IT_TILE_R;
+  rules[th] = row_rule(pack_item_info<G>(it * THREADS + t0 + (th >> 4)), th & 15, nl);   // 16 items x 16 row slots: one per thread
 #pragma unroll
   for (int r = 0; r < 8; ++r) {
     const int e = th + 256 * r;
@@ -668,13 +683,15 @@ __device__ __forceinline__ QuadRows quad_rows(int inf, int u, int nl) {
   return q;
 }
 
+template <class G = Geometry>
 __global__ __launch_bounds__(256) void spectrum_gather_real(const float* __restrict__ rr, float4* __restrict__ rec, int nl, long nbatch) {
+  constexpr int THREADS = G::THREADS, REC_F4 = G::REC_F4, TILES = THREADS / IT_TILE_R;
   __shared__ float vals[IT_TILE_R * VLD_R];
   __shared__ QuadRows quads[IT_TILE_R * 4];
   const int th = threadIdx.x;
   const long z0 = (long)blockIdx.x * ZR;
-  const int it = blockIdx.y >> 5, t0 = (blockIdx.y & 31) * IT_TILE_R;
-  if (th < IT_TILE_R * 4) quads[th] = quad_rows(pack_item_info(it * THREADS + t0 + (th >> 2)), th & 3, nl);
+  const int it = blockIdx.y / TILES, t0 = (blockIdx.y % TILES) * IT_TILE_R;
+  if (th < IT_TILE_R * 4) quads[th] = quad_rows(pack_item_info<G>(it * THREADS + t0 + (th >> 2)), th & 3, nl);
   __syncthreads();
   {
     const int zz = th & 31, u = (th >> 5) & 3, sub = th >> 7;
