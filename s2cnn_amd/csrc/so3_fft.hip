@@ -556,9 +556,13 @@ struct PlaneMoments {
   const float* params = nullptr;   // [2][nfeature]
 };
 
-// 2 b_out (the sums come per plane) where the real synthesis b_in -> b_out can form them, else 0
+// Pairs of sums per volume where the real synthesis b_in -> b_out of a complex spectrum can form them: 2 b_out (one per plane)
+// on the two-stage path, 1 from the per-volume kernels of the 32^3 grid, else 0
 int moment_parts(int b_in, int b_out) {
-  if (!sizes_ok(b_out, b_in, 1) || fused_path(b_out, b_in, 0, true) || 2 * b_out == 64) return 0;
+  if (!sizes_ok(b_out, b_in, 1)) return 0;
+  const FusedKind k = fused_kind(b_out, b_in, 0, true);
+  if (k == FUSED_32) return 1;
+  if (k != FUSED_NONE || 2 * b_out == 64) return 0;
   const plane_real::Plan plan = plane_real::plan_inv(2 * b_out, b_in < b_out ? b_in : b_out, 2 * b_out);
   return plan.pl > 0 && plan.alias ? 2 * b_out : 0;
 }
@@ -577,8 +581,11 @@ int synthesis_impl(const float* xhat, const float* table, const float* packed_ta
   if ((!real_basis && !s2cnn::aligned8(xhat)) || (complex_out && !s2cnn::aligned8(out))) return S2CNN_EALIGN;
   if (packed_table && !s2cnn::aligned16(packed_table)) return S2CNN_EALIGN;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (const FusedKind k = fused_kind(b_out, b_in, complex_out, true))
-    return fused_synthesis(k, xhat, table, packed_table, out, workspace, workspace_bytes, b_in, nbatch, real_basis, bias, bias ? nfeature : 1, relu, bits, st);
+  if (const FusedKind k = fused_kind(b_out, b_in, complex_out, true)) {
+    if (mom.yref && bias) return S2CNN_EINVAL;
+    return fused_synthesis(k, xhat, table, packed_table, out, workspace, workspace_bytes, b_in, nbatch, real_basis, bias,
+                           (bias || mom.yref) ? nfeature : 1, relu, bits, st, mom.out, mom.yref, mom.params);
+  }
   const size_t need = s2cnn_so3_synthesis_workspace(b_in, b_out, nbatch, complex_out);
   if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
   const int n2 = 2 * b_out, nb = b_in < b_out ? b_in : b_out;

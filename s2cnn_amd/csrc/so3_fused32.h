@@ -48,7 +48,7 @@ constexpr size_t PACKED_FLOATS = (size_t)NJ * NIT * 2 * THREADS * 4;
 constexpr int REC_F4 = NIT * 4 * THREADS;
 constexpr size_t REC_BYTES = (size_t)REC_F4 * 16;          // 32768
 inline size_t scratch_bytes(long nbatch) { return (size_t)nbatch * REC_BYTES; }
-constexpr int WAVES_PER_SIMD = 4;          // four workgroups per compute unit
+constexpr int WAVES_PER_SIMD = 4;          // four workgroups per compute unit (five or six cost registers and time)
 
 __host__ __device__ constexpr int slot_of(int k) { return 8 * (k & 3) + (k >> 2); }    // where bin (or sample) k of a line sits
 __host__ __device__ constexpr int index_of(int s) { return (s >> 3) + 4 * (s & 7); }   // which bin (or sample) slot s holds
@@ -320,8 +320,11 @@ __global__ __launch_bounds__(THREADS, WAVES_PER_SIMD) void synthesis_kernel(cons
                                                                            int nfeature, int relu, float2* __restrict__ moments,
                                                                            const float* __restrict__ yref, const float* __restrict__ params) {
   __shared__ __attribute__((aligned(16))) float2 work[LDS_ELEMS];
-  __shared__ __attribute__((aligned(16))) float4 stg_p[NITEMS];      // the item's share of the bins [+a,n], [-a,-n]
-  __shared__ __attribute__((aligned(16))) float4 stg_m[NITEMS];      //                              [-a,n], [+a,-n]
+  // places 0 .. NITEMS-1: one per item; ZERO_PLACE: never written, read for the degree groups a column does not have;
+  // DUMP_PLACE: written by the threads without an item, never read
+  constexpr int ZERO_PLACE = NITEMS, DUMP_PLACE = NITEMS + 1, NPLACES = NITEMS + 2;
+  __shared__ __attribute__((aligned(16))) float4 stg_p[NPLACES];     // the item's share of the bins [+a,n], [-a,-n]
+  __shared__ __attribute__((aligned(16))) float4 stg_m[NPLACES];     //                              [-a,n], [+a,-n]
   const long z = volume_of_block(nbatch);
   if (z < 0) return;
   const int t = threadIdx.x;
@@ -332,7 +335,7 @@ __global__ __launch_bounds__(THREADS, WAVES_PER_SIMD) void synthesis_kernel(cons
   Twiddles tw;
   make_twiddles<true>(tw);
   for (int i = t; i < LDS_ELEMS; i += THREADS) work[i] = make_float2(0.f, 0.f);
-  for (int i = t; i < NITEMS; i += THREADS) { stg_p[i] = make_float4(0.f, 0.f, 0.f, 0.f); stg_m[i] = make_float4(0.f, 0.f, 0.f, 0.f); }   // places of skipped rounds stay zero
+  for (int i = t; i < NPLACES; i += THREADS) { stg_p[i] = make_float4(0.f, 0.f, 0.f, 0.f); stg_m[i] = make_float4(0.f, 0.f, 0.f, 0.f); }   // places of skipped rounds stay zero
 
   const __amdgpu_buffer_rsrc_t rr = make_rsrc(rec + (size_t)z * REC_F4, (unsigned)REC_BYTES);
   const __amdgpu_buffer_rsrc_t rt = make_rsrc(Tf, (unsigned)(PACKED_FLOATS * 4));
@@ -343,12 +346,12 @@ __global__ __launch_bounds__(THREADS, WAVES_PER_SIMD) void synthesis_kernel(cons
   if constexpr (MOM == 2) { mom_a = params[z % nfeature]; mom_b = params[nfeature + z % nfeature]; }
 
   float2 xp[NA][4], xm[NA][4];
-  int place[NA];                 // staging place of the item, -1: none; bit 30: n is odd
+  int place[NA];                 // staging place of the item; bit 30: n is odd
 #pragma unroll
   for (int it = 0; it < NA; ++it) {
     int c, a, n;
     const bool ok = decode_item(it * THREADS + t, c, a, n);
-    place[it] = ok ? (stage_offset(c) + a * (4 * c + 4) + n) | ((n & 1) << 30) : -1;
+    place[it] = ok ? (stage_offset(c) + a * (4 * c + 4) + n) | ((n & 1) << 30) : DUMP_PLACE;
     const float4 v0 = buf_load_f32x4(rr, toff, (it * 4 + 0) * (THREADS * 16)), v1 = buf_load_f32x4(rr, toff, (it * 4 + 1) * (THREADS * 16));
     const float4 v2 = buf_load_f32x4(rr, toff, (it * 4 + 2) * (THREADS * 16)), v3 = buf_load_f32x4(rr, toff, (it * 4 + 3) * (THREADS * 16));
     xp[it][0] = make_float2(v0.x, v0.y); xp[it][1] = make_float2(v0.z, v0.w);
@@ -378,33 +381,38 @@ __global__ __launch_bounds__(THREADS, WAVES_PER_SIMD) void synthesis_kernel(cons
       Sm.x = fmaf(a2[u], xm[it][u].x, Sm.x); Sm.y = fmaf(a2[u], xm[it][u].y, Sm.y);
       Qm.x = fmaf(b1, xm[it][u].x, Qm.x);    Qm.y = fmaf(b1, xm[it][u].y, Qm.y);
     }
-    if (place[it] < 0) return;
     const unsigned sb = ((unsigned)place[it] << 1) & 0x80000000u;
     const int pos = place[it] & 0xffff;
     const float qpx = flip(Qp.x, sb), qpy = flip(Qp.y, sb), qmx = flip(Qm.x, sb), qmy = flip(Qm.y, sb);
     stg_p[pos] = make_float4(Sp.x - qpy, Sp.y + qpx, Sp.x + qpy, qpx - Sp.y);
     stg_m[pos] = make_float4(Sm.x - qmy, Sm.y + qmx, Sm.x + qmy, qmx - Sm.y);
   };
-  // staging -> work (natural order): thread t takes the column a = t / 16, n = t % 16
-  auto reduce = [&]() {
+  // staging -> work (natural order): thread t takes the column a = t / 16, n = t % 16.  No branches: a degree group the
+  // column does not have reads the zero place, a bin that does not exist (-0) goes to the pad column of its row.
+  int red_pos[NA == 1 ? 3 : 4], red_dst[4];
+  {
     const int a = t >> 4, n = t & 15;
     const int cmin = (a > n ? a : n) >> 2;
+#pragma unroll
+    for (int c = 0; c < (NA == 1 ? 3 : 4); ++c) red_pos[c] = c >= cmin ? stage_offset(c) + a * (4 * c + 4) + n : ZERO_PLACE;
+    const int rp = a * PITCH, rm = ((32 - a) & 31) * PITCH;
+    red_dst[0] = rp + n;                                  // [+a, n]
+    red_dst[1] = n > 0 ? rm + 32 - n : rm + 32;           // [-a,-n]
+    red_dst[2] = a > 0 ? rm + n : rp + 32;                // [-a, n]
+    red_dst[3] = a > 0 && n > 0 ? rp + 32 - n : rp + 32;  // [+a,-n]
+  }
+  auto reduce = [&]() {
     float4 s0 = make_float4(0.f, 0.f, 0.f, 0.f), s1 = s0;
 #pragma unroll
     for (int c = 0; c < (NA == 1 ? 3 : 4); ++c) {
-      if (c < cmin) continue;
-      const int pos = stage_offset(c) + a * (4 * c + 4) + n;
-      const float4 u0 = stg_p[pos], u1 = stg_m[pos];
+      const float4 u0 = stg_p[red_pos[c]], u1 = stg_m[red_pos[c]];
       s0 = make_float4(s0.x + u0.x, s0.y + u0.y, s0.z + u0.z, s0.w + u0.w);
       s1 = make_float4(s1.x + u1.x, s1.y + u1.y, s1.z + u1.z, s1.w + u1.w);
     }
-    const int rp = a * PITCH, rm = ((32 - a) & 31) * PITCH;
-    work[rp + n] = make_float2(s0.x, s0.y);
-    if (n > 0) work[rm + 32 - n] = make_float2(s0.z, s0.w);
-    if (a > 0) {
-      work[rm + n] = make_float2(s1.x, s1.y);
-      if (n > 0) work[rp + 32 - n] = make_float2(s1.z, s1.w);
-    }
+    work[red_dst[0]] = make_float2(s0.x, s0.y);
+    work[red_dst[1]] = make_float2(s0.z, s0.w);
+    work[red_dst[2]] = make_float2(s1.x, s1.y);
+    work[red_dst[3]] = make_float2(s1.z, s1.w);
     // the bins of m = 16 and n = 16 hold what the last transform left there: cleared again
     if (t < 32) { work[16 * PITCH + t] = make_float2(0.f, 0.f); work[t * PITCH + 16] = make_float2(0.f, 0.f); }
   };

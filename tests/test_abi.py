@@ -62,10 +62,16 @@ def test_argument_rejection_without_gpu():
     assert lib.s2cnn_so3_analysis_workspace(32, 32, 256, 0) == 256 * 28 * 512 * 16 + packed   # one record per volume (7 items x 4 float4 x 512 threads), no intermediate planes
     assert lib.s2cnn_so3_synthesis_workspace(40, 32, 256, 0) == 256 * 28 * 512 * 16 + packed
     packed16 = lib.s2cnn_so3_packed_table_bytes(16, 16, 0)
-    assert packed16 == 31 * 32 * 256 * 4                                            # small problems: 16 x 16 table values per beta
-    assert lib.s2cnn_so3_packed_table_bytes(16, 16, 1) == 31 * 16 * 16 * 32 * 4        # ... and a 16 x 32 tile per degree in the synthesis
+    assert packed16 == 16 * 2 * 2 * 256 * 4 * 4                                      # the 32^3 grid has the same path: 16 beta pairs x 2 items x 2 x 256 threads x 4 degrees
+    assert lib.s2cnn_so3_packed_table_bytes(12, 16, 1) == packed16
+    assert lib.s2cnn_so3_analysis_workspace(16, 16, 256, 0) == 256 * 8 * 256 * 16 + packed16    # records of 2 items x 4 float4 x 256 threads
+    assert lib.s2cnn_so3_synthesis_workspace(20, 16, 256, 0) == 256 * 8 * 256 * 16 + packed16
+    packed12 = lib.s2cnn_so3_packed_table_bytes(12, 12, 0)
+    assert packed12 == 23 * 24 * 256 * 4                                            # small problems of the two-stage path: 16 x 16 table values per beta
+    assert lib.s2cnn_so3_packed_table_bytes(12, 12, 1) == 23 * 12 * 16 * 32 * 4        # ... and a 16 x 32 tile per degree in the synthesis
     assert lib.s2cnn_so3_packed_table_bytes(22, 22, 0) == 43 * 44 * 1024 * 4 and lib.s2cnn_so3_packed_table_bytes(22, 22, 1) == 43 * 22 * 2048 * 4
-    assert lib.s2cnn_so3_analysis_workspace(16, 16, 256, 0) == 256 * 32 * 31 * 16 * 8 + packed16
+    assert lib.s2cnn_so3_analysis_workspace(12, 12, 256, 0) == 256 * 24 * 23 * 12 * 8 + packed12
+    assert lib.s2cnn_so3_relu_bits_bytes(32, 3) == 3 * 64 * 64 * 8 and lib.s2cnn_so3_relu_bits_bytes(16, 3) == 0     # bit masks: the 64^3 grid only
     assert lib.s2cnn_so3_analysis(ctypes.c_void_p(0x1008), fake, fake, fake, null, 0, 32, 32, 1, 0, null) == -3   # 64^3 real input: 16-byte alignment
     assert lib.s2cnn_so3_synthesis_workspace(4, 6, 3, 1) == 16 * 12 * 7 * 7 * 8      # batch padded to the z tile, no fast path
     # more than 32 frequencies / degrees or 64 betas: one packed table per part of the Wigner stage; none beyond 64 / 128
@@ -86,7 +92,8 @@ def test_argument_rejection_without_gpu():
     assert lib.s2cnn_bn_backward_from_moments(fake, 0, 3, 1, 16.0, fake, fake, 1, fake, fake, null) == -1
     # sums per plane out of the synthesis: where it stages whole planes, not on the 64^3 grid
     assert lib.s2cnn_so3_synthesis_moment_parts(22, 22) == 44 and lib.s2cnn_so3_synthesis_moment_parts(7, 22) == 44
-    assert lib.s2cnn_so3_synthesis_moment_parts(16, 16) == 32 and lib.s2cnn_so3_synthesis_moment_parts(32, 32) == 0
+    assert lib.s2cnn_so3_synthesis_moment_parts(12, 12) == 24 and lib.s2cnn_so3_synthesis_moment_parts(32, 32) == 0
+    assert lib.s2cnn_so3_synthesis_moment_parts(16, 16) == 1 and lib.s2cnn_so3_synthesis_moment_parts(10, 16) == 1      # per volume on the 32^3 grid
     assert lib.s2cnn_so3_synthesis_real_moments(fake, fake, null, fake, fake, 1 << 30, 32, 32, 3, null, 1, fake, null, null, null) == -1
     assert lib.s2cnn_so3_synthesis_real_moments(fake, fake, null, fake, fake, 1 << 30, 22, 22, 4, null, 3, fake, fake, fake, null) == -1   # 4 volumes, 3 features
     assert lib.s2cnn_so3_synthesis_real_basis_moment_parts(32, 32, 0) == 1 and lib.s2cnn_so3_synthesis_real_basis_moment_parts(32, 32, 1) == 0

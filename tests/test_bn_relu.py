@@ -68,6 +68,35 @@ def test_sums_formed_by_the_synthesis(hip, b_in, b_out):
     assert mean_err.max().item() < 1e-6 and _rel(mom.double()[:, 1], want[:, 1]) < 2e-5
 
 
+@pytest.mark.parametrize("b_in,b_out", [(16, 16), (9, 16), (12, 12)])
+def test_sums_formed_by_the_synthesis_of_a_complex_spectrum(hip, b_in, b_out):
+    """The same sums from s2cnn_so3_synthesis_real_moments (complex spectrum): per plane on the two-stage path, per volume
+    from the per-volume kernels of the 32^3 grid; both kinds of sums, against float64 sums of the output."""
+    from s2cnn_amd.soft import so3_fft as F
+    parts = F._hip.lib().s2cnn_so3_synthesis_moment_parts(b_in, b_out)
+    assert parts == (1 if b_out == 16 else 2 * b_out)
+    gen = torch.Generator().manual_seed(b_in * 100 + b_out + 3)
+    nspec = b_in * (4 * b_in ** 2 - 1) // 3
+    xh = torch.randn(nspec, 2, 3, 2, generator=gen).cuda()
+    bias = torch.tensor([0.5, -1.0, 2.0]).cuda()
+    mom = torch.full((6 * parts, 2), float("nan")).cuda()
+    y = F.so3_rifft(xh, b_out=b_out, bias=bias, moments=(mom, None, None))
+    assert torch.equal(y, F.so3_rifft(xh, b_out=b_out, bias=bias))
+    yd = y.double().view(6 * parts, -1)
+    want = _sum_and_squared_deviations(yd)
+    mean_err = ((mom.double()[:, 0] - want[:, 0]) / yd.size(1)).abs() / yd.std(-1)
+    assert mean_err.max().item() < 1e-6 and _rel(mom.double()[:, 1], want[:, 1]) < 2e-5
+    w = torch.randn(2, 3, 2 * b_out, 2 * b_out, 2 * b_out, generator=gen).cuda()
+    ab = torch.tensor([[0.7, 1.3, 2.0], [0.1, 0.4, -0.5]]).cuda()
+    mom = torch.full((6 * parts, 2), float("nan")).cuda()
+    g = F.so3_rifft(xh, for_grad=True, b_out=b_out, moments=(mom, w, ab))
+    assert torch.equal(g, F.so3_rifft(xh, for_grad=True, b_out=b_out))
+    m = ab[0].view(1, 3, 1, 1, 1) * w + ab[1].view(1, 3, 1, 1, 1) > 0
+    gm = (g * m).double().view(6, parts, -1)
+    want = torch.stack([gm.sum(-1), (gm * w.double().view(6, parts, -1)).sum(-1)], -1).view(-1, 2)
+    assert (mom.double() - want).abs().max().item() < 2e-5 * want.abs().max().item()
+
+
 @pytest.mark.parametrize("ratio", [100.0, 1000.0])
 @pytest.mark.parametrize("b_in,b_out", [(32, 32), (16, 16), (22, 22), (6, 6)])
 def test_statistics_of_a_signal_with_a_large_mean(hip, b_in, b_out, ratio):
