@@ -20,7 +20,7 @@
 #include "so3_plane_fft64.h"
 #include "so3_wigner_tiled.h"
 #include "so3_fused64.h"
-#include "so3_fused32.h"
+#include "so3_fused4r.h"
 #include "so3_plane_dft_real.h"
 #include <mutex>
 
@@ -296,22 +296,52 @@ __global__ void add_bias_kernel(float* __restrict__ y, const float* __restrict__
   }
 }
 
-// Real signals on the 64^3 and 32^3 grids go through the per-volume kernels of so3_fused64.h / so3_fused32.h (the planes
-// never leave the CU).
-enum FusedKind { FUSED_NONE = 0, FUSED_64, FUSED_32 };
+// Real signals on the 64^3, 44^3 and 32^3 grids go through the per-volume kernels of so3_fused64.h / so3_fused4r.h (the
+// planes never leave the CU).
+using fused4r::Grid32;
+using fused4r::Grid44;
+enum FusedKind { FUSED_NONE = 0, FUSED_64, FUSED_44, FUSED_32 };
+int fused_bandwidth(FusedKind k) { return k == FUSED_64 ? 32 : k == FUSED_44 ? 22 : 16; }
 FusedKind fused_kind(int b_grid, int b_spec, int cplx, bool synthesis) {
   if (cplx) return FUSED_NONE;
-  if (b_grid == 32 && (synthesis || b_spec <= 32)) return FUSED_64;
-  if (b_grid == 16 && (synthesis || b_spec <= 16)) return FUSED_32;
-  return FUSED_NONE;
+  const FusedKind k = b_grid == 32 ? FUSED_64 : b_grid == 22 ? FUSED_44 : b_grid == 16 ? FUSED_32 : FUSED_NONE;
+  return synthesis || b_spec <= b_grid ? k : FUSED_NONE;
 }
 bool fused_path(int b_grid, int b_spec, int cplx, bool synthesis) { return fused_kind(b_grid, b_spec, cplx, synthesis) != FUSED_NONE; }
-size_t fused_scratch_bytes(FusedKind k, long nbatch) { return k == FUSED_64 ? fused64::scratch_bytes(nbatch) : fused32::scratch_bytes(nbatch); }
-size_t fused_packed_floats(FusedKind k) { return k == FUSED_64 ? fused64::PACKED_FLOATS : fused32::PACKED_FLOATS; }
+size_t fused_scratch_bytes(FusedKind k, long nbatch) {
+  return k == FUSED_64 ? fused64::scratch_bytes(nbatch) : k == FUSED_44 ? Grid44::scratch_bytes(nbatch) : Grid32::scratch_bytes(nbatch);
+}
+size_t fused_packed_floats(FusedKind k) { return k == FUSED_64 ? fused64::PACKED_FLOATS : k == FUSED_44 ? Grid44::PACKED_FLOATS : Grid32::PACKED_FLOATS; }
 // table [2 b_grid][nspec(b_spec)] -> the packed table of the per-volume kernels, degrees below nl
 void fused_pack_table(FusedKind k, hipStream_t st, const float* table, float* packed, int b_spec, int nl) {
-  if (k == FUSED_64) hipLaunchKernelGGL(fused64::pack_table, dim3(1024), dim3(256), 0, st, table, packed, s2cnn::so3_nspec(b_spec), nl);
-  else hipLaunchKernelGGL(fused32::pack_table, dim3(256), dim3(256), 0, st, table, packed, s2cnn::so3_nspec(b_spec), nl);
+  const long stride = s2cnn::so3_nspec(b_spec);
+  if (k == FUSED_64) hipLaunchKernelGGL(fused64::pack_table, dim3(1024), dim3(256), 0, st, table, packed, stride, nl);
+  else if (k == FUSED_44) hipLaunchKernelGGL(fused4r::pack_table<Grid44>, dim3(512), dim3(256), 0, st, table, packed, stride, nl);
+  else hipLaunchKernelGGL(fused4r::pack_table<Grid32>, dim3(256), dim3(256), 0, st, table, packed, stride, nl);
+}
+// per-volume kernel + the pass between its records and the spectral rows, for the grids of so3_fused4r.h
+template <class G>
+void fused4r_analysis(const s2cnn::Input& in, const float* Tf, float4* rec, float* out, int b_out, long nbatch, bool real_basis, hipStream_t st) {
+  const unsigned tiles_r = (unsigned)((nbatch + fused64::ZR - 1) / fused64::ZR), tiles_c = (unsigned)((nbatch + fused64::ZT - 1) / fused64::ZT);
+  const int rounds = G::active_rounds(b_out);
+  fused4r::launch_analysis<G>(b_out, st, in, Tf, rec, nbatch);
+  if (real_basis)
+    hipLaunchKernelGGL(fused64::spectrum_scatter_real<G>, dim3(tiles_r, rounds * (G::THREADS / fused64::IT_TILE_R)), dim3(256), 0, st, rec, out, b_out, nbatch);
+  else
+    hipLaunchKernelGGL(fused64::spectrum_scatter<G>, dim3(tiles_c, rounds * (G::THREADS / fused64::IT_TILE)), dim3(256), 0, st, rec,
+                       reinterpret_cast<float2*>(out), b_out, nbatch);
+}
+template <class G>
+void fused4r_synthesis(const float* xhat, const float* Tf, float4* rec, float* out, int nl, long nbatch, bool real_basis, const float* bias,
+                       int nfeature, int relu, hipStream_t st, float2* mom, const float* yref, const float* params) {
+  const unsigned tiles_r = (unsigned)((nbatch + fused64::ZR - 1) / fused64::ZR), tiles_c = (unsigned)((nbatch + fused64::ZT - 1) / fused64::ZT);
+  const int rounds = G::active_rounds(nl);
+  if (real_basis)
+    hipLaunchKernelGGL(fused64::spectrum_gather_real<G>, dim3(tiles_r, rounds * (G::THREADS / fused64::IT_TILE_R)), dim3(256), 0, st, xhat, rec, nl, nbatch);
+  else
+    hipLaunchKernelGGL(fused64::spectrum_gather<G>, dim3(tiles_c, rounds * (G::THREADS / fused64::IT_TILE)), dim3(256), 0, st,
+                       reinterpret_cast<const float2*>(xhat), rec, nl, nbatch);
+  fused4r::launch_synthesis<G>(nl, st, rec, Tf, out, nbatch, bias, nfeature, relu, mom, yref, params);
 }
 
 // Bytes of the intermediate; batch items padded to the z tile of the tiled Wigner kernels.
@@ -371,13 +401,10 @@ int fused_analysis(FusedKind kind, const s2cnn::Input& in, const float* table, c
     fused64::launch_analysis(b_out, st, in, Tf, rec, nbatch);
     if (real_basis) hipLaunchKernelGGL(fused64::spectrum_scatter_real<>, dim3(tiles_r, rounds * 32), dim3(256), 0, st, rec, out, b_out, nbatch);
     else hipLaunchKernelGGL(fused64::spectrum_scatter<>, dim3(tiles_c, rounds * 16), dim3(256), 0, st, rec, outc, b_out, nbatch);
+  } else if (kind == FUSED_44) {
+    fused4r_analysis<Grid44>(in, Tf, rec, out, b_out, nbatch, real_basis, st);
   } else {
-    const int rounds = fused32::active_rounds(b_out);
-    fused32::launch_analysis(b_out, st, in, Tf, rec, nbatch);
-    if (real_basis)
-      hipLaunchKernelGGL(fused64::spectrum_scatter_real<fused32::Geometry>, dim3(tiles_r, rounds * 16), dim3(256), 0, st, rec, out, b_out, nbatch);
-    else
-      hipLaunchKernelGGL(fused64::spectrum_scatter<fused32::Geometry>, dim3(tiles_c, rounds * 8), dim3(256), 0, st, rec, outc, b_out, nbatch);
+    fused4r_analysis<Grid32>(in, Tf, rec, out, b_out, nbatch, real_basis, st);
   }
   return s2cnn::launch_status();
 }
@@ -388,7 +415,7 @@ int fused_synthesis(FusedKind kind, const float* xhat, const float* table, const
                     const float* params = nullptr) {
   if (!s2cnn::aligned16(out) || !s2cnn::aligned16(bits) || !s2cnn::aligned8(moments) || !s2cnn::aligned16(yref)) return S2CNN_EALIGN;
   if (bits && kind != FUSED_64) return S2CNN_EINVAL;
-  const int b_grid = kind == FUSED_64 ? 32 : 16;
+  const int b_grid = fused_bandwidth(kind);
   const int nl = b_in < b_grid ? b_in : b_grid;
   const size_t need = round256(fused_scratch_bytes(kind, nbatch)) + fused_packed_floats(kind) * sizeof(float);
   if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
@@ -407,11 +434,10 @@ int fused_synthesis(FusedKind kind, const float* xhat, const float* table, const
     if (real_basis) hipLaunchKernelGGL(fused64::spectrum_gather_real<>, dim3(tiles_r, rounds * 32), dim3(256), 0, st, xhat, rec, nl, nbatch);
     else hipLaunchKernelGGL(fused64::spectrum_gather<>, dim3(tiles_c, rounds * 16), dim3(256), 0, st, xc, rec, nl, nbatch);
     fused64::launch_synthesis(nl, st, rec, Tf, out, nbatch, bias, nfeature, relu, bits, mom, yref, params);
+  } else if (kind == FUSED_44) {
+    fused4r_synthesis<Grid44>(xhat, Tf, rec, out, nl, nbatch, real_basis, bias, nfeature, relu, st, mom, yref, params);
   } else {
-    const int rounds = fused32::active_rounds(nl);
-    if (real_basis) hipLaunchKernelGGL(fused64::spectrum_gather_real<fused32::Geometry>, dim3(tiles_r, rounds * 16), dim3(256), 0, st, xhat, rec, nl, nbatch);
-    else hipLaunchKernelGGL(fused64::spectrum_gather<fused32::Geometry>, dim3(tiles_c, rounds * 8), dim3(256), 0, st, xc, rec, nl, nbatch);
-    fused32::launch_synthesis(nl, st, rec, Tf, out, nbatch, bias, nfeature, relu, mom, yref, params);
+    fused4r_synthesis<Grid32>(xhat, Tf, rec, out, nl, nbatch, real_basis, bias, nfeature, relu, st, mom, yref, params);
   }
   return s2cnn::launch_status();
 }
@@ -561,7 +587,7 @@ struct PlaneMoments {
 int moment_parts(int b_in, int b_out) {
   if (!sizes_ok(b_out, b_in, 1)) return 0;
   const FusedKind k = fused_kind(b_out, b_in, 0, true);
-  if (k == FUSED_32) return 1;
+  if (k == FUSED_32 || k == FUSED_44) return 1;
   if (k != FUSED_NONE || 2 * b_out == 64) return 0;
   const plane_real::Plan plan = plane_real::plan_inv(2 * b_out, b_in < b_out ? b_in : b_out, 2 * b_out);
   return plan.pl > 0 && plan.alias ? 2 * b_out : 0;
@@ -750,7 +776,7 @@ extern "C" int s2cnn_so3_synthesis_real_basis_moment_parts(int b_in, int b_out, 
   if (!sizes_ok(b_out, b_in, 1) || !real_basis_synthesis(b_in, b_out)) return 0;
   const FusedKind k = fused_kind(b_out, b_in, 0, true);
   if (k == FUSED_NONE) return moment_parts(b_in, b_out);
-  return !grad || k == FUSED_32 || b_in <= fused64::GRAD_MOMENTS_MAX_NL ? 1 : 0;
+  return !grad || k != FUSED_64 || b_in <= fused64::GRAD_MOMENTS_MAX_NL ? 1 : 0;
 }
 
 extern "C" int s2cnn_so3_synthesis_real_basis_moments(const float* r, const float* table, const float* packed_table, float* out,

@@ -69,7 +69,9 @@ def test_argument_rejection_without_gpu():
     packed12 = lib.s2cnn_so3_packed_table_bytes(12, 12, 0)
     assert packed12 == 23 * 24 * 256 * 4                                            # small problems of the two-stage path: 16 x 16 table values per beta
     assert lib.s2cnn_so3_packed_table_bytes(12, 12, 1) == 23 * 12 * 16 * 32 * 4        # ... and a 16 x 32 tile per degree in the synthesis
-    assert lib.s2cnn_so3_packed_table_bytes(22, 22, 0) == 43 * 44 * 1024 * 4 and lib.s2cnn_so3_packed_table_bytes(22, 22, 1) == 43 * 22 * 2048 * 4
+    assert lib.s2cnn_so3_packed_table_bytes(22, 22, 0) == 22 * 3 * 2 * 512 * 4 * 4 == lib.s2cnn_so3_packed_table_bytes(7, 22, 1)     # and the 44^3 grid: 22 beta pairs x 3 items x 2 x 512 threads
+    assert lib.s2cnn_so3_analysis_workspace(22, 7, 10, 0) == 10 * 12 * 512 * 16 + 22 * 3 * 2 * 512 * 4 * 4
+    assert lib.s2cnn_so3_packed_table_bytes(20, 20, 0) == 39 * 40 * 1024 * 4 and lib.s2cnn_so3_packed_table_bytes(20, 20, 1) == 39 * 20 * 2048 * 4
     assert lib.s2cnn_so3_analysis_workspace(12, 12, 256, 0) == 256 * 24 * 23 * 12 * 8 + packed12
     assert lib.s2cnn_so3_relu_bits_bytes(32, 3) == 3 * 64 * 64 * 8 and lib.s2cnn_so3_relu_bits_bytes(16, 3) == 0     # bit masks: the 64^3 grid only
     assert lib.s2cnn_so3_analysis(ctypes.c_void_p(0x1008), fake, fake, fake, null, 0, 32, 32, 1, 0, null) == -3   # 64^3 real input: 16-byte alignment
@@ -91,13 +93,15 @@ def test_argument_rejection_without_gpu():
     assert lib.s2cnn_bn_forward_from_moments(fake, 2, 3, 1, 16.0, null, null, null, null, 1e-5, 0.1, 0, fake, fake, null) == -1   # evaluation mode without running statistics
     assert lib.s2cnn_bn_backward_from_moments(fake, 0, 3, 1, 16.0, fake, fake, 1, fake, fake, null) == -1
     # sums per plane out of the synthesis: where it stages whole planes, not on the 64^3 grid
-    assert lib.s2cnn_so3_synthesis_moment_parts(22, 22) == 44 and lib.s2cnn_so3_synthesis_moment_parts(7, 22) == 44
+    assert lib.s2cnn_so3_synthesis_moment_parts(20, 20) == 40 and lib.s2cnn_so3_synthesis_moment_parts(7, 20) == 40
     assert lib.s2cnn_so3_synthesis_moment_parts(12, 12) == 24 and lib.s2cnn_so3_synthesis_moment_parts(32, 32) == 0
     assert lib.s2cnn_so3_synthesis_moment_parts(16, 16) == 1 and lib.s2cnn_so3_synthesis_moment_parts(10, 16) == 1      # per volume on the 32^3 grid
+    assert lib.s2cnn_so3_synthesis_moment_parts(22, 22) == 1 and lib.s2cnn_so3_synthesis_moment_parts(7, 22) == 1       # ... and on the 44^3 grid
     assert lib.s2cnn_so3_synthesis_real_moments(fake, fake, null, fake, fake, 1 << 30, 32, 32, 3, null, 1, fake, null, null, null) == -1
     assert lib.s2cnn_so3_synthesis_real_moments(fake, fake, null, fake, fake, 1 << 30, 22, 22, 4, null, 3, fake, fake, fake, null) == -1   # 4 volumes, 3 features
     assert lib.s2cnn_so3_synthesis_real_basis_moment_parts(32, 32, 0) == 1 and lib.s2cnn_so3_synthesis_real_basis_moment_parts(32, 32, 1) == 0
-    assert lib.s2cnn_so3_synthesis_real_basis_moment_parts(22, 32, 1) == 1 and lib.s2cnn_so3_synthesis_real_basis_moment_parts(22, 22, 0) == 44
+    assert lib.s2cnn_so3_synthesis_real_basis_moment_parts(22, 32, 1) == 1 and lib.s2cnn_so3_synthesis_real_basis_moment_parts(20, 20, 0) == 40
+    assert lib.s2cnn_so3_synthesis_real_basis_moment_parts(22, 22, 0) == 1 and lib.s2cnn_so3_synthesis_real_basis_moment_parts(22, 22, 1) == 1
     assert lib.s2cnn_so3_synthesis_real_basis_moment_parts(70, 70, 0) == 0
     assert lib.s2cnn_so3_synthesis_real_basis_moments(fake, fake, null, fake, fake, 1 << 30, 70, 70, 3, null, 1, fake, null, null, null) == -1    # no tiled stage at this size
     assert lib.s2cnn_so3_synthesis_real_basis_moments(fake, fake, null, fake, fake, 1 << 30, 32, 32, 3, null, 1, null, null, null, null) == -1    # nowhere to write the sums

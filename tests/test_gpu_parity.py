@@ -74,7 +74,7 @@ def test_s2_mm_forward_backward(hip, nl, B, Fi, Fo):
 
 
 # ------------------------------------------------------------------ SO(3) transforms
-SO3_PAIRS = [(2, 9), (6, 6), (9, 2), (10, 11), (11, 10), (7, 5), (4, 6), (16, 16), (16, 10), (20, 16), (32, 32), (32, 12), (12, 32)]   # first five: tests/so3_fft.py:102
+SO3_PAIRS = [(2, 9), (6, 6), (9, 2), (10, 11), (11, 10), (7, 5), (4, 6), (16, 16), (16, 10), (20, 16), (22, 22), (22, 18), (32, 32), (32, 12), (12, 32)]   # first five: tests/so3_fft.py:102
 
 
 @pytest.mark.parametrize("b_in,b_out", SO3_PAIRS)
@@ -128,32 +128,32 @@ def test_so3_one_kernel_path_batches(hip, nz):
             close(PSO3.so3_rifft(s.cuda(), for_grad, 32), O.so3_rifft(s.double(), for_grad, 32), f"rifft {b_spec}->32 for_grad={for_grad}")
 
 
-@pytest.mark.parametrize("nz", [1, 9, 20])
-def test_so3_one_kernel_path_of_the_32_grid(hip, nz):
-    """Real signals on the 32^3 grid have per-volume kernels of their own (256 threads per volume, two item rounds): batch
-    sizes that leave XCD slots empty, spectra that skip the second round (below degree 12) and over-long ones, both tables;
-    repeated calls agree bit for bit, and a truncated spectrum gives what its zero-extended form gives."""
+@pytest.mark.parametrize("b,nz", [(16, 1), (16, 9), (16, 20), (22, 1), (22, 9), (22, 20)])
+def test_so3_one_kernel_path_of_the_32_and_44_grids(hip, b, nz):
+    """Real signals on the 32^3 and 44^3 grids have per-volume kernels of their own (a line of 4 x 8 or 4 x 11 points, two
+    or three item rounds): batch sizes that leave XCD slots empty, spectra that skip the later rounds and over-long ones,
+    both tables; repeated calls agree bit for bit, and a truncated spectrum gives what its zero-extended form gives."""
     from s2cnn_amd.soft.so3_fft import so3_rifft_real_basis, so3_rfft_real_basis
-    print(f"so3 one-kernel path of the 32 grid nz={nz}", flush=True)
-    x = rnd((nz, 32, 32, 32), 150 + nz)
+    print(f"so3 one-kernel path of the {2 * b}^3 grid nz={nz}", flush=True)
+    x = rnd((nz, 2 * b, 2 * b, 2 * b), 150 + nz)
     for for_grad in (False, True):
-        for b_out in (16, 13, 12, 7, 1):
-            close(PSO3.so3_rfft(x.cuda(), for_grad, b_out), O.so3_rfft(x.double(), for_grad, b_out), f"rfft 16->{b_out} for_grad={for_grad}")
-        for b_spec in (16, 12, 9, 19, 1):
+        for b_out in (b, b - 3, b - 4, 7, 1):
+            close(PSO3.so3_rfft(x.cuda(), for_grad, b_out), O.so3_rfft(x.double(), for_grad, b_out), f"rfft {b}->{b_out} for_grad={for_grad}")
+        for b_spec in (b, b - 4, 9, b + 3, 1):
             s = rnd((O.nspec_so3(b_spec), nz, 2), 160 + b_spec)
-            close(PSO3.so3_rifft(s.cuda(), for_grad, 16), O.so3_rifft(s.double(), for_grad, 16), f"rifft {b_spec}->16 for_grad={for_grad}")
+            close(PSO3.so3_rifft(s.cuda(), for_grad, b), O.so3_rifft(s.double(), for_grad, b), f"rifft {b_spec}->{b} for_grad={for_grad}")
     xg = x.cuda()
     bias = rnd((1,), 170).cuda()
-    for b in (16, 10):
-        r = rnd((O.nspec_so3(b), nz, 1), 171 + b).cuda()
-        a1, y1 = so3_rfft_real_basis(xg, b_out=b), so3_rifft_real_basis(r, b_out=16, bias=bias)
+    for bs in (b, b - 6):
+        r = rnd((O.nspec_so3(bs), nz, 1), 171 + bs).cuda()
+        a1, y1 = so3_rfft_real_basis(xg, b_out=bs), so3_rifft_real_basis(r, b_out=b, bias=bias)
         for _ in range(3):
-            assert torch.equal(so3_rfft_real_basis(xg, b_out=b), a1)
-            assert torch.equal(so3_rifft_real_basis(r, b_out=16, bias=bias), y1)
-        rz = torch.zeros(O.nspec_so3(16), nz, 1, device="cuda")
+            assert torch.equal(so3_rfft_real_basis(xg, b_out=bs), a1)
+            assert torch.equal(so3_rifft_real_basis(r, b_out=b, bias=bias), y1)
+        rz = torch.zeros(O.nspec_so3(b), nz, 1, device="cuda")
         rz[:r.size(0)] = r
-        close(y1, so3_rifft_real_basis(rz, b_out=16, bias=bias).cpu().double(), f"synthesis from {b} degrees")
-        close(a1, so3_rfft_real_basis(xg, b_out=16)[:a1.size(0)].cpu().double(), f"analysis to {b} degrees")
+        close(y1, so3_rifft_real_basis(rz, b_out=b, bias=bias).cpu().double(), f"synthesis from {bs} degrees")
+        close(a1, so3_rfft_real_basis(xg, b_out=b)[:a1.size(0)].cpu().double(), f"analysis to {bs} degrees")
 
 
 def test_so3_one_kernel_path_is_reproducible(hip):
@@ -186,7 +186,7 @@ def test_so3_one_kernel_path_is_reproducible(hip):
 def test_so3_transforms_without_prepacked_table(hip):
     """packed_table = NULL (the library repacks into its workspace) gives the same bits as the prepacked path."""
     from s2cnn_amd import _hip
-    for b_in, b_out in [(32, 32), (16, 16), (16, 9), (10, 6)]:
+    for b_in, b_out in [(32, 32), (16, 16), (16, 9), (22, 22), (22, 13), (10, 6)]:
         nz = 5
         x = rnd((nz, 2 * b_in, 2 * b_in, 2 * b_in), 17).cuda()
         want = PSO3.so3_rfft(x, b_out=b_out)
@@ -397,6 +397,7 @@ def test_s2_convolution_parity(hip, real_basis):
                                               (32, 22, 6, 3), (32, 26, 2, 1),   # their truncated instantiations
                                               (10, 32, 6, 3),     # synthesis onto the 64^3 grid from a short spectrum
                                               (16, 16, 4, 2), (16, 10, 6, 3), (10, 16, 6, 3), (16, 18, 2, 1),   # the per-volume kernels of the 32^3 grid
+                                              (22, 22, 4, 2), (22, 18, 2, 1), (12, 22, 6, 3), (22, 24, 2, 1),   # ... and of the 44^3 grid
                                               (32, 34, 2, 1),     # 64-point plane kernel + Wigner stage
                                               (22, 7, 6, 2), (6, 6, 10, 5), (5, 9, 3, 1), (11, 4, 2, 1),   # folded plane kernels
                                               (36, 36, 2, 1), (40, 33, 2, 2)])   # ... with the Wigner stage in parts
