@@ -116,8 +116,14 @@ __device__ __forceinline__ void dft_r(float2 (&v)[R], Emit emit) {
 
 // The grid of N = 4 R points per axis and how a workgroup of T threads (a power of two) is laid over it;
 // W = waves per SIMD the kernels are compiled for (workgroups per compute unit x T / 256).
-template <int R_, int T, int W>
+// LATE: the analysis issues the loads of the next plane pair after the transform of the current one instead of before it
+// (fewer registers held through the transform, less time for the loads).
+// DMA: those loads go straight to LDS (buffer loads with the lds bit: lane i of a wave writes word i of a 256-byte row of
+// its own), so no registers hold them while they are in flight; a wave waits for its own loads and reads back its own rows.
+template <int R_, int T, int W, bool LATE_ = false, bool DMA_ = false>
 struct Grid {
+  static constexpr bool LATE = LATE_;
+  static constexpr bool DMA = DMA_;
   static constexpr int R = R_;
   static constexpr int N = 4 * R;
   static constexpr int H = N / 2;               // bandwidth: frequencies 0 <= a, n < H; also the number of beta pairs
@@ -164,8 +170,8 @@ struct Grid {
   }
 };
 
-using Grid32 = Grid<8, 256, 4>;        // 32^3: four workgroups per compute unit
-using Grid44 = Grid<11, 512, 4>;       // 44^3: two
+using Grid32 = Grid<8, 256, 4>;                    // 32^3: four workgroups per compute unit, plane loads through registers
+using Grid44 = Grid<11, 512, 4, false, true>;       // 44^3: two (one, with all the registers it wants, is slower)
 
 // Packed table, as fused64::pack_table: float index ((((j*NIT + it)*2 + h)*THREADS + t)*4 + u) holds
 // 0.5 * T[j, l = 4c+u, m = (h ? -a : +a), n] for the item of place it*THREADS + t.  T is [N][nspec_stride].
@@ -282,9 +288,28 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void analysis_kernel
   const unsigned toff = t * 16;
   float pa[4], pb[4];
   float ma[MASKED ? 4 : 1], mb[MASKED ? 4 : 1];
-  float4 t1[NA], t2[NA];
+  // DMA: [tensor][plane][j1][thread] words, filled by the loads themselves
+  __shared__ __attribute__((aligned(16))) float landing[G::DMA ? (MASKED ? 16 : 8) * THREADS : 1];
+  const int wave_first = __builtin_amdgcn_readfirstlane(t & ~63);       // first thread of this wave
+  // table registers: item it in slot it % SLOTS; a slot is refilled when its item is done.  With the plane loads going to
+  // LDS there are registers for all items, and no table load queues up behind the plane loads.
+  constexpr int SLOTS = G::DMA || NA < 2 ? NA : 2;
+  float4 t1[SLOTS], t2[SLOTS];
 
   auto load_planes = [&](int j) {        // rows R j1 + d of the planes j and N-1-j: contiguous over the workgroup
+    if constexpr (G::DMA) {
+      typedef __attribute__((address_space(3))) void* lds_ptr;
+#pragma unroll
+      for (int j1 = 0; j1 < 4; ++j1) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr)(landing + (0 + j1) * THREADS + wave_first), 4, (int)xoff, (j * N * N + j1 * R * N) * 4, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr)(landing + (4 + j1) * THREADS + wave_first), 4, (int)xoff, ((N - 1 - j) * N * N + j1 * R * N) * 4, 0, 0);
+        if constexpr (MASKED) {
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rm, (lds_ptr)(landing + (8 + j1) * THREADS + wave_first), 4, (int)xoff, (j * N * N + j1 * R * N) * 4, 0, 0);
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rm, (lds_ptr)(landing + (12 + j1) * THREADS + wave_first), 4, (int)xoff, ((N - 1 - j) * N * N + j1 * R * N) * 4, 0, 0);
+        }
+      }
+      return;
+    }
 #pragma unroll
     for (int j1 = 0; j1 < 4; ++j1) {
       pa[j1] = buf_load_f32(rx, xoff, (j * N * N + j1 * R * N) * 4);
@@ -295,16 +320,23 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void analysis_kernel
       }
     }
   };
-  auto load_table = [&](int j) {
-#pragma unroll
-    for (int it = 0; it < NA; ++it) {
-      t1[it] = buf_load_f32x4(rt, toff, ((j * NIT + it) * 2 + 0) * (THREADS * 16));
-      t2[it] = buf_load_f32x4(rt, toff, ((j * NIT + it) * 2 + 1) * (THREADS * 16));
-    }
+  auto load_table = [&](int j, int it) {
+    t1[it % SLOTS] = buf_load_f32x4(rt, toff, ((j * NIT + it) * 2 + 0) * (THREADS * 16));
+    t2[it % SLOTS] = buf_load_f32x4(rt, toff, ((j * NIT + it) * 2 + 1) * (THREADS * 16));
   };
   // pass A of the alpha axis out of the registers: 4-point transforms over j1, twiddle, -> work[R k1 + d][lo]
   auto stage_c1 = [&]() {
     float2 v[4];
+    if constexpr (G::DMA) {        // this wave's loads have landed (vmcnt = 0), then its own words are read back
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int j1 = 0; j1 < 4; ++j1) {
+        pa[j1] = landing[(0 + j1) * THREADS + t];
+        pb[j1] = landing[(4 + j1) * THREADS + t];
+        if constexpr (MASKED) { ma[j1] = landing[(8 + j1) * THREADS + t]; mb[j1] = landing[(12 + j1) * THREADS + t]; }
+      }
+    }
 #pragma unroll
     for (int j1 = 0; j1 < 4; ++j1) {
       if constexpr (MASK == 1) v[j1] = make_float2(s2cnn::relu_pass(pa[j1], ma[j1]), s2cnn::relu_pass(pb[j1], mb[j1]));
@@ -350,8 +382,8 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void analysis_kernel
     const float2 Qp = make_float2(flip(za.y + za.w, sb), flip(za.z - za.x, sb));
     const float2 Pm = make_float2(zb.x + zb.z, zb.y - zb.w);
     const float2 Qm = make_float2(flip(zb.y + zb.w, sb), flip(zb.z - zb.x, sb));
-    const float a1[4] = {t1[it].x, t1[it].y, t1[it].z, t1[it].w};
-    const float a2[4] = {t2[it].x, t2[it].y, t2[it].z, t2[it].w};
+    const float a1[4] = {t1[it % SLOTS].x, t1[it % SLOTS].y, t1[it % SLOTS].z, t1[it % SLOTS].w};
+    const float a2[4] = {t2[it % SLOTS].x, t2[it % SLOTS].y, t2[it % SLOTS].z, t2[it % SLOTS].w};
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       // (-1)^(l-n) = (-1)^u (-1)^n for l = 4c+u: the sign of odd u goes into the table operand
@@ -363,21 +395,36 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void analysis_kernel
     }
   };
 
-  load_planes(0);
+  // The barriers of a step order LDS accesses only.  With loads on their way to LDS, __syncthreads() would wait for them
+  // too (its fence covers every write to LDS): there the barrier is taken once this wave's own LDS accesses are done.
+  auto step_barrier = [&]() {
+    if constexpr (G::DMA) {
+      __builtin_amdgcn_s_waitcnt(0xC07F);           // lgkmcnt(0)
+      __builtin_amdgcn_s_barrier();
+    } else {
+      __syncthreads();
+    }
+  };
   __syncthreads();                                  // cleared quads
+  load_planes(0);
   for (int j = 0; j < NJ; ++j) {
     stage_c1();
-    load_planes(j + 1 < NJ ? j + 1 : NJ - 1);       // clamped, not branched: in flight during the step
-    __syncthreads();
+    if constexpr (!G::LATE) { __builtin_amdgcn_sched_barrier(0); load_planes(j + 1 < NJ ? j + 1 : NJ - 1); }      // clamped, not branched: in flight during the step
+    step_barrier();
     if (t >= G::B_COLS_FIRST && t < G::B_COLS_FIRST + G::B_THREADS) pass_b<G, false, false>(work, t - G::B_COLS_FIRST);
-    __syncthreads();
+    step_barrier();
     pass_a<G, false, true>(work, tw, lo, d);
-    __syncthreads();
+    step_barrier();
     if (t < G::B_THREADS) stage_r2();
-    load_table(j);                                  // only now: its registers are not held through the transform
-    __syncthreads();
 #pragma unroll
-    for (int it = 0; it < NA; ++it) accumulate(it);
+    for (int it = 0; it < SLOTS; ++it) load_table(j, it);     // only now: their registers are not held through the transform
+    if constexpr (G::LATE) load_planes(j + 1 < NJ ? j + 1 : NJ - 1);
+    step_barrier();
+#pragma unroll
+    for (int it = 0; it < NA; ++it) {
+      accumulate(it);
+      if (it + SLOTS < NA) { __builtin_amdgcn_sched_barrier(0); load_table(j, it + SLOTS); __builtin_amdgcn_sched_barrier(0); }
+    }
   }
 
   const __amdgpu_buffer_rsrc_t rr = make_rsrc(rec + (size_t)z * G::REC_F4, (unsigned)G::REC_BYTES);
