@@ -296,28 +296,43 @@ __global__ void add_bias_kernel(float* __restrict__ y, const float* __restrict__
   }
 }
 
-// Real signals on the 64^3, 44^3 and 32^3 grids go through the per-volume kernels of so3_fused64.h / so3_fused4r.h (the
-// planes never leave the CU).
+// Real signals on the 64^3, 44^3, 32^3 and 20^3 grids go through the per-volume kernels of so3_fused64.h / so3_fused4r.h
+// (the planes never leave the CU).
+using fused4r::Grid20;
 using fused4r::Grid32;
 using fused4r::Grid44;
-enum FusedKind { FUSED_NONE = 0, FUSED_64, FUSED_44, FUSED_32 };
-int fused_bandwidth(FusedKind k) { return k == FUSED_64 ? 32 : k == FUSED_44 ? 22 : 16; }
+enum FusedKind { FUSED_NONE = 0, FUSED_64, FUSED_44, FUSED_32, FUSED_20 };
+int fused_bandwidth(FusedKind k) { return k == FUSED_64 ? 32 : k == FUSED_44 ? 22 : k == FUSED_32 ? 16 : 10; }
 FusedKind fused_kind(int b_grid, int b_spec, int cplx, bool synthesis) {
   if (cplx) return FUSED_NONE;
-  const FusedKind k = b_grid == 32 ? FUSED_64 : b_grid == 22 ? FUSED_44 : b_grid == 16 ? FUSED_32 : FUSED_NONE;
+  const FusedKind k = b_grid == 32 ? FUSED_64 : b_grid == 22 ? FUSED_44 : b_grid == 16 ? FUSED_32 : b_grid == 10 ? FUSED_20 : FUSED_NONE;
   return synthesis || b_spec <= b_grid ? k : FUSED_NONE;
 }
 bool fused_path(int b_grid, int b_spec, int cplx, bool synthesis) { return fused_kind(b_grid, b_spec, cplx, synthesis) != FUSED_NONE; }
-size_t fused_scratch_bytes(FusedKind k, long nbatch) {
-  return k == FUSED_64 ? fused64::scratch_bytes(nbatch) : k == FUSED_44 ? Grid44::scratch_bytes(nbatch) : Grid32::scratch_bytes(nbatch);
+// f.template operator()<G>() for the grid G of a kind other than FUSED_64
+template <class F>
+auto with_grid(FusedKind k, F f) {
+  if (k == FUSED_44) return f(Grid44{});
+  if (k == FUSED_32) return f(Grid32{});
+  return f(Grid20{});
 }
-size_t fused_packed_floats(FusedKind k) { return k == FUSED_64 ? fused64::PACKED_FLOATS : k == FUSED_44 ? Grid44::PACKED_FLOATS : Grid32::PACKED_FLOATS; }
+size_t fused_scratch_bytes(FusedKind k, long nbatch) {
+  if (k == FUSED_64) return fused64::scratch_bytes(nbatch);
+  return with_grid(k, [&](auto g) { return decltype(g)::scratch_bytes(nbatch); });
+}
+size_t fused_packed_floats(FusedKind k) {
+  if (k == FUSED_64) return fused64::PACKED_FLOATS;
+  return with_grid(k, [](auto g) { return (size_t) decltype(g)::PACKED_FLOATS; });
+}
 // table [2 b_grid][nspec(b_spec)] -> the packed table of the per-volume kernels, degrees below nl
 void fused_pack_table(FusedKind k, hipStream_t st, const float* table, float* packed, int b_spec, int nl) {
   const long stride = s2cnn::so3_nspec(b_spec);
-  if (k == FUSED_64) hipLaunchKernelGGL(fused64::pack_table, dim3(1024), dim3(256), 0, st, table, packed, stride, nl);
-  else if (k == FUSED_44) hipLaunchKernelGGL(fused4r::pack_table<Grid44>, dim3(512), dim3(256), 0, st, table, packed, stride, nl);
-  else hipLaunchKernelGGL(fused4r::pack_table<Grid32>, dim3(256), dim3(256), 0, st, table, packed, stride, nl);
+  if (k == FUSED_64) { hipLaunchKernelGGL(fused64::pack_table, dim3(1024), dim3(256), 0, st, table, packed, stride, nl); return; }
+  with_grid(k, [&](auto g) {
+    using G = decltype(g);
+    hipLaunchKernelGGL(fused4r::pack_table<G>, dim3((unsigned)((G::PACKED_FLOATS + 1023) / 1024)), dim3(256), 0, st, table, packed, stride, nl);
+    return 0;
+  });
 }
 // per-volume kernel + the pass between its records and the spectral rows, for the grids of so3_fused4r.h
 template <class G>
@@ -401,10 +416,8 @@ int fused_analysis(FusedKind kind, const s2cnn::Input& in, const float* table, c
     fused64::launch_analysis(b_out, st, in, Tf, rec, nbatch);
     if (real_basis) hipLaunchKernelGGL(fused64::spectrum_scatter_real<>, dim3(tiles_r, rounds * 32), dim3(256), 0, st, rec, out, b_out, nbatch);
     else hipLaunchKernelGGL(fused64::spectrum_scatter<>, dim3(tiles_c, rounds * 16), dim3(256), 0, st, rec, outc, b_out, nbatch);
-  } else if (kind == FUSED_44) {
-    fused4r_analysis<Grid44>(in, Tf, rec, out, b_out, nbatch, real_basis, st);
   } else {
-    fused4r_analysis<Grid32>(in, Tf, rec, out, b_out, nbatch, real_basis, st);
+    with_grid(kind, [&](auto g) { fused4r_analysis<decltype(g)>(in, Tf, rec, out, b_out, nbatch, real_basis, st); return 0; });
   }
   return s2cnn::launch_status();
 }
@@ -434,10 +447,11 @@ int fused_synthesis(FusedKind kind, const float* xhat, const float* table, const
     if (real_basis) hipLaunchKernelGGL(fused64::spectrum_gather_real<>, dim3(tiles_r, rounds * 32), dim3(256), 0, st, xhat, rec, nl, nbatch);
     else hipLaunchKernelGGL(fused64::spectrum_gather<>, dim3(tiles_c, rounds * 16), dim3(256), 0, st, xc, rec, nl, nbatch);
     fused64::launch_synthesis(nl, st, rec, Tf, out, nbatch, bias, nfeature, relu, bits, mom, yref, params);
-  } else if (kind == FUSED_44) {
-    fused4r_synthesis<Grid44>(xhat, Tf, rec, out, nl, nbatch, real_basis, bias, nfeature, relu, st, mom, yref, params);
   } else {
-    fused4r_synthesis<Grid32>(xhat, Tf, rec, out, nl, nbatch, real_basis, bias, nfeature, relu, st, mom, yref, params);
+    with_grid(kind, [&](auto g) {
+      fused4r_synthesis<decltype(g)>(xhat, Tf, rec, out, nl, nbatch, real_basis, bias, nfeature, relu, st, mom, yref, params);
+      return 0;
+    });
   }
   return s2cnn::launch_status();
 }
@@ -587,7 +601,7 @@ struct PlaneMoments {
 int moment_parts(int b_in, int b_out) {
   if (!sizes_ok(b_out, b_in, 1)) return 0;
   const FusedKind k = fused_kind(b_out, b_in, 0, true);
-  if (k == FUSED_32 || k == FUSED_44) return 1;
+  if (k != FUSED_NONE && k != FUSED_64) return 1;
   if (k != FUSED_NONE || 2 * b_out == 64) return 0;
   const plane_real::Plan plan = plane_real::plan_inv(2 * b_out, b_in < b_out ? b_in : b_out, 2 * b_out);
   return plan.pl > 0 && plan.alias ? 2 * b_out : 0;

@@ -2,8 +2,8 @@
 // the form of the 64^3 kernels of so3_fused64.h: a workgroup owns one volume, keeps its half spectrum in registers and
 // walks over beta, so the transformed planes never leave the compute unit.  What is the same (the beta fold, the sign
 // rules, the ITEMS, the quad layout, the per-volume records and the passes between records and spectral rows) is described
-// there; this file says what differs.  Instantiated for the 32^3 grid (R = 8, bandwidth 16) and the 44^3 grid (R = 11,
-// bandwidth 22).
+// there; this file says what differs.  Instantiated for the grids 20^3 (R = 5, bandwidth 10), 32^3 (R = 8, bandwidth 16)
+// and 44^3 (R = 11, bandwidth 22).
 //
 // A volume of these grids is a fraction of the work of a 64^3 volume, so SEVERAL volumes are resident on a compute unit at
 // once, each in another phase of its step: what the 64^3 kernels arrange inside one workgroup (two halves of the waves in
@@ -60,7 +60,7 @@ template <int R, int Q> struct Trig {
 
 // R-point DFT out of registers, natural order in; every output X[k] is handed to emit(k, X[k]) as soon as it is formed, so
 // no second set of registers holds the outputs.  Sign of the exponent: - (forward) / + (INV).
-// X[k] = v0 + sum_{j=1..H} ( p_j cos(2 pi j k / R) -+ i m_j sin(2 pi j k / R) ) (+ (-1)^k v_{R/2} for even R),
+// X[k] = v0 + sum_{j=1..H} ( p_j cos(2 pi j k / R) -+ i m_j sin(2 pi j k / R) ) for odd R,
 // p_j = v_j + v_{R-j}, m_j = v_j - v_{R-j} (formed in place: v_j <- p_j, v_{R-j} <- m_j), H = (R - 1) / 2; X[R - k] has the
 // other sign of the sine part.
 template <int R, int K, int J>
@@ -76,7 +76,6 @@ template <int R, bool INV, int K, class Emit>
 __device__ __forceinline__ void dft_fold_outputs(const float2 (&v)[R], Emit& emit) {
   if constexpr (K <= (R - 1) / 2) {
     float2 C = v[0], S = make_float2(0.f, 0.f);
-    if constexpr (R % 2 == 0) { C.x += (K & 1) ? -v[R / 2].x : v[R / 2].x; C.y += (K & 1) ? -v[R / 2].y : v[R / 2].y; }
     dft_fold_term<R, K, 1>(v, C, S);
     // forward: X[K] = C - i S, X[R-K] = C + i S; inverse: the other way round
     const float2 lo = make_float2(C.x + S.y, C.y - S.x), hi = make_float2(C.x - S.y, C.y + S.x);
@@ -92,6 +91,7 @@ __device__ __forceinline__ void dft_r(float2 (&v)[R], Emit emit) {
 #pragma unroll
     for (int k = 0; k < 8; ++k) emit(k, v[k]);
   } else {
+    static_assert(R % 2 == 1, "the folded sum is written for odd R");
     constexpr int H = (R - 1) / 2;
     float2 sum = v[0];
 #pragma unroll
@@ -100,14 +100,6 @@ __device__ __forceinline__ void dft_r(float2 (&v)[R], Emit emit) {
       v[j] = make_float2(a.x + b.x, a.y + b.y);
       v[R - j] = make_float2(a.x - b.x, a.y - b.y);
       sum.x += v[j].x; sum.y += v[j].y;
-    }
-    if constexpr (R % 2 == 0) {
-      const float2 vmid = v[R / 2];
-      float2 alt = make_float2(v[0].x + ((R / 2) & 1 ? -vmid.x : vmid.x), v[0].y + ((R / 2) & 1 ? -vmid.y : vmid.y));
-#pragma unroll
-      for (int j = 1; j <= H; ++j) { alt.x += (j & 1) ? -v[j].x : v[j].x; alt.y += (j & 1) ? -v[j].y : v[j].y; }
-      emit(R / 2, alt);
-      sum.x += vmid.x; sum.y += vmid.y;
     }
     emit(0, sum);
     dft_fold_outputs<R, INV, 1>(v, emit);
@@ -170,6 +162,7 @@ struct Grid {
   }
 };
 
+using Grid20 = Grid<5, 128, 4>;                    // 20^3: eight
 using Grid32 = Grid<8, 256, 4>;                    // 32^3: four workgroups per compute unit, plane loads through registers
 using Grid44 = Grid<11, 512, 4, false, true>;       // 44^3: two (one, with all the registers it wants, is slower)
 
@@ -456,8 +449,9 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void synthesis_kerne
   constexpr int ZERO_PLACE = G::NITEMS, DUMP_PLACE = G::NITEMS + 1, NPLACES = G::NITEMS + 2;
   // degree groups that the NA rounds hold at least in part (the others are zero)
   constexpr int GROUPS = [] { int g = 0; for (int c = 0; c < G::NCG; ++c) if (G::offset(c) < NA * THREADS) g = c + 1; return g; }();
-  __shared__ __attribute__((aligned(16))) float4 stg_p[NPLACES];     // the item's share of the bins [+a,n], [-a,-n]
-  __shared__ __attribute__((aligned(16))) float4 stg_m[NPLACES];     //                              [-a,n], [+a,-n]
+  __shared__ __attribute__((aligned(16))) float4 stg[2 * NPLACES];
+  float4* const stg_p = stg;                 // the item's share of the bins [+a,n], [-a,-n]
+  float4* const stg_m = stg + NPLACES;       //                              [-a,n], [+a,-n]
   const long z = volume_of_block(nbatch);
   if (z < 0) return;
   const int t = threadIdx.x;
@@ -615,10 +609,10 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void synthesis_kerne
   // the sums of the B_THREADS threads that hold samples (2 R NJ each) through LDS, pairwise, always in the same order;
   // threads without samples enter with a count of zero
   constexpr int PAD = G::B_THREADS <= 128 ? 128 : G::B_THREADS <= 256 ? 256 : 512;
-  static_assert(PAD <= THREADS && 3 * PAD * 8 <= G::LDS_ELEMS * 8, "reduction does not fit");
+  static_assert(PAD <= THREADS && 3 * PAD * 8 <= (int)sizeof(stg), "reduction does not fit");
   if constexpr (MOM == 1) {                         // (mean, squared deviations, count) per thread, merged in float64
     __syncthreads();
-    double* red = reinterpret_cast<double*>(work);  // [3][PAD]: mean, M2, count
+    double* red = reinterpret_cast<double*>(stg);    // [3][PAD]: mean, M2, count
     constexpr double NT_SAMPLES = 2.0 * R * NJ;
     if (t < PAD) { red[t] = 0.0; red[PAD + t] = 0.0; red[2 * PAD + t] = 0.0; }
     __syncthreads();
@@ -645,7 +639,7 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void synthesis_kerne
   }
   if constexpr (MOM == 2) {
     __syncthreads();
-    float* red = reinterpret_cast<float*>(work);
+    float* red = reinterpret_cast<float*>(stg);
     if (t < PAD) { red[t] = 0.f; red[PAD + t] = 0.f; }
     __syncthreads();
     if (in_store) { red[t - G::B_COLS_FIRST] = ms1; red[PAD + t - G::B_COLS_FIRST] = ms2; }

@@ -14,7 +14,7 @@ from s2cnn_amd.soft import so3_fft as P
 
 pytestmark = pytest.mark.gpu
 
-PAIRS = [(32, 32), (32, 22), (22, 22), (22, 7), (22, 18), (16, 16), (16, 10), (12, 12), (10, 6), (6, 6), (7, 7), (3, 3)]
+PAIRS = [(32, 32), (32, 22), (22, 22), (22, 7), (22, 18), (16, 16), (16, 10), (12, 12), (10, 10), (10, 6), (6, 6), (7, 7), (3, 3)]
 
 
 def _rel(got, want):
@@ -47,12 +47,12 @@ def test_volume_moments(hip):
         assert (got - want).abs().max().item() < 2e-5 * want.abs().max().item(), n2    # a sample at the threshold may fall either way
 
 
-@pytest.mark.parametrize("b_in,b_out", [(32, 32), (22, 32), (26, 32), (16, 16), (10, 16), (20, 16), (22, 22), (7, 22), (18, 22), (12, 12), (6, 6)])
+@pytest.mark.parametrize("b_in,b_out", [(32, 32), (22, 32), (26, 32), (16, 16), (10, 16), (20, 16), (22, 22), (7, 22), (18, 22), (10, 10), (6, 10), (12, 12), (6, 6)])
 def test_sums_formed_by_the_synthesis(hip, b_in, b_out):
     """(sum y, sum (y - mean)^2) per volume (64^3, 44^3 and 32^3 grids) or per plane (two-stage path) written by the synthesis that
     produces y, against float64 sums of that y; y itself bit for bit the output of the synthesis without the sums."""
     parts = P.synthesis_moment_parts(b_in, b_out)
-    assert parts == (1 if b_out in (32, 22, 16) else 2 * b_out)
+    assert parts == (1 if b_out in (32, 22, 16, 10) else 2 * b_out)
     g = torch.Generator().manual_seed(b_in * 100 + b_out)
     nspec = b_in * (4 * b_in ** 2 - 1) // 3
     r = torch.randn(nspec, 2, 3, generator=g).cuda()
@@ -68,13 +68,13 @@ def test_sums_formed_by_the_synthesis(hip, b_in, b_out):
     assert mean_err.max().item() < 1e-6 and _rel(mom.double()[:, 1], want[:, 1]) < 2e-5
 
 
-@pytest.mark.parametrize("b_in,b_out", [(16, 16), (9, 16), (22, 22), (12, 12)])
+@pytest.mark.parametrize("b_in,b_out", [(16, 16), (9, 16), (22, 22), (10, 10), (12, 12)])
 def test_sums_formed_by_the_synthesis_of_a_complex_spectrum(hip, b_in, b_out):
     """The same sums from s2cnn_so3_synthesis_real_moments (complex spectrum): per plane on the two-stage path, per volume
     from the per-volume kernels of the 32^3 grid; both kinds of sums, against float64 sums of the output."""
     from s2cnn_amd.soft import so3_fft as F
     parts = F._hip.lib().s2cnn_so3_synthesis_moment_parts(b_in, b_out)
-    assert parts == (1 if b_out in (22, 16) else 2 * b_out)
+    assert parts == (1 if b_out in (22, 16, 10) else 2 * b_out)
     gen = torch.Generator().manual_seed(b_in * 100 + b_out + 3)
     nspec = b_in * (4 * b_in ** 2 - 1) // 3
     xh = torch.randn(nspec, 2, 3, 2, generator=gen).cuda()
@@ -98,7 +98,7 @@ def test_sums_formed_by_the_synthesis_of_a_complex_spectrum(hip, b_in, b_out):
 
 
 @pytest.mark.parametrize("ratio", [100.0, 1000.0])
-@pytest.mark.parametrize("b_in,b_out", [(32, 32), (16, 16), (22, 22), (12, 12), (6, 6)])
+@pytest.mark.parametrize("b_in,b_out", [(32, 32), (16, 16), (22, 22), (10, 10), (12, 12), (6, 6)])
 def test_statistics_of_a_signal_with_a_large_mean(hip, b_in, b_out, ratio):
     """A mean `ratio` times the standard deviation: the batch variance that the normalisation forms from the library's sums
     (the synthesis's own, and s2cnn_volume_moments) must keep its digits, as nn.BatchNorm3d's does; E[y^2] - mean^2 from
@@ -123,13 +123,13 @@ def test_statistics_of_a_signal_with_a_large_mean(hip, b_in, b_out, ratio):
         assert _rel(got_var, want_var) < 1e-3, (nparts, got_var, want_var)
 
 
-@pytest.mark.parametrize("b_in,b_out", [(22, 32), (26, 32), (28, 32), (16, 16), (10, 16), (22, 22), (7, 22), (18, 22), (12, 12), (6, 6)])
+@pytest.mark.parametrize("b_in,b_out", [(22, 32), (26, 32), (28, 32), (16, 16), (10, 16), (22, 22), (7, 22), (18, 22), (10, 10), (6, 10), (12, 12), (6, 6)])
 def test_gradient_sums_formed_by_the_synthesis(hip, b_in, b_out):
     """(sum g m, sum g m y), m = (a y + b > 0), with g the output of the synthesis and y a second tensor, per volume or per
     plane, against float64 sums; none on the 64^3 grid for a spectrum of all 32 degrees."""
     assert P.synthesis_moment_parts(32, 32, grad=True) == 0
     parts = P.synthesis_moment_parts(b_in, b_out, grad=True)
-    assert parts == (1 if b_out in (32, 22, 16) else 2 * b_out)
+    assert parts == (1 if b_out in (32, 22, 16, 10) else 2 * b_out)
     gen = torch.Generator().manual_seed(b_in * 100 + b_out + 7)
     nspec = b_in * (4 * b_in ** 2 - 1) // 3
     r = torch.randn(nspec, 2, 3, generator=gen).cuda()

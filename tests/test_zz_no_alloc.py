@@ -33,6 +33,7 @@ def _both(lib, x, table, packed, b_in, b_out):
                                                          (16, 16, 21, 6),     # the per-volume kernels of the 32^3 grid
                                                          (16, 10, 9, 3),
                                                          (22, 22, 7, 3),      # ... and of the 44^3 grid
+                                                         (10, 10, 50, 3),     # ... and of the 20^3 grid
                                                          (12, 8, 40, 7),      # two-stage path: scratch = transformed planes
                                                          (6, 6, 33, 1)])
 def test_static_scratch_analysis_equals_workspace_analysis(hip, b_in, b_out, n_first, n_second):
