@@ -205,8 +205,9 @@ def measure_rows(torch, dev, with_cpu):
     add("so3_ifft complex b=32 N=16", gpu_ms(lambda: PSO3.so3_ifft(sc)), byc, "B", t, 1 / 16, "1 volume of 16")
     del xc, sc
     # --- real SO(3) transforms on the grids below 64^3, spectrum in the real basis as inside the layers: the 44^3 grid of
-    # config 5 (b = 22, 32 x 100 volumes) and the 32^3 grid of the reference's SHREC17 model (b = 16, 32 x 100 volumes)
-    for bs, nv in ((22, 3200), (16, 3200)):
+    # config 5 (b = 22, 32 x 100 volumes) and the 32^3 and 20^3 grids of the reference's SHREC17 model (b = 16 and 10,
+    # 32 x 100 volumes)
+    for bs, nv in ((22, 3200), (16, 3200), (10, 3200)):
         xs = torch.randn(nv, 2 * bs, 2 * bs, 2 * bs, device=dev)
         rs = PSO3.so3_rfft_real_basis(xs)
         bys = 4.0 * xs.numel() + 4.0 * rs.numel()

@@ -269,10 +269,10 @@ int s2cnn_volume_moments(const float *x, float *out, long nvol, long n, void *st
 int s2cnn_bn_relu_grad_moments(const float *g, const float *y, const float *params, int nfeature, float *out,
                                long nvol, long n, void *stream);
 /* Where the synthesis that produces y (or the gradient g) stages whole planes in LDS it can form those sums itself, one
- * pair per plane, and the separate read is not needed; the per-volume kernels of the 32^3 grid (b_out = 16) form one pair
- * per volume.  s2cnn_so3_synthesis_moment_parts(b_in, b_out) = pairs per volume (2 b_out, or 1 for b_out = 16) where
+ * pair per plane, and the separate read is not needed; the per-volume kernels of the 44^3, 32^3 and 20^3 grids (b_out = 22,
+ * 16, 10) form one pair per volume.  s2cnn_so3_synthesis_moment_parts(b_in, b_out) = pairs per volume (2 b_out, or 1 on those grids) where
  * s2cnn_so3_synthesis_real_moments can do that (real signals, complex spectrum; other arguments as
- * s2cnn_so3_synthesis_real_bias; with yref: no bias on the 32^3 grid), else 0.  moments [nbatch][pairs][2]; yref = NULL:
+ * s2cnn_so3_synthesis_real_bias; with yref: no bias on those three grids), else 0.  moments [nbatch][pairs][2]; yref = NULL:
  * (sum y, sum (y - mean of the part)^2) of the output; yref = the tensor y and params = ab: (sum g m, sum g m y) with the
  * output as g. */
 int s2cnn_so3_synthesis_moment_parts(int b_in, int b_out);
@@ -284,7 +284,7 @@ int s2cnn_so3_synthesis_real_moments(const float *xhat, const float *table, cons
  * grid, whose per-volume kernel forms the sums over the volume it writes: one pair per volume (with yref: no bias, and
  * on the 64^3 grid spectra of at most 28 degrees, for which the kernel has registers to spare).
  * s2cnn_so3_synthesis_real_basis_moment_parts(b_in, b_out, grad = whether yref is given) = pairs per volume (1 on the
- * 64^3 and 32^3 grids, 2 b_out elsewhere) where it can, else 0 (and the entry point returns -1); moments [nbatch][pairs][2]. */
+ * 64^3, 44^3, 32^3 and 20^3 grids, 2 b_out elsewhere) where it can, else 0 (and the entry point returns -1); moments [nbatch][pairs][2]. */
 int s2cnn_so3_synthesis_real_basis_moment_parts(int b_in, int b_out, int grad);
 int s2cnn_so3_synthesis_real_basis_moments(const float *r, const float *table, const float *packed_table, float *out,
                                            void *workspace, size_t workspace_bytes, int b_in, int b_out, long nbatch,

@@ -399,7 +399,7 @@ bool real_basis_analysis(int b_in, int b_out) {
 // real_basis: the spectrum is stored in the real basis (one float per entry) instead of complex pairs.
 int fused_analysis(FusedKind kind, const s2cnn::Input& in, const float* table, const float* packed_table, float* out,
                    void* workspace, size_t workspace_bytes, int b_out, long nbatch, bool real_basis, hipStream_t st) {
-  if (!s2cnn::aligned16(in.x) || !s2cnn::aligned16(in.w)) return S2CNN_EALIGN;
+  if (kind == FUSED_64 && (!s2cnn::aligned16(in.x) || !s2cnn::aligned16(in.w))) return S2CNN_EALIGN;     // the other grids: any float pointer
   const size_t need = round256(fused_scratch_bytes(kind, nbatch)) + fused_packed_floats(kind) * sizeof(float);
   if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return S2CNN_EWORKSPACE;
   float4* rec = static_cast<float4*>(workspace);
@@ -426,7 +426,8 @@ int fused_synthesis(FusedKind kind, const float* xhat, const float* table, const
                     size_t workspace_bytes, int b_in, long nbatch, bool real_basis, const float* bias, int nfeature, int relu,
                     unsigned long long* bits, hipStream_t st, float* moments = nullptr, const float* yref = nullptr,
                     const float* params = nullptr) {
-  if (!s2cnn::aligned16(out) || !s2cnn::aligned16(bits) || !s2cnn::aligned8(moments) || !s2cnn::aligned16(yref)) return S2CNN_EALIGN;
+  if (kind == FUSED_64 && (!s2cnn::aligned16(out) || !s2cnn::aligned16(bits) || !s2cnn::aligned16(yref))) return S2CNN_EALIGN;
+  if (!s2cnn::aligned8(moments)) return S2CNN_EALIGN;
   if (bits && kind != FUSED_64) return S2CNN_EINVAL;
   const int b_grid = fused_bandwidth(kind);
   const int nl = b_in < b_grid ? b_in : b_grid;

@@ -207,6 +207,37 @@ def test_so3_transforms_without_prepacked_table(hip):
         assert torch.equal(out, want)
 
 
+@pytest.mark.parametrize("b", [10, 16, 22])
+def test_so3_per_volume_kernels_take_any_float_pointer(hip, b):
+    """Through the raw C ABI: the per-volume kernels of the 20^3, 32^3 and 44^3 grids ask for no more than float alignment
+    of the signal, the mask and the output (the 64^3 grid wants 16 bytes and says so with S2CNN_EALIGN)."""
+    from s2cnn_amd import _hip
+    nz = 3
+    n3 = nz * (2 * b) ** 3
+    big = rnd((2 * n3 + 8,), 33).cuda()
+    x = big[1:1 + n3].view(nz, 2 * b, 2 * b, 2 * b)                    # 4 bytes past a 16-byte boundary
+    assert x.data_ptr() % 16 == 4
+    table = PSO3._setup_wigner(b, b, True, x.device)
+    want = PSO3.so3_rfft(x.clone())
+    out = torch.empty_like(want)
+    ws = _hip.workspace(hip.s2cnn_so3_analysis_workspace(b, b, nz, 0), x.device)
+    _hip.check(hip.s2cnn_so3_analysis(_hip.ptr(x), _hip.ptr(table), None, _hip.ptr(out), _hip.ptr(ws), ws.numel(), b, b, nz, 0, _hip.stream_ptr()))
+    assert torch.equal(out, want)
+    s = rnd((O.nspec_so3(b), nz, 2), 34).cuda()
+    want = PSO3.so3_rifft(s)
+    y = big[n3 + 3:2 * n3 + 3].view(nz, 2 * b, 2 * b, 2 * b)
+    assert y.data_ptr() % 16 == 12
+    table = PSO3._setup_wigner(b, b, False, x.device)
+    ws = _hip.workspace(hip.s2cnn_so3_synthesis_workspace(b, b, nz, 0), x.device)
+    _hip.check(hip.s2cnn_so3_synthesis(_hip.ptr(s), _hip.ptr(table), None, _hip.ptr(y), _hip.ptr(ws), ws.numel(), b, b, nz, 0, _hip.stream_ptr()))
+    assert torch.equal(y, want)
+    x64 = rnd((64 ** 3 + 4,), 35).cuda()[1:]
+    ws = _hip.workspace(hip.s2cnn_so3_analysis_workspace(32, 32, 1, 0), x.device)
+    t64 = PSO3._setup_wigner(32, 32, True, x.device)
+    o64 = torch.empty(O.nspec_so3(32), 1, 2, device="cuda")
+    assert hip.s2cnn_so3_analysis(_hip.ptr(x64), _hip.ptr(t64), None, _hip.ptr(o64), _hip.ptr(ws), ws.numel(), 32, 32, 1, 0, _hip.stream_ptr()) == -3
+
+
 def test_so3_reference_identities_on_gpu(hip):
     """tests/so3_fft.py:8-24 and :34-91 of the reference, run on the HIP path."""
     b_in, b_out = 7, 5
