@@ -482,8 +482,13 @@ int run(const float* a, const float* b, float* c, int nl, int RI, int CI, int KI
   hipStream_t st = static_cast<hipStream_t>(stream);
   // the fast loaders address a degree with 32-bit byte offsets
   const bool small = Lmax * Lmax * RI * KI < (1L << 30) && Lmax * Lmax * CI * KI < (1L << 30);
-  const bool fast = a4 && b4 && (KI % TK == 0 || TK % KI == 0) && small;
-  const bool fast2 = a4 && b4 && !fast && KI > TK && KI % 4 == 0 && small;     // 100 features: stages that run over a block boundary
+  const bool divides = (KI % TK == 0 || TK % KI == 0) && small;                 // block size and K stage divide one another
+  const bool crosses = !divides && KI > TK && small;                           // 100 features: stages that run over a block boundary
+  const bool fast = a4 && b4 && divides;
+  const bool fast2 = a4 && b4 && crosses && KI % 4 == 0;
+  // the same two loaders with 8-byte accesses: even sizes that are no multiples of four (50, 70 features)
+  const bool fast_v2 = !fast && a2 && b2 && divides && KI % 2 == 0;
+  const bool fast2_v2 = !fast2 && a2 && b2 && crosses && KI % 2 == 0;
 #define S2CNN_LAUNCH(VA, VB, FAST)                                                                                    \
   do {                                                                                                                \
     if (narrow) hipLaunchKernelGGL((so3_block_mm_real_kernel<MODE, VA, VB, FAST, 1>), dim3(grid), dim3(NT), 0, st, p); \
@@ -491,6 +496,8 @@ int run(const float* a, const float* b, float* c, int nl, int RI, int CI, int KI
   } while (0)
   if (fast) S2CNN_LAUNCH(4, 4, 1);
   else if (fast2) S2CNN_LAUNCH(4, 4, 2);
+  else if (fast_v2) S2CNN_LAUNCH(2, 2, 1);
+  else if (fast2_v2) S2CNN_LAUNCH(2, 2, 2);
   else if (a4 && b4) S2CNN_LAUNCH(4, 4, 0);
   else if (a4 && b2) S2CNN_LAUNCH(4, 2, 0);
   else if (a2 && b4) S2CNN_LAUNCH(2, 4, 0);

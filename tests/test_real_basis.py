@@ -138,7 +138,10 @@ def test_basis_kernels_against_dense(hip, nl, cols):
                                         # one operand with 16-byte accesses, the other with 4-byte ones
                                         (5, 6, 20, 7), (4, 3, 7, 8), (7, 32, 100, 55),
                                         # even sizes that are no multiples of four: 8-byte accesses, alone and beside 16-byte ones
-                                        (6, 2, 50, 70), (5, 6, 10, 14), (4, 16, 70, 350), (5, 4, 6, 20), (5, 2, 20, 6), (3, 6, 2, 2)])
+                                        (6, 2, 50, 70), (5, 6, 10, 14), (4, 16, 70, 350), (5, 4, 6, 20), (5, 2, 20, 6), (3, 6, 2, 2),
+                                        # ... through the scalar-stepped loaders: blocks that divide the stage (16, 2) and blocks
+                                        # that stages run across (34, 50, 66, 70), ragged last stages
+                                        (7, 16, 50, 70), (5, 6, 34, 66), (6, 6, 16, 18), (4, 10, 66, 34), (9, 2, 38, 2)])
 def test_so3_mm_real_forward_backward(hip, nl, B, Fi, Fo):
     import s2cnn_amd
     print(f"so3_mm_real nl={nl} B={B} Fi={Fi} Fo={Fo}", flush=True)
