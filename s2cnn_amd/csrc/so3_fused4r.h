@@ -402,7 +402,10 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void analysis_kernel
   load_planes(0);
   for (int j = 0; j < NJ; ++j) {
     stage_c1();
-    if constexpr (!G::LATE) { __builtin_amdgcn_sched_barrier(0); load_planes(j + 1 < NJ ? j + 1 : NJ - 1); }      // clamped, not branched: in flight during the step
+    // the next plane pair, in flight during the step.  Into registers: clamped, not branched (a branch would make the loads
+    // synchronous); into LDS: none after the last pair (nothing would read them)
+    if constexpr (!G::LATE && !G::DMA) load_planes(j + 1 < NJ ? j + 1 : NJ - 1);
+    if constexpr (!G::LATE && G::DMA) { __builtin_amdgcn_sched_barrier(0); if (j + 1 < NJ) load_planes(j + 1); }
     step_barrier();
     if (t >= G::B_COLS_FIRST && t < G::B_COLS_FIRST + G::B_THREADS) pass_b<G, false, false>(work, t - G::B_COLS_FIRST);
     step_barrier();
@@ -411,7 +414,8 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void analysis_kernel
     if (t < G::B_THREADS) stage_r2();
 #pragma unroll
     for (int it = 0; it < SLOTS; ++it) load_table(j, it);     // only now: their registers are not held through the transform
-    if constexpr (G::LATE) load_planes(j + 1 < NJ ? j + 1 : NJ - 1);
+    if constexpr (G::LATE && !G::DMA) load_planes(j + 1 < NJ ? j + 1 : NJ - 1);
+    if constexpr (G::LATE && G::DMA) { if (j + 1 < NJ) load_planes(j + 1); }
     step_barrier();
 #pragma unroll
     for (int it = 0; it < NA; ++it) {
