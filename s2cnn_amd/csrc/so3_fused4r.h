@@ -108,13 +108,11 @@ __device__ __forceinline__ void dft_r(float2 (&v)[R], Emit emit) {
 
 // The grid of N = 4 R points per axis and how a workgroup of T threads (a power of two) is laid over it;
 // W = waves per SIMD the kernels are compiled for (workgroups per compute unit x T / 256).
-// LATE: the analysis issues the loads of the next plane pair after the transform of the current one instead of before it
-// (fewer registers held through the transform, less time for the loads).
-// DMA: those loads go straight to LDS (buffer loads with the lds bit: lane i of a wave writes word i of a 256-byte row of
-// its own), so no registers hold them while they are in flight; a wave waits for its own loads and reads back its own rows.
-template <int R_, int T, int W, bool LATE_ = false, bool DMA_ = false>
+// DMA: the analysis sends the loads of the next plane pair straight to LDS (buffer loads with the lds bit: lane i of a wave
+// writes word i of a 256-byte row of its own), so no registers hold them while they are in flight; a wave waits for its own
+// loads and reads back its own rows.
+template <int R_, int T, int W, bool DMA_ = false>
 struct Grid {
-  static constexpr bool LATE = LATE_;
   static constexpr bool DMA = DMA_;
   static constexpr int R = R_;
   static constexpr int N = 4 * R;
@@ -164,7 +162,7 @@ struct Grid {
 
 using Grid20 = Grid<5, 128, 4>;                    // 20^3: eight
 using Grid32 = Grid<8, 256, 4>;                    // 32^3: four workgroups per compute unit, plane loads through registers
-using Grid44 = Grid<11, 512, 4, false, true>;       // 44^3: two (one, with all the registers it wants, is slower)
+using Grid44 = Grid<11, 512, 4, true>;       // 44^3: two (one, with all the registers it wants, is slower)
 
 // Packed table, as fused64::pack_table: float index ((((j*NIT + it)*2 + h)*THREADS + t)*4 + u) holds
 // 0.5 * T[j, l = 4c+u, m = (h ? -a : +a), n] for the item of place it*THREADS + t.  T is [N][nspec_stride].
@@ -284,10 +282,7 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void analysis_kernel
   // DMA: [tensor][plane][j1][thread] words, filled by the loads themselves
   __shared__ __attribute__((aligned(16))) float landing[G::DMA ? (MASKED ? 16 : 8) * THREADS : 1];
   const int wave_first = __builtin_amdgcn_readfirstlane(t & ~63);       // first thread of this wave
-  // table registers: item it in slot it % SLOTS; a slot is refilled when its item is done.  With the plane loads going to
-  // LDS there are registers for all items, and no table load queues up behind the plane loads.
-  constexpr int SLOTS = G::DMA || NA < 2 ? NA : 2;
-  float4 t1[SLOTS], t2[SLOTS];
+  float4 t1[NA], t2[NA];
 
   auto load_planes = [&](int j) {        // rows R j1 + d of the planes j and N-1-j: contiguous over the workgroup
     if constexpr (G::DMA) {
@@ -314,8 +309,8 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void analysis_kernel
     }
   };
   auto load_table = [&](int j, int it) {
-    t1[it % SLOTS] = buf_load_f32x4(rt, toff, ((j * NIT + it) * 2 + 0) * (THREADS * 16));
-    t2[it % SLOTS] = buf_load_f32x4(rt, toff, ((j * NIT + it) * 2 + 1) * (THREADS * 16));
+    t1[it] = buf_load_f32x4(rt, toff, ((j * NIT + it) * 2 + 0) * (THREADS * 16));
+    t2[it] = buf_load_f32x4(rt, toff, ((j * NIT + it) * 2 + 1) * (THREADS * 16));
   };
   // pass A of the alpha axis out of the registers: 4-point transforms over j1, twiddle, -> work[R k1 + d][lo]
   auto stage_c1 = [&]() {
@@ -375,8 +370,8 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void analysis_kernel
     const float2 Qp = make_float2(flip(za.y + za.w, sb), flip(za.z - za.x, sb));
     const float2 Pm = make_float2(zb.x + zb.z, zb.y - zb.w);
     const float2 Qm = make_float2(flip(zb.y + zb.w, sb), flip(zb.z - zb.x, sb));
-    const float a1[4] = {t1[it % SLOTS].x, t1[it % SLOTS].y, t1[it % SLOTS].z, t1[it % SLOTS].w};
-    const float a2[4] = {t2[it % SLOTS].x, t2[it % SLOTS].y, t2[it % SLOTS].z, t2[it % SLOTS].w};
+    const float a1[4] = {t1[it].x, t1[it].y, t1[it].z, t1[it].w};
+    const float a2[4] = {t2[it].x, t2[it].y, t2[it].z, t2[it].w};
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       // (-1)^(l-n) = (-1)^u (-1)^n for l = 4c+u: the sign of odd u goes into the table operand
@@ -404,8 +399,8 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void analysis_kernel
     stage_c1();
     // the next plane pair, in flight during the step.  Into registers: clamped, not branched (a branch would make the loads
     // synchronous); into LDS: none after the last pair (nothing would read them)
-    if constexpr (!G::LATE && !G::DMA) load_planes(j + 1 < NJ ? j + 1 : NJ - 1);
-    if constexpr (!G::LATE && G::DMA) { __builtin_amdgcn_sched_barrier(0); if (j + 1 < NJ) load_planes(j + 1); }
+    if constexpr (!G::DMA) load_planes(j + 1 < NJ ? j + 1 : NJ - 1);
+    else { __builtin_amdgcn_sched_barrier(0); if (j + 1 < NJ) load_planes(j + 1); }
     step_barrier();
     if (t >= G::B_COLS_FIRST && t < G::B_COLS_FIRST + G::B_THREADS) pass_b<G, false, false>(work, t - G::B_COLS_FIRST);
     step_barrier();
@@ -413,15 +408,10 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void analysis_kernel
     step_barrier();
     if (t < G::B_THREADS) stage_r2();
 #pragma unroll
-    for (int it = 0; it < SLOTS; ++it) load_table(j, it);     // only now: their registers are not held through the transform
-    if constexpr (G::LATE && !G::DMA) load_planes(j + 1 < NJ ? j + 1 : NJ - 1);
-    if constexpr (G::LATE && G::DMA) { if (j + 1 < NJ) load_planes(j + 1); }
+    for (int it = 0; it < NA; ++it) load_table(j, it);        // only now: their registers are not held through the transform
     step_barrier();
 #pragma unroll
-    for (int it = 0; it < NA; ++it) {
-      accumulate(it);
-      if (it + SLOTS < NA) { __builtin_amdgcn_sched_barrier(0); load_table(j, it + SLOTS); __builtin_amdgcn_sched_barrier(0); }
-    }
+    for (int it = 0; it < NA; ++it) accumulate(it);
   }
 
   const __amdgpu_buffer_rsrc_t rr = make_rsrc(rec + (size_t)z * G::REC_F4, (unsigned)G::REC_BYTES);
@@ -520,6 +510,9 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void synthesis_kerne
   };
   // staging -> work (natural order): thread t < NR^2 takes the column a = t / NR, n = t % NR.  No branches inside: a
   // degree group the column does not have reads the zero place, a bin that does not exist (-0) goes to the pad column.
+  // the thread's reduction indices, kept in LDS where registers are short (three item rounds): [index][thread] words
+  constexpr bool RED_LDS = NA >= 3;
+  __shared__ unsigned short red_tab[RED_LDS ? (GROUPS + 4) * THREADS : 1];
   int red_pos[GROUPS], red_dst[4];
   const bool in_red = NR * NR == THREADS || t < NR * NR;
   {
@@ -532,20 +525,27 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void synthesis_kerne
     red_dst[1] = n > 0 ? rm + N - n : rm + N;             // [-a,-n]
     red_dst[2] = a > 0 ? rm + n : rp + N;                 // [-a, n]
     red_dst[3] = a > 0 && n > 0 ? rp + N - n : rp + N;    // [+a,-n]
+    if constexpr (RED_LDS) {
+#pragma unroll
+      for (int c = 0; c < GROUPS; ++c) red_tab[c * THREADS + t] = (unsigned short)red_pos[c];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) red_tab[(GROUPS + q) * THREADS + t] = (unsigned short)red_dst[q];
+    }
   }
   auto reduce = [&]() {
     if (in_red) {
       float4 s0 = make_float4(0.f, 0.f, 0.f, 0.f), s1 = s0;
 #pragma unroll
       for (int c = 0; c < GROUPS; ++c) {
-        const float4 u0 = stg_p[red_pos[c]], u1 = stg_m[red_pos[c]];
+        const int pos = RED_LDS ? (int)red_tab[c * THREADS + t] : red_pos[c];
+        const float4 u0 = stg_p[pos], u1 = stg_m[pos];
         s0 = make_float4(s0.x + u0.x, s0.y + u0.y, s0.z + u0.z, s0.w + u0.w);
         s1 = make_float4(s1.x + u1.x, s1.y + u1.y, s1.z + u1.z, s1.w + u1.w);
       }
-      work[red_dst[0]] = make_float2(s0.x, s0.y);
-      work[red_dst[1]] = make_float2(s0.z, s0.w);
-      work[red_dst[2]] = make_float2(s1.x, s1.y);
-      work[red_dst[3]] = make_float2(s1.z, s1.w);
+      work[RED_LDS ? (int)red_tab[(GROUPS + 0) * THREADS + t] : red_dst[0]] = make_float2(s0.x, s0.y);
+      work[RED_LDS ? (int)red_tab[(GROUPS + 1) * THREADS + t] : red_dst[1]] = make_float2(s0.z, s0.w);
+      work[RED_LDS ? (int)red_tab[(GROUPS + 2) * THREADS + t] : red_dst[2]] = make_float2(s1.x, s1.y);
+      work[RED_LDS ? (int)red_tab[(GROUPS + 3) * THREADS + t] : red_dst[3]] = make_float2(s1.z, s1.w);
     }
     // the bins of m = N/2 and n = N/2 hold what the last transform left there: cleared again
     if (t < N) { work[(N / 2) * PITCH + t] = make_float2(0.f, 0.f); work[t * PITCH + N / 2] = make_float2(0.f, 0.f); }
