@@ -587,24 +587,45 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void synthesis_kerne
   __syncthreads();                                  // cleared work and staging
 #pragma unroll
   for (int it = 0; it < NA; ++it) contribute(it);
-  load_table(1);
+  if (G::B_COLS_FIRST < (G::B_THREADS + 63) / 64 * 64) load_table(1);
   __syncthreads();
   reduce();
   __syncthreads();
+  // The shares of pair j + 1 are formed while pair j is in the plane.  Where the B passes of the two axes have waves of
+  // their own (SPLIT), every wave forms its shares while it would otherwise wait for one of them: the waves beyond those
+  // of the row pass B during that pass, the others during the last pass and its stores; their table values are loaded
+  // right before.
+  constexpr int ROW_B_END = (G::B_THREADS + 63) / 64 * 64;
+  constexpr bool SPLIT = ROW_B_END <= G::B_COLS_FIRST;
+  const bool early = t >= ROW_B_END;
   for (int j = 0; j < NJ; ++j) {
-    if (j + 1 < NJ) {                               // the shares of pair j + 1, while pair j is in the plane
+    const bool more = j + 1 < NJ;
+    if (!SPLIT && more) {
 #pragma unroll
       for (int it = 0; it < NA; ++it) contribute(it);
     }
+    if (SPLIT && more && early) load_table(j + 1);
     pass_a<G, true, true>(work, tw, lo, d);
     __syncthreads();
     if (t < G::B_THREADS) pass_b<G, true, true>(work, t);
+    if (SPLIT && more) {
+      if (early) {
+#pragma unroll
+        for (int it = 0; it < NA; ++it) contribute(it);
+      } else {
+        load_table(j + 1);
+      }
+    }
     __syncthreads();
     pass_a<G, true, false>(work, tw, lo, d);
     __syncthreads();
     if (in_store) stage_c2_store(j, t - G::B_COLS_FIRST);
-    if (j + 1 < NJ) {
-      load_table(j + 2 < NJ ? j + 2 : NJ - 1);      // only now: its registers are not held through the transform
+    if (SPLIT && more && !early) {
+#pragma unroll
+      for (int it = 0; it < NA; ++it) contribute(it);
+    }
+    if (more) {
+      if (!SPLIT) load_table(j + 2 < NJ ? j + 2 : NJ - 1);      // only now: its registers are not held through the transform
       __syncthreads();
       reduce();
       __syncthreads();
