@@ -387,8 +387,10 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void analysis_kernel
   // too (its fence covers every write to LDS): there the barrier is taken once this wave's own LDS accesses are done.
   auto step_barrier = [&]() {
     if constexpr (G::DMA) {
+      asm volatile("" ::: "memory");                // the compiler moves no memory access across the barrier ...
       __builtin_amdgcn_s_waitcnt(0xC07F);           // lgkmcnt(0)
       __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");                // ... in either direction
     } else {
       __syncthreads();
     }
