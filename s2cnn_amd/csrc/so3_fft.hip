@@ -338,13 +338,13 @@ void fused_pack_table(FusedKind k, hipStream_t st, const float* table, float* pa
 template <class G>
 void fused4r_analysis(const s2cnn::Input& in, const float* Tf, float4* rec, float* out, int b_out, long nbatch, bool real_basis, hipStream_t st) {
   const unsigned tiles_r = (unsigned)((nbatch + fused64::ZR - 1) / fused64::ZR), tiles_c = (unsigned)((nbatch + fused64::ZT - 1) / fused64::ZT);
-  const int rounds = G::active_rounds(b_out);
-  fused4r::launch_analysis<G>(b_out, st, in, Tf, rec, nbatch);
+  const int rounds = G::active_rounds(b_out), nparts = G::parts(nbatch);
+  fused4r::launch_analysis<G>(b_out, st, in, Tf, rec, nbatch, nparts);
   if (real_basis)
-    hipLaunchKernelGGL(fused64::spectrum_scatter_real<G>, dim3(tiles_r, rounds * (G::THREADS / fused64::IT_TILE_R)), dim3(256), 0, st, rec, out, b_out, nbatch);
+    hipLaunchKernelGGL(fused64::spectrum_scatter_real<G>, dim3(tiles_r, rounds * (G::THREADS / fused64::IT_TILE_R)), dim3(256), 0, st, rec, out, b_out, nbatch, nparts);
   else
     hipLaunchKernelGGL(fused64::spectrum_scatter<G>, dim3(tiles_c, rounds * (G::THREADS / fused64::IT_TILE)), dim3(256), 0, st, rec,
-                       reinterpret_cast<float2*>(out), b_out, nbatch);
+                       reinterpret_cast<float2*>(out), b_out, nbatch, nparts);
 }
 template <class G>
 void fused4r_synthesis(const float* xhat, const float* Tf, float4* rec, float* out, int nl, long nbatch, bool real_basis, const float* bias,
@@ -356,7 +356,7 @@ void fused4r_synthesis(const float* xhat, const float* Tf, float4* rec, float* o
   else
     hipLaunchKernelGGL(fused64::spectrum_gather<G>, dim3(tiles_c, rounds * (G::THREADS / fused64::IT_TILE)), dim3(256), 0, st,
                        reinterpret_cast<const float2*>(xhat), rec, nl, nbatch);
-  fused4r::launch_synthesis<G>(nl, st, rec, Tf, out, nbatch, bias, nfeature, relu, mom, yref, params);
+  fused4r::launch_synthesis<G>(nl, st, rec, Tf, out, nbatch, bias, nfeature, relu, G::parts(nbatch), mom, yref, params);
 }
 
 // Bytes of the intermediate; batch items padded to the z tile of the tiled Wigner kernels.
@@ -414,8 +414,8 @@ int fused_analysis(FusedKind kind, const s2cnn::Input& in, const float* table, c
   if (kind == FUSED_64) {
     const int rounds = fused64::active_rounds(b_out);
     fused64::launch_analysis(b_out, st, in, Tf, rec, nbatch);
-    if (real_basis) hipLaunchKernelGGL(fused64::spectrum_scatter_real<>, dim3(tiles_r, rounds * 32), dim3(256), 0, st, rec, out, b_out, nbatch);
-    else hipLaunchKernelGGL(fused64::spectrum_scatter<>, dim3(tiles_c, rounds * 16), dim3(256), 0, st, rec, outc, b_out, nbatch);
+    if (real_basis) hipLaunchKernelGGL(fused64::spectrum_scatter_real<>, dim3(tiles_r, rounds * 32), dim3(256), 0, st, rec, out, b_out, nbatch, 1);
+    else hipLaunchKernelGGL(fused64::spectrum_scatter<>, dim3(tiles_c, rounds * 16), dim3(256), 0, st, rec, outc, b_out, nbatch, 1);
   } else {
     with_grid(kind, [&](auto g) { fused4r_analysis<decltype(g)>(in, Tf, rec, out, b_out, nbatch, real_basis, st); return 0; });
   }

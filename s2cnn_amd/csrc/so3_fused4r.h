@@ -152,7 +152,13 @@ struct Grid {
     a = r / width(c); n = r - a * width(c);
     return true;
   }
-  static size_t scratch_bytes(long nbatch) { return (size_t)nbatch * REC_BYTES; }
+  // workgroups per volume: a power of two, at least four beta pairs each, no more than fill the chip once
+  static int parts(long nbatch) {
+    int p = 1;
+    while (2 * p * 4 <= NJ && 2 * p * nbatch <= 256) p *= 2;
+    return p;
+  }
+  static size_t scratch_bytes(long nbatch) { return (size_t)nbatch * parts(nbatch) * REC_BYTES; }
   // item rounds that carry degrees below nl
   static int active_rounds(int nl) {
     const int groups = nl >= NR ? NCG : (nl + 3) / 4;
@@ -226,18 +232,25 @@ __device__ __forceinline__ void pass_b(float2* buf, int u) {
 // ---------------------------------------------------------------------------------------------
 // analysis: x [nbatch][N][N][N] real -> records of the half spectrum n >= 0
 // NA: item rounds with degrees below the output bandwidth; MASK: s2cnn::Prologue (bit masks, 2, are not supported)
+// nparts: workgroups per volume.  Few volumes do not fill the chip with one workgroup each: part p of a volume then takes
+// the beta pairs p NJ / nparts .. (p+1) NJ / nparts - 1 and writes a record of its own ([volume][part]); the pass to the
+// spectral rows adds the parts in their order.
 // ---------------------------------------------------------------------------------------------
 template <class G, int NA, int MASK>
 __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void analysis_kernel(const float* __restrict__ x, const float* __restrict__ mask,
                                                                                 const float* __restrict__ Tf, float4* __restrict__ rec,
-                                                                                long nbatch, const float* __restrict__ params, int nfeature) {
+                                                                                long nbatch, const float* __restrict__ params, int nfeature,
+                                                                                int nparts) {
   static_assert(MASK != 2, "bit masks exist on the 64^3 grid only");
   constexpr bool MASKED = MASK == 1 || MASK == 4;
   constexpr int N = G::N, R = G::R, PITCH = G::PITCH, THREADS = G::THREADS, NJ = G::NJ, NR = G::NR, NIT = G::NIT;
   __shared__ __attribute__((aligned(16))) float2 work[G::LDS_ELEMS];
   __shared__ __attribute__((aligned(16))) float2 quad[G::QUAD_ELEMS];
-  const long z = volume_of_block(nbatch);
-  if (z < 0) return;
+  const long vp = volume_of_block(nbatch * nparts);
+  if (vp < 0) return;
+  const long z = vp / nparts;
+  const int part = (int)(vp - z * nparts);
+  const int j0 = part * NJ / nparts, j1 = (part + 1) * NJ / nparts;
   const int t = threadIdx.x;
   const int lo = t % N, d = t / N;
   const bool in_a = G::A_THREADS == THREADS || t < G::A_THREADS;
@@ -396,13 +409,13 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void analysis_kernel
     }
   };
   __syncthreads();                                  // cleared quads
-  load_planes(0);
-  for (int j = 0; j < NJ; ++j) {
+  load_planes(j0);
+  for (int j = j0; j < j1; ++j) {
     stage_c1();
     // the next plane pair, in flight during the step.  Into registers: clamped, not branched (a branch would make the loads
     // synchronous); into LDS: none after the last pair (nothing would read them)
-    if constexpr (!G::DMA) load_planes(j + 1 < NJ ? j + 1 : NJ - 1);
-    else { __builtin_amdgcn_sched_barrier(0); if (j + 1 < NJ) load_planes(j + 1); }
+    if constexpr (!G::DMA) load_planes(j + 1 < j1 ? j + 1 : j1 - 1);
+    else { __builtin_amdgcn_sched_barrier(0); if (j + 1 < j1) load_planes(j + 1); }
     step_barrier();
     if (t >= G::B_COLS_FIRST && t < G::B_COLS_FIRST + G::B_THREADS) pass_b<G, false, false>(work, t - G::B_COLS_FIRST);
     step_barrier();
@@ -416,7 +429,7 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void analysis_kernel
     for (int it = 0; it < NA; ++it) accumulate(it);
   }
 
-  const __amdgpu_buffer_rsrc_t rr = make_rsrc(rec + (size_t)z * G::REC_F4, (unsigned)G::REC_BYTES);
+  const __amdgpu_buffer_rsrc_t rr = make_rsrc(rec + (size_t)vp * G::REC_F4, (unsigned)G::REC_BYTES);      // record [z][part]
 #pragma unroll
   for (int it = 0; it < NA; ++it) {                 // the pass that follows reads these rounds only
     buf_store_f32x4(make_float4(accp[it][0].x, accp[it][0].y, accp[it][1].x, accp[it][1].y), rr, toff, (it * 4 + 0) * (THREADS * 16));
@@ -432,12 +445,14 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void analysis_kernel
 // Every item adds its share of the bins of a plane pair to a place of its own in a staging area (its number); a reduction
 // sums the places of each column (a, n), one per degree group c >= max(a, n) / 4, in that order, into the plane.
 // bias, relu, MOM, moments, yref, params: as fused64::synthesis_kernel (no bit masks).
+// nparts: workgroups per volume (1 with MOM): part p reads the volume's record and writes the planes of its beta pairs.
 // ---------------------------------------------------------------------------------------------
 template <class G, int NA, int MOM>
 __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void synthesis_kernel(const float4* __restrict__ rec, const float* __restrict__ Tf,
                                                                                  float* __restrict__ y, long nbatch, const float* __restrict__ bias,
                                                                                  int nfeature, int relu, float2* __restrict__ moments,
-                                                                                 const float* __restrict__ yref, const float* __restrict__ params) {
+                                                                                 const float* __restrict__ yref, const float* __restrict__ params,
+                                                                                 int nparts) {
   constexpr int N = G::N, R = G::R, PITCH = G::PITCH, THREADS = G::THREADS, NJ = G::NJ, NR = G::NR, NIT = G::NIT;
   __shared__ __attribute__((aligned(16))) float2 work[G::LDS_ELEMS];
   // places 0 .. NITEMS-1: one per item; ZERO_PLACE: never written, read for the degree groups a column does not have;
@@ -448,8 +463,11 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void synthesis_kerne
   __shared__ __attribute__((aligned(16))) float4 stg[2 * NPLACES];
   float4* const stg_p = stg;                 // the item's share of the bins [+a,n], [-a,-n]
   float4* const stg_m = stg + NPLACES;       //                              [-a,n], [+a,-n]
-  const long z = volume_of_block(nbatch);
-  if (z < 0) return;
+  const long vp = volume_of_block(nbatch * nparts);
+  if (vp < 0) return;
+  const long z = vp / nparts;
+  const int part = (int)(vp - z * nparts);
+  const int j0 = part * NJ / nparts, j1 = (part + 1) * NJ / nparts;
   const int t = threadIdx.x;
   const int lo = t % N, d = t / N;
   const float bz = bias ? bias[z % nfeature] : 0.f;
@@ -570,7 +588,7 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void synthesis_kerne
     dft_r<R, true>(v, [&](int k, float2 x) {
       float ra = x.x + bz, rb = x.y + bz;
       if constexpr (MOM == 1) {
-        if (j == 0 && k == 0) mpivot = ra;
+        if (j == j0 && k == 0) mpivot = ra;
         const float da = ra - mpivot, db = rb - mpivot;
         ms1 += da + db; ms2 = fmaf(da, da, fmaf(db, db, ms2));
       }
@@ -585,11 +603,11 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void synthesis_kerne
   };
   const bool in_store = t >= G::B_COLS_FIRST && t < G::B_COLS_FIRST + G::B_THREADS;
 
-  load_table(0);
+  load_table(j0);
   __syncthreads();                                  // cleared work and staging
 #pragma unroll
   for (int it = 0; it < NA; ++it) contribute(it);
-  if (G::B_COLS_FIRST < (G::B_THREADS + 63) / 64 * 64) load_table(1);
+  if (G::B_COLS_FIRST < (G::B_THREADS + 63) / 64 * 64) load_table(j0 + 1 < j1 ? j0 + 1 : j1 - 1);
   __syncthreads();
   reduce();
   __syncthreads();
@@ -600,8 +618,8 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void synthesis_kerne
   constexpr int ROW_B_END = (G::B_THREADS + 63) / 64 * 64;
   constexpr bool SPLIT = ROW_B_END <= G::B_COLS_FIRST;
   const bool early = t >= ROW_B_END;
-  for (int j = 0; j < NJ; ++j) {
-    const bool more = j + 1 < NJ;
+  for (int j = j0; j < j1; ++j) {
+    const bool more = j + 1 < j1;
     if (!SPLIT && more) {
 #pragma unroll
       for (int it = 0; it < NA; ++it) contribute(it);
@@ -627,7 +645,7 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void synthesis_kerne
       for (int it = 0; it < NA; ++it) contribute(it);
     }
     if (more) {
-      if (!SPLIT) load_table(j + 2 < NJ ? j + 2 : NJ - 1);      // only now: its registers are not held through the transform
+      if (!SPLIT) load_table(j + 2 < j1 ? j + 2 : j1 - 1);      // only now: its registers are not held through the transform
       __syncthreads();
       reduce();
       __syncthreads();
@@ -681,43 +699,44 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void synthesis_kerne
 
 // Launchers: the instantiation whose item rounds cover the nl degrees present.
 template <class G, int MASK>
-inline void launch_analysis_m(int nl, hipStream_t st, const s2cnn::Input& in, const float* Tf, float4* rec, long nbatch) {
-  const dim3 grid(grid_size(nbatch)), block(G::THREADS);
+inline void launch_analysis_m(int nl, hipStream_t st, const s2cnn::Input& in, const float* Tf, float4* rec, long nbatch, int nparts) {
+  const dim3 grid(grid_size(nbatch * nparts)), block(G::THREADS);
   const int na = G::active_rounds(nl);
   static_assert(G::NIT <= 3, "add the instantiations of more rounds");
-  if (na <= 1) hipLaunchKernelGGL((analysis_kernel<G, 1, MASK>), grid, block, 0, st, in.x, in.w, Tf, rec, nbatch, in.params, in.nfeature);
-  else if (na == 2 || G::NIT < 3) hipLaunchKernelGGL((analysis_kernel<G, (G::NIT < 2 ? G::NIT : 2), MASK>), grid, block, 0, st, in.x, in.w, Tf, rec, nbatch, in.params, in.nfeature);
-  else hipLaunchKernelGGL((analysis_kernel<G, G::NIT, MASK>), grid, block, 0, st, in.x, in.w, Tf, rec, nbatch, in.params, in.nfeature);
+  if (na <= 1) hipLaunchKernelGGL((analysis_kernel<G, 1, MASK>), grid, block, 0, st, in.x, in.w, Tf, rec, nbatch, in.params, in.nfeature, nparts);
+  else if (na == 2 || G::NIT < 3) hipLaunchKernelGGL((analysis_kernel<G, (G::NIT < 2 ? G::NIT : 2), MASK>), grid, block, 0, st, in.x, in.w, Tf, rec, nbatch, in.params, in.nfeature, nparts);
+  else hipLaunchKernelGGL((analysis_kernel<G, G::NIT, MASK>), grid, block, 0, st, in.x, in.w, Tf, rec, nbatch, in.params, in.nfeature, nparts);
 }
 
 // in: the signal and what is done to it in the loads (s2cnn::Input; not PRO_BITS)
 template <class G>
-inline void launch_analysis(int nl, hipStream_t st, const s2cnn::Input& in, const float* Tf, float4* rec, long nbatch) {
+inline void launch_analysis(int nl, hipStream_t st, const s2cnn::Input& in, const float* Tf, float4* rec, long nbatch, int nparts) {
   switch (in.kind) {
-    case s2cnn::PRO_MASK: launch_analysis_m<G, 1>(nl, st, in, Tf, rec, nbatch); break;
-    case s2cnn::PRO_AFFINE_RELU: launch_analysis_m<G, 3>(nl, st, in, Tf, rec, nbatch); break;
-    case s2cnn::PRO_BN_RELU_GRAD: launch_analysis_m<G, 4>(nl, st, in, Tf, rec, nbatch); break;
-    default: launch_analysis_m<G, 0>(nl, st, in, Tf, rec, nbatch);
+    case s2cnn::PRO_MASK: launch_analysis_m<G, 1>(nl, st, in, Tf, rec, nbatch, nparts); break;
+    case s2cnn::PRO_AFFINE_RELU: launch_analysis_m<G, 3>(nl, st, in, Tf, rec, nbatch, nparts); break;
+    case s2cnn::PRO_BN_RELU_GRAD: launch_analysis_m<G, 4>(nl, st, in, Tf, rec, nbatch, nparts); break;
+    default: launch_analysis_m<G, 0>(nl, st, in, Tf, rec, nbatch, nparts);
   }
 }
 
 template <class G, int MOM>
 inline void launch_synthesis_m(int nl, hipStream_t st, const float4* rec, const float* Tf, float* y, long nbatch, const float* bias,
-                               int nfeature, int relu, float2* moments, const float* yref, const float* params) {
-  const dim3 grid(grid_size(nbatch)), block(G::THREADS);
+                               int nfeature, int relu, float2* moments, const float* yref, const float* params, int nparts) {
+  const dim3 grid(grid_size(nbatch * nparts)), block(G::THREADS);
   const int na = G::active_rounds(nl);
-  if (na <= 1) hipLaunchKernelGGL((synthesis_kernel<G, 1, MOM>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, moments, yref, params);
-  else if (na == 2 || G::NIT < 3) hipLaunchKernelGGL((synthesis_kernel<G, (G::NIT < 2 ? G::NIT : 2), MOM>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, moments, yref, params);
-  else hipLaunchKernelGGL((synthesis_kernel<G, G::NIT, MOM>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, moments, yref, params);
+  if (na <= 1) hipLaunchKernelGGL((synthesis_kernel<G, 1, MOM>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, moments, yref, params, nparts);
+  else if (na == 2 || G::NIT < 3) hipLaunchKernelGGL((synthesis_kernel<G, (G::NIT < 2 ? G::NIT : 2), MOM>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, moments, yref, params, nparts);
+  else hipLaunchKernelGGL((synthesis_kernel<G, G::NIT, MOM>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, moments, yref, params, nparts);
 }
 
 // moments: NULL, or two sums per volume: those of the output, or, with yref and params, those of the gradient of a normalisation
+// (one workgroup per volume then, whatever nparts says)
 template <class G>
 inline void launch_synthesis(int nl, hipStream_t st, const float4* rec, const float* Tf, float* y, long nbatch, const float* bias,
-                             int nfeature, int relu, float2* moments = nullptr, const float* yref = nullptr, const float* params = nullptr) {
-  if (moments && yref) launch_synthesis_m<G, 2>(nl, st, rec, Tf, y, nbatch, bias, nfeature, relu, moments, yref, params);
-  else if (moments) launch_synthesis_m<G, 1>(nl, st, rec, Tf, y, nbatch, bias, nfeature, relu, moments, nullptr, nullptr);
-  else launch_synthesis_m<G, 0>(nl, st, rec, Tf, y, nbatch, bias, nfeature, relu, nullptr, nullptr, nullptr);
+                             int nfeature, int relu, int nparts, float2* moments = nullptr, const float* yref = nullptr, const float* params = nullptr) {
+  if (moments && yref) launch_synthesis_m<G, 2>(nl, st, rec, Tf, y, nbatch, bias, nfeature, relu, moments, yref, params, 1);
+  else if (moments) launch_synthesis_m<G, 1>(nl, st, rec, Tf, y, nbatch, bias, nfeature, relu, moments, nullptr, nullptr, 1);
+  else launch_synthesis_m<G, 0>(nl, st, rec, Tf, y, nbatch, bias, nfeature, relu, nullptr, nullptr, nullptr, nparts);
 }
 
 }  // namespace fused4r

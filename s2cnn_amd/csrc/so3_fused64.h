@@ -520,8 +520,9 @@ __device__ __forceinline__ int row_index(int info, int u, int kind, int nl) {
   return lmn_index(l, m, kind >= 2 ? -n : n);
 }
 
+// nparts: records per volume ([volume][part], see so3_fused4r.h); their sum is the volume's record
 template <class G = Geometry>
-__global__ __launch_bounds__(256) void spectrum_scatter(const float4* __restrict__ rec, float2* __restrict__ out, int nl, long nbatch) {
+__global__ __launch_bounds__(256) void spectrum_scatter(const float4* __restrict__ rec, float2* __restrict__ out, int nl, long nbatch, int nparts) {
   constexpr int THREADS = G::THREADS, REC_F4 = G::REC_F4, TILES = THREADS / IT_TILE;
   __shared__ float vals[IT_TILE * VLD];
   __shared__ int info[IT_TILE];
@@ -534,7 +535,11 @@ __global__ __launch_bounds__(256) void spectrum_scatter(const float4* __restrict
     const int e = th + 256 * r;
     const int item = e & 31, q = (e >> 5) & 3, zz = e >> 7;
     float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (z0 + zz < nbatch) v = rec[(size_t)(z0 + zz) * REC_F4 + (it * 4 + q) * THREADS + t0 + item];
+    if (z0 + zz < nbatch)
+      for (int p = 0; p < nparts; ++p) {
+        const float4 w = rec[((size_t)(z0 + zz) * nparts + p) * REC_F4 + (it * 4 + q) * THREADS + t0 + item];
+        v = make_float4(v.x + w.x, v.y + w.y, v.z + w.z, v.w + w.w);
+      }
     float* d = vals + item * VLD + (4 * q) * ZT + zz;
     d[0] = v.x; d[ZT] = v.y; d[2 * ZT] = v.z; d[3 * ZT] = v.w;
   }
@@ -637,7 +642,7 @@ __device__ __forceinline__ RowRule row_rule(int inf, int rs, int nl) {
 }
 
 template <class G = Geometry>
-__global__ __launch_bounds__(256) void spectrum_scatter_real(const float4* __restrict__ rec, float* __restrict__ out, int nl, long nbatch) {
+__global__ __launch_bounds__(256) void spectrum_scatter_real(const float4* __restrict__ rec, float* __restrict__ out, int nl, long nbatch, int nparts) {
   constexpr int THREADS = G::THREADS, REC_F4 = G::REC_F4, TILES = THREADS / IT_TILE_R;
   __shared__ float vals[IT_TILE_R * VLD_R];
   __shared__ RowRule rules[IT_TILE_R * 16];
@@ -650,7 +655,11 @@ __global__ __launch_bounds__(256) void spectrum_scatter_real(const float4* __res
     const int e = th + 256 * r;
     const int item = e & 15, q = (e >> 4) & 3, zz = e >> 6;
     float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (z0 + zz < nbatch) v = rec[(size_t)(z0 + zz) * REC_F4 + (it * 4 + q) * THREADS + t0 + item];
+    if (z0 + zz < nbatch)
+      for (int p = 0; p < nparts; ++p) {
+        const float4 w = rec[((size_t)(z0 + zz) * nparts + p) * REC_F4 + (it * 4 + q) * THREADS + t0 + item];
+        v = make_float4(v.x + w.x, v.y + w.y, v.z + w.z, v.w + w.w);
+      }
     float* d = vals + item * VLD_R + (4 * q) * ZR + zz;
     d[0] = v.x; d[ZR] = v.y; d[2 * ZR] = v.z; d[3 * ZR] = v.w;
   }

@@ -70,7 +70,9 @@ def test_argument_rejection_without_gpu():
     assert packed12 == 23 * 24 * 256 * 4                                            # small problems of the two-stage path: 16 x 16 table values per beta
     assert lib.s2cnn_so3_packed_table_bytes(12, 12, 1) == 23 * 12 * 16 * 32 * 4        # ... and a 16 x 32 tile per degree in the synthesis
     assert lib.s2cnn_so3_packed_table_bytes(22, 22, 0) == 22 * 3 * 2 * 512 * 4 * 4 == lib.s2cnn_so3_packed_table_bytes(7, 22, 1)     # and the 44^3 grid: 22 beta pairs x 3 items x 2 x 512 threads
-    assert lib.s2cnn_so3_analysis_workspace(22, 7, 10, 0) == 10 * 12 * 512 * 16 + 22 * 3 * 2 * 512 * 4 * 4
+    assert lib.s2cnn_so3_analysis_workspace(22, 7, 200, 0) == 200 * 12 * 512 * 16 + 22 * 3 * 2 * 512 * 4 * 4
+    assert lib.s2cnn_so3_analysis_workspace(22, 7, 10, 0) == 10 * 4 * 12 * 512 * 16 + 22 * 3 * 2 * 512 * 4 * 4     # few volumes: four workgroups and records per volume
+    assert lib.s2cnn_so3_analysis_workspace(16, 16, 100, 0) == 100 * 2 * 8 * 256 * 16 + packed16                    # two
     assert lib.s2cnn_so3_packed_table_bytes(20, 20, 0) == 39 * 40 * 1024 * 4 and lib.s2cnn_so3_packed_table_bytes(20, 20, 1) == 39 * 20 * 2048 * 4
     assert lib.s2cnn_so3_analysis_workspace(12, 12, 256, 0) == 256 * 24 * 23 * 12 * 8 + packed12
     assert lib.s2cnn_so3_relu_bits_bytes(32, 3) == 3 * 64 * 64 * 8 and lib.s2cnn_so3_relu_bits_bytes(16, 3) == 0     # bit masks: the 64^3 grid only
