@@ -168,13 +168,13 @@ int s2cnn_so3_analysis(const float *x, const float *table, const float *packed_t
  * with its scratch in a buffer that the library itself holds, S2CNN_STATIC_SCRATCH_BYTES per GPU from the
  * moment the library is loaded until the process ends.  Calls nothing that allocates.
  *   - sizes whose s2cnn_so3_analysis_workspace(...) exceeds S2CNN_STATIC_SCRATCH_BYTES are rejected with
- *     S2CNN_ETOOBIG (real signals on the 64^3 grid: up to 130 volumes per call);
+ *     S2CNN_ETOOBIG (real signals on the 64^3 grid: up to 276 volumes per call);
  *   - all calls on one GPU share that GPU's buffer: calls that overlap in time on one GPU (different
  *     streams or threads) race; calls on one stream are ordered and safe;
  *   - the first call on a GPU resolves the buffer's address for it (no allocation; make it outside a graph capture);
  *   - results are those of s2cnn_so3_analysis bit for bit.
  */
-#define S2CNN_STATIC_SCRATCH_BYTES (32u << 20)
+#define S2CNN_STATIC_SCRATCH_BYTES (64u << 20)
 int s2cnn_so3_analysis_static(const float *x, const float *table, const float *packed_table, float *out,
                               int b_in, int b_out, long nbatch, int complex_in, void *stream);
 

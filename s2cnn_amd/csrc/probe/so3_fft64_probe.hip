@@ -18,12 +18,12 @@ extern "C" int s2cnn_so3_fft64_probe(const float* x, float* y, const float* pack
   float4* rec = static_cast<float4*>(workspace);
   const dim3 grid(grid_size(nbatch)), block(THREADS);
   if (direction == 0) {
-    if (probe == 1) hipLaunchKernelGGL((analysis_kernel<7, 0, 1>), grid, block, 0, st, x, nullptr, packed_table, rec, nbatch, nullptr, 1);
-    else if (probe == 2) hipLaunchKernelGGL((analysis_kernel<7, 0, 2>), grid, block, 0, st, x, nullptr, packed_table, rec, nbatch, nullptr, 1);
-    else hipLaunchKernelGGL((analysis_kernel<7, 0, 0>), grid, block, 0, st, x, nullptr, packed_table, rec, nbatch, nullptr, 1);
+    if (probe == 1) hipLaunchKernelGGL((analysis_kernel<7, 0, 1>), grid, block, 0, st, x, nullptr, packed_table, rec, nbatch, nullptr, 1, 1);
+    else if (probe == 2) hipLaunchKernelGGL((analysis_kernel<7, 0, 2>), grid, block, 0, st, x, nullptr, packed_table, rec, nbatch, nullptr, 1, 1);
+    else hipLaunchKernelGGL((analysis_kernel<7, 0, 0>), grid, block, 0, st, x, nullptr, packed_table, rec, nbatch, nullptr, 1, 1);
   } else {
-    if (probe == 1) hipLaunchKernelGGL((synthesis_kernel<7, 1>), grid, block, 0, st, rec, packed_table, y, nbatch, nullptr, 1, 0, nullptr, nullptr, nullptr, nullptr);
-    else hipLaunchKernelGGL((synthesis_kernel<7, 0>), grid, block, 0, st, rec, packed_table, y, nbatch, nullptr, 1, 0, nullptr, nullptr, nullptr, nullptr);
+    if (probe == 1) hipLaunchKernelGGL((synthesis_kernel<7, 1>), grid, block, 0, st, rec, packed_table, y, nbatch, nullptr, 1, 0, nullptr, nullptr, nullptr, nullptr, 1);
+    else hipLaunchKernelGGL((synthesis_kernel<7, 0>), grid, block, 0, st, rec, packed_table, y, nbatch, nullptr, 1, 0, nullptr, nullptr, nullptr, nullptr, 1);
   }
   return s2cnn::launch_status();
 }

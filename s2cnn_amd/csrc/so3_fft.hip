@@ -412,10 +412,10 @@ int fused_analysis(FusedKind kind, const s2cnn::Input& in, const float* table, c
   const unsigned tiles_r = (unsigned)((nbatch + fused64::ZR - 1) / fused64::ZR), tiles_c = (unsigned)((nbatch + fused64::ZT - 1) / fused64::ZT);
   float2* outc = reinterpret_cast<float2*>(out);
   if (kind == FUSED_64) {
-    const int rounds = fused64::active_rounds(b_out);
-    fused64::launch_analysis(b_out, st, in, Tf, rec, nbatch);
-    if (real_basis) hipLaunchKernelGGL(fused64::spectrum_scatter_real<>, dim3(tiles_r, rounds * 32), dim3(256), 0, st, rec, out, b_out, nbatch, 1);
-    else hipLaunchKernelGGL(fused64::spectrum_scatter<>, dim3(tiles_c, rounds * 16), dim3(256), 0, st, rec, outc, b_out, nbatch, 1);
+    const int rounds = fused64::active_rounds(b_out), nparts = fused64::parts(nbatch);
+    fused64::launch_analysis(b_out, st, in, Tf, rec, nbatch, nparts);
+    if (real_basis) hipLaunchKernelGGL(fused64::spectrum_scatter_real<>, dim3(tiles_r, rounds * 32), dim3(256), 0, st, rec, out, b_out, nbatch, nparts);
+    else hipLaunchKernelGGL(fused64::spectrum_scatter<>, dim3(tiles_c, rounds * 16), dim3(256), 0, st, rec, outc, b_out, nbatch, nparts);
   } else {
     with_grid(kind, [&](auto g) { fused4r_analysis<decltype(g)>(in, Tf, rec, out, b_out, nbatch, real_basis, st); return 0; });
   }
@@ -447,7 +447,7 @@ int fused_synthesis(FusedKind kind, const float* xhat, const float* table, const
     const int rounds = fused64::active_rounds(nl);
     if (real_basis) hipLaunchKernelGGL(fused64::spectrum_gather_real<>, dim3(tiles_r, rounds * 32), dim3(256), 0, st, xhat, rec, nl, nbatch);
     else hipLaunchKernelGGL(fused64::spectrum_gather<>, dim3(tiles_c, rounds * 16), dim3(256), 0, st, xc, rec, nl, nbatch);
-    fused64::launch_synthesis(nl, st, rec, Tf, out, nbatch, bias, nfeature, relu, bits, mom, yref, params);
+    fused64::launch_synthesis(nl, st, rec, Tf, out, nbatch, bias, nfeature, relu, bits, mom, yref, params, fused64::parts(nbatch));
   } else {
     with_grid(kind, [&](auto g) {
       fused4r_synthesis<decltype(g)>(xhat, Tf, rec, out, nl, nbatch, real_basis, bias, nfeature, relu, st, mom, yref, params);

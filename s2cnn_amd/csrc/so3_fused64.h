@@ -179,7 +179,13 @@ inline unsigned grid_size(long nbatch) { return (unsigned)(8 * ((nbatch + 7) / 8
 // (re, im, re, im); q = 1: (+a) u = 2, 3; q = 2, 3: the same for (-a).
 constexpr int REC_F4 = NIT * 4 * THREADS;                 // float4 per record
 constexpr size_t REC_BYTES = (size_t)REC_F4 * 16;         // 229376
-inline size_t scratch_bytes(long nbatch) { return (size_t)nbatch * REC_BYTES; }
+// workgroups per volume: a power of two, at least four beta pairs each, no more than fill the chip once
+inline int parts(long nbatch) {
+  int p = 1;
+  while (2 * p * 4 <= NJ && 2 * p * nbatch <= 256) p *= 2;
+  return p;
+}
+inline size_t scratch_bytes(long nbatch) { return (size_t)nbatch * parts(nbatch) * REC_BYTES; }
 
 // ---------------------------------------------------------------------------------------------
 // analysis: x [nbatch][64][64][64] real -> records of the half spectrum n >= 0
@@ -218,17 +224,21 @@ __host__ __device__ inline size_t bits_index(long z, int beta, int d) { return (
 // PROBE (measurement only, results meaningless): 1: the Wigner contraction of an item reduced to one add per table
 // operand (table loads, LDS reads of the quads and everything else kept); 2: the table loads gone as well.  What is left
 // is the plane pipeline: loads, the 2-D transform through LDS with its barriers, the quad layout, the record.
-template <int NA, int MASK, int PROBE = 0>
+template <int NA, int MASK, int PROBE = 0, bool SPLIT = false>
 __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MASK == 0 || MASK == 2 || MASK == 3)) void analysis_kernel(const float* __restrict__ x, const float* __restrict__ mask,
                                                            const float* __restrict__ Tf, float4* __restrict__ rec, long nbatch,
-                                                           const float* __restrict__ params, int nfeature) {
+                                                           const float* __restrict__ params, int nfeature, int nparts) {
   constexpr bool MASKED = MASK == 1 || MASK == 4;      // a second tensor is loaded beside x
   using namespace fft64;
   __shared__ __attribute__((aligned(16))) float2 work[LDS_ELEMS];
   constexpr int NR = rows_kept(NA), QUAD_ELEMS = quad_elems(NR);
   __shared__ __attribute__((aligned(16))) float2 quad[2][QUAD_ELEMS];
-  const long z = volume_of_block(nbatch);
-  if (z < 0) return;
+  // nparts workgroups per volume (few volumes do not fill the chip with one each): part p takes the beta pairs
+  // p NJ / nparts .. (p+1) NJ / nparts - 1 and writes a record of its own, [volume][part]; spectrum_scatter adds them
+  const long vp = volume_of_block(nbatch * nparts);
+  if (vp < 0) return;
+  const long z = vp / nparts;
+  const int j0 = SPLIT ? (int)(vp - z * nparts) * NJ / nparts : 0, j1 = SPLIT ? ((int)(vp - z * nparts) + 1) * NJ / nparts : NJ;
   const int t = threadIdx.x;
   const int lo = t & 63, d = t >> 6;
   Twiddles twl;
@@ -386,18 +396,18 @@ __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MASK == 0 || MASK == 2 
   };
 
   // first plane pair: transformed alone
-  load_planes(0);
-  load_table(0, 0);
-  if constexpr (NA > 1) load_table(0, 1);
-  if constexpr (NA > 2) load_table(0, 2);
-  if constexpr (NA > 3) load_table(0, 3);
+  load_planes(j0);
+  load_table(j0, 0);
+  if constexpr (NA > 1) load_table(j0, 1);
+  if constexpr (NA > 2) load_table(j0, 2);
+  if constexpr (NA > 3) load_table(j0, 3);
   __syncthreads();                              // cleared quads
   stage_c1();
-  load_planes(1);
+  load_planes(j0 + 1);                          // a part has at least two pairs
   __syncthreads();
   fft_pass<false, 3>(work, twl); __syncthreads();
   fft_pass<false, 0>(work, twl); __syncthreads();
-  stage_r2(quad[0]); __syncthreads();
+  stage_r2(quad[j0 & 1]); __syncthreads();
 
   // step j: contract pair j out of quad[j & 1] while pair j+1 is transformed into quad[(j+1) & 1].
   // The scheduling fences keep the parts of a stage in program order.
@@ -415,10 +425,10 @@ __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MASK == 0 || MASK == 2 
   // wave of either kind, so its LDS-bound and its FMA-bound half of a stage overlap.
   if (d < 4) {
     constexpr unsigned FR = FRESH_LO;
-    for (int j = 0; j < NJ - 1; ++j) {
+    for (int j = j0; j < j1 - 1; ++j) {
       const float2* cur = quad[j & 1];
       float2* nxt = quad[(j + 1) & 1];
-      const int jp = j + 2 < NJ ? j + 2 : NJ - 1;     // clamped, not branched: a branch would make the loads synchronous
+      const int jp = j + 2 < j1 ? j + 2 : j1 - 1;     // clamped, not branched: a branch would make the loads synchronous
       stage_c1(); S2CNN_FENCE();
       S2CNN_PLANES(0) S2CNN_ACC(0, j, 4) S2CNN_PLANES(1) S2CNN_ACC(1, j, 5)
       __syncthreads();
@@ -434,10 +444,10 @@ __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MASK == 0 || MASK == 2 
     }
   } else {
     constexpr unsigned FR = FRESH_HI;
-    for (int j = 0; j < NJ - 1; ++j) {
+    for (int j = j0; j < j1 - 1; ++j) {
       const float2* cur = quad[j & 1];
       float2* nxt = quad[(j + 1) & 1];
-      const int jp = j + 2 < NJ ? j + 2 : NJ - 1;
+      const int jp = j + 2 < j1 ? j + 2 : j1 - 1;
       S2CNN_ACC(0, j, 4) S2CNN_ACC(1, j, 5)
       stage_c1(); S2CNN_FENCE();
       S2CNN_PLANES(0) S2CNN_PLANES(1)
@@ -462,11 +472,11 @@ __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MASK == 0 || MASK == 2 
     }
   }
   {
-    const float2* cur = quad[(NJ - 1) & 1];
+    const float2* cur = quad[(j1 - 1) & 1];
 #define S2CNN_LAST(k)                                                                                    \
   if constexpr ((k) < NA) {                                                                              \
     accumulate(cur, k, FRESH_LO | FRESH_HI);                                                             \
-    if constexpr ((k) + 4 < NA) { S2CNN_FENCE(); load_table(NJ - 1, (k) + 4); S2CNN_FENCE(); }           \
+    if constexpr ((k) + 4 < NA) { S2CNN_FENCE(); load_table(j1 - 1, (k) + 4); S2CNN_FENCE(); }           \
   }
     S2CNN_LAST(0) S2CNN_LAST(1) S2CNN_LAST(2) S2CNN_LAST(3) S2CNN_LAST(4) S2CNN_LAST(5) S2CNN_LAST(6)
 #undef S2CNN_LAST
@@ -475,7 +485,7 @@ __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MASK == 0 || MASK == 2 
 #undef S2CNN_PLANES
 #undef S2CNN_FENCE
 
-  const __amdgpu_buffer_rsrc_t rr = make_rsrc(rec + (size_t)z * REC_F4, (unsigned)REC_BYTES);
+  const __amdgpu_buffer_rsrc_t rr = make_rsrc(rec + (size_t)vp * REC_F4, (unsigned)REC_BYTES);      // record [z][part]
 #pragma unroll
   for (int it = 0; it < NA; ++it) {            // the pass that follows reads these rounds only
     buf_store_f32x4(make_float4(accp[it][0].x, accp[it][0].y, accp[it][1].x, accp[it][1].y), rr, toff, (it * 4 + 0) * (THREADS * 16));
@@ -759,11 +769,11 @@ __global__ __launch_bounds__(256) void spectrum_gather_real(const float* __restr
 //   2: (sum v m, sum v m w) with w = yref at the same sample and m = (a w + b > 0), a = params[f], b = params[nfeature + f],
 //      f = z % nfeature: the two reductions of the gradient of such a normalisation followed by max(., 0), with the
 //      output as the incoming gradient (s2cnn::bn_relu_grad).
-template <int NA, int PROBE = 0, int MOM = 0>
+template <int NA, int PROBE = 0, int MOM = 0, bool SPLIT = false>
 __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MOM == 0)) void synthesis_kernel(const float4* __restrict__ rec, const float* __restrict__ Tf,
                                                             float* __restrict__ y, long nbatch, const float* __restrict__ bias, int nfeature,
                                                             int relu, unsigned long long* __restrict__ bits, float2* __restrict__ moments,
-                                                            const float* __restrict__ yref, const float* __restrict__ params) {
+                                                            const float* __restrict__ yref, const float* __restrict__ params, int nparts) {
   using namespace fft64;
   __shared__ __attribute__((aligned(16))) float2 work[LDS_ELEMS];
   float ms1 = 0.f, ms2 = 0.f;
@@ -772,8 +782,11 @@ __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MOM == 0)) void synthes
   constexpr int NCOL = NR * NR;                                               // columns (a, n)
   __shared__ __attribute__((aligned(16))) float4 stg_p[2 * NCOL];             // [run of the column][NR a + n]: the run's share of the bins [+a,n], [-a,-n]
   __shared__ __attribute__((aligned(16))) float4 stg_m[2 * NCOL];             //                                                            [-a,n], [+a,-n]
-  const long z = volume_of_block(nbatch);
-  if (z < 0) return;
+  // nparts workgroups per volume (1 with MOM): part p reads the volume's record and writes the planes of its beta pairs
+  const long vp = volume_of_block(nbatch * nparts);
+  if (vp < 0) return;
+  const long z = vp / nparts;
+  const int j0 = SPLIT ? (int)(vp - z * nparts) * NJ / nparts : 0, j1 = SPLIT ? ((int)(vp - z * nparts) + 1) * NJ / nparts : NJ;
   const int t = threadIdx.x;
   const int lo = t & 63, d = t >> 6;
   const float bz = bias ? bias[z % nfeature] : 0.f;
@@ -898,7 +911,7 @@ __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MOM == 0)) void synthes
     for (int k = 0; k < 8; ++k) {
       float ra = v[k].x + bz, rb = v[k].y + bz;
       if constexpr (MOM == 1) {
-        if (j == 0 && k == 0) mpivot = ra;
+        if (j == j0 && k == 0) mpivot = ra;
         const float da = ra - mpivot, db = rb - mpivot;
         ms1 += da + db; ms2 = fmaf(da, da, fmaf(db, db, ms2));
       }
@@ -926,18 +939,18 @@ __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MOM == 0)) void synthes
 #define S2CNN_CON(k, P)                                                                                  \
   if constexpr ((k) < NA) {                                                                              \
     contribute(k, FR); S2CNN_FENCE();                                                                    \
-    if constexpr ((k) + 4 < NA) load_table((P) < NJ ? (P) : NJ - 1, (k) + 4);                            \
-    else load_table((P) + 1 < NJ ? (P) + 1 : NJ - 1, (k) & 3);                                           \
+    if constexpr ((k) + 4 < NA) load_table((P) < j1 ? (P) : j1 - 1, (k) + 4);                            \
+    else load_table((P) + 1 < j1 ? (P) + 1 : j1 - 1, (k) & 3);                                           \
     S2CNN_FENCE();                                                                                       \
   }
-  load_table(0, 0);
-  if constexpr (NA > 1) load_table(0, 1);
-  if constexpr (NA > 2) load_table(0, 2);
-  if constexpr (NA > 3) load_table(0, 3);
+  load_table(j0, 0);
+  if constexpr (NA > 1) load_table(j0, 1);
+  if constexpr (NA > 2) load_table(j0, 2);
+  if constexpr (NA > 3) load_table(j0, 3);
   __syncthreads();
   {
     constexpr unsigned FR = FRESH_LO | FRESH_HI;
-    S2CNN_CON(0, 0) S2CNN_CON(1, 0) S2CNN_CON(2, 0) S2CNN_CON(3, 0) S2CNN_CON(4, 0) S2CNN_CON(5, 0) S2CNN_CON(6, 0)
+    S2CNN_CON(0, j0) S2CNN_CON(1, j0) S2CNN_CON(2, j0) S2CNN_CON(3, j0) S2CNN_CON(4, j0) S2CNN_CON(5, j0) S2CNN_CON(6, j0)
   }
   __syncthreads();
   reduce();
@@ -948,7 +961,7 @@ __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MOM == 0)) void synthes
   // and the FMA-bound half of a stage overlap.
   if (d < 4) {
     constexpr unsigned FR = FRESH_LO;
-    for (int j = 0; j < NJ - 1; ++j) {
+    for (int j = j0; j < j1 - 1; ++j) {
       fft_pass<true, 0>(work, twl); S2CNN_FENCE();
       S2CNN_CON(0, j + 1) S2CNN_CON(1, j + 1)
       __syncthreads();
@@ -966,7 +979,7 @@ __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MOM == 0)) void synthes
     }
   } else {
     constexpr unsigned FR = FRESH_HI;
-    for (int j = 0; j < NJ - 1; ++j) {
+    for (int j = j0; j < j1 - 1; ++j) {
       S2CNN_CON(0, j + 1) S2CNN_CON(1, j + 1)
       fft_pass<true, 0>(work, twl);
       __syncthreads();
@@ -988,7 +1001,7 @@ __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MOM == 0)) void synthes
   fft_pass<true, 0>(work, twl); __syncthreads();
   fft_pass<true, 1>(work, twl); __syncthreads();
   fft_pass<true, 2>(work, twl); __syncthreads();
-  stage_c2_store(NJ - 1);
+  stage_c2_store(j1 - 1);
   if constexpr (MOM == 1) {                         // (mean, squared deviations) of every thread's 2 x 8 x 32 samples, merged pairwise in float64
     __syncthreads();
     double* red = reinterpret_cast<double*>(work);
@@ -1025,22 +1038,29 @@ __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MOM == 0)) void synthes
 inline int active_rounds(int nl) { return nl <= 24 ? 3 : nl <= 28 ? 6 : NIT; }
 
 // Launchers: the instantiation whose item rounds cover the nl degrees present.
+template <int MASK, bool SPLIT>
+inline void launch_analysis_ms(int nl, hipStream_t st, const s2cnn::Input& in, const float* Tf, float4* rec, long nbatch, int nparts) {
+  const dim3 grid(grid_size(nbatch * nparts)), block(THREADS);
+  if (nl <= 24) hipLaunchKernelGGL((analysis_kernel<3, MASK, 0, SPLIT>), grid, block, 0, st, in.x, in.w, Tf, rec, nbatch, in.params, in.nfeature, nparts);
+  else if (nl <= 28) hipLaunchKernelGGL((analysis_kernel<6, MASK, 0, SPLIT>), grid, block, 0, st, in.x, in.w, Tf, rec, nbatch, in.params, in.nfeature, nparts);
+  else hipLaunchKernelGGL((analysis_kernel<7, MASK, 0, SPLIT>), grid, block, 0, st, in.x, in.w, Tf, rec, nbatch, in.params, in.nfeature, nparts);
+}
+
+// one workgroup per volume runs the instantiation whose plane loop has constant bounds
 template <int MASK>
-inline void launch_analysis_m(int nl, hipStream_t st, const s2cnn::Input& in, const float* Tf, float4* rec, long nbatch) {
-  const dim3 grid(grid_size(nbatch)), block(THREADS);
-  if (nl <= 24) hipLaunchKernelGGL((analysis_kernel<3, MASK>), grid, block, 0, st, in.x, in.w, Tf, rec, nbatch, in.params, in.nfeature);
-  else if (nl <= 28) hipLaunchKernelGGL((analysis_kernel<6, MASK>), grid, block, 0, st, in.x, in.w, Tf, rec, nbatch, in.params, in.nfeature);
-  else hipLaunchKernelGGL((analysis_kernel<7, MASK>), grid, block, 0, st, in.x, in.w, Tf, rec, nbatch, in.params, in.nfeature);
+inline void launch_analysis_m(int nl, hipStream_t st, const s2cnn::Input& in, const float* Tf, float4* rec, long nbatch, int nparts) {
+  if (nparts > 1) launch_analysis_ms<MASK, true>(nl, st, in, Tf, rec, nbatch, nparts);
+  else launch_analysis_ms<MASK, false>(nl, st, in, Tf, rec, nbatch, 1);
 }
 
 // in: the signal and what is done to it in the loads (s2cnn::Input)
-inline void launch_analysis(int nl, hipStream_t st, const s2cnn::Input& in, const float* Tf, float4* rec, long nbatch) {
+inline void launch_analysis(int nl, hipStream_t st, const s2cnn::Input& in, const float* Tf, float4* rec, long nbatch, int nparts = 1) {
   switch (in.kind) {
-    case s2cnn::PRO_MASK: launch_analysis_m<1>(nl, st, in, Tf, rec, nbatch); break;
-    case s2cnn::PRO_BITS: launch_analysis_m<2>(nl, st, in, Tf, rec, nbatch); break;
-    case s2cnn::PRO_AFFINE_RELU: launch_analysis_m<3>(nl, st, in, Tf, rec, nbatch); break;
-    case s2cnn::PRO_BN_RELU_GRAD: launch_analysis_m<4>(nl, st, in, Tf, rec, nbatch); break;
-    default: launch_analysis_m<0>(nl, st, in, Tf, rec, nbatch);
+    case s2cnn::PRO_MASK: launch_analysis_m<1>(nl, st, in, Tf, rec, nbatch, nparts); break;
+    case s2cnn::PRO_BITS: launch_analysis_m<2>(nl, st, in, Tf, rec, nbatch, nparts); break;
+    case s2cnn::PRO_AFFINE_RELU: launch_analysis_m<3>(nl, st, in, Tf, rec, nbatch, nparts); break;
+    case s2cnn::PRO_BN_RELU_GRAD: launch_analysis_m<4>(nl, st, in, Tf, rec, nbatch, nparts); break;
+    default: launch_analysis_m<0>(nl, st, in, Tf, rec, nbatch, nparts);
   }
 }
 
@@ -1050,24 +1070,32 @@ constexpr int GRAD_MOMENTS_MAX_NL = 28;
 
 // moments: NULL, or two sums per volume (see MOM): those of the output, or, with yref and params (nl <= GRAD_MOMENTS_MAX_NL
 // only), those of the gradient of a normalisation
+// nparts: workgroups per volume where no sums are formed (one with `moments`)
 inline void launch_synthesis(int nl, hipStream_t st, const float4* rec, const float* Tf, float* y, long nbatch, const float* bias,
                              int nfeature, int relu, unsigned long long* bits, float2* moments = nullptr, const float* yref = nullptr,
-                             const float* params = nullptr) {
-  const dim3 grid(grid_size(nbatch)), block(THREADS);
+                             const float* params = nullptr, int nparts = 1) {
+  if (moments) nparts = 1;
+  const dim3 grid(grid_size(nbatch * nparts)), block(THREADS);
   if (moments && yref) {
-    if (nl <= 24) hipLaunchKernelGGL((synthesis_kernel<3, 0, 2>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, yref, params);
-    else hipLaunchKernelGGL((synthesis_kernel<6, 0, 2>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, yref, params);
+    if (nl <= 24) hipLaunchKernelGGL((synthesis_kernel<3, 0, 2>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, yref, params, nparts);
+    else hipLaunchKernelGGL((synthesis_kernel<6, 0, 2>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, yref, params, nparts);
     return;
   }
   if (moments) {
-    if (nl <= 24) hipLaunchKernelGGL((synthesis_kernel<3, 0, 1>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, nullptr, nullptr);
-    else if (nl <= 28) hipLaunchKernelGGL((synthesis_kernel<6, 0, 1>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, nullptr, nullptr);
-    else hipLaunchKernelGGL((synthesis_kernel<7, 0, 1>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, nullptr, nullptr);
+    if (nl <= 24) hipLaunchKernelGGL((synthesis_kernel<3, 0, 1>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, nullptr, nullptr, nparts);
+    else if (nl <= 28) hipLaunchKernelGGL((synthesis_kernel<6, 0, 1>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, nullptr, nullptr, nparts);
+    else hipLaunchKernelGGL((synthesis_kernel<7, 0, 1>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, nullptr, nullptr, nparts);
     return;
   }
-  if (nl <= 24) hipLaunchKernelGGL((synthesis_kernel<3>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, nullptr, nullptr, nullptr);
-  else if (nl <= 28) hipLaunchKernelGGL((synthesis_kernel<6>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, nullptr, nullptr, nullptr);
-  else hipLaunchKernelGGL((synthesis_kernel<7>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, nullptr, nullptr, nullptr);
+  if (nparts > 1) {
+    if (nl <= 24) hipLaunchKernelGGL((synthesis_kernel<3, 0, 0, true>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, nullptr, nullptr, nullptr, nparts);
+    else if (nl <= 28) hipLaunchKernelGGL((synthesis_kernel<6, 0, 0, true>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, nullptr, nullptr, nullptr, nparts);
+    else hipLaunchKernelGGL((synthesis_kernel<7, 0, 0, true>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, nullptr, nullptr, nullptr, nparts);
+    return;
+  }
+  if (nl <= 24) hipLaunchKernelGGL((synthesis_kernel<3>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, nullptr, nullptr, nullptr, 1);
+  else if (nl <= 28) hipLaunchKernelGGL((synthesis_kernel<6>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, nullptr, nullptr, nullptr, 1);
+  else hipLaunchKernelGGL((synthesis_kernel<7>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, nullptr, nullptr, nullptr, 1);
 }
 
 }  // namespace fused64

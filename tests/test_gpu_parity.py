@@ -881,7 +881,7 @@ def test_so3_rft_kernel_spectrum(hip, factorised, monkeypatch):
 def test_so3_transforms_beyond_32_bit_offsets(hip, b, nz):
     """Batches whose tensors pass 2^31 elements (and 2^33 bytes): the last volumes must get the bits they get in a batch of
     their own, for the complex-pair and the real-basis spectra (per-volume kernels of the 64^3 and 44^3 grids).  The small
-    batches are 200 volumes: below 129 the analysis of the 44^3 grid gives a volume to several workgroups, which adds the
+    batches are 200 volumes: below 129 the analysis gives a volume to several workgroups, which adds the
     beta sum up in another order (the same numbers to rounding, not to the bit)."""
     if torch.cuda.mem_get_info()[0] < 60 * 2 ** 30:
         pytest.skip("needs 60 GiB of free device memory")
@@ -930,15 +930,20 @@ def test_s2_transforms_and_integral_beyond_32_bit_offsets(hip):
 
 
 def test_so3_round_trip_at_the_benchmark_size(hip):
-    """[256, 64, 64, 64] (the transform benchmark): every volume of the batch gets the bits it gets alone (the result
-    of a volume does not depend on the workgroup that takes it), and analysis o synthesis is the identity on spectra."""
+    """[256, 64, 64, 64] (the transform benchmark): every volume of the batch gets the bits it gets in another batch
+    that is split the same way (the result of a volume does not depend on the workgroup that takes it; 128 volumes
+    or fewer are split along beta over several workgroups, whose partial sums are added in another order, so a volume
+    alone agrees to rounding only), and analysis o synthesis is the identity on spectra."""
     g = torch.Generator(device="cuda").manual_seed(33)
     x = torch.randn(256, 64, 64, 64, device="cuda", generator=g)
     s = PSO3.so3_rfft(x)
     y = PSO3.so3_rifft(s)
+    for i in (0, 126):
+        assert torch.equal(PSO3.so3_rfft(x[i:i + 130].contiguous()), s[:, i:i + 130]), i
+        assert torch.equal(PSO3.so3_rifft(s[:, i:i + 130].contiguous()), y[i:i + 130]), i
     for i in (0, 7, 100, 255):
-        assert torch.equal(PSO3.so3_rfft(x[i:i + 1].contiguous())[:, 0], s[:, i]), i
-        assert torch.equal(PSO3.so3_rifft(s[:, i:i + 1].contiguous())[0], y[i]), i
+        close(PSO3.so3_rfft(x[i:i + 1].contiguous())[:, 0], s[:, i].cpu(), f"rfft of volume {i} alone")
+        assert torch.equal(PSO3.so3_rifft(s[:, i:i + 1].contiguous())[0], y[i]), i      # the synthesis adds nothing across workgroups
     s2 = PSO3.so3_rfft(y)
     rel = ((s2 - s).norm() / s.norm()).item()
     print(f"analysis(synthesis(s)) - s: rel L2 {rel:.2e}", flush=True)

@@ -30,6 +30,7 @@ def _both(lib, x, table, packed, b_in, b_out):
 
 @pytest.mark.parametrize("b_in,b_out,n_first,n_second", [(32, 32, 9, 4),      # per-volume kernels: scratch = one record per volume
                                                          (32, 22, 5, 2),      # truncated spectrum
+                                                         (32, 32, 128, 100),  # the largest scratch of few volumes: two records per volume
                                                          (16, 16, 21, 6),     # the per-volume kernels of the 32^3 grid
                                                          (16, 10, 9, 3),
                                                          (22, 22, 7, 3),      # ... and of the 44^3 grid
@@ -90,8 +91,8 @@ def test_static_scratch_analysis_allocates_nothing(hip):
 def test_static_scratch_rejects_what_does_not_fit(hip):
     dev = torch.device("cuda:0")
     fake = ctypes.c_void_p(torch.empty(64, device=dev).data_ptr())
-    limit = 32 << 20
-    assert hip.s2cnn_so3_analysis_workspace(32, 32, 147, 0) > limit
-    assert hip.s2cnn_so3_analysis_static(fake, fake, fake, fake, 32, 32, 147, 0, None) == -4     # S2CNN_ETOOBIG, before any launch
+    limit = 64 << 20
+    assert hip.s2cnn_so3_analysis_workspace(32, 32, 277, 0) > limit
+    assert hip.s2cnn_so3_analysis_static(fake, fake, fake, fake, 32, 32, 277, 0, None) == -4     # S2CNN_ETOOBIG, before any launch
     assert b"static" in hip.s2cnn_strerror(-4)
     assert hip.s2cnn_so3_analysis_static(None, fake, fake, fake, 32, 32, 1, 0, None) == -1
