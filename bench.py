@@ -436,7 +436,8 @@ def measure_fft_floor(torch, dev, nvol=256, reps=10):
     out = {}
     variants = [("analysis kernel", 0, 0), ("analysis kernel, no contraction multiply-adds", 0, 1),
                 ("analysis kernel, no contraction and no table loads", 0, 2),
-                ("synthesis kernel", 1, 0), ("synthesis kernel, no contraction multiply-adds", 1, 1)]
+                ("synthesis kernel", 1, 0), ("synthesis kernel, no contraction multiply-adds", 1, 1),
+                ("synthesis kernel, the contraction's multiply-adds as 4x4x1 matrix instructions", 1, 2)]
     for name, direction, probe in variants:
         def run():
             _hip.check(P.s2cnn_so3_fft64_probe(_hip.ptr(x), _hip.ptr(y), _hip.ptr(packed[direction]), _hip.ptr(ws), ws.numel(), nvol,

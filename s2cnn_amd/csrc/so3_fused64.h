@@ -830,12 +830,23 @@ __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MOM == 0)) void synthes
   // complex plane Z = S + i S' at [m,n], its Hermitian partner conj S + i conj S' at [-m,-n]
   // the sums of the current run: S = sum_l t1 xs, S' = sum_l s t2 xs at (+a, n), t1 <-> t2 at (-a, n)
   float2 Sp = make_float2(0.f, 0.f), Qp = make_float2(0.f, 0.f), Sm = make_float2(0.f, 0.f), Qm = make_float2(0.f, 0.f);
+  typedef float macc_t __attribute__((ext_vector_type(4)));
+  [[maybe_unused]] macc_t macc[4] = {};
   // fresh: as in analysis_kernel; a run can only end in front of a round that starts one, or in the last round
   auto contribute = [&](int it, unsigned fresh) {
     const float4 ta = t1[table_slot(it)], tb = t2[table_slot(it)];
     const float a1[4] = {ta.x, ta.y, ta.z, ta.w};
     const float a2[4] = {tb.x, tb.y, tb.z, tb.w};
-    if constexpr (PROBE != 0) {
+    if constexpr (PROBE == 2) {
+      // what the contraction would cost on the matrix pipe: 4 groups of 16 items x 4 degrees, one 4x4x1 instruction each
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        macc[0] = __builtin_amdgcn_mfma_f32_4x4x1f32(a1[u], xp[it][u].x, macc[0], 0, 0, 0);
+        macc[1] = __builtin_amdgcn_mfma_f32_4x4x1f32(a2[u], xp[it][u].y, macc[1], 0, 0, 0);
+        macc[2] = __builtin_amdgcn_mfma_f32_4x4x1f32(a1[u], xm[it][u].x, macc[2], 0, 0, 0);
+        macc[3] = __builtin_amdgcn_mfma_f32_4x4x1f32(a2[u], xm[it][u].y, macc[3], 0, 0, 0);
+      }
+    } else if constexpr (PROBE != 0) {
       Sp.x += a1[0] + xp[it][0].x; Sm.x += a2[0] + xm[it][0].x;
     } else {
 #pragma unroll
@@ -856,8 +867,15 @@ __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MOM == 0)) void synthes
       const float qpx = flip(Qp.x, sb), qpy = flip(Qp.y, sb), qmx = flip(Qm.x, sb), qmy = flip(Qm.y, sb);
       const unsigned col32 = e & 0x3ffu;                                        // 32 a + n
       const unsigned pos = ((e >> 14) & 1u) * NCOL + col32 - (32 - NR) * (col32 >> 5);
+      if constexpr (PROBE == 2) {
+        stg_p[pos] = make_float4(macc[0].x - macc[1].y, macc[0].y + macc[1].x, macc[0].x + macc[1].y, macc[1].x - macc[0].y);
+        stg_m[pos] = make_float4(macc[2].x - macc[3].y, macc[2].y + macc[3].x, macc[2].x + macc[3].y, macc[3].x - macc[2].y);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) macc[g] = macc_t{qpx, qpy, qmx, qmy};
+      } else {
       stg_p[pos] = make_float4(Sp.x - qpy, Sp.y + qpx, Sp.x + qpy, qpx - Sp.y);
       stg_m[pos] = make_float4(Sm.x - qmy, Sm.y + qmx, Sm.x + qmy, qmx - Sm.y);
+      }
       Sp = make_float2(0.f, 0.f); Qp = Sp; Sm = Sp; Qm = Sp;
     }
   };
