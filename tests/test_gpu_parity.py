@@ -157,6 +157,23 @@ def test_so3_one_kernel_path_of_the_20_32_and_44_grids(hip, b, nz):
         close(a1, so3_rfft_real_basis(xg, b_out=b)[:a1.size(0)].cpu().double(), f"analysis to {bs} degrees")
 
 
+@pytest.mark.parametrize("b", [10, 16, 22, 32])
+def test_so3_few_volumes_split_along_beta(hip, b):
+    """Below 129 volumes the per-volume kernels give a volume to 2, 4 or 8 workgroups along beta.  The analysis then adds
+    partial records (another order of the beta sum: equal to rounding), the synthesis writes the same planes from the same
+    record (equal to the bit).  130 volumes run unsplit; 100, 40 and 3 of them run with 2, 4 and up to 8 parts."""
+    print(f"so3 beta split b={b}", flush=True)
+    x = rnd((130, 2 * b, 2 * b, 2 * b), 180 + b).cuda()
+    m = rnd((130, 2 * b, 2 * b, 2 * b), 181 + b).cuda()
+    s = PSO3.so3_rfft(x)
+    sm = PSO3.so3_rfft(x, mask=m)
+    y = PSO3.so3_rifft(s)
+    for n in (100, 40, 3):
+        close(PSO3.so3_rfft(x[:n].contiguous()), s[:, :n].cpu(), f"rfft of {n} volumes")
+        close(PSO3.so3_rfft(x[:n].contiguous(), mask=m[:n].contiguous()), sm[:, :n].cpu(), f"masked rfft of {n} volumes")
+        assert torch.equal(PSO3.so3_rifft(s[:, :n].contiguous()), y[:n]), n
+
+
 def test_so3_one_kernel_path_is_reproducible(hip):
     """Both directions on the 64^3 grid form their sums in a fixed order: repeated calls agree bit for bit
     (this also guards the store sequence of the synthesis kernel, which once mixed two stores up now and then)."""
