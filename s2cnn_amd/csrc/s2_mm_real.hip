@@ -18,7 +18,8 @@
 namespace {
 
 constexpr int KC = 8;       // input features per register pass
-constexpr int NSPLIT = 4;   // forward: workgroups along n per (l, r)
+constexpr int NSPLIT = 8;   // forward: workgroups along n per (l, r)
+constexpr int IPT = 2;      // forward: batch items per thread
 constexpr int IB = 4;       // grad x: batch items per workgroup
 
 template <int VEC> struct Pack;
@@ -43,6 +44,13 @@ template <> struct Pack<4> {
   static __device__ __forceinline__ float dot(float4 a, float4 b) { return fmaf(a.x, b.x, fmaf(a.y, b.y, fmaf(a.z, b.z, a.w * b.w))); }
 };
 
+// a store of data that this kernel does not read again
+typedef float ext2_t __attribute__((ext_vector_type(2)));
+typedef float ext4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void stream_store(float v, float* p) { __builtin_nontemporal_store(v, p); }
+__device__ __forceinline__ void stream_store(float2 v, float2* p) { __builtin_nontemporal_store(ext2_t{v.x, v.y}, reinterpret_cast<ext2_t*>(p)); }
+__device__ __forceinline__ void stream_store(float4 v, float4* p) { __builtin_nontemporal_store(ext4_t{v.x, v.y, v.z, v.w}, reinterpret_cast<ext4_t*>(p)); }
+
 __device__ inline int isqrt_floor(int v) {
   int l = (int)sqrtf((float)v);
   while (l * l > v) --l;
@@ -50,9 +58,10 @@ __device__ inline int isqrt_floor(int v) {
   return l;
 }
 
-// ---- forward.  grid.x = nl^2 (l, r), grid.y = part of the s range, grid.z = tile of 256 (i pair, j group) outputs.
-// A thread owns two batch items and VEC output features: x[l,r,i,:] stays in registers while it walks s, so per s it
-// reads KC pieces of the row y[l,s] once for both items and writes two pieces of the row z[l,r,s].
+// ---- forward.  grid.x = nl^2 (l, r), grid.y = part of the s range, grid.z = tile of 256 (item group, j group) outputs.
+// A thread owns IPT batch items (ngroup apart, so that the lanes of a store cover whole rows of z) and VEC output
+// features: x[l,r,i,:] stays in registers while it walks s, so per s it reads KC pieces of the row y[l,s] once for all
+// its items and writes IPT pieces of the row z[l,r,s].
 template <int VEC>
 __global__ __launch_bounds__(256) void s2_mm_real_fwd_kernel(const float* __restrict__ x, const float* __restrict__ y,
                                                              float* __restrict__ z, int nl, int nbatch, int fi, int fo) {
@@ -61,37 +70,39 @@ __global__ __launch_bounds__(256) void s2_mm_real_fwd_kernel(const float* __rest
   const int l = isqrt_floor(lr), r = lr - l * l - l;
   const int L = 2 * l + 1;
   const int s_lo = (int)((long)blockIdx.y * L / NSPLIT), s_hi = (int)((long)(blockIdx.y + 1) * L / NSPLIT);
-  const int fov = fo / VEC, npair = (nbatch + 1) / 2;
+  const int fov = fo / VEC, ngroup = (nbatch + IPT - 1) / IPT;
   const int o = blockIdx.z * 256 + threadIdx.x;
-  if (o >= npair * fov || s_lo >= s_hi) return;
+  if (o >= ngroup * fov || s_lo >= s_hi) return;
   const int ip = o / fov, jv = o - ip * fov;
-  const int i0 = 2 * ip, i1 = i0 + 1 < nbatch ? i0 + 1 : i0;       // odd batch: the last pair computes its item twice
-  const float* x0 = x + ((size_t)lr * nbatch + i0) * fi;
-  const float* x1 = x + ((size_t)lr * nbatch + i1) * fi;
+  int item[IPT];
+#pragma unroll
+  for (int q = 0; q < IPT; ++q) item[q] = ip + q * ngroup < nbatch ? ip + q * ngroup : -1;    // item[0] always exists
   const size_t zrow = (size_t)l * (4 * l * l - 1) / 3 + (size_t)(l + r) * L;
   for (int k0 = 0; k0 < fi; k0 += KC) {
-    float xa[KC], xb[KC];
+    float xa[IPT][KC];
 #pragma unroll
-    for (int u = 0; u < KC; ++u) {
-      xa[u] = k0 + u < fi ? x0[k0 + u] : 0.f;
-      xb[u] = k0 + u < fi ? x1[k0 + u] : 0.f;
+    for (int q = 0; q < IPT; ++q) {
+      const float* xq = x + ((size_t)lr * nbatch + (item[q] < 0 ? ip : item[q])) * fi;
+#pragma unroll
+      for (int u = 0; u < KC; ++u) xa[q][u] = k0 + u < fi ? xq[k0 + u] : 0.f;
     }
     for (int s = s_lo; s < s_hi; ++s) {
       const vec_t* ys = reinterpret_cast<const vec_t*>(y + ((size_t)(l * l + s) * fi + k0) * fo) + jv;
-      vec_t* z0 = reinterpret_cast<vec_t*>(z + ((zrow + s) * nbatch + i0) * fo) + jv;
-      vec_t* z1 = reinterpret_cast<vec_t*>(z + ((zrow + s) * nbatch + i1) * fo) + jv;
-      vec_t a0 = Pack<VEC>::zero(), a1 = Pack<VEC>::zero();
-      if (k0 > 0) { a0 = *z0; a1 = *z1; }                          // later feature passes accumulate
+      vec_t* zs = reinterpret_cast<vec_t*>(z + (zrow + s) * nbatch * fo) + jv;
+      vec_t acc[IPT];
+#pragma unroll
+      for (int q = 0; q < IPT; ++q) acc[q] = (k0 > 0 && item[q] >= 0) ? zs[(size_t)item[q] * fov] : Pack<VEC>::zero();   // later feature passes accumulate
 #pragma unroll
       for (int u = 0; u < KC; ++u) {
         if (k0 + u < fi) {
           const vec_t b = ys[(size_t)u * fov];
-          Pack<VEC>::fma(xa[u], b, a0);
-          Pack<VEC>::fma(xb[u], b, a1);
+#pragma unroll
+          for (int q = 0; q < IPT; ++q) Pack<VEC>::fma(xa[q][u], b, acc[q]);
         }
       }
-      *z0 = a0;
-      if (i1 != i0) *z1 = a1;
+#pragma unroll
+      for (int q = 0; q < IPT; ++q)
+        if (item[q] >= 0) stream_store(acc[q], zs + (size_t)item[q] * fov);
     }
   }
 }
@@ -219,7 +230,7 @@ extern "C" int s2cnn_s2_mm_real_fwd(const float* x, const float* y, float* z, in
   s2cnn::clear_stale_error();
   if (int rc = check(x, y, z, nl, nbatch, f_in, f_out)) return rc;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const int npair = (nbatch + 1) / 2;
+  const int npair = (nbatch + IPT - 1) / IPT;      // item groups of the forward kernel
   if (vec4(y, z, z, f_out)) {
     const dim3 grid(nl * nl, NSPLIT, (unsigned)(((long)npair * (f_out / 4) + 255) / 256));
     hipLaunchKernelGGL(s2_mm_real_fwd_kernel<4>, grid, dim3(256), 0, st, x, y, z, nl, nbatch, f_in, f_out);

@@ -31,6 +31,7 @@ using fft64::fft8;
 using fused64::buf_load_f32;
 using fused64::buf_load_f32x4;
 using fused64::buf_store_f32;
+using fused64::buf_store_f32_stream;
 using fused64::buf_store_f32x4;
 using fused64::flip;
 using fused64::lmn_index;
@@ -597,8 +598,8 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void synthesis_kerne
         ms1 += ga + gb; ms2 = fmaf(ga, w[k].x, fmaf(gb, w[k].y, ms2));
       }
       if (relu) { ra = s2cnn::relu_f(ra); rb = s2cnn::relu_f(rb); }
-      buf_store_f32(ra, ry, yoff, (j * N * N + k * 4 * N) * 4);
-      buf_store_f32(rb, ry, yoff, ((N - 1 - j) * N * N + k * 4 * N) * 4);
+      buf_store_f32_stream(ra, ry, yoff, (j * N * N + k * 4 * N) * 4);
+      buf_store_f32_stream(rb, ry, yoff, ((N - 1 - j) * N * N + k * 4 * N) * 4);
     });
   };
   const bool in_store = t >= G::B_COLS_FIRST && t < G::B_COLS_FIRST + G::B_THREADS;

@@ -61,6 +61,11 @@ __device__ __forceinline__ float4 buf_load_f32x4(__amdgpu_buffer_rsrc_t r, unsig
 __device__ __forceinline__ void buf_store_f32(float x, __amdgpu_buffer_rsrc_t r, unsigned voff, unsigned soff) {
   __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(x), r, (int)voff, (int)soff, 0);
 }
+// the same store with the non-temporal hint (cache policy bit 1): for output that this kernel and the next ones on the
+// stream do not find in a cache anyway (a transform's result planes)
+__device__ __forceinline__ void buf_store_f32_stream(float x, __amdgpu_buffer_rsrc_t r, unsigned voff, unsigned soff) {
+  __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(x), r, (int)voff, (int)soff, 2);
+}
 __device__ __forceinline__ void buf_store_f32x4(float4 x, __amdgpu_buffer_rsrc_t r, unsigned voff, unsigned soff) {
   u32x4 v; v.x = __float_as_uint(x.x); v.y = __float_as_uint(x.y); v.z = __float_as_uint(x.z); v.w = __float_as_uint(x.w);
   __builtin_amdgcn_raw_buffer_store_b128(v, r, (int)voff, (int)soff, 0);
@@ -938,8 +943,8 @@ __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MOM == 0)) void synthes
         ms1 += ga + gb; ms2 = fmaf(ga, w[k].x, fmaf(gb, w[k].y, ms2));
       }
       if (relu) { ra = s2cnn::relu_f(ra); rb = s2cnn::relu_f(rb); }
-      buf_store_f32(ra, ry, yoff, (j * 4096 + k * 512) * 4);
-      buf_store_f32(rb, ry, yoff, ((63 - j) * 4096 + k * 512) * 4);
+      buf_store_f32_stream(ra, ry, yoff, (j * 4096 + k * 512) * 4);
+      buf_store_f32_stream(rb, ry, yoff, ((63 - j) * 4096 + k * 512) * 4);
       if (bits) {                                   // the gradient of max(., 0) passes where the output is not <= 0 (a NaN passes)
         const unsigned long long qa = __ballot(!(ra <= 0.f)), qb = __ballot(!(rb <= 0.f));
         if (lo == k) { wa = qa; wb = qb; }
