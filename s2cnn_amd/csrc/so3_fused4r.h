@@ -29,6 +29,7 @@ namespace fused4r {
 using fft64::fft4;
 using fft64::fft8;
 using fused64::buf_load_f32;
+using fused64::buf_load_f32_stream;
 using fused64::buf_load_f32x4;
 using fused64::buf_store_f32;
 using fused64::buf_store_f32_stream;
@@ -303,22 +304,22 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void analysis_kernel
       typedef __attribute__((address_space(3))) void* lds_ptr;
 #pragma unroll
       for (int j1 = 0; j1 < 4; ++j1) {
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr)(landing + (0 + j1) * THREADS + wave_first), 4, (int)xoff, (j * N * N + j1 * R * N) * 4, 0, 0);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr)(landing + (4 + j1) * THREADS + wave_first), 4, (int)xoff, ((N - 1 - j) * N * N + j1 * R * N) * 4, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr)(landing + (0 + j1) * THREADS + wave_first), 4, (int)xoff, (j * N * N + j1 * R * N) * 4, 0, 2);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr)(landing + (4 + j1) * THREADS + wave_first), 4, (int)xoff, ((N - 1 - j) * N * N + j1 * R * N) * 4, 0, 2);
         if constexpr (MASKED) {
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(rm, (lds_ptr)(landing + (8 + j1) * THREADS + wave_first), 4, (int)xoff, (j * N * N + j1 * R * N) * 4, 0, 0);
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(rm, (lds_ptr)(landing + (12 + j1) * THREADS + wave_first), 4, (int)xoff, ((N - 1 - j) * N * N + j1 * R * N) * 4, 0, 0);
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rm, (lds_ptr)(landing + (8 + j1) * THREADS + wave_first), 4, (int)xoff, (j * N * N + j1 * R * N) * 4, 0, 2);
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rm, (lds_ptr)(landing + (12 + j1) * THREADS + wave_first), 4, (int)xoff, ((N - 1 - j) * N * N + j1 * R * N) * 4, 0, 2);
         }
       }
       return;
     }
 #pragma unroll
     for (int j1 = 0; j1 < 4; ++j1) {
-      pa[j1] = buf_load_f32(rx, xoff, (j * N * N + j1 * R * N) * 4);
-      pb[j1] = buf_load_f32(rx, xoff, ((N - 1 - j) * N * N + j1 * R * N) * 4);
+      pa[j1] = buf_load_f32_stream(rx, xoff, (j * N * N + j1 * R * N) * 4);
+      pb[j1] = buf_load_f32_stream(rx, xoff, ((N - 1 - j) * N * N + j1 * R * N) * 4);
       if constexpr (MASKED) {
-        ma[j1] = buf_load_f32(rm, xoff, (j * N * N + j1 * R * N) * 4);
-        mb[j1] = buf_load_f32(rm, xoff, ((N - 1 - j) * N * N + j1 * R * N) * 4);
+        ma[j1] = buf_load_f32_stream(rm, xoff, (j * N * N + j1 * R * N) * 4);
+        mb[j1] = buf_load_f32_stream(rm, xoff, ((N - 1 - j) * N * N + j1 * R * N) * 4);
       }
     }
   };
@@ -581,7 +582,7 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void synthesis_kerne
     if constexpr (MOM == 2) {
 #pragma unroll
       for (int k = 0; k < R; ++k)
-        w[k] = make_float2(buf_load_f32(rw, yoff, (j * N * N + k * 4 * N) * 4), buf_load_f32(rw, yoff, ((N - 1 - j) * N * N + k * 4 * N) * 4));
+        w[k] = make_float2(buf_load_f32_stream(rw, yoff, (j * N * N + k * 4 * N) * 4), buf_load_f32_stream(rw, yoff, ((N - 1 - j) * N * N + k * 4 * N) * 4));
     }
     const float2* line = work + G::slot_of(u % N) + R * (u / N) * PITCH;
 #pragma unroll

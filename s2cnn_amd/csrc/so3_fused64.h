@@ -54,6 +54,10 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, un
 __device__ __forceinline__ float buf_load_f32(__amdgpu_buffer_rsrc_t r, unsigned voff, unsigned soff) {
   return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, (int)voff, (int)soff, 0));
 }
+// a load with the non-temporal hint: input that is read once (a transform's signal planes)
+__device__ __forceinline__ float buf_load_f32_stream(__amdgpu_buffer_rsrc_t r, unsigned voff, unsigned soff) {
+  return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, (int)voff, (int)soff, 2));
+}
 __device__ __forceinline__ float4 buf_load_f32x4(__amdgpu_buffer_rsrc_t r, unsigned voff, unsigned soff) {
   const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, (int)soff, 0);
   return make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
@@ -301,11 +305,11 @@ __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MASK == 0 || MASK == 2 
   float4 t1[4], t2[4];
 
   auto load_rows = [&](int j, int j1) {      // row 8 j1 + d of the planes j and 63-j: one full row (256 bytes) per wave and load
-    pa[j1] = buf_load_f32(rx, xoff, (j * 4096 + j1 * 512) * 4);
-    pb[j1] = buf_load_f32(rx, xoff, ((63 - j) * 4096 + j1 * 512) * 4);
+    pa[j1] = buf_load_f32_stream(rx, xoff, (j * 4096 + j1 * 512) * 4);
+    pb[j1] = buf_load_f32_stream(rx, xoff, ((63 - j) * 4096 + j1 * 512) * 4);
     if constexpr (MASKED) {
-      ma[j1] = buf_load_f32(rm, xoff, (j * 4096 + j1 * 512) * 4);
-      mb[j1] = buf_load_f32(rm, xoff, ((63 - j) * 4096 + j1 * 512) * 4);
+      ma[j1] = buf_load_f32_stream(rm, xoff, (j * 4096 + j1 * 512) * 4);
+      mb[j1] = buf_load_f32_stream(rm, xoff, ((63 - j) * 4096 + j1 * 512) * 4);
     }
     if constexpr (MASK == 2) {
       ba[j1] = bits[bits_index(z, j, du) + j1];
@@ -923,7 +927,7 @@ __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MOM == 0)) void synthes
     if constexpr (MOM == 2) {
 #pragma unroll
       for (int k = 0; k < 8; ++k)
-        w[k] = make_float2(buf_load_f32(rw, yoff, (j * 4096 + k * 512) * 4), buf_load_f32(rw, yoff, ((63 - j) * 4096 + k * 512) * 4));
+        w[k] = make_float2(buf_load_f32_stream(rw, yoff, (j * 4096 + k * 512) * 4), buf_load_f32_stream(rw, yoff, ((63 - j) * 4096 + k * 512) * 4));
     }
     const float2* line = work + sigma(lo) + 8 * d * PITCH;
 #pragma unroll
