@@ -49,4 +49,21 @@ __device__ __forceinline__ float bn_relu_grad(float g, float w, float a, float b
   return fmaf(q, w, p) + relu_pass(a * g, fmaf(a, w, b));
 }
 
+// Accesses with the non-temporal hint, for data that is streamed: written once and not found in a cache by its reader
+// anyway (hundreds of megabytes), or read once.  On this chip such stores run at up to 1.5 times the rate of plain ones.
+typedef float ext2_t __attribute__((ext_vector_type(2)));
+typedef float ext4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void stream_store(float v, float* p) { __builtin_nontemporal_store(v, p); }
+__device__ __forceinline__ void stream_store(float2 v, float2* p) { __builtin_nontemporal_store(ext2_t{v.x, v.y}, reinterpret_cast<ext2_t*>(p)); }
+__device__ __forceinline__ void stream_store(float4 v, float4* p) { __builtin_nontemporal_store(ext4_t{v.x, v.y, v.z, v.w}, reinterpret_cast<ext4_t*>(p)); }
+__device__ __forceinline__ float stream_load(const float* p) { return __builtin_nontemporal_load(p); }
+__device__ __forceinline__ float2 stream_load(const float2* p) {
+  const ext2_t v = __builtin_nontemporal_load(reinterpret_cast<const ext2_t*>(p));
+  return make_float2(v.x, v.y);
+}
+__device__ __forceinline__ float4 stream_load(const float4* p) {
+  const ext4_t v = __builtin_nontemporal_load(reinterpret_cast<const ext4_t*>(p));
+  return make_float4(v.x, v.y, v.z, v.w);
+}
+
 }  // namespace s2cnn

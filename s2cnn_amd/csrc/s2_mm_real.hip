@@ -44,13 +44,6 @@ template <> struct Pack<4> {
   static __device__ __forceinline__ float dot(float4 a, float4 b) { return fmaf(a.x, b.x, fmaf(a.y, b.y, fmaf(a.z, b.z, a.w * b.w))); }
 };
 
-// a store of data that this kernel does not read again
-typedef float ext2_t __attribute__((ext_vector_type(2)));
-typedef float ext4_t __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ void stream_store(float v, float* p) { __builtin_nontemporal_store(v, p); }
-__device__ __forceinline__ void stream_store(float2 v, float2* p) { __builtin_nontemporal_store(ext2_t{v.x, v.y}, reinterpret_cast<ext2_t*>(p)); }
-__device__ __forceinline__ void stream_store(float4 v, float4* p) { __builtin_nontemporal_store(ext4_t{v.x, v.y, v.z, v.w}, reinterpret_cast<ext4_t*>(p)); }
-
 __device__ inline int isqrt_floor(int v) {
   int l = (int)sqrtf((float)v);
   while (l * l > v) --l;
@@ -102,7 +95,7 @@ __global__ __launch_bounds__(256) void s2_mm_real_fwd_kernel(const float* __rest
       }
 #pragma unroll
       for (int q = 0; q < IPT; ++q)
-        if (item[q] >= 0) stream_store(acc[q], zs + (size_t)item[q] * fov);
+        if (item[q] >= 0) s2cnn::stream_store(acc[q], zs + (size_t)item[q] * fov);
     }
   }
 }
@@ -131,7 +124,7 @@ __global__ __launch_bounds__(256) void s2_mm_real_gradx_kernel(const float* __re
     const vec_t* g = reinterpret_cast<const vec_t*>(gz + ((zrow + s) * nbatch + i0) * fo) + jv;
     vec_t a[IB];
 #pragma unroll
-    for (int q = 0; q < IB; ++q) a[q] = i0 + q < nbatch ? g[(size_t)q * fov] : Pack<VEC>::zero();
+    for (int q = 0; q < IB; ++q) a[q] = i0 + q < nbatch ? s2cnn::stream_load(g + (size_t)q * fov) : Pack<VEC>::zero();
     const vec_t* yy = reinterpret_cast<const vec_t*>(y + ((size_t)(l * l + s) * fi + k0) * fo) + jv;
 #pragma unroll
     for (int u = 0; u < KC; ++u) {
@@ -185,7 +178,7 @@ __global__ __launch_bounds__(256) void s2_mm_real_grady_kernel(const float* __re
   int rr = slice / nbatch, i = slice - rr * nbatch;                // walks the pairs with stride SL
   const int dr = SL / nbatch, di = SL - dr * nbatch;
   for (int p = slice; p < total; p += SL) {
-    const vec_t a = jv < fov ? reinterpret_cast<const vec_t*>(gz + ((zcol + (size_t)rr * L) * nbatch + i) * fo)[jv] : Pack<VEC>::zero();
+    const vec_t a = jv < fov ? s2cnn::stream_load(reinterpret_cast<const vec_t*>(gz + ((zcol + (size_t)rr * L) * nbatch + i) * fo) + jv) : Pack<VEC>::zero();
     const float* xx = x + ((size_t)(l * l + rr) * nbatch + i) * fi + k0;
 #pragma unroll
     for (int u = 0; u < KC; ++u)

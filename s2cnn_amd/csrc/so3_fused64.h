@@ -246,7 +246,7 @@ __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MASK == 0 || MASK == 2 
   // p NJ / nparts .. (p+1) NJ / nparts - 1 and writes a record of its own, [volume][part]; spectrum_scatter adds them
   const long vp = volume_of_block(nbatch * nparts);
   if (vp < 0) return;
-  const long z = vp / nparts;
+  const long z = SPLIT ? vp / nparts : vp;
   const int j0 = SPLIT ? (int)(vp - z * nparts) * NJ / nparts : 0, j1 = SPLIT ? ((int)(vp - z * nparts) + 1) * NJ / nparts : NJ;
   const int t = threadIdx.x;
   const int lo = t & 63, d = t >> 6;
@@ -794,7 +794,7 @@ __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MOM == 0)) void synthes
   // nparts workgroups per volume (1 with MOM): part p reads the volume's record and writes the planes of its beta pairs
   const long vp = volume_of_block(nbatch * nparts);
   if (vp < 0) return;
-  const long z = vp / nparts;
+  const long z = SPLIT ? vp / nparts : vp;
   const int j0 = SPLIT ? (int)(vp - z * nparts) * NJ / nparts : 0, j1 = SPLIT ? ((int)(vp - z * nparts) + 1) * NJ / nparts : NJ;
   const int t = threadIdx.x;
   const int lo = t & 63, d = t >> 6;

@@ -58,16 +58,16 @@ __global__ __launch_bounds__(256) void rft_expand_kernel(const float* __restrict
     }
     float* row = y + c0;
     if (a > 0 && n > 0) {
-      *reinterpret_cast<float4*>(row + (size_t)ip * ncols) = lin4(1.f, Ar, s, Cr);
-      *reinterpret_cast<float4*>(row + (size_t)lmn_index(l, a, -n) * ncols) = lin4(-1.f, Ai, -s, Ci);
-      *reinterpret_cast<float4*>(row + (size_t)im * ncols) = lin4(1.f, Ai, -s, Ci);
-      *reinterpret_cast<float4*>(row + (size_t)lmn_index(l, -a, -n) * ncols) = lin4(1.f, Ar, -s, Cr);
+      s2cnn::stream_store(lin4(1.f, Ar, s, Cr), reinterpret_cast<float4*>(row + (size_t)ip * ncols));
+      s2cnn::stream_store(lin4(-1.f, Ai, -s, Ci), reinterpret_cast<float4*>(row + (size_t)lmn_index(l, a, -n) * ncols));
+      s2cnn::stream_store(lin4(1.f, Ai, -s, Ci), reinterpret_cast<float4*>(row + (size_t)im * ncols));
+      s2cnn::stream_store(lin4(1.f, Ar, -s, Cr), reinterpret_cast<float4*>(row + (size_t)lmn_index(l, -a, -n) * ncols));
     } else if (a > 0) {
-      *reinterpret_cast<float4*>(row + (size_t)ip * ncols) = lin4(RSQRT2, Ar, s * RSQRT2, Cr);
-      *reinterpret_cast<float4*>(row + (size_t)im * ncols) = lin4(RSQRT2, Ai, -s * RSQRT2, Ci);
+      s2cnn::stream_store(lin4(RSQRT2, Ar, s * RSQRT2, Cr), reinterpret_cast<float4*>(row + (size_t)ip * ncols));
+      s2cnn::stream_store(lin4(RSQRT2, Ai, -s * RSQRT2, Ci), reinterpret_cast<float4*>(row + (size_t)im * ncols));
     } else if (n > 0) {
-      *reinterpret_cast<float4*>(row + (size_t)ip * ncols) = lin4(SQRT2, Ar, 0.f, zero);
-      *reinterpret_cast<float4*>(row + (size_t)lmn_index(l, 0, -n) * ncols) = lin4(-SQRT2, Ai, 0.f, zero);
+      s2cnn::stream_store(lin4(SQRT2, Ar, 0.f, zero), reinterpret_cast<float4*>(row + (size_t)ip * ncols));
+      s2cnn::stream_store(lin4(-SQRT2, Ai, 0.f, zero), reinterpret_cast<float4*>(row + (size_t)lmn_index(l, 0, -n) * ncols));
     } else {
       *reinterpret_cast<float4*>(row + (size_t)ip * ncols) = Ar;
     }
@@ -94,23 +94,23 @@ __global__ __launch_bounds__(256) void rft_expand_grad_kernel(const float* __res
     const float* row = gy + c0;
     float4 gAr, gAi, gCr = zero, gCi = zero;
     if (a > 0 && n > 0) {
-      const float4 gpp = *reinterpret_cast<const float4*>(row + (size_t)ip * ncols);
-      const float4 gpm = *reinterpret_cast<const float4*>(row + (size_t)lmn_index(l, a, -n) * ncols);
-      const float4 gmp = *reinterpret_cast<const float4*>(row + (size_t)im * ncols);
-      const float4 gmm = *reinterpret_cast<const float4*>(row + (size_t)lmn_index(l, -a, -n) * ncols);
+      const float4 gpp = s2cnn::stream_load(reinterpret_cast<const float4*>(row + (size_t)ip * ncols));
+      const float4 gpm = s2cnn::stream_load(reinterpret_cast<const float4*>(row + (size_t)lmn_index(l, a, -n) * ncols));
+      const float4 gmp = s2cnn::stream_load(reinterpret_cast<const float4*>(row + (size_t)im * ncols));
+      const float4 gmm = s2cnn::stream_load(reinterpret_cast<const float4*>(row + (size_t)lmn_index(l, -a, -n) * ncols));
       gAr = lin4(1.f, gpp, 1.f, gmm); gAi = lin4(-1.f, gpm, 1.f, gmp);
       gCr = lin4(s, gpp, -s, gmm);    gCi = lin4(-s, gpm, -s, gmp);
     } else if (a > 0) {
-      const float4 gpp = *reinterpret_cast<const float4*>(row + (size_t)ip * ncols);
-      const float4 gmp = *reinterpret_cast<const float4*>(row + (size_t)im * ncols);
+      const float4 gpp = s2cnn::stream_load(reinterpret_cast<const float4*>(row + (size_t)ip * ncols));
+      const float4 gmp = s2cnn::stream_load(reinterpret_cast<const float4*>(row + (size_t)im * ncols));
       gAr = lin4(RSQRT2, gpp, 0.f, zero);     gAi = lin4(RSQRT2, gmp, 0.f, zero);
       gCr = lin4(s * RSQRT2, gpp, 0.f, zero); gCi = lin4(-s * RSQRT2, gmp, 0.f, zero);
     } else if (n > 0) {
-      const float4 gpp = *reinterpret_cast<const float4*>(row + (size_t)ip * ncols);
-      const float4 gpm = *reinterpret_cast<const float4*>(row + (size_t)lmn_index(l, 0, -n) * ncols);
+      const float4 gpp = s2cnn::stream_load(reinterpret_cast<const float4*>(row + (size_t)ip * ncols));
+      const float4 gpm = s2cnn::stream_load(reinterpret_cast<const float4*>(row + (size_t)lmn_index(l, 0, -n) * ncols));
       gAr = lin4(SQRT2, gpp, 0.f, zero); gAi = lin4(-SQRT2, gpm, 0.f, zero);
     } else {
-      gAr = *reinterpret_cast<const float4*>(row + (size_t)ip * ncols); gAi = zero;
+      gAr = s2cnn::stream_load(reinterpret_cast<const float4*>(row + (size_t)ip * ncols)); gAi = zero;
     }
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
