@@ -66,4 +66,13 @@ __device__ __forceinline__ float4 stream_load(const float4* p) {
   return make_float4(v.x, v.y, v.z, v.w);
 }
 
+// The hint chosen at run time by a uniform flag.  Tensors of at least STREAM_BYTES are streamed: they pass no cache on
+// their way to their reader (256 MB of memory-side cache); smaller ones are left to the caches.
+constexpr size_t STREAM_BYTES = (size_t)256 << 20;
+template <class V> __device__ __forceinline__ void store_policy(V v, V* p, bool stream) {
+  if (stream) stream_store(v, p);
+  else *p = v;
+}
+template <class V> __device__ __forceinline__ V load_policy(const V* p, bool stream) { return stream ? stream_load(p) : *p; }
+
 }  // namespace s2cnn

@@ -71,6 +71,7 @@ __global__ __launch_bounds__(256) void s2_mm_real_fwd_kernel(const float* __rest
 #pragma unroll
   for (int q = 0; q < IPT; ++q) item[q] = ip + q * ngroup < nbatch ? ip + q * ngroup : -1;    // item[0] always exists
   const size_t zrow = (size_t)l * (4 * l * l - 1) / 3 + (size_t)(l + r) * L;
+  const bool stream = (size_t)nl * (4 * nl * nl - 1) / 3 * nbatch * fo * 4 >= s2cnn::STREAM_BYTES;     // z passes no cache: uniform
   for (int k0 = 0; k0 < fi; k0 += KC) {
     float xa[IPT][KC];
 #pragma unroll
@@ -95,7 +96,7 @@ __global__ __launch_bounds__(256) void s2_mm_real_fwd_kernel(const float* __rest
       }
 #pragma unroll
       for (int q = 0; q < IPT; ++q)
-        if (item[q] >= 0) s2cnn::stream_store(acc[q], zs + (size_t)item[q] * fov);
+        if (item[q] >= 0) s2cnn::store_policy(acc[q], zs + (size_t)item[q] * fov, stream);
     }
   }
 }
@@ -124,7 +125,7 @@ __global__ __launch_bounds__(256) void s2_mm_real_gradx_kernel(const float* __re
     const vec_t* g = reinterpret_cast<const vec_t*>(gz + ((zrow + s) * nbatch + i0) * fo) + jv;
     vec_t a[IB];
 #pragma unroll
-    for (int q = 0; q < IB; ++q) a[q] = i0 + q < nbatch ? s2cnn::stream_load(g + (size_t)q * fov) : Pack<VEC>::zero();
+    for (int q = 0; q < IB; ++q) a[q] = i0 + q < nbatch ? g[(size_t)q * fov] : Pack<VEC>::zero();
     const vec_t* yy = reinterpret_cast<const vec_t*>(y + ((size_t)(l * l + s) * fi + k0) * fo) + jv;
 #pragma unroll
     for (int u = 0; u < KC; ++u) {
@@ -178,7 +179,7 @@ __global__ __launch_bounds__(256) void s2_mm_real_grady_kernel(const float* __re
   int rr = slice / nbatch, i = slice - rr * nbatch;                // walks the pairs with stride SL
   const int dr = SL / nbatch, di = SL - dr * nbatch;
   for (int p = slice; p < total; p += SL) {
-    const vec_t a = jv < fov ? s2cnn::stream_load(reinterpret_cast<const vec_t*>(gz + ((zcol + (size_t)rr * L) * nbatch + i) * fo) + jv) : Pack<VEC>::zero();
+    const vec_t a = jv < fov ? reinterpret_cast<const vec_t*>(gz + ((zcol + (size_t)rr * L) * nbatch + i) * fo)[jv] : Pack<VEC>::zero();
     const float* xx = x + ((size_t)(l * l + rr) * nbatch + i) * fi + k0;
 #pragma unroll
     for (int u = 0; u < KC; ++u)

@@ -30,6 +30,9 @@ using fft64::fft4;
 using fft64::fft8;
 using fused64::buf_load_f32;
 using fused64::buf_load_f32_stream;
+using fused64::buf_load_f32_policy;
+using fused64::buf_store_f32_policy;
+using fused64::STREAM_BYTES;
 using fused64::buf_load_f32x4;
 using fused64::buf_store_f32;
 using fused64::buf_store_f32_stream;
@@ -238,7 +241,7 @@ __device__ __forceinline__ void pass_b(float2* buf, int u) {
 // the beta pairs p NJ / nparts .. (p+1) NJ / nparts - 1 and writes a record of its own ([volume][part]); the pass to the
 // spectral rows adds the parts in their order.
 // ---------------------------------------------------------------------------------------------
-template <class G, int NA, int MASK>
+template <class G, int NA, int MASK, bool STREAM>
 __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void analysis_kernel(const float* __restrict__ x, const float* __restrict__ mask,
                                                                                 const float* __restrict__ Tf, float4* __restrict__ rec,
                                                                                 long nbatch, const float* __restrict__ params, int nfeature,
@@ -253,6 +256,7 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void analysis_kernel
   const long z = vp / nparts;
   const int part = (int)(vp - z * nparts);
   const int j0 = part * NJ / nparts, j1 = (part + 1) * NJ / nparts;
+  constexpr bool stream = STREAM;        // the signal passes no cache (see s2cnn::STREAM_BYTES): non-temporal loads / stores
   const int t = threadIdx.x;
   const int lo = t % N, d = t / N;
   const bool in_a = G::A_THREADS == THREADS || t < G::A_THREADS;
@@ -302,24 +306,36 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void analysis_kernel
   auto load_planes = [&](int j) {        // rows R j1 + d of the planes j and N-1-j: contiguous over the workgroup
     if constexpr (G::DMA) {
       typedef __attribute__((address_space(3))) void* lds_ptr;
+      if constexpr (stream) {       // the cache policy is an immediate of the instruction
 #pragma unroll
-      for (int j1 = 0; j1 < 4; ++j1) {
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr)(landing + (0 + j1) * THREADS + wave_first), 4, (int)xoff, (j * N * N + j1 * R * N) * 4, 0, 2);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr)(landing + (4 + j1) * THREADS + wave_first), 4, (int)xoff, ((N - 1 - j) * N * N + j1 * R * N) * 4, 0, 2);
-        if constexpr (MASKED) {
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(rm, (lds_ptr)(landing + (8 + j1) * THREADS + wave_first), 4, (int)xoff, (j * N * N + j1 * R * N) * 4, 0, 2);
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(rm, (lds_ptr)(landing + (12 + j1) * THREADS + wave_first), 4, (int)xoff, ((N - 1 - j) * N * N + j1 * R * N) * 4, 0, 2);
+        for (int j1 = 0; j1 < 4; ++j1) {
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr)(landing + (0 + j1) * THREADS + wave_first), 4, (int)xoff, (j * N * N + j1 * R * N) * 4, 0, 2);
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr)(landing + (4 + j1) * THREADS + wave_first), 4, (int)xoff, ((N - 1 - j) * N * N + j1 * R * N) * 4, 0, 2);
+          if constexpr (MASKED) {
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rm, (lds_ptr)(landing + (8 + j1) * THREADS + wave_first), 4, (int)xoff, (j * N * N + j1 * R * N) * 4, 0, 2);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rm, (lds_ptr)(landing + (12 + j1) * THREADS + wave_first), 4, (int)xoff, ((N - 1 - j) * N * N + j1 * R * N) * 4, 0, 2);
+          }
+        }
+      } else {
+#pragma unroll
+        for (int j1 = 0; j1 < 4; ++j1) {
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr)(landing + (0 + j1) * THREADS + wave_first), 4, (int)xoff, (j * N * N + j1 * R * N) * 4, 0, 0);
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr)(landing + (4 + j1) * THREADS + wave_first), 4, (int)xoff, ((N - 1 - j) * N * N + j1 * R * N) * 4, 0, 0);
+          if constexpr (MASKED) {
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rm, (lds_ptr)(landing + (8 + j1) * THREADS + wave_first), 4, (int)xoff, (j * N * N + j1 * R * N) * 4, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rm, (lds_ptr)(landing + (12 + j1) * THREADS + wave_first), 4, (int)xoff, ((N - 1 - j) * N * N + j1 * R * N) * 4, 0, 0);
+          }
         }
       }
       return;
     }
 #pragma unroll
     for (int j1 = 0; j1 < 4; ++j1) {
-      pa[j1] = buf_load_f32_stream(rx, xoff, (j * N * N + j1 * R * N) * 4);
-      pb[j1] = buf_load_f32_stream(rx, xoff, ((N - 1 - j) * N * N + j1 * R * N) * 4);
+      pa[j1] = buf_load_f32_policy(rx, xoff, (j * N * N + j1 * R * N) * 4, stream);
+      pb[j1] = buf_load_f32_policy(rx, xoff, ((N - 1 - j) * N * N + j1 * R * N) * 4, stream);
       if constexpr (MASKED) {
-        ma[j1] = buf_load_f32_stream(rm, xoff, (j * N * N + j1 * R * N) * 4);
-        mb[j1] = buf_load_f32_stream(rm, xoff, ((N - 1 - j) * N * N + j1 * R * N) * 4);
+        ma[j1] = buf_load_f32_policy(rm, xoff, (j * N * N + j1 * R * N) * 4, stream);
+        mb[j1] = buf_load_f32_policy(rm, xoff, ((N - 1 - j) * N * N + j1 * R * N) * 4, stream);
       }
     }
   };
@@ -449,7 +465,7 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void analysis_kernel
 // bias, relu, MOM, moments, yref, params: as fused64::synthesis_kernel (no bit masks).
 // nparts: workgroups per volume (1 with MOM): part p reads the volume's record and writes the planes of its beta pairs.
 // ---------------------------------------------------------------------------------------------
-template <class G, int NA, int MOM>
+template <class G, int NA, int MOM, bool STREAM>
 __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void synthesis_kernel(const float4* __restrict__ rec, const float* __restrict__ Tf,
                                                                                  float* __restrict__ y, long nbatch, const float* __restrict__ bias,
                                                                                  int nfeature, int relu, float2* __restrict__ moments,
@@ -470,6 +486,7 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void synthesis_kerne
   const long z = vp / nparts;
   const int part = (int)(vp - z * nparts);
   const int j0 = part * NJ / nparts, j1 = (part + 1) * NJ / nparts;
+  constexpr bool stream = STREAM;        // the signal passes no cache (see s2cnn::STREAM_BYTES): non-temporal loads / stores
   const int t = threadIdx.x;
   const int lo = t % N, d = t / N;
   const float bz = bias ? bias[z % nfeature] : 0.f;
@@ -582,7 +599,7 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void synthesis_kerne
     if constexpr (MOM == 2) {
 #pragma unroll
       for (int k = 0; k < R; ++k)
-        w[k] = make_float2(buf_load_f32_stream(rw, yoff, (j * N * N + k * 4 * N) * 4), buf_load_f32_stream(rw, yoff, ((N - 1 - j) * N * N + k * 4 * N) * 4));
+        w[k] = make_float2(buf_load_f32_policy(rw, yoff, (j * N * N + k * 4 * N) * 4, stream), buf_load_f32_policy(rw, yoff, ((N - 1 - j) * N * N + k * 4 * N) * 4, stream));
     }
     const float2* line = work + G::slot_of(u % N) + R * (u / N) * PITCH;
 #pragma unroll
@@ -599,8 +616,8 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void synthesis_kerne
         ms1 += ga + gb; ms2 = fmaf(ga, w[k].x, fmaf(gb, w[k].y, ms2));
       }
       if (relu) { ra = s2cnn::relu_f(ra); rb = s2cnn::relu_f(rb); }
-      buf_store_f32_stream(ra, ry, yoff, (j * N * N + k * 4 * N) * 4);
-      buf_store_f32_stream(rb, ry, yoff, ((N - 1 - j) * N * N + k * 4 * N) * 4);
+      buf_store_f32_policy(ra, ry, yoff, (j * N * N + k * 4 * N) * 4, stream);
+      buf_store_f32_policy(rb, ry, yoff, ((N - 1 - j) * N * N + k * 4 * N) * 4, stream);
     });
   };
   const bool in_store = t >= G::B_COLS_FIRST && t < G::B_COLS_FIRST + G::B_THREADS;
@@ -700,14 +717,21 @@ __global__ __launch_bounds__(G::THREADS, G::WAVES_PER_SIMD) void synthesis_kerne
 }
 
 // Launchers: the instantiation whose item rounds cover the nl degrees present.
-template <class G, int MASK>
-inline void launch_analysis_m(int nl, hipStream_t st, const s2cnn::Input& in, const float* Tf, float4* rec, long nbatch, int nparts) {
+template <class G, int MASK, bool STREAM>
+inline void launch_analysis_ms(int nl, hipStream_t st, const s2cnn::Input& in, const float* Tf, float4* rec, long nbatch, int nparts) {
   const dim3 grid(grid_size(nbatch * nparts)), block(G::THREADS);
   const int na = G::active_rounds(nl);
   static_assert(G::NIT <= 3, "add the instantiations of more rounds");
-  if (na <= 1) hipLaunchKernelGGL((analysis_kernel<G, 1, MASK>), grid, block, 0, st, in.x, in.w, Tf, rec, nbatch, in.params, in.nfeature, nparts);
-  else if (na == 2 || G::NIT < 3) hipLaunchKernelGGL((analysis_kernel<G, (G::NIT < 2 ? G::NIT : 2), MASK>), grid, block, 0, st, in.x, in.w, Tf, rec, nbatch, in.params, in.nfeature, nparts);
-  else hipLaunchKernelGGL((analysis_kernel<G, G::NIT, MASK>), grid, block, 0, st, in.x, in.w, Tf, rec, nbatch, in.params, in.nfeature, nparts);
+  if (na <= 1) hipLaunchKernelGGL((analysis_kernel<G, 1, MASK, STREAM>), grid, block, 0, st, in.x, in.w, Tf, rec, nbatch, in.params, in.nfeature, nparts);
+  else if (na == 2 || G::NIT < 3) hipLaunchKernelGGL((analysis_kernel<G, (G::NIT < 2 ? G::NIT : 2), MASK, STREAM>), grid, block, 0, st, in.x, in.w, Tf, rec, nbatch, in.params, in.nfeature, nparts);
+  else hipLaunchKernelGGL((analysis_kernel<G, G::NIT, MASK, STREAM>), grid, block, 0, st, in.x, in.w, Tf, rec, nbatch, in.params, in.nfeature, nparts);
+}
+// a signal of s2cnn::STREAM_BYTES or more passes no cache: the instantiation with non-temporal loads
+template <class G> inline bool streamed(long nbatch) { return (size_t)nbatch * (G::N * G::N * G::N * 4) >= s2cnn::STREAM_BYTES; }
+template <class G, int MASK>
+inline void launch_analysis_m(int nl, hipStream_t st, const s2cnn::Input& in, const float* Tf, float4* rec, long nbatch, int nparts) {
+  if (streamed<G>(nbatch)) launch_analysis_ms<G, MASK, true>(nl, st, in, Tf, rec, nbatch, nparts);
+  else launch_analysis_ms<G, MASK, false>(nl, st, in, Tf, rec, nbatch, nparts);
 }
 
 // in: the signal and what is done to it in the loads (s2cnn::Input; not PRO_BITS)
@@ -721,14 +745,20 @@ inline void launch_analysis(int nl, hipStream_t st, const s2cnn::Input& in, cons
   }
 }
 
+template <class G, int MOM, bool STREAM>
+inline void launch_synthesis_ms(int nl, hipStream_t st, const float4* rec, const float* Tf, float* y, long nbatch, const float* bias,
+                                int nfeature, int relu, float2* moments, const float* yref, const float* params, int nparts) {
+  const dim3 grid(grid_size(nbatch * nparts)), block(G::THREADS);
+  const int na = G::active_rounds(nl);
+  if (na <= 1) hipLaunchKernelGGL((synthesis_kernel<G, 1, MOM, STREAM>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, moments, yref, params, nparts);
+  else if (na == 2 || G::NIT < 3) hipLaunchKernelGGL((synthesis_kernel<G, (G::NIT < 2 ? G::NIT : 2), MOM, STREAM>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, moments, yref, params, nparts);
+  else hipLaunchKernelGGL((synthesis_kernel<G, G::NIT, MOM, STREAM>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, moments, yref, params, nparts);
+}
 template <class G, int MOM>
 inline void launch_synthesis_m(int nl, hipStream_t st, const float4* rec, const float* Tf, float* y, long nbatch, const float* bias,
                                int nfeature, int relu, float2* moments, const float* yref, const float* params, int nparts) {
-  const dim3 grid(grid_size(nbatch * nparts)), block(G::THREADS);
-  const int na = G::active_rounds(nl);
-  if (na <= 1) hipLaunchKernelGGL((synthesis_kernel<G, 1, MOM>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, moments, yref, params, nparts);
-  else if (na == 2 || G::NIT < 3) hipLaunchKernelGGL((synthesis_kernel<G, (G::NIT < 2 ? G::NIT : 2), MOM>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, moments, yref, params, nparts);
-  else hipLaunchKernelGGL((synthesis_kernel<G, G::NIT, MOM>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, moments, yref, params, nparts);
+  if (streamed<G>(nbatch)) launch_synthesis_ms<G, MOM, true>(nl, st, rec, Tf, y, nbatch, bias, nfeature, relu, moments, yref, params, nparts);
+  else launch_synthesis_ms<G, MOM, false>(nl, st, rec, Tf, y, nbatch, bias, nfeature, relu, moments, yref, params, nparts);
 }
 
 // moments: NULL, or two sums per volume: those of the output, or, with yref and params, those of the gradient of a normalisation

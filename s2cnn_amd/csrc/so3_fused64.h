@@ -65,11 +65,20 @@ __device__ __forceinline__ float4 buf_load_f32x4(__amdgpu_buffer_rsrc_t r, unsig
 __device__ __forceinline__ void buf_store_f32(float x, __amdgpu_buffer_rsrc_t r, unsigned voff, unsigned soff) {
   __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(x), r, (int)voff, (int)soff, 0);
 }
+// the hint chosen at run time by a uniform flag (the instruction carries it as an immediate, so there are two of them)
+__device__ __forceinline__ float buf_load_f32_policy(__amdgpu_buffer_rsrc_t r, unsigned voff, unsigned soff, bool stream) {
+  return stream ? buf_load_f32_stream(r, voff, soff) : buf_load_f32(r, voff, soff);
+}
 // the same store with the non-temporal hint (cache policy bit 1): for output that this kernel and the next ones on the
 // stream do not find in a cache anyway (a transform's result planes)
 __device__ __forceinline__ void buf_store_f32_stream(float x, __amdgpu_buffer_rsrc_t r, unsigned voff, unsigned soff) {
   __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(x), r, (int)voff, (int)soff, 2);
 }
+__device__ __forceinline__ void buf_store_f32_policy(float x, __amdgpu_buffer_rsrc_t r, unsigned voff, unsigned soff, bool stream) {
+  if (stream) buf_store_f32_stream(x, r, voff, soff);
+  else buf_store_f32(x, r, voff, soff);
+}
+using s2cnn::STREAM_BYTES;
 __device__ __forceinline__ void buf_store_f32x4(float4 x, __amdgpu_buffer_rsrc_t r, unsigned voff, unsigned soff) {
   u32x4 v; v.x = __float_as_uint(x.x); v.y = __float_as_uint(x.y); v.z = __float_as_uint(x.z); v.w = __float_as_uint(x.w);
   __builtin_amdgcn_raw_buffer_store_b128(v, r, (int)voff, (int)soff, 0);
@@ -233,7 +242,7 @@ __host__ __device__ inline size_t bits_index(long z, int beta, int d) { return (
 // PROBE (measurement only, results meaningless): 1: the Wigner contraction of an item reduced to one add per table
 // operand (table loads, LDS reads of the quads and everything else kept); 2: the table loads gone as well.  What is left
 // is the plane pipeline: loads, the 2-D transform through LDS with its barriers, the quad layout, the record.
-template <int NA, int MASK, int PROBE = 0, bool SPLIT = false>
+template <int NA, int MASK, int PROBE = 0, bool SPLIT = false, bool STREAM = false>
 __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MASK == 0 || MASK == 2 || MASK == 3)) void analysis_kernel(const float* __restrict__ x, const float* __restrict__ mask,
                                                            const float* __restrict__ Tf, float4* __restrict__ rec, long nbatch,
                                                            const float* __restrict__ params, int nfeature, int nparts) {
@@ -248,6 +257,7 @@ __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MASK == 0 || MASK == 2 
   if (vp < 0) return;
   const long z = SPLIT ? vp / nparts : vp;
   const int j0 = SPLIT ? (int)(vp - z * nparts) * NJ / nparts : 0, j1 = SPLIT ? ((int)(vp - z * nparts) + 1) * NJ / nparts : NJ;
+  constexpr bool stream = STREAM;        // the signal passes no cache (see s2cnn::STREAM_BYTES): non-temporal loads / stores
   const int t = threadIdx.x;
   const int lo = t & 63, d = t >> 6;
   Twiddles twl;
@@ -305,11 +315,11 @@ __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MASK == 0 || MASK == 2 
   float4 t1[4], t2[4];
 
   auto load_rows = [&](int j, int j1) {      // row 8 j1 + d of the planes j and 63-j: one full row (256 bytes) per wave and load
-    pa[j1] = buf_load_f32_stream(rx, xoff, (j * 4096 + j1 * 512) * 4);
-    pb[j1] = buf_load_f32_stream(rx, xoff, ((63 - j) * 4096 + j1 * 512) * 4);
+    pa[j1] = buf_load_f32_policy(rx, xoff, (j * 4096 + j1 * 512) * 4, stream);
+    pb[j1] = buf_load_f32_policy(rx, xoff, ((63 - j) * 4096 + j1 * 512) * 4, stream);
     if constexpr (MASKED) {
-      ma[j1] = buf_load_f32_stream(rm, xoff, (j * 4096 + j1 * 512) * 4);
-      mb[j1] = buf_load_f32_stream(rm, xoff, ((63 - j) * 4096 + j1 * 512) * 4);
+      ma[j1] = buf_load_f32_policy(rm, xoff, (j * 4096 + j1 * 512) * 4, stream);
+      mb[j1] = buf_load_f32_policy(rm, xoff, ((63 - j) * 4096 + j1 * 512) * 4, stream);
     }
     if constexpr (MASK == 2) {
       ba[j1] = bits[bits_index(z, j, du) + j1];
@@ -778,7 +788,7 @@ __global__ __launch_bounds__(256) void spectrum_gather_real(const float* __restr
 //   2: (sum v m, sum v m w) with w = yref at the same sample and m = (a w + b > 0), a = params[f], b = params[nfeature + f],
 //      f = z % nfeature: the two reductions of the gradient of such a normalisation followed by max(., 0), with the
 //      output as the incoming gradient (s2cnn::bn_relu_grad).
-template <int NA, int PROBE = 0, int MOM = 0, bool SPLIT = false>
+template <int NA, int PROBE = 0, int MOM = 0, bool SPLIT = false, bool STREAM = false>
 __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MOM == 0)) void synthesis_kernel(const float4* __restrict__ rec, const float* __restrict__ Tf,
                                                             float* __restrict__ y, long nbatch, const float* __restrict__ bias, int nfeature,
                                                             int relu, unsigned long long* __restrict__ bits, float2* __restrict__ moments,
@@ -796,6 +806,7 @@ __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MOM == 0)) void synthes
   if (vp < 0) return;
   const long z = SPLIT ? vp / nparts : vp;
   const int j0 = SPLIT ? (int)(vp - z * nparts) * NJ / nparts : 0, j1 = SPLIT ? ((int)(vp - z * nparts) + 1) * NJ / nparts : NJ;
+  constexpr bool stream = STREAM;        // the signal passes no cache (see s2cnn::STREAM_BYTES): non-temporal loads / stores
   const int t = threadIdx.x;
   const int lo = t & 63, d = t >> 6;
   const float bz = bias ? bias[z % nfeature] : 0.f;
@@ -927,7 +938,7 @@ __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MOM == 0)) void synthes
     if constexpr (MOM == 2) {
 #pragma unroll
       for (int k = 0; k < 8; ++k)
-        w[k] = make_float2(buf_load_f32_stream(rw, yoff, (j * 4096 + k * 512) * 4), buf_load_f32_stream(rw, yoff, ((63 - j) * 4096 + k * 512) * 4));
+        w[k] = make_float2(buf_load_f32_policy(rw, yoff, (j * 4096 + k * 512) * 4, stream), buf_load_f32_policy(rw, yoff, ((63 - j) * 4096 + k * 512) * 4, stream));
     }
     const float2* line = work + sigma(lo) + 8 * d * PITCH;
 #pragma unroll
@@ -947,8 +958,8 @@ __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MOM == 0)) void synthes
         ms1 += ga + gb; ms2 = fmaf(ga, w[k].x, fmaf(gb, w[k].y, ms2));
       }
       if (relu) { ra = s2cnn::relu_f(ra); rb = s2cnn::relu_f(rb); }
-      buf_store_f32_stream(ra, ry, yoff, (j * 4096 + k * 512) * 4);
-      buf_store_f32_stream(rb, ry, yoff, ((63 - j) * 4096 + k * 512) * 4);
+      buf_store_f32_policy(ra, ry, yoff, (j * 4096 + k * 512) * 4, stream);
+      buf_store_f32_policy(rb, ry, yoff, ((63 - j) * 4096 + k * 512) * 4, stream);
       if (bits) {                                   // the gradient of max(., 0) passes where the output is not <= 0 (a NaN passes)
         const unsigned long long qa = __ballot(!(ra <= 0.f)), qb = __ballot(!(rb <= 0.f));
         if (lo == k) { wa = qa; wb = qb; }
@@ -1065,19 +1076,23 @@ __global__ __launch_bounds__(THREADS, waves_per_simd(NA, MOM == 0)) void synthes
 inline int active_rounds(int nl) { return nl <= 24 ? 3 : nl <= 28 ? 6 : NIT; }
 
 // Launchers: the instantiation whose item rounds cover the nl degrees present.
-template <int MASK, bool SPLIT>
+template <int MASK, bool SPLIT, bool STREAM>
 inline void launch_analysis_ms(int nl, hipStream_t st, const s2cnn::Input& in, const float* Tf, float4* rec, long nbatch, int nparts) {
   const dim3 grid(grid_size(nbatch * nparts)), block(THREADS);
-  if (nl <= 24) hipLaunchKernelGGL((analysis_kernel<3, MASK, 0, SPLIT>), grid, block, 0, st, in.x, in.w, Tf, rec, nbatch, in.params, in.nfeature, nparts);
-  else if (nl <= 28) hipLaunchKernelGGL((analysis_kernel<6, MASK, 0, SPLIT>), grid, block, 0, st, in.x, in.w, Tf, rec, nbatch, in.params, in.nfeature, nparts);
-  else hipLaunchKernelGGL((analysis_kernel<7, MASK, 0, SPLIT>), grid, block, 0, st, in.x, in.w, Tf, rec, nbatch, in.params, in.nfeature, nparts);
+  if (nl <= 24) hipLaunchKernelGGL((analysis_kernel<3, MASK, 0, SPLIT, STREAM>), grid, block, 0, st, in.x, in.w, Tf, rec, nbatch, in.params, in.nfeature, nparts);
+  else if (nl <= 28) hipLaunchKernelGGL((analysis_kernel<6, MASK, 0, SPLIT, STREAM>), grid, block, 0, st, in.x, in.w, Tf, rec, nbatch, in.params, in.nfeature, nparts);
+  else hipLaunchKernelGGL((analysis_kernel<7, MASK, 0, SPLIT, STREAM>), grid, block, 0, st, in.x, in.w, Tf, rec, nbatch, in.params, in.nfeature, nparts);
 }
+
+// a signal of s2cnn::STREAM_BYTES or more passes no cache: the instantiations with non-temporal loads / stores
+inline bool streamed(long nbatch) { return (size_t)nbatch * (N * N * N * 4) >= s2cnn::STREAM_BYTES; }
 
 // one workgroup per volume runs the instantiation whose plane loop has constant bounds
 template <int MASK>
 inline void launch_analysis_m(int nl, hipStream_t st, const s2cnn::Input& in, const float* Tf, float4* rec, long nbatch, int nparts) {
-  if (nparts > 1) launch_analysis_ms<MASK, true>(nl, st, in, Tf, rec, nbatch, nparts);
-  else launch_analysis_ms<MASK, false>(nl, st, in, Tf, rec, nbatch, 1);
+  if (nparts > 1) launch_analysis_ms<MASK, true, false>(nl, st, in, Tf, rec, nbatch, nparts);
+  else if (streamed(nbatch)) launch_analysis_ms<MASK, false, true>(nl, st, in, Tf, rec, nbatch, 1);
+  else launch_analysis_ms<MASK, false, false>(nl, st, in, Tf, rec, nbatch, 1);
 }
 
 // in: the signal and what is done to it in the loads (s2cnn::Input)
@@ -1098,31 +1113,27 @@ constexpr int GRAD_MOMENTS_MAX_NL = 28;
 // moments: NULL, or two sums per volume (see MOM): those of the output, or, with yref and params (nl <= GRAD_MOMENTS_MAX_NL
 // only), those of the gradient of a normalisation
 // nparts: workgroups per volume where no sums are formed (one with `moments`)
+template <int MOM, bool SPLIT, bool STREAM>
+inline void launch_synthesis_ms(int nl, hipStream_t st, const float4* rec, const float* Tf, float* y, long nbatch, const float* bias,
+                                int nfeature, int relu, unsigned long long* bits, float2* moments, const float* yref, const float* params, int nparts) {
+  const dim3 grid(grid_size(nbatch * nparts)), block(THREADS);
+  if (nl <= 24) hipLaunchKernelGGL((synthesis_kernel<3, 0, MOM, SPLIT, STREAM>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, yref, params, nparts);
+  else if (nl <= 28 || MOM == 2) hipLaunchKernelGGL((synthesis_kernel<6, 0, MOM, SPLIT, STREAM>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, yref, params, nparts);
+  else hipLaunchKernelGGL((synthesis_kernel<(MOM == 2 ? 6 : 7), 0, MOM, SPLIT, STREAM>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, yref, params, nparts);
+}
+template <int MOM>
+inline void launch_synthesis_m(int nl, hipStream_t st, const float4* rec, const float* Tf, float* y, long nbatch, const float* bias,
+                               int nfeature, int relu, unsigned long long* bits, float2* moments, const float* yref, const float* params, int nparts) {
+  if (MOM == 0 && nparts > 1) launch_synthesis_ms<0, true, false>(nl, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, nullptr, nullptr, nullptr, nparts);
+  else if (streamed(nbatch)) launch_synthesis_ms<MOM, false, true>(nl, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, yref, params, 1);
+  else launch_synthesis_ms<MOM, false, false>(nl, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, yref, params, 1);
+}
 inline void launch_synthesis(int nl, hipStream_t st, const float4* rec, const float* Tf, float* y, long nbatch, const float* bias,
                              int nfeature, int relu, unsigned long long* bits, float2* moments = nullptr, const float* yref = nullptr,
                              const float* params = nullptr, int nparts = 1) {
-  if (moments) nparts = 1;
-  const dim3 grid(grid_size(nbatch * nparts)), block(THREADS);
-  if (moments && yref) {
-    if (nl <= 24) hipLaunchKernelGGL((synthesis_kernel<3, 0, 2>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, yref, params, nparts);
-    else hipLaunchKernelGGL((synthesis_kernel<6, 0, 2>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, yref, params, nparts);
-    return;
-  }
-  if (moments) {
-    if (nl <= 24) hipLaunchKernelGGL((synthesis_kernel<3, 0, 1>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, nullptr, nullptr, nparts);
-    else if (nl <= 28) hipLaunchKernelGGL((synthesis_kernel<6, 0, 1>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, nullptr, nullptr, nparts);
-    else hipLaunchKernelGGL((synthesis_kernel<7, 0, 1>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, nullptr, nullptr, nparts);
-    return;
-  }
-  if (nparts > 1) {
-    if (nl <= 24) hipLaunchKernelGGL((synthesis_kernel<3, 0, 0, true>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, nullptr, nullptr, nullptr, nparts);
-    else if (nl <= 28) hipLaunchKernelGGL((synthesis_kernel<6, 0, 0, true>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, nullptr, nullptr, nullptr, nparts);
-    else hipLaunchKernelGGL((synthesis_kernel<7, 0, 0, true>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, nullptr, nullptr, nullptr, nparts);
-    return;
-  }
-  if (nl <= 24) hipLaunchKernelGGL((synthesis_kernel<3>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, nullptr, nullptr, nullptr, 1);
-  else if (nl <= 28) hipLaunchKernelGGL((synthesis_kernel<6>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, nullptr, nullptr, nullptr, 1);
-  else hipLaunchKernelGGL((synthesis_kernel<7>), grid, block, 0, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, nullptr, nullptr, nullptr, 1);
+  if (moments && yref) launch_synthesis_m<2>(nl, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, yref, params, 1);      // nl <= GRAD_MOMENTS_MAX_NL
+  else if (moments) launch_synthesis_m<1>(nl, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, moments, nullptr, nullptr, 1);
+  else launch_synthesis_m<0>(nl, st, rec, Tf, y, nbatch, bias, nfeature, relu, bits, nullptr, nullptr, nullptr, nparts);
 }
 
 }  // namespace fused64

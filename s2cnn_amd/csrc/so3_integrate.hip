@@ -21,13 +21,14 @@ __global__ __launch_bounds__(256) void so3_integrate_kernel(const float* __restr
   float acc = 0.f;
   if (plane % 4096 == 0 && (reinterpret_cast<uintptr_t>(x) & 15u) == 0) {
     // 16-byte loads, four in flight per thread (4 KB per workgroup and step)
+    const bool stream = (size_t)gridDim.x * plane * n2 * 4 >= s2cnn::STREAM_BYTES;     // a tensor that passes no cache
     const float4* x4 = reinterpret_cast<const float4*>(xs);
     const size_t p4 = plane / 4;
     for (int bt = 0; bt < n2; ++bt) {
       float4 s0 = make_float4(0.f, 0.f, 0.f, 0.f), s1 = s0, s2 = s0, s3 = s0;
       const float4* pl = x4 + bt * p4 + threadIdx.x;
       for (size_t i = 0; i < p4; i += 1024) {
-        const float4 v0 = f4(s2cnn::stream_load(pl + i)), v1 = f4(s2cnn::stream_load(pl + i + 256)), v2 = f4(s2cnn::stream_load(pl + i + 512)), v3 = f4(s2cnn::stream_load(pl + i + 768));
+        const float4 v0 = f4(s2cnn::load_policy(pl + i, stream)), v1 = f4(s2cnn::load_policy(pl + i + 256, stream)), v2 = f4(s2cnn::load_policy(pl + i + 512, stream)), v3 = f4(s2cnn::load_policy(pl + i + 768, stream));
         s0.x += v0.x; s0.y += v0.y; s0.z += v0.z; s0.w += v0.w;
         s1.x += v1.x; s1.y += v1.y; s1.z += v1.z; s1.w += v1.w;
         s2.x += v2.x; s2.y += v2.y; s2.z += v2.z; s2.w += v2.w;
@@ -74,10 +75,11 @@ __global__ __launch_bounds__(256) void so3_integrate_grad_kernel(const float* __
   if ((reinterpret_cast<uintptr_t>(gx) & 15u) == 0) {      // n2 is even: every plane is a whole number of 16-byte words
     float4* dst4 = reinterpret_cast<float4*>(dst);
     const int p4 = (int)(plane / 4);
+    const bool stream = (size_t)gridDim.x * plane * n2 * 4 >= s2cnn::STREAM_BYTES;     // a tensor that passes no cache
     for (int bt = 0; bt < n2; ++bt) {
       const float v = gv * w[bt];
       const float4 v4 = make_float4(v, v, v, v);
-      for (int i = threadIdx.x; i < p4; i += blockDim.x) s2cnn::stream_store(v4, dst4 + (size_t)bt * p4 + i);
+      for (int i = threadIdx.x; i < p4; i += blockDim.x) s2cnn::store_policy(v4, dst4 + (size_t)bt * p4 + i, stream);
     }
     return;
   }

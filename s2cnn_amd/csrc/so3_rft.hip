@@ -35,6 +35,7 @@ __global__ __launch_bounds__(256) void rft_expand_kernel(const float* __restrict
   if (c0 >= ncols) return;
   const long nspec = (long)b * (4L * b * b - 1) / 3;
   const size_t R = (size_t)(2 * b - 1) * b * 2;
+  const bool stream = (size_t)nspec * (size_t)ncols * 4 >= s2cnn::STREAM_BYTES;    // the spectrum is streamed: uniform
   const size_t rp = (size_t)((a + b - 1) * b + n) * 2, rm = (size_t)((-a + b - 1) * b + n) * 2;
   float4 pr[NB], pi[NB], mr[NB], mi[NB];
 #pragma unroll
@@ -58,16 +59,16 @@ __global__ __launch_bounds__(256) void rft_expand_kernel(const float* __restrict
     }
     float* row = y + c0;
     if (a > 0 && n > 0) {
-      s2cnn::stream_store(lin4(1.f, Ar, s, Cr), reinterpret_cast<float4*>(row + (size_t)ip * ncols));
-      s2cnn::stream_store(lin4(-1.f, Ai, -s, Ci), reinterpret_cast<float4*>(row + (size_t)lmn_index(l, a, -n) * ncols));
-      s2cnn::stream_store(lin4(1.f, Ai, -s, Ci), reinterpret_cast<float4*>(row + (size_t)im * ncols));
-      s2cnn::stream_store(lin4(1.f, Ar, -s, Cr), reinterpret_cast<float4*>(row + (size_t)lmn_index(l, -a, -n) * ncols));
+      s2cnn::store_policy(lin4(1.f, Ar, s, Cr), reinterpret_cast<float4*>(row + (size_t)ip * ncols), stream);
+      s2cnn::store_policy(lin4(-1.f, Ai, -s, Ci), reinterpret_cast<float4*>(row + (size_t)lmn_index(l, a, -n) * ncols), stream);
+      s2cnn::store_policy(lin4(1.f, Ai, -s, Ci), reinterpret_cast<float4*>(row + (size_t)im * ncols), stream);
+      s2cnn::store_policy(lin4(1.f, Ar, -s, Cr), reinterpret_cast<float4*>(row + (size_t)lmn_index(l, -a, -n) * ncols), stream);
     } else if (a > 0) {
-      s2cnn::stream_store(lin4(RSQRT2, Ar, s * RSQRT2, Cr), reinterpret_cast<float4*>(row + (size_t)ip * ncols));
-      s2cnn::stream_store(lin4(RSQRT2, Ai, -s * RSQRT2, Ci), reinterpret_cast<float4*>(row + (size_t)im * ncols));
+      s2cnn::store_policy(lin4(RSQRT2, Ar, s * RSQRT2, Cr), reinterpret_cast<float4*>(row + (size_t)ip * ncols), stream);
+      s2cnn::store_policy(lin4(RSQRT2, Ai, -s * RSQRT2, Ci), reinterpret_cast<float4*>(row + (size_t)im * ncols), stream);
     } else if (n > 0) {
-      s2cnn::stream_store(lin4(SQRT2, Ar, 0.f, zero), reinterpret_cast<float4*>(row + (size_t)ip * ncols));
-      s2cnn::stream_store(lin4(-SQRT2, Ai, 0.f, zero), reinterpret_cast<float4*>(row + (size_t)lmn_index(l, 0, -n) * ncols));
+      s2cnn::store_policy(lin4(SQRT2, Ar, 0.f, zero), reinterpret_cast<float4*>(row + (size_t)ip * ncols), stream);
+      s2cnn::store_policy(lin4(-SQRT2, Ai, 0.f, zero), reinterpret_cast<float4*>(row + (size_t)lmn_index(l, 0, -n) * ncols), stream);
     } else {
       *reinterpret_cast<float4*>(row + (size_t)ip * ncols) = Ar;
     }
@@ -83,6 +84,7 @@ __global__ __launch_bounds__(256) void rft_expand_grad_kernel(const float* __res
   if (c0 >= ncols) return;
   const long nspec = (long)b * (4L * b * b - 1) / 3;
   const size_t R = (size_t)(2 * b - 1) * b * 2;
+  const bool stream = (size_t)nspec * (size_t)ncols * 4 >= s2cnn::STREAM_BYTES;    // the spectrum is streamed: uniform
   const size_t rp = (size_t)((a + b - 1) * b + n) * 2, rm = (size_t)((-a + b - 1) * b + n) * 2;
   const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
   float4 pr[NB], pi[NB], mr[NB], mi[NB];
@@ -94,23 +96,23 @@ __global__ __launch_bounds__(256) void rft_expand_grad_kernel(const float* __res
     const float* row = gy + c0;
     float4 gAr, gAi, gCr = zero, gCi = zero;
     if (a > 0 && n > 0) {
-      const float4 gpp = s2cnn::stream_load(reinterpret_cast<const float4*>(row + (size_t)ip * ncols));
-      const float4 gpm = s2cnn::stream_load(reinterpret_cast<const float4*>(row + (size_t)lmn_index(l, a, -n) * ncols));
-      const float4 gmp = s2cnn::stream_load(reinterpret_cast<const float4*>(row + (size_t)im * ncols));
-      const float4 gmm = s2cnn::stream_load(reinterpret_cast<const float4*>(row + (size_t)lmn_index(l, -a, -n) * ncols));
+      const float4 gpp = s2cnn::load_policy(reinterpret_cast<const float4*>(row + (size_t)ip * ncols), stream);
+      const float4 gpm = s2cnn::load_policy(reinterpret_cast<const float4*>(row + (size_t)lmn_index(l, a, -n) * ncols), stream);
+      const float4 gmp = s2cnn::load_policy(reinterpret_cast<const float4*>(row + (size_t)im * ncols), stream);
+      const float4 gmm = s2cnn::load_policy(reinterpret_cast<const float4*>(row + (size_t)lmn_index(l, -a, -n) * ncols), stream);
       gAr = lin4(1.f, gpp, 1.f, gmm); gAi = lin4(-1.f, gpm, 1.f, gmp);
       gCr = lin4(s, gpp, -s, gmm);    gCi = lin4(-s, gpm, -s, gmp);
     } else if (a > 0) {
-      const float4 gpp = s2cnn::stream_load(reinterpret_cast<const float4*>(row + (size_t)ip * ncols));
-      const float4 gmp = s2cnn::stream_load(reinterpret_cast<const float4*>(row + (size_t)im * ncols));
+      const float4 gpp = s2cnn::load_policy(reinterpret_cast<const float4*>(row + (size_t)ip * ncols), stream);
+      const float4 gmp = s2cnn::load_policy(reinterpret_cast<const float4*>(row + (size_t)im * ncols), stream);
       gAr = lin4(RSQRT2, gpp, 0.f, zero);     gAi = lin4(RSQRT2, gmp, 0.f, zero);
       gCr = lin4(s * RSQRT2, gpp, 0.f, zero); gCi = lin4(-s * RSQRT2, gmp, 0.f, zero);
     } else if (n > 0) {
-      const float4 gpp = s2cnn::stream_load(reinterpret_cast<const float4*>(row + (size_t)ip * ncols));
-      const float4 gpm = s2cnn::stream_load(reinterpret_cast<const float4*>(row + (size_t)lmn_index(l, 0, -n) * ncols));
+      const float4 gpp = s2cnn::load_policy(reinterpret_cast<const float4*>(row + (size_t)ip * ncols), stream);
+      const float4 gpm = s2cnn::load_policy(reinterpret_cast<const float4*>(row + (size_t)lmn_index(l, 0, -n) * ncols), stream);
       gAr = lin4(SQRT2, gpp, 0.f, zero); gAi = lin4(-SQRT2, gpm, 0.f, zero);
     } else {
-      gAr = s2cnn::stream_load(reinterpret_cast<const float4*>(row + (size_t)ip * ncols)); gAi = zero;
+      gAr = s2cnn::load_policy(reinterpret_cast<const float4*>(row + (size_t)ip * ncols), stream); gAi = zero;
     }
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
