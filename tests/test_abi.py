@@ -40,7 +40,7 @@ def test_measurement_entry_is_not_in_the_product_library():
     if os.path.exists(_hip.PROBE_LIB_PATH):
         probe = _hip.probe_lib()
         fake, null = ctypes.c_void_p(0x1000), ctypes.c_void_p(0)
-        assert probe.s2cnn_so3_fft64_probe(fake, fake, fake, fake, 1 << 30, 2, 1, 2, null) == -1     # the synthesis has no probe 2
+        assert probe.s2cnn_so3_fft64_probe(fake, fake, fake, fake, 1 << 30, 2, 1, 3, null) == -1     # there is no probe 3
         assert probe.s2cnn_so3_fft64_probe(fake, fake, fake, fake, 0, 2, 0, 1, null) == -2           # workspace too small
 
 
