@@ -21,44 +21,6 @@ __device__ inline int isqrt_floor(int v) {
   return l;
 }
 
-// ---- forward: grid.x = nl^2 (l,m), grid.y = quarter of the n range, grid.z = tile of 256 (i,j) outputs.
-// A thread owns one (i, j): x[l,m,i,:] stays in registers while it walks n, so per n it reads one coalesced
-// row of y and writes one coalesced row of z; consecutive n are consecutive blocks of z.
-constexpr int NSPLIT = 4;
-
-__global__ __launch_bounds__(256) void s2_mm_fwd_kernel(const float2* __restrict__ x, const float2* __restrict__ y,
-                                                        float2* __restrict__ z, int nl, int nbatch, int fi, int fo) {
-  const int lm = blockIdx.x;
-  const int l = isqrt_floor(lm), m = lm - l * l - l;
-  const int L = 2 * l + 1;
-  const int n_lo = (int)((long)blockIdx.y * L / NSPLIT), n_hi = (int)((long)(blockIdx.y + 1) * L / NSPLIT);
-  const int o = blockIdx.z * 256 + threadIdx.x;
-  if (o >= nbatch * fo || n_lo >= n_hi) return;
-  const int i = o / fo, j = o - i * fo;
-  const float2* xs = x + ((size_t)lm * nbatch + i) * fi;
-  const size_t zbase = (size_t)l * (4 * l * l - 1) / 3 + (size_t)(l + m) * L;
-  for (int k0 = 0; k0 < fi; k0 += KC) {
-    float2 xr[KC];
-#pragma unroll
-    for (int u = 0; u < KC; ++u) xr[u] = k0 + u < fi ? xs[k0 + u] : make_float2(0.f, 0.f);
-    for (int nn = n_lo; nn < n_hi; ++nn) {
-      const float2* ys = y + ((size_t)(l * l + nn) * fi + k0) * fo + j;
-      float2* zp = z + (zbase + nn) * nbatch * fo + o;
-      float re = 0.f, im = 0.f;
-      if (k0 > 0) { const float2 p = *zp; re = p.x; im = p.y; }     // later feature passes accumulate
-#pragma unroll
-      for (int u = 0; u < KC; ++u) {
-        if (k0 + u < fi) {
-          const float2 b = ys[(size_t)u * fo];
-          re += xr[u].x * b.x + xr[u].y * b.y;
-          im += xr[u].y * b.x - xr[u].x * b.y;
-        }
-      }
-      *zp = make_float2(re, im);
-    }
-  }
-}
-
 // CV complex numbers per lane along j: 2 (16-byte accesses) when F_out is even and the rows start on 16-byte boundaries
 template <int CV> struct CPack;
 template <> struct CPack<1> {
@@ -68,6 +30,11 @@ template <> struct CPack<1> {
   static __device__ __forceinline__ void dot(float2 a, float2 b, float2& acc) {
     acc.x = fmaf(a.x, b.x, fmaf(-a.y, b.y, acc.x));
     acc.y = fmaf(a.x, b.y, fmaf(a.y, b.x, acc.y));
+  }
+  // acc[entry] += s * conj(b[entry]) for a complex scalar s
+  static __device__ __forceinline__ void scal_conj(float2 s, float2 b, float2& acc) {
+    acc.x = fmaf(s.x, b.x, fmaf(s.y, b.y, acc.x));
+    acc.y = fmaf(s.y, b.x, fmaf(-s.x, b.y, acc.y));
   }
   // acc[entry] += conj(a[entry]) * s for a complex scalar s
   static __device__ __forceinline__ void conj_axpy(float2 a, float2 s, float2& acc) {
@@ -82,6 +49,12 @@ template <> struct CPack<2> {
     acc.x = fmaf(a.x, b.x, fmaf(-a.y, b.y, fmaf(a.z, b.z, fmaf(-a.w, b.w, acc.x))));
     acc.y = fmaf(a.x, b.y, fmaf(a.y, b.x, fmaf(a.z, b.w, fmaf(a.w, b.z, acc.y))));
   }
+  static __device__ __forceinline__ void scal_conj(float2 s, float4 b, float4& acc) {
+    acc.x = fmaf(s.x, b.x, fmaf(s.y, b.y, acc.x));
+    acc.y = fmaf(s.y, b.x, fmaf(-s.x, b.y, acc.y));
+    acc.z = fmaf(s.x, b.z, fmaf(s.y, b.w, acc.z));
+    acc.w = fmaf(s.y, b.z, fmaf(-s.x, b.w, acc.w));
+  }
   static __device__ __forceinline__ void conj_axpy(float4 a, float2 s, float4& acc) {
     acc.x = fmaf(a.x, s.x, fmaf(a.y, s.y, acc.x));
     acc.y = fmaf(a.x, s.y, fmaf(-a.y, s.x, acc.y));
@@ -89,6 +62,59 @@ template <> struct CPack<2> {
     acc.w = fmaf(a.z, s.y, fmaf(-a.w, s.x, acc.w));
   }
 };
+
+// ---- forward: grid.x = nl^2 (l,m), grid.y = part of the n range, grid.z = tile of 256 (item group, j group) outputs.
+// A thread owns IPT batch items (ngroup apart, so that the lanes of a store cover whole rows of z) and CV output
+// features: x[l,m,i,:] stays in registers while it walks n, so per n it reads KC pieces of the row y[l,n] once for all
+// its items and writes IPT pieces of the row z[l,m,n]; consecutive n are consecutive blocks of z.
+constexpr int NSPLIT = 8;
+constexpr int IPT = 2;
+
+template <int CV>
+__global__ __launch_bounds__(256) void s2_mm_fwd_kernel(const float2* __restrict__ x, const float2* __restrict__ y,
+                                                        float2* __restrict__ z, int nl, int nbatch, int fi, int fo) {
+  typedef typename CPack<CV>::type vec_t;
+  const int lm = blockIdx.x;
+  const int l = isqrt_floor(lm), m = lm - l * l - l;
+  const int L = 2 * l + 1;
+  const int n_lo = (int)((long)blockIdx.y * L / NSPLIT), n_hi = (int)((long)(blockIdx.y + 1) * L / NSPLIT);
+  const int fov = fo / CV, ngroup = (nbatch + IPT - 1) / IPT;
+  const int o = blockIdx.z * 256 + threadIdx.x;
+  if (o >= ngroup * fov || n_lo >= n_hi) return;
+  const int ip = o / fov, jv = o - ip * fov;
+  int item[IPT];
+#pragma unroll
+  for (int q = 0; q < IPT; ++q) item[q] = ip + q * ngroup < nbatch ? ip + q * ngroup : -1;    // item[0] always exists
+  const size_t zbase = (size_t)l * (4 * l * l - 1) / 3 + (size_t)(l + m) * L;
+  const bool stream = (size_t)nl * (4 * nl * nl - 1) / 3 * nbatch * fo * 8 >= s2cnn::STREAM_BYTES;     // z passes no cache: uniform
+  for (int k0 = 0; k0 < fi; k0 += KC) {
+    float2 xr[IPT][KC];
+#pragma unroll
+    for (int q = 0; q < IPT; ++q) {
+      const float2* xs = x + ((size_t)lm * nbatch + (item[q] < 0 ? ip : item[q])) * fi;
+#pragma unroll
+      for (int u = 0; u < KC; ++u) xr[q][u] = k0 + u < fi ? xs[k0 + u] : make_float2(0.f, 0.f);
+    }
+    for (int nn = n_lo; nn < n_hi; ++nn) {
+      const vec_t* ys = reinterpret_cast<const vec_t*>(y + ((size_t)(l * l + nn) * fi + k0) * fo) + jv;
+      vec_t* zs = reinterpret_cast<vec_t*>(z + (zbase + nn) * nbatch * fo) + jv;
+      vec_t acc[IPT];
+#pragma unroll
+      for (int q = 0; q < IPT; ++q) acc[q] = (k0 > 0 && item[q] >= 0) ? zs[(size_t)item[q] * fov] : CPack<CV>::zero();   // later feature passes accumulate
+#pragma unroll
+      for (int u = 0; u < KC; ++u) {
+        if (k0 + u < fi) {
+          const vec_t b = ys[(size_t)u * fov];
+#pragma unroll
+          for (int q = 0; q < IPT; ++q) CPack<CV>::scal_conj(xr[q][u], b, acc[q]);
+        }
+      }
+#pragma unroll
+      for (int q = 0; q < IPT; ++q)
+        if (item[q] >= 0) s2cnn::store_policy(acc[q], zs + (size_t)item[q] * fov, stream);
+    }
+  }
+}
 
 constexpr int IB = 4;   // grad x: batch items per workgroup
 
@@ -208,10 +234,15 @@ int check(const void* a, const void* b, const void* c, int nl, int nbatch, int f
 extern "C" int s2cnn_s2_mm_fwd(const float* x, const float* y, float* z, int nl, int nbatch, int f_in, int f_out, void* stream) {
   s2cnn::clear_stale_error();
   if (int rc = check(x, y, z, nl, nbatch, f_in, f_out)) return rc;
-  hipLaunchKernelGGL(s2_mm_fwd_kernel, dim3(nl * nl, NSPLIT, (unsigned)(((long)nbatch * f_out + 255) / 256)), dim3(256), 0,
-                     static_cast<hipStream_t>(stream),
-                     reinterpret_cast<const float2*>(x), reinterpret_cast<const float2*>(y), reinterpret_cast<float2*>(z),
-                     nl, nbatch, f_in, f_out);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const float2 *x2 = reinterpret_cast<const float2*>(x), *y2 = reinterpret_cast<const float2*>(y);
+  const long ngroup = (nbatch + IPT - 1) / IPT;
+  if (f_out % 2 == 0 && s2cnn::aligned16(y) && s2cnn::aligned16(z))
+    hipLaunchKernelGGL(s2_mm_fwd_kernel<2>, dim3(nl * nl, NSPLIT, (unsigned)((ngroup * (f_out / 2) + 255) / 256)), dim3(256), 0, st,
+                       x2, y2, reinterpret_cast<float2*>(z), nl, nbatch, f_in, f_out);
+  else
+    hipLaunchKernelGGL(s2_mm_fwd_kernel<1>, dim3(nl * nl, NSPLIT, (unsigned)((ngroup * f_out + 255) / 256)), dim3(256), 0, st,
+                       x2, y2, reinterpret_cast<float2*>(z), nl, nbatch, f_in, f_out);
   return s2cnn::launch_status();
 }
 
