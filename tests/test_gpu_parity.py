@@ -925,6 +925,28 @@ def test_so3_transforms_beyond_32_bit_offsets(hip, b, nz):
     torch.cuda.empty_cache()
 
 
+@pytest.mark.parametrize("b,nz", [(16, 2100), (10, 8400), (22, 800), (32, 260)])
+def test_so3_streamed_batches_equal_cached_ones(hip, b, nz):
+    """Signals of 256 MB or more are loaded and stored with the non-temporal hint (instantiations of their own of the
+    per-volume kernels); the hint changes no arithmetic: 200 volumes of such a batch get the bits they get in a batch of
+    their own, which takes the plain instantiations, in both directions and with a second tensor in the loads."""
+    n = 2 * b
+    assert nz * n ** 3 * 4 >= 256 << 20 and 200 * n ** 3 * 4 < 256 << 20
+    print(f"streamed batch b={b} nz={nz}", flush=True)
+    g = torch.Generator(device="cuda").manual_seed(7 * b)
+    x = torch.randn(nz, n, n, n, device="cuda", generator=g)
+    m = torch.randn(nz, n, n, n, device="cuda", generator=g)
+    for lo in (0, nz - 200):
+        sl = slice(lo, lo + 200)
+        r = PSO3.so3_rfft_real_basis(x)
+        assert torch.equal(r[:, sl], PSO3.so3_rfft_real_basis(x[sl].contiguous()))
+        rm = PSO3.so3_rfft_real_basis(x, mask=m)
+        assert torch.equal(rm[:, sl], PSO3.so3_rfft_real_basis(x[sl].contiguous(), mask=m[sl].contiguous()))
+        y = PSO3.so3_rifft_real_basis(r)
+        assert torch.equal(y[sl], PSO3.so3_rifft_real_basis(r[:, sl].contiguous()))
+        del r, rm, y
+
+
 def test_s2_transforms_and_integral_beyond_32_bit_offsets(hip):
     """The same property for the S^2 transforms ([33 000, 256, 256] -> b 32 and back) and for so3_integrate."""
     if torch.cuda.mem_get_info()[0] < 60 * 2 ** 30:
