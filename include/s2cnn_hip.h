@@ -101,9 +101,12 @@ int s2cnn_so3_mm_real_grady(const float *gz, const float *x, float *gy,
  *   dtab [nbeta, nspec(b)]               d^l_{mn}(beta_i), degree-major then m then n
  *   y    [nspec(b), ncols]               in the real basis of s2cnn_so3_spectrum_to_real
  * expand_real      : y from G              expand_real_grad : gG from gy (the adjoint)
+ * expand           : the same spectrum as complex pairs, y [nspec(b), ncols, 2]: the output of so3_rft (so3_ft.py:24);
+ *                    its adjoint is s2cnn_so3_spectrum_to_real followed by expand_real_grad
  * nbeta <= 4, ncols a multiple of 4, G / y / gy / gG 16-byte aligned.
  */
 int s2cnn_so3_rft_expand_real(const float *G, const float *dtab, float *y, int b, int nbeta, long ncols, void *stream);
+int s2cnn_so3_rft_expand(const float *G, const float *dtab, float *y, int b, int nbeta, long ncols, void *stream);
 int s2cnn_so3_rft_expand_real_grad(const float *gy, const float *dtab, float *gG, int b, int nbeta, long ncols, void *stream);
 
 /* ---- S^2 x S^2 -> SO(3) spectral outer products -------------------------------------

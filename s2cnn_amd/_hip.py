@@ -34,6 +34,7 @@ SIGNATURES = {
     "s2cnn_so3_spectrum_to_real": (_int, [_c_float_p, _c_float_p, _int, _long, _vp]),
     "s2cnn_so3_spectrum_to_complex": (_int, [_c_float_p, _c_float_p, _int, _long, _vp]),
     "s2cnn_so3_rft_expand_real": (_int, [_c_float_p, _c_float_p, _c_float_p, _int, _int, _long, _vp]),
+    "s2cnn_so3_rft_expand": (_int, [_c_float_p, _c_float_p, _c_float_p, _int, _int, _long, _vp]),
     "s2cnn_so3_rft_expand_real_grad": (_int, [_c_float_p, _c_float_p, _c_float_p, _int, _int, _long, _vp]),
     "s2cnn_s2_mm_fwd": (_int, _MM_SIG),
     "s2cnn_s2_mm_gradx": (_int, _MM_SIG),

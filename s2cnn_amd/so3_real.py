@@ -138,7 +138,7 @@ class _SO3RftRealFactorised(torch.autograd.Function):
     """x [ncols, n_grid] -> y [nspec, ncols]: plane coefficients per beta group by a batched GEMM, then the
     expansion over the degrees (s2cnn_so3_rft_expand_real) and its adjoint."""
     @staticmethod
-    def forward(ctx, x2, b, plan):
+    def forward(ctx, x2, b, plan, complex_out=False):
         idx, valid, E, dtab = plan[:4]
         _hip.require_gpu_f32(x2)
         ncols = x2.size(0)
@@ -146,15 +146,20 @@ class _SO3RftRealFactorised(torch.autograd.Function):
             xg = x2.t()[idx] * valid.unsqueeze(-1)                # [nbeta, P, ncols]
             G = torch.bmm(E.transpose(1, 2), xg).contiguous()    # [nbeta, R, ncols]
         _hip.require_gpu_f32(G)
-        y = x2.new_empty((b * (4 * b * b - 1) // 3, ncols))
-        _hip.call("s2cnn_so3_rft_expand_real", _hip.ptr(G), _hip.ptr(dtab), _hip.ptr(y), b, idx.size(0), ncols, _hip.stream_ptr())
-        ctx.plan, ctx.b, ctx.n_grid = plan, b, x2.size(1)
+        nspec = b * (4 * b * b - 1) // 3
+        y = x2.new_empty((nspec, ncols, 2) if complex_out else (nspec, ncols))
+        _hip.call("s2cnn_so3_rft_expand" if complex_out else "s2cnn_so3_rft_expand_real",
+                  _hip.ptr(G), _hip.ptr(dtab), _hip.ptr(y), b, idx.size(0), ncols, _hip.stream_ptr())
+        ctx.plan, ctx.b, ctx.n_grid, ctx.complex_out = plan, b, x2.size(1), complex_out
         return y
 
     @staticmethod
     def backward(ctx, gy):
         idx, valid, E, dtab, sel, idx_sel = ctx.plan
         gy = gy.contiguous()
+        if ctx.complex_out:      # the adjoint of the change of basis, then the adjoint of the real-basis expansion
+            _hip.require_gpu_f32(gy)
+            gy = _convert("s2cnn_so3_spectrum_to_real", gy, gy.shape[:-1])
         _hip.require_gpu_f32(gy)
         ncols = gy.size(1)
         gG = gy.new_empty((idx.size(0), E.size(2), ncols))
@@ -163,7 +168,26 @@ class _SO3RftRealFactorised(torch.autograd.Function):
             gxg = torch.bmm(E, gG)                                # [nbeta, P, ncols]
         gx = gy.new_zeros((ctx.n_grid, ncols))
         gx.index_add_(0, idx_sel, gxg.reshape(-1, ncols).index_select(0, sel))   # no boolean masks: they would sync with the host
-        return gx.t(), None, None
+        return gx.t(), None, None, None
+
+
+def so3_rft_complex(x, b, grid):
+    """
+    so3_rft (s2cnn/so3_ft.py:8-24) of a real kernel on a grid with few distinct beta values: the factorised transform with
+    its expansion written as complex pairs; None where the factorisation does not apply (the caller takes the dense product)
+    :param x: [..., beta_alpha_gamma]
+    :return: [l * m * n, ..., complex] or None
+    """
+    sz = x.size()
+    ncols = x.numel() // sz[-1]
+    if not (x.is_cuda and x.dtype == torch.float32 and ncols % 4 == 0):
+        return None
+    plan = _setup_so3_rft_plan(b, tuple(grid), x.device)
+    if plan is None:
+        return None
+    assert sz[-1] == len(grid)
+    out = _SO3RftRealFactorised.apply(x.reshape(-1, sz[-1]), b, plan, True)
+    return out.view(-1, *sz[:-1], 2)
 
 
 def so3_rft_real(x, b, grid):

@@ -894,6 +894,26 @@ def test_so3_rft_kernel_spectrum(hip, factorised, monkeypatch):
     close(kg.grad, ko.grad, "so3_rft grad")
 
 
+@pytest.mark.parametrize("shape", [(30, 50), (4, 3), (32, 33 * 4), (1, 1024), (2, 514)])
+def test_so3_rft_complex_expansion_equals_dense_product(hip, shape, monkeypatch):
+    """so3_rft of a real kernel (so3_ft.py:8-24): the factorised transform writes its expansion as complex pairs, a
+    thread's columns in two pairs half a tile (512 columns) apart; column counts that end inside either half of a tile,
+    against the dense product with the matrix of Wigner-D samples, values and gradient."""
+    b = 6
+    grid = s2cnn_amd.so3_near_identity_grid(n_alpha=6, n_beta=3, n_gamma=4)
+    k = rnd((*shape, len(grid)), 97).cuda()
+    w = rnd((O.nspec_so3(b), *shape, 2), 98).cuda()
+    out = {}
+    for factorised in (True, False):
+        monkeypatch.setattr(s2cnn_amd.so3_rft, "factorised", factorised)
+        kg = k.clone().requires_grad_()
+        y = s2cnn_amd.so3_rft(kg, b, grid)
+        (y * w).sum().backward()
+        out[factorised] = (y.detach(), kg.grad)
+    close(out[True][0], out[False][0].cpu(), f"so3_rft {shape}")
+    close(out[True][1], out[False][1].cpu(), f"so3_rft grad {shape}")
+
+
 @pytest.mark.parametrize("b,nz", [(32, 8200), (22, 25300)])
 def test_so3_transforms_beyond_32_bit_offsets(hip, b, nz):
     """Batches whose tensors pass 2^31 elements (and 2^33 bytes): the last volumes must get the bits they get in a batch of
