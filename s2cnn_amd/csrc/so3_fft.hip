@@ -414,8 +414,8 @@ int fused_analysis(FusedKind kind, const s2cnn::Input& in, const float* table, c
   if (kind == FUSED_64) {
     const int rounds = fused64::active_rounds(b_out), nparts = fused64::parts(nbatch);
     fused64::launch_analysis(b_out, st, in, Tf, rec, nbatch, nparts);
-    if (real_basis) hipLaunchKernelGGL(fused64::spectrum_scatter_real<>, dim3(tiles_r, rounds * 32), dim3(256), 0, st, rec, out, b_out, nbatch, nparts);
-    else hipLaunchKernelGGL(fused64::spectrum_scatter<>, dim3(tiles_c, rounds * 16), dim3(256), 0, st, rec, outc, b_out, nbatch, nparts);
+    if (real_basis) hipLaunchKernelGGL(fused64::spectrum_scatter_real<>, dim3(tiles_r, rounds * (fused64::THREADS / fused64::IT_TILE_R)), dim3(256), 0, st, rec, out, b_out, nbatch, nparts);
+    else hipLaunchKernelGGL(fused64::spectrum_scatter<>, dim3(tiles_c, rounds * (fused64::THREADS / fused64::IT_TILE)), dim3(256), 0, st, rec, outc, b_out, nbatch, nparts);
   } else {
     with_grid(kind, [&](auto g) { fused4r_analysis<decltype(g)>(in, Tf, rec, out, b_out, nbatch, real_basis, st); return 0; });
   }
@@ -445,8 +445,8 @@ int fused_synthesis(FusedKind kind, const float* xhat, const float* table, const
   float2* mom = reinterpret_cast<float2*>(moments);
   if (kind == FUSED_64) {
     const int rounds = fused64::active_rounds(nl);
-    if (real_basis) hipLaunchKernelGGL(fused64::spectrum_gather_real<>, dim3(tiles_r, rounds * 32), dim3(256), 0, st, xhat, rec, nl, nbatch);
-    else hipLaunchKernelGGL(fused64::spectrum_gather<>, dim3(tiles_c, rounds * 16), dim3(256), 0, st, xc, rec, nl, nbatch);
+    if (real_basis) hipLaunchKernelGGL(fused64::spectrum_gather_real<>, dim3(tiles_r, rounds * (fused64::THREADS / fused64::IT_TILE_R)), dim3(256), 0, st, xhat, rec, nl, nbatch);
+    else hipLaunchKernelGGL(fused64::spectrum_gather<>, dim3(tiles_c, rounds * (fused64::THREADS / fused64::IT_TILE)), dim3(256), 0, st, xc, rec, nl, nbatch);
     fused64::launch_synthesis(nl, st, rec, Tf, out, nbatch, bias, nfeature, relu, bits, mom, yref, params, fused64::parts(nbatch));
   } else {
     with_grid(kind, [&](auto g) {

@@ -642,10 +642,11 @@ __global__ __launch_bounds__(256) void spectrum_gather(const float2* __restrict_
 // and backwards (records hold twice the complex value, the table carries 1/2):
 //     2 A = (cc + ss, sc - cs)   2 C = s (cc - ss, -(cs + sc))   with cc, cs, sc, ss = R[+a,+n], R[+a,-n], R[-a,+n], R[-a,-n]
 //     a = 0: sqrt2 (cc, -cs), C unused     n = 0: sqrt2 (cc, sc), s sqrt2 (cc, -sc)     a = n = 0: (2 cc, 0)
-// Tiles of 32 volumes (128-byte pieces of a row) and 16 items; grid (ceil(nbatch / 32), rounds * G::THREADS / 16).
+// Tiles of ZR volumes (4 ZR-byte pieces of a row) and IT_TILE_R items; grid (ceil(nbatch / ZR), rounds * G::THREADS / IT_TILE_R).
 // ---------------------------------------------------------------------------------------------
-constexpr int ZR = 32;
-constexpr int IT_TILE_R = 16;
+constexpr int ZR = 32;                      // volumes per tile: 32 or 64
+constexpr int IT_TILE_R = 512 / ZR;         // items per tile: the tile holds 512 x 16 floats
+static_assert(IT_TILE_R * 16 <= 256 && 4 * ZR <= 256 && 256 % ZR == 0 && 16 % (256 / ZR) == 0, "thread mappings of the real-basis record passes");
 constexpr int VLD_R = 16 * ZR + 1;
 constexpr float SQRT2 = 1.41421356237309504880f, RSQRT2 = 0.70710678118654752440f;
 
@@ -678,11 +679,11 @@ __global__ __launch_bounds__(256) void spectrum_scatter_real(const float4* __res
   const int th = threadIdx.x;
   const long z0 = (long)blockIdx.x * ZR;
   const int it = blockIdx.y / TILES, t0 = (blockIdx.y % TILES) * IT_TILE_R;
-  rules[th] = row_rule(pack_item_info<G>(it * THREADS + t0 + (th >> 4)), th & 15, nl);   // 16 items x 16 row slots: one per thread
+  if (th < IT_TILE_R * 16) rules[th] = row_rule(pack_item_info<G>(it * THREADS + t0 + (th >> 4)), th & 15, nl);   // items x 16 row slots: one per thread
 #pragma unroll
   for (int r = 0; r < 8; ++r) {
     const int e = th + 256 * r;
-    const int item = e & 15, q = (e >> 4) & 3, zz = e >> 6;
+    const int item = e % IT_TILE_R, q = (e / IT_TILE_R) & 3, zz = e / (4 * IT_TILE_R);
     float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
     if (z0 + zz < nbatch)
       for (int p = 0; p < nparts; ++p) {
@@ -693,12 +694,13 @@ __global__ __launch_bounds__(256) void spectrum_scatter_real(const float4* __res
     d[0] = v.x; d[ZR] = v.y; d[2 * ZR] = v.z; d[3 * ZR] = v.w;
   }
   __syncthreads();
-  const int zz = th & 31, sub = th >> 5;       // 8 row slots at a time, 32 volumes (128 bytes of a row) each
+  constexpr int NSLOT = 256 / ZR;              // row slots at a time, ZR volumes (4 ZR bytes of a row) each
+  const int zz = th % ZR, sub = th / ZR;
   if (z0 + zz >= nbatch) return;
   float* dst = out + z0 + zz;
-  for (int p = 0; p < 2 * IT_TILE_R; ++p) {
-    const int item = p >> 1;
-    const RowRule r = rules[item * 16 + (p & 1) * 8 + sub];
+  for (int p = 0; p < (16 / NSLOT) * IT_TILE_R; ++p) {
+    const int item = p / (16 / NSLOT);
+    const RowRule r = rules[item * 16 + (p % (16 / NSLOT)) * NSLOT + sub];
     if (r.row < 0) continue;
     const float* v = vals + item * VLD_R + r.comp * ZR + zz;
     dst[(size_t)r.row * nbatch] = r.alpha * v[0] + r.beta * v[8 * ZR];
@@ -732,10 +734,10 @@ __global__ __launch_bounds__(256) void spectrum_gather_real(const float* __restr
   if (th < IT_TILE_R * 4) quads[th] = quad_rows(pack_item_info<G>(it * THREADS + t0 + (th >> 2)), th & 3, nl);
   __syncthreads();
   {
-    const int zz = th & 31, u = (th >> 5) & 3, sub = th >> 7;
+    const int zz = th % ZR, u = (th / ZR) & 3, sub = th / (4 * ZR);
     const long zc = z0 + zz < nbatch ? z0 + zz : nbatch - 1;
     const float* src = rr + zc;
-    for (int item = sub; item < IT_TILE_R; item += 2) {
+    for (int item = sub; item < IT_TILE_R; item += (256 / (4 * ZR) > 0 ? 256 / (4 * ZR) : 1)) {
       const QuadRows q = quads[item * 4 + u];
       float2 A = make_float2(0.f, 0.f), C = A;
       if (q.rows[0] >= 0) {
@@ -759,7 +761,7 @@ __global__ __launch_bounds__(256) void spectrum_gather_real(const float* __restr
 #pragma unroll
   for (int r = 0; r < 8; ++r) {
     const int e = th + 256 * r;
-    const int item = e & 15, q = (e >> 4) & 3, zz = e >> 6;
+    const int item = e % IT_TILE_R, q = (e / IT_TILE_R) & 3, zz = e / (4 * IT_TILE_R);
     if (z0 + zz >= nbatch) continue;
     const float* d = vals + item * VLD_R + (4 * q) * ZR + zz;
     rec[(size_t)(z0 + zz) * REC_F4 + (it * 4 + q) * THREADS + t0 + item] = make_float4(d[0], d[ZR], d[2 * ZR], d[3 * ZR]);
