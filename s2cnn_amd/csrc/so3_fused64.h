@@ -563,12 +563,13 @@ __global__ __launch_bounds__(256) void spectrum_scatter(const float4* __restrict
   for (int r = 0; r < 8; ++r) {
     const int e = th + 256 * r;
     const int item = e & 31, q = (e >> 5) & 3, zz = e >> 7;
-    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (z0 + zz < nbatch)
-      for (int p = 0; p < nparts; ++p) {
-        const float4 w = rec[((size_t)(z0 + zz) * nparts + p) * REC_F4 + (it * 4 + q) * THREADS + t0 + item];
-        v = make_float4(v.x + w.x, v.y + w.y, v.z + w.z, v.w + w.w);
-      }
+    // a volume past the end reads the last one (its values are not stored): no branch around the loads
+    const size_t zc = (size_t)(z0 + zz < nbatch ? z0 + zz : nbatch - 1);
+    float4 v = rec[zc * nparts * REC_F4 + (it * 4 + q) * THREADS + t0 + item];
+    for (int p = 1; p < nparts; ++p) {
+      const float4 w = rec[(zc * nparts + p) * REC_F4 + (it * 4 + q) * THREADS + t0 + item];
+      v = make_float4(v.x + w.x, v.y + w.y, v.z + w.z, v.w + w.w);
+    }
     float* d = vals + item * VLD + (4 * q) * ZT + zz;
     d[0] = v.x; d[ZT] = v.y; d[2 * ZT] = v.z; d[3 * ZT] = v.w;
   }
@@ -606,20 +607,28 @@ __global__ __launch_bounds__(256) void spectrum_gather(const float2* __restrict_
     const int zz = th & 15, u = (th >> 4) & 3, pm = (th >> 6) & 1, sub = th >> 7;
     const int comp = 4 * (pm * 2 + (u >> 1)) + 2 * (u & 1);
     const long zc = z0 + zz < nbatch ? z0 + zz : nbatch - 1;
-    for (int item = sub; item < IT_TILE; item += 2) {
-      const int inf = info[item];
+    // all loads of the thread's items first (an entry that does not exist reads row 0 instead and is not used), so that
+    // their latencies overlap; then the sums
+    constexpr int NI = IT_TILE / 2;
+    float2 v0[NI], v1[NI];
+    float sg[NI];                                               // 0: no such entry
+#pragma unroll
+    for (int k = 0; k < NI; ++k) {
+      const int inf = info[sub + 2 * k];
       const int r0 = row_index(inf, u, pm, nl);                 // (+-a, n)
-      float re = 0.f, im = 0.f;
-      if (r0 >= 0) {
-        const int a = (inf >> 8) & 0xff, n = (inf >> 16) & 0xff;
-        const int l = 4 * (inf & 0xff) + u;
-        const int r1 = lmn_index(l, pm ? a : -a, -n);           // the partner (-+a, -n); exists for every n
-        const float2 v0 = xh[(size_t)r0 * nbatch + zc], v1 = xh[(size_t)r1 * nbatch + zc];
-        const float sg = ((a - n) & 1) ? -1.f : 1.f;
-        re = v0.x + sg * v1.x; im = v0.y - sg * v1.y;
-      }
-      vals[item * VLD + comp * ZT + zz] = re;
-      vals[item * VLD + (comp + 1) * ZT + zz] = im;
+      const int a = (inf >> 8) & 0xff, n = (inf >> 16) & 0xff;
+      const int l = 4 * (inf & 0xff) + u;
+      const int r1 = r0 >= 0 ? lmn_index(l, pm ? a : -a, -n) : 0;   // the partner (-+a, -n); exists for every n
+      v0[k] = xh[(size_t)(r0 < 0 ? 0 : r0) * nbatch + zc];
+      v1[k] = xh[(size_t)r1 * nbatch + zc];
+      sg[k] = r0 < 0 ? 0.f : ((a - n) & 1) ? -1.f : 1.f;
+    }
+#pragma unroll
+    for (int k = 0; k < NI; ++k) {
+      const int item = sub + 2 * k;
+      const bool has = sg[k] != 0.f;
+      vals[item * VLD + comp * ZT + zz] = has ? v0[k].x + sg[k] * v1[k].x : 0.f;
+      vals[item * VLD + (comp + 1) * ZT + zz] = has ? v0[k].y - sg[k] * v1[k].y : 0.f;
     }
   }
   __syncthreads();
@@ -684,12 +693,14 @@ __global__ __launch_bounds__(256) void spectrum_scatter_real(const float4* __res
   for (int r = 0; r < 8; ++r) {
     const int e = th + 256 * r;
     const int item = e % IT_TILE_R, q = (e / IT_TILE_R) & 3, zz = e / (4 * IT_TILE_R);
-    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (z0 + zz < nbatch)
-      for (int p = 0; p < nparts; ++p) {
-        const float4 w = rec[((size_t)(z0 + zz) * nparts + p) * REC_F4 + (it * 4 + q) * THREADS + t0 + item];
-        v = make_float4(v.x + w.x, v.y + w.y, v.z + w.z, v.w + w.w);
-      }
+    // a volume past the end reads the last one (its values are not stored): no branch around the loads, so the eight of
+    // a thread are in flight together
+    const size_t zc = (size_t)(z0 + zz < nbatch ? z0 + zz : nbatch - 1);
+    float4 v = rec[zc * nparts * REC_F4 + (it * 4 + q) * THREADS + t0 + item];
+    for (int p = 1; p < nparts; ++p) {
+      const float4 w = rec[(zc * nparts + p) * REC_F4 + (it * 4 + q) * THREADS + t0 + item];
+      v = make_float4(v.x + w.x, v.y + w.y, v.z + w.z, v.w + w.w);
+    }
     float* d = vals + item * VLD_R + (4 * q) * ZR + zz;
     d[0] = v.x; d[ZR] = v.y; d[2 * ZR] = v.z; d[3 * ZR] = v.w;
   }
@@ -734,26 +745,37 @@ __global__ __launch_bounds__(256) void spectrum_gather_real(const float* __restr
   if (th < IT_TILE_R * 4) quads[th] = quad_rows(pack_item_info<G>(it * THREADS + t0 + (th >> 2)), th & 3, nl);
   __syncthreads();
   {
+    constexpr int NSUB = 256 / (4 * ZR), NI = IT_TILE_R / NSUB;      // items per thread
     const int zz = th % ZR, u = (th / ZR) & 3, sub = th / (4 * ZR);
     const long zc = z0 + zz < nbatch ? z0 + zz : nbatch - 1;
     const float* src = rr + zc;
-    for (int item = sub; item < IT_TILE_R; item += (256 / (4 * ZR) > 0 ? 256 / (4 * ZR) : 1)) {
-      const QuadRows q = quads[item * 4 + u];
+    // all loads of the thread's items first (a row that does not exist reads row 0 instead: a valid address, and the
+    // value is not used), so that their latencies overlap; then the combinations
+    QuadRows qs[NI];
+    float cc[NI], cs[NI], sc[NI], ss[NI];
+#pragma unroll
+    for (int k = 0; k < NI; ++k) {
+      qs[k] = quads[(sub + k * NSUB) * 4 + u];
+      const QuadRows& q = qs[k];
+      cc[k] = src[(size_t)(q.rows[0] < 0 ? 0 : q.rows[0]) * nbatch];
+      cs[k] = src[(size_t)(q.rows[1] < 0 ? 0 : q.rows[1]) * nbatch];
+      sc[k] = src[(size_t)(q.rows[2] < 0 ? 0 : q.rows[2]) * nbatch];
+      ss[k] = src[(size_t)(q.rows[3] < 0 ? 0 : q.rows[3]) * nbatch];
+    }
+#pragma unroll
+    for (int k = 0; k < NI; ++k) {
+      const QuadRows& q = qs[k];
       float2 A = make_float2(0.f, 0.f), C = A;
       if (q.rows[0] >= 0) {
         const bool hn = q.rows[1] >= 0, ha = q.rows[2] >= 0;
-        const float cc = src[(size_t)q.rows[0] * nbatch];
-        const float cs = hn ? src[(size_t)q.rows[1] * nbatch] : 0.f;
-        const float sc = ha ? src[(size_t)q.rows[2] * nbatch] : 0.f;
-        const float ss = q.rows[3] >= 0 ? src[(size_t)q.rows[3] * nbatch] : 0.f;
         const float s = q.s;
-        if (ha && hn) { A = make_float2(cc + ss, sc - cs); C = make_float2(s * (cc - ss), -s * (cs + sc)); }
-        else if (ha)  { A = make_float2(SQRT2 * cc, SQRT2 * sc); C = make_float2(s * SQRT2 * cc, -s * SQRT2 * sc); }
-        else if (hn)  { A = make_float2(SQRT2 * cc, -SQRT2 * cs); }
-        else          { A = make_float2(2.f * cc, 0.f); }
+        if (ha && hn) { A = make_float2(cc[k] + ss[k], sc[k] - cs[k]); C = make_float2(s * (cc[k] - ss[k]), -s * (cs[k] + sc[k])); }
+        else if (ha)  { A = make_float2(SQRT2 * cc[k], SQRT2 * sc[k]); C = make_float2(s * SQRT2 * cc[k], -s * SQRT2 * sc[k]); }
+        else if (hn)  { A = make_float2(SQRT2 * cc[k], -SQRT2 * cs[k]); }
+        else          { A = make_float2(2.f * cc[k], 0.f); }
       }
       const int comp = 4 * (u >> 1) + 2 * (u & 1);
-      float* d = vals + item * VLD_R + comp * ZR + zz;
+      float* d = vals + (sub + k * NSUB) * VLD_R + comp * ZR + zz;
       d[0] = A.x; d[ZR] = A.y; d[8 * ZR] = C.x; d[9 * ZR] = C.y;
     }
   }
